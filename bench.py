@@ -1,0 +1,198 @@
+"""Benchmark of the hot path on one MI355X.
+
+Headline: bf16 GEMM 4096^3 (f32 accumulation, bf16 output), TFLOP/s and fraction of the
+dense bf16 MFMA peak, with the CPU restatement of the reference's loop nest timed beside
+it.  `python bench.py --gpus 1 --steps K --warmup W` prints ONE JSON line.
+"""
+
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_FP8_TFLOPS = 5000.0
+PEAK_F32_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def time_region(fn, steps, warmup):
+    """(wall seconds, event seconds) for `steps` calls after `warmup` untimed calls."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return t1 - t0, start.elapsed_time(stop) * 1e-3
+
+
+def cpu_baseline_gemm_bf16(n: int, target_seconds: float = 12.0):
+    """The oracle's C loop nest (i-j-k, f32 multiply then add) on all host cores, on a
+    bounded slab of rows of the same 4096^3 problem."""
+    import numpy as np
+
+    lib_path = ROOT / "oracle" / "_build" / "libcpu_ref.so"
+    if not lib_path.is_file():
+        from lighthouse_amd import build as lh_build
+
+        lh_build.build_oracle()
+    lib = ctypes.CDLL(str(lib_path))
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+    rng = np.random.default_rng(0)
+    b = (rng.standard_normal((n, n)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+
+    def run(rows):
+        a = (rng.standard_normal((rows, n)).astype(np.float32).view(np.uint32) >> 16).astype(np.uint16)
+        out = np.zeros((rows, n), np.uint16)
+        t0 = time.perf_counter()
+        lib.lhref_matmul_bf16(out.ctypes.data_as(ctypes.c_void_p), a.ctypes.data_as(ctypes.c_void_p),
+                              b.ctypes.data_as(ctypes.c_void_p), None, ctypes.c_int64(rows), ctypes.c_int64(n),
+                              ctypes.c_int64(n), ctypes.c_uint32(0), ctypes.c_int(cores))
+        return time.perf_counter() - t0
+
+    probe_rows = cores
+    t = run(probe_rows)
+    rows = int(max(cores, min(n, probe_rows * target_seconds / max(t, 1e-6))))
+    rows = (rows // cores) * cores
+    t = run(rows)
+    flops = 2.0 * rows * n * n
+    return {
+        "value": flops / t / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+        "sample": f"{rows} of {n} rows of the same {n}^3 bf16 GEMM (i-j-k scalar loop nest, OpenMP over rows), {t:.1f} s",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (one MI355X per box); use --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    import torch
+
+    from lighthouse_amd import ops
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    n = 4096
+    g = torch.Generator(device="cuda").manual_seed(0xC0FFEE + 2)
+    a = torch.randn(n, n, device="cuda", generator=g).to(torch.bfloat16)
+    b = torch.randn(n, n, device="cuda", generator=g).to(torch.bfloat16)
+    bias = torch.randn(n, device="cuda", generator=g).to(torch.bfloat16)
+    out = torch.empty(n, n, device="cuda", dtype=torch.bfloat16)
+
+    flops = 2.0 * n * n * n
+    wall, ev = time_region(lambda: ops.gemm(a, b, out=out), args.steps, args.warmup)
+    value = flops * args.steps / wall / 1e12
+    achieved = flops * args.steps / ev / 1e12
+
+    extras = {}
+    if not args.no_extras:
+        def rate(fn, work, steps=20, warmup=5):
+            _, e = time_region(fn, steps, warmup)
+            return work * steps / e
+
+        extras["gemm_bf16_4096_bias_relu_tflops"] = rate(lambda: ops.gemm(a, b, bias, relu=True, out=out), flops) / 1e12
+        shape = (4, 16, 2048, 64)
+        q, k, v = (torch.randn(shape, device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
+        o = torch.empty_like(q)
+        aflops = 4.0 * 4 * 16 * 2048 * 2048 * 64
+        extras["attention_bf16_noncausal_tflops"] = rate(lambda: ops.attention(q, k, v, out=o), aflops) / 1e12
+        extras["attention_bf16_causal_tflops"] = rate(lambda: ops.attention(q, k, v, causal=True, out=o), aflops / 2) / 1e12
+        a32 = torch.rand(1024, 1024, device="cuda", generator=g) * 2 - 1
+        b32 = torch.rand(1024, 1024, device="cuda", generator=g) * 2 - 1
+        bias32 = torch.rand(1024, device="cuda", generator=g) * 2 - 1
+        o32 = torch.empty(1024, 1024, device="cuda")
+        extras["gemm_f32_1024_bias_relu_tflops"] = rate(lambda: ops.gemm(a32, b32, bias32, relu=True, out=o32), 2.0 * 1024**3) / 1e12
+        n8 = 8192
+        a8 = (torch.randn(n8, n8, device="cuda", generator=g)).clamp(-4, 4).to(torch.float8_e4m3fn)
+        b8 = (torch.randn(n8, n8, device="cuda", generator=g)).clamp(-4, 4).to(torch.float8_e4m3fn)
+        o8 = torch.empty(n8, n8, device="cuda", dtype=torch.bfloat16)
+        extras["gemm_fp8_8192_tflops"] = rate(lambda: ops.gemm_fp8(a8, b8, 0.01, 0.01, out=o8), 2.0 * n8**3, 10, 3) / 1e12
+        a8d = a8[:16].contiguous()
+        o8d = torch.empty(16, n8, device="cuda", dtype=torch.bfloat16)
+        dec_bytes = n8 * n8 + 16 * n8 + 16 * n8 * 2
+        extras["gemm_fp8_decode_16x8192x8192_gbs"] = rate(lambda: ops.gemm_fp8(a8d, b8, 0.01, 0.01, out=o8d), dec_bytes) / 1e9
+        del a8, b8, o8
+        M, C = 8192, 768
+        x = torch.randn(M, C, device="cuda", generator=g)
+        gam, bet = torch.ones(C, device="cuda"), torch.zeros(C, device="cuda")
+        y = torch.empty_like(x)
+        extras["layer_norm_f32_8192x768_gbs"] = rate(lambda: ops.layer_norm(x, gam, bet, out=y), 2.0 * M * C * 4) / 1e9
+        hdn = torch.randn(M, 4 * C, device="cuda", generator=g)
+        ho = torch.empty_like(hdn)
+        extras["gelu_f32_8192x3072_gbs"] = rate(lambda: ops.gelu_tanh(hdn, out=ho), 2.0 * M * 4 * C * 4) / 1e9
+        for dt, name in ((torch.float32, "f32"), (torch.bfloat16, "bf16")):
+            B, T, H = 8, 1024, 12
+            p = {}
+            for nm, shp in (("w_qkv", (C, 3 * C)), ("w_o", (C, C)), ("w_fc", (C, 4 * C)), ("w_proj", (4 * C, C))):
+                p[nm] = (torch.randn(shp, device="cuda", generator=g) * 0.02).to(dt)
+            for nm, ln in (("b_qkv", 3 * C), ("b_o", C), ("b_fc", 4 * C), ("b_proj", C)):
+                p[nm] = torch.zeros(ln, device="cuda", dtype=dt)
+            for nm in ("ln1_g", "ln2_g"):
+                p[nm] = torch.ones(C, device="cuda")
+            for nm in ("ln1_b", "ln2_b"):
+                p[nm] = torch.zeros(C, device="cuda")
+            xb = torch.randn(B, T, C, device="cuda", generator=g)
+            yb = torch.empty_like(xb)
+            ws = torch.empty(ops.nanogpt_block_workspace_bytes(B, T, C, dt), dtype=torch.uint8, device="cuda")
+            bflops = 128849018880.0  # causal-halved attention
+            extras[f"nanogpt_block_{name}_tflops"] = rate(lambda: ops.nanogpt_block(xb, p, H, out=yb, workspace=ws), bflops, 10, 3) / 1e12
+        extras = {k: round(float(v), 3) for k, v in extras.items()}
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline_gemm_bf16(n)
+
+    line = {
+        "metric": "GEMM & flash-attn TFLOP/s, % of MI355X MFMA peak; speedup vs host-CPU lh-run",
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "bf16 GEMM M=N=K=4096, A,B ~ N(0,1), f32 accumulation, bf16 output, no epilogue",
+                   "kernel": "gemm16_fast<bf16,256,256,2,4>"},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None},
+        "cpu_baseline": cpu,
+        "pct_of_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
+        "speedup_vs_cpu": (value / cpu["value"]) if cpu else None,
+        "other_workloads": extras,
+        "device": ops.device_info(),
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

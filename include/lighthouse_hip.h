@@ -1,0 +1,272 @@
+/*
+ * lighthouse_hip.h -- C ABI of liblighthouse_hip.so, the MI355X (gfx950) runtime
+ * target for Lighthouse's GPU payloads.
+ *
+ * Lighthouse's Runner JIT-compiles a payload module and calls the resulting native
+ * symbol through ctypes with "packed" arguments (lighthouse/execution/runner.py:
+ * 196-215): one void* per argument, each pointing at a pointer to a ranked memref
+ * descriptor {allocated, aligned, offset, sizes[rank], strides[rank]} with strides
+ * in ELEMENTS (lighthouse/utils/memref.py:5-44, lighthouse/utils/torch.py:41-66),
+ * or at an int64 for scalars.  This library offers the same calling convention for
+ * hand-written kernels instead of JIT'd code (the lh_hip_payload_* functions), plus
+ * the plain pointer/size form underneath (lh_hip_gemm, lh_hip_attention, ...), plus
+ * the device-memory helpers that replace the JIT'd gpu_alloc/gpu_dealloc/gpu_copy
+ * functions of lighthouse/ingress/mlir_gen/gpu_utils.py:6-45.
+ *
+ * Conventions
+ *  - Every function returns 0 on success or a negative lh_status; the message of the
+ *    last failure on the calling thread is lh_hip_last_error().  No C++ exception
+ *    crosses this boundary.  (The reference's JIT'd functions return void and cannot
+ *    report errors; the Python wrapper maps these codes to ValueError/RuntimeError as
+ *    lighthouse/execution/runner.py:113,175,179,191 do.)
+ *  - All data pointers are DEVICE pointers unless a parameter is named host_*.
+ *  - `stream` is a hipStream_t passed as void*; NULL selects the default stream.
+ *    Plain-pointer entry points only enqueue work; lh_hip_payload_* entry points
+ *    return after the work has finished, like a JIT'd payload call does.
+ *  - The caller owns every buffer; no entry point allocates results
+ *    (lighthouse/dialects/transform/transform_ext/ops/convert_func_results_to_args.py:14-24).
+ *  - Matrices are row-major; `ld*` are leading dimensions in elements.
+ */
+#ifndef LIGHTHOUSE_HIP_H
+#define LIGHTHOUSE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum lh_status {
+  LH_OK = 0,
+  LH_ERR_INVALID = -1,     /* bad shape / stride / flag / null pointer  -> ValueError   */
+  LH_ERR_UNSUPPORTED = -2, /* valid request with no kernel              -> ValueError   */
+  LH_ERR_RUNTIME = -3      /* HIP runtime failure                       -> RuntimeError */
+} lh_status;
+
+/* Element types (the MLIR element types the payload generators accept). */
+typedef enum lh_dtype {
+  LH_F32 = 0,
+  LH_BF16 = 1,
+  LH_F16 = 2,
+  LH_F8E4M3 = 3, /* OCP e4m3fn */
+  LH_F64 = 4,
+  LH_I8 = 5,
+  LH_I16 = 6,
+  LH_I32 = 7,
+  LH_I64 = 8
+} lh_dtype;
+
+/* GEMM epilogue / layout flags; names follow generate_gpu_matmul_payload's keyword
+ * arguments (lighthouse/ingress/mlir_gen/gpu_matmul_payload.py:5-36). */
+#define LH_GEMM_HAS_BIAS 1u
+#define LH_GEMM_HAS_RELU 2u
+#define LH_GEMM_ACCUMULATE_C 4u
+#define LH_GEMM_TRANSPOSE_A 8u
+#define LH_GEMM_TRANSPOSE_B 16u
+#define LH_GEMM_HAS_GELU 32u /* tanh-GELU on the accumulator instead of ReLU (nanoGPT MLP) */
+
+/* ---------------------------------------------------------------- runtime ---- */
+
+/* Message of the last error raised on this thread ("" if none). */
+const char* lh_hip_last_error(void);
+
+typedef struct lh_device_info {
+  char arch[64];            /* gcnArchName, e.g. "gfx950:sramecc+:xnack-" */
+  char name[128];
+  int32_t compute_units;
+  int32_t clock_khz;        /* engine clock */
+  int32_t memory_clock_khz;
+  int32_t memory_bus_bits;
+  int32_t lds_bytes_per_cu; /* max shared memory per block */
+  int32_t wavefront_size;
+  int64_t hbm_bytes;
+} lh_device_info;
+
+/* Replaces nothing in the reference; feeds the roofline report
+ * (the reference keeps vendor constants in lighthouse/schedule/xegpu/xegpu_specs.py:20-35). */
+int lh_hip_device_info(lh_device_info* out);
+int lh_hip_device_count(int32_t* out);
+
+/* Device memory: replace gpu_alloc_* / gpu_dealloc_* / gpu_copy_* helpers that
+ * GPUMemoryManager invokes (lighthouse/execution/memory_manager.py:97-151). */
+int lh_hip_alloc(void** dev_ptr, size_t bytes);
+int lh_hip_free(void* dev_ptr);
+int lh_hip_memcpy_h2d(void* dev_dst, const void* host_src, size_t bytes);
+int lh_hip_memcpy_d2h(void* host_dst, const void* dev_src, size_t bytes);
+int lh_hip_memcpy_d2d(void* dev_dst, const void* dev_src, size_t bytes);
+int lh_hip_memset(void* dev_ptr, int value, size_t bytes);
+int lh_hip_sync(void* stream);
+
+/* --------------------------------------------------- plain pointer kernels ---- */
+
+/*
+ * out[M,N] = epilogue(A.B) ; the matmul/MLP-layer payload, emit_mlp_layer
+ * (lighthouse/ingress/mlir_gen/gpu_mlp_payload.py:110-156): f32 accumulation from 0 or
+ * from `out` (ACCUMULATE_C), + bias[n] extended to f32, conversion to out_dtype, then
+ * ReLU.  A is [M,K] (or [K,M] with TRANSPOSE_A), B is [K,N] (or [N,K] with TRANSPOSE_B).
+ * ab_dtype in {F32, BF16, F16}; out_dtype F32 or ab_dtype; bias has out_dtype.
+ */
+int lh_hip_gemm(void* out, const void* a, const void* b, const void* bias, int64_t M, int64_t N, int64_t K,
+                int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype, int32_t out_dtype, uint32_t flags,
+                void* stream);
+
+/*
+ * fp8 GEMM of the benchmark's quantised configuration (no counterpart in the
+ * reference): out[M,N] = out_dtype( (Aq.Bq)_f32 * (scale_a*scale_b) ), Aq [M,K] and
+ * Bq [K,N] hold OCP e4m3fn codes; out_dtype BF16 or F32.
+ */
+int lh_hip_gemm_fp8(void* out, const void* a_q, const void* b_q, float scale_a, float scale_b, int64_t M,
+                    int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int32_t out_dtype, void* stream);
+
+/*
+ * Fused attention forward, the payload of generate_gpu_attention_payload
+ * (lighthouse/ingress/mlir_gen/gpu_attention_payload.py:12-132) in the fused form of
+ * ReplaceWithFusedAttentionOp (lighthouse/dialects/transform/transform_ext/ops/
+ * replace_with_fused_attention.py:332-455): O = softmax(Q K^T * scale [+ causal mask]) V
+ * with f32 running max / sum / accumulator.  Tensors are [Z,H,T,d] with element strides
+ * (sz, sh, st) per tensor and unit stride along d, so (T, H*d) projection buffers can be
+ * passed as strided views without a copy (examples/xegpu/nanoGPT_payload.py:198-217).
+ * dtype in {BF16, F16, F32}; d must be 64.
+ */
+typedef struct lh_strides3 {
+  int64_t z, h, t;
+} lh_strides3;
+int lh_hip_attention(void* out, const void* q, const void* k, const void* v, int64_t Z, int64_t H, int64_t T,
+                     int64_t d, lh_strides3 so, lh_strides3 sq, lh_strides3 sk, lh_strides3 sv, float scale,
+                     int32_t causal, int32_t dtype, void* stream);
+
+/*
+ * Row LayerNorm, emit_layer_norm_generics
+ * (lighthouse/ingress/mlir_gen/gpu_layer_norm_payload.py:15-87): x [M,N] (x_dtype F32 or
+ * BF16), gamma/beta [N] f32, statistics in f32, out [M,N] in out_dtype (F32 or BF16; BF16
+ * fuses the cast that follows every LayerNorm in examples/xegpu/nanoGPT_payload.py:299-317).
+ */
+int lh_hip_layer_norm(void* out, const void* x, const float* gamma, const float* beta, int64_t M, int64_t N,
+                      float eps, int32_t x_dtype, int32_t out_dtype, void* stream);
+
+/* Row softmax, generate_gpu_softmax_payload (lighthouse/ingress/mlir_gen/gpu_softmax_payload.py:11-65). */
+int lh_hip_softmax(void* out, const void* x, int64_t M, int64_t N, int32_t dtype, void* stream);
+
+/* Elementwise kernels of the nanoGPT payload builder (examples/xegpu/nanoGPT_payload.py:123-181). */
+/* out = tanh-GELU(x), n elements (no counterpart in the reference; benchmark's MLP activation). */
+int lh_hip_gelu_tanh(void* out, const void* x, int64_t n, int32_t dtype, void* stream);
+/* out[m,n] = x[m,n] + bias[n], optional ReLU (Builder.bias :141-163). x, bias, out share dtype. */
+int lh_hip_bias_act(void* out, const void* x, const void* bias, int64_t M, int64_t N, int32_t relu,
+                    int32_t dtype, void* stream);
+/* out = a + b (Builder.add :166-181). */
+int lh_hip_add(void* out, const void* a, const void* b, int64_t n, int32_t dtype, void* stream);
+/* out = convert(x) between F32/BF16/F16 (Builder.cast_f16 :123-138). */
+int lh_hip_cast(void* out, const void* x, int64_t n, int32_t src_dtype, int32_t dst_dtype, void* stream);
+
+/*
+ * One pre-LayerNorm GPT-2 block forward (op order of _emit_block_fused,
+ * examples/xegpu/nanoGPT_payload.py:299-317, with the benchmark's fused QKV projection,
+ * causal mask and tanh-GELU).  x, y: [B*T, C] f32 residual stream.  Weights are stored
+ * [in, out] in `dtype` (F32 or BF16) with biases in the same type; LayerNorm parameters
+ * are f32.  `workspace` must hold lh_hip_nanogpt_block_workspace_bytes(...) bytes.
+ */
+typedef struct lh_nanogpt_block_params {
+  const float* ln1_g;
+  const float* ln1_b;
+  const void* w_qkv; /* [C, 3C] */
+  const void* b_qkv; /* [3C]    */
+  const void* w_o;   /* [C, C]  */
+  const void* b_o;   /* [C]     */
+  const float* ln2_g;
+  const float* ln2_b;
+  const void* w_fc;   /* [C, 4C] */
+  const void* b_fc;   /* [4C]    */
+  const void* w_proj; /* [4C, C] */
+  const void* b_proj; /* [C]     */
+} lh_nanogpt_block_params;
+size_t lh_hip_nanogpt_block_workspace_bytes(int64_t B, int64_t T, int64_t C, int32_t dtype);
+int lh_hip_nanogpt_block(float* y, const float* x, const lh_nanogpt_block_params* p, int64_t B, int64_t T,
+                         int64_t C, int64_t n_head, float eps, int32_t dtype, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------- packed-argument payloads ---- */
+
+/*
+ * The calling convention of a JIT'd `payload` symbol: args[i] points at a pointer to the
+ * i-th memref descriptor, output first (lighthouse/ingress/mlir_gen/gpu_mlp_payload.py:44-48,
+ * gpu_attention_payload.py:48-50, gpu_layer_norm_payload.py:122-124).  A memref descriptor
+ * carries no element type (lighthouse/execution/memory_manager.py:112), so each payload
+ * takes an attribute struct with the types and options its generator was called with.
+ * These functions validate shapes and strides, run on the library's stream and return
+ * after the device finished.
+ */
+typedef struct lh_matmul_attrs {
+  int32_t ab_dtype;
+  int32_t out_dtype;
+  uint32_t flags; /* LH_GEMM_* */
+} lh_matmul_attrs;
+/* args: out[M,N], A, B[, bias[N]] */
+int lh_hip_payload_matmul(void** args, int32_t nargs, const lh_matmul_attrs* attrs);
+
+typedef struct lh_matmul_fp8_attrs {
+  int32_t out_dtype;
+  float scale_a;
+  float scale_b;
+} lh_matmul_fp8_attrs;
+/* args: out[M,N], Aq[M,K], Bq[K,N] */
+int lh_hip_payload_matmul_fp8(void** args, int32_t nargs, const lh_matmul_fp8_attrs* attrs);
+
+typedef struct lh_attention_attrs {
+  int32_t dtype;
+  int32_t causal;
+  float scale; /* <= 0 selects 1/sqrt(d) */
+} lh_attention_attrs;
+/* args: out, Q, K, V, each rank-4 [Z,H,T,d] */
+int lh_hip_payload_attention(void** args, int32_t nargs, const lh_attention_attrs* attrs);
+
+typedef struct lh_layer_norm_attrs {
+  int32_t x_dtype;
+  int32_t out_dtype;
+  float eps;
+} lh_layer_norm_attrs;
+/* args: out[M,N], x[M,N], gamma[N], beta[N] */
+int lh_hip_payload_layer_norm(void** args, int32_t nargs, const lh_layer_norm_attrs* attrs);
+
+typedef struct lh_elementwise_attrs {
+  int32_t kind;      /* lh_elementwise_kind */
+  int32_t dtype;     /* element type of the operands */
+  int32_t dst_dtype; /* CAST only */
+  int32_t relu;      /* BIAS only */
+} lh_elementwise_attrs;
+typedef enum lh_elementwise_kind {
+  LH_EW_SOFTMAX = 0, /* args: out[M,N], x[M,N] */
+  LH_EW_GELU = 1,    /* args: out, x */
+  LH_EW_BIAS = 2,    /* args: out[M,N], x[M,N], bias[N] */
+  LH_EW_ADD = 3,     /* args: out, a, b */
+  LH_EW_CAST = 4     /* args: out, x */
+} lh_elementwise_kind;
+int lh_hip_payload_elementwise(void** args, int32_t nargs, const lh_elementwise_attrs* attrs);
+
+typedef struct lh_nanogpt_block_attrs {
+  int32_t dtype; /* F32 or BF16: type of the weights, biases and matmul inputs */
+  int32_t n_head;
+  int32_t B;
+  int32_t T;
+  float eps;
+} lh_nanogpt_block_attrs;
+/* args: y[B*T,C], x[B*T,C], ln1_g[C], ln1_b[C], w_qkv[C,3C], b_qkv[3C], w_o[C,C], b_o[C], ln2_g[C], ln2_b[C],
+ * w_fc[C,4C], b_fc[4C], w_proj[4C,C], b_proj[C], workspace[bytes] (i8). */
+int lh_hip_payload_nanogpt_block(void** args, int32_t nargs, const lh_nanogpt_block_attrs* attrs);
+
+/*
+ * The `__benchmark` wrapper (WrapInBenchingFuncOp, lighthouse/dialects/transform/
+ * transform_ext/ops/wrap_in_benching_func.py:29-65): calls the payload `nwarmup` times
+ * untimed, then `nruns` times, each bracketed by a wall clock read with the device idle
+ * on both sides; the durations in seconds go to host_times[0..nruns).  `payload` selects
+ * the entry point by its name without the "lh_hip_payload_" prefix ("matmul",
+ * "matmul_fp8", "attention", "layer_norm", "elementwise", "nanogpt_block"); `attrs` is that entry point's
+ * attribute struct.
+ */
+int lh_hip_payload_benchmark(const char* payload, void** args, int32_t nargs, const void* attrs,
+                             double* host_times, int64_t nruns, int64_t nwarmup);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LIGHTHOUSE_HIP_H */

@@ -1,0 +1,365 @@
+// C ABI entry points: argument validation, the plain-pointer GEMM calls, the nanoGPT block,
+// and the packed-argument (memref descriptor) payload calls with their benchmark wrapper.
+#include <chrono>
+#include <cstring>
+
+#include "gemm_common.h"
+
+namespace lh {
+
+static int gemm_common_checks(const char* who, const void* out, const void* a, const void* b, const void* bias,
+                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, uint32_t flags) {
+  LH_REQUIRE(out && a && b, "%s: null pointer", who);
+  LH_REQUIRE(M > 0 && N > 0 && K > 0, "%s: empty problem M=%lld N=%lld K=%lld", who, (long long)M, (long long)N,
+             (long long)K);
+  LH_REQUIRE(M < (1ll << 31) && N < (1ll << 31) && K < (1ll << 31), "%s: dimension exceeds 2^31", who);
+  const bool ta = flags & LH_GEMM_TRANSPOSE_A, tb = flags & LH_GEMM_TRANSPOSE_B;
+  LH_REQUIRE(lda >= (ta ? M : K), "%s: lda %lld too small", who, (long long)lda);
+  LH_REQUIRE(ldb >= (tb ? K : N), "%s: ldb %lld too small", who, (long long)ldb);
+  LH_REQUIRE(ldc >= N, "%s: ldc %lld too small", who, (long long)ldc);
+  LH_REQUIRE(!(flags & LH_GEMM_HAS_BIAS) || bias != nullptr, "%s: HAS_BIAS set but bias is null", who);
+  LH_REQUIRE(!((flags & LH_GEMM_HAS_RELU) && (flags & LH_GEMM_HAS_GELU)), "%s: RELU and GELU are exclusive", who);
+  const uint32_t known = LH_GEMM_HAS_BIAS | LH_GEMM_HAS_RELU | LH_GEMM_ACCUMULATE_C | LH_GEMM_TRANSPOSE_A |
+                         LH_GEMM_TRANSPOSE_B | LH_GEMM_HAS_GELU;
+  LH_REQUIRE((flags & ~known) == 0, "%s: unknown flag bits 0x%x", who, flags & ~known);
+  return LH_OK;
+}
+
+// Internal form with a separate accumulator input and bias type.
+int gemm_run(void* out, const void* c, const void* a, const void* b, const void* bias, int64_t M, int64_t N, int64_t K,
+             int64_t lda, int64_t ldb, int64_t ldc, int ab_dtype, int out_dtype, int bias_dtype, uint32_t flags,
+             hipStream_t s) {
+  GemmArgs g;
+  g.out = out; g.c = c; g.a = a; g.b = b; g.bias = bias;
+  g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+  g.flags = flags; g.out_dt = out_dtype; g.bias_dt = bias_dtype; g.alpha = 1.0f;
+  if (ab_dtype == LH_F32) return gemm32(g, s);
+  return gemm16(g, ab_dtype, s);
+}
+
+// ---- memref descriptors ------------------------------------------------------------------
+struct Memref {
+  char* base;  // aligned pointer
+  int64_t offset;
+  const int64_t* sizes;
+  const int64_t* strides;
+  void* data(size_t elem) const { return base + offset * (int64_t)elem; }
+};
+
+// args[i] points at a pointer to {allocated, aligned, offset, sizes[rank], strides[rank]}.
+static bool get_memref(void** args, int i, Memref* m) {
+  if (args == nullptr || args[i] == nullptr) return false;
+  char* desc = *reinterpret_cast<char**>(args[i]);
+  if (desc == nullptr) return false;
+  void* aligned;
+  std::memcpy(&aligned, desc + sizeof(void*), sizeof(void*));
+  std::memcpy(&m->offset, desc + 2 * sizeof(void*), sizeof(int64_t));
+  m->base = reinterpret_cast<char*>(aligned);
+  m->sizes = reinterpret_cast<const int64_t*>(desc + 2 * sizeof(void*) + sizeof(int64_t));
+  return m->base != nullptr;
+}
+static bool get_memref(void** args, int i, int rank, Memref* m) {
+  if (!get_memref(args, i, m)) return false;
+  m->strides = m->sizes + rank;
+  return true;
+}
+
+static int sync_default() {
+  LH_HIP_CHECK(hipStreamSynchronize(nullptr));
+  return LH_OK;
+}
+
+}  // namespace lh
+
+using namespace lh;
+
+extern "C" {
+
+int lh_hip_gemm(void* out, const void* a, const void* b, const void* bias, int64_t M, int64_t N, int64_t K, int64_t lda,
+                int64_t ldb, int64_t ldc, int32_t ab_dtype, int32_t out_dtype, uint32_t flags, void* stream) {
+  int rc = gemm_common_checks("lh_hip_gemm", out, a, b, bias, M, N, K, lda, ldb, ldc, flags);
+  if (rc) return rc;
+  if (!(ab_dtype == LH_F32 || ab_dtype == LH_BF16 || ab_dtype == LH_F16))
+    return fail(LH_ERR_UNSUPPORTED, "lh_hip_gemm: unsupported A/B dtype %d", ab_dtype);
+  if (!(out_dtype == LH_F32 || (out_dtype == ab_dtype)))
+    return fail(LH_ERR_UNSUPPORTED, "lh_hip_gemm: out dtype %d must be f32 or the A/B dtype %d", out_dtype, ab_dtype);
+  return gemm_run(out, out, a, b, bias, M, N, K, lda, ldb, ldc, ab_dtype, out_dtype, out_dtype, flags,
+                  reinterpret_cast<hipStream_t>(stream));
+}
+
+int lh_hip_gemm_fp8(void* out, const void* a_q, const void* b_q, float scale_a, float scale_b, int64_t M, int64_t N,
+                    int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int32_t out_dtype, void* stream) {
+  int rc = gemm_common_checks("lh_hip_gemm_fp8", out, a_q, b_q, nullptr, M, N, K, lda, ldb, ldc, 0);
+  if (rc) return rc;
+  if (!(out_dtype == LH_BF16 || out_dtype == LH_F32))
+    return fail(LH_ERR_UNSUPPORTED, "lh_hip_gemm_fp8: out dtype %d must be bf16 or f32", out_dtype);
+  GemmArgs g;
+  g.out = out; g.c = out; g.a = a_q; g.b = b_q; g.bias = nullptr;
+  g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+  g.flags = 0; g.out_dt = out_dtype; g.bias_dt = out_dtype;
+  g.alpha = scale_a * scale_b;
+  return gemm8(g, reinterpret_cast<hipStream_t>(stream));
+}
+
+// ---- nanoGPT block -------------------------------------------------------------------------
+static size_t align256(size_t b) { return (b + 255) & ~(size_t)255; }
+
+size_t lh_hip_nanogpt_block_workspace_bytes(int64_t B, int64_t T, int64_t C, int32_t dtype) {
+  const size_t e = dtype_size(dtype);
+  const size_t rows = (size_t)B * T;
+  return align256(rows * C * e)         /* LayerNorm output */
+         + align256(rows * 3 * C * e)   /* q | k | v */
+         + align256(rows * C * e)       /* attention output */
+         + align256(rows * C * 4)       /* residual stream after attention */
+         + align256(rows * 4 * C * e);  /* MLP hidden */
+}
+
+int lh_hip_nanogpt_block(float* y, const float* x, const lh_nanogpt_block_params* p, int64_t B, int64_t T, int64_t C,
+                         int64_t n_head, float eps, int32_t dtype, void* workspace, size_t workspace_bytes,
+                         void* stream) {
+  LH_REQUIRE(y && x && p && workspace, "lh_hip_nanogpt_block: null pointer");
+  LH_REQUIRE(dtype == LH_F32 || dtype == LH_BF16, "lh_hip_nanogpt_block: dtype must be f32 or bf16");
+  LH_REQUIRE(B > 0 && T > 0 && C > 0 && n_head > 0 && C % n_head == 0, "lh_hip_nanogpt_block: bad shape");
+  LH_REQUIRE(workspace_bytes >= lh_hip_nanogpt_block_workspace_bytes(B, T, C, dtype),
+             "lh_hip_nanogpt_block: workspace too small (%zu bytes)", workspace_bytes);
+  LH_REQUIRE(aligned16(workspace), "lh_hip_nanogpt_block: workspace must be 16-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const size_t e = dtype_size(dtype);
+  const int64_t rows = B * T, hs = C / n_head;
+  char* w = reinterpret_cast<char*>(workspace);
+  void* ln = w;            w += align256((size_t)rows * C * e);
+  void* qkv = w;           w += align256((size_t)rows * 3 * C * e);
+  void* att = w;           w += align256((size_t)rows * C * e);
+  float* a = (float*)w;    w += align256((size_t)rows * C * 4);
+  void* hid = w;
+  int rc;
+  // ln1 = LN(x), rounded to the matmul input type.
+  if ((rc = lh_hip_layer_norm(ln, x, p->ln1_g, p->ln1_b, rows, C, eps, LH_F32, dtype, s))) return rc;
+  // qkv = ln1 Wqkv + bqkv
+  if ((rc = gemm_run(qkv, nullptr, ln, p->w_qkv, p->b_qkv, rows, 3 * C, C, C, 3 * C, 3 * C, dtype, dtype, dtype,
+                     LH_GEMM_HAS_BIAS, s)))
+    return rc;
+  // Causal attention on (B, H, T, hs) strided views of the (B*T, 3C) projection buffer.
+  {
+    lh_strides3 sqkv = {T * 3 * C, hs, 3 * C};
+    lh_strides3 so = {T * C, hs, C};
+    const char* qp = reinterpret_cast<const char*>(qkv);
+    if ((rc = lh_hip_attention(att, qp, qp + (size_t)C * e, qp + (size_t)2 * C * e, B, n_head, T, hs, so, sqkv, sqkv,
+                               sqkv, 0.0f, 1, dtype, s)))
+      return rc;
+  }
+  // a = x + att Wo + bo
+  if ((rc = gemm_run(a, x, att, p->w_o, p->b_o, rows, C, C, C, C, C, dtype, LH_F32, dtype,
+                     LH_GEMM_HAS_BIAS | LH_GEMM_ACCUMULATE_C, s)))
+    return rc;
+  // ln2 = LN(a)
+  if ((rc = lh_hip_layer_norm(ln, a, p->ln2_g, p->ln2_b, rows, C, eps, LH_F32, dtype, s))) return rc;
+  // h = gelu(ln2 W1 + b1)
+  if ((rc = gemm_run(hid, nullptr, ln, p->w_fc, p->b_fc, rows, 4 * C, C, C, 4 * C, 4 * C, dtype, dtype, dtype,
+                     LH_GEMM_HAS_BIAS | LH_GEMM_HAS_GELU, s)))
+    return rc;
+  // y = a + h W2 + b2
+  return gemm_run(y, a, hid, p->w_proj, p->b_proj, rows, C, 4 * C, 4 * C, C, C, dtype, LH_F32, dtype,
+                  LH_GEMM_HAS_BIAS | LH_GEMM_ACCUMULATE_C, s);
+}
+
+// ---- packed-argument payloads -------------------------------------------------------------
+
+int lh_hip_payload_matmul(void** args, int32_t nargs, const lh_matmul_attrs* at) {
+  LH_REQUIRE(args && at, "lh_hip_payload_matmul: null argument");
+  const bool has_bias = at->flags & LH_GEMM_HAS_BIAS;
+  LH_REQUIRE(nargs == (has_bias ? 4 : 3), "lh_hip_payload_matmul: expected %d arguments, got %d", has_bias ? 4 : 3,
+             nargs);
+  Memref o, a, b, bias;
+  LH_REQUIRE(get_memref(args, 0, 2, &o) && get_memref(args, 1, 2, &a) && get_memref(args, 2, 2, &b),
+             "lh_hip_payload_matmul: bad memref descriptor");
+  const bool ta = at->flags & LH_GEMM_TRANSPOSE_A, tb = at->flags & LH_GEMM_TRANSPOSE_B;
+  const int64_t M = o.sizes[0], N = o.sizes[1];
+  const int64_t K = ta ? a.sizes[0] : a.sizes[1];
+  LH_REQUIRE((ta ? a.sizes[1] : a.sizes[0]) == M, "lh_hip_payload_matmul: A shape does not match out rows");
+  LH_REQUIRE((tb ? b.sizes[1] : b.sizes[0]) == K && (tb ? b.sizes[0] : b.sizes[1]) == N,
+             "lh_hip_payload_matmul: B shape [%lld,%lld] does not match K=%lld N=%lld", (long long)b.sizes[0],
+             (long long)b.sizes[1], (long long)K, (long long)N);
+  LH_REQUIRE(o.strides[1] == 1 && a.strides[1] == 1 && b.strides[1] == 1,
+             "lh_hip_payload_matmul: innermost stride must be 1");
+  const void* bias_p = nullptr;
+  if (has_bias) {
+    LH_REQUIRE(get_memref(args, 3, 1, &bias), "lh_hip_payload_matmul: bad bias descriptor");
+    LH_REQUIRE(bias.sizes[0] == N && bias.strides[0] == 1, "lh_hip_payload_matmul: bias must be contiguous [N]");
+    bias_p = bias.data(dtype_size(at->out_dtype));
+  }
+  int rc = lh_hip_gemm(o.data(dtype_size(at->out_dtype)), a.data(dtype_size(at->ab_dtype)),
+                       b.data(dtype_size(at->ab_dtype)), bias_p, M, N, K, a.strides[0], b.strides[0], o.strides[0],
+                       at->ab_dtype, at->out_dtype, at->flags, nullptr);
+  if (rc) return rc;
+  return sync_default();
+}
+
+int lh_hip_payload_matmul_fp8(void** args, int32_t nargs, const lh_matmul_fp8_attrs* at) {
+  LH_REQUIRE(args && at, "lh_hip_payload_matmul_fp8: null argument");
+  LH_REQUIRE(nargs == 3, "lh_hip_payload_matmul_fp8: expected 3 arguments, got %d", nargs);
+  Memref o, a, b;
+  LH_REQUIRE(get_memref(args, 0, 2, &o) && get_memref(args, 1, 2, &a) && get_memref(args, 2, 2, &b),
+             "lh_hip_payload_matmul_fp8: bad memref descriptor");
+  const int64_t M = o.sizes[0], N = o.sizes[1], K = a.sizes[1];
+  LH_REQUIRE(a.sizes[0] == M && b.sizes[0] == K && b.sizes[1] == N, "lh_hip_payload_matmul_fp8: shape mismatch");
+  LH_REQUIRE(o.strides[1] == 1 && a.strides[1] == 1 && b.strides[1] == 1,
+             "lh_hip_payload_matmul_fp8: innermost stride must be 1");
+  int rc = lh_hip_gemm_fp8(o.data(dtype_size(at->out_dtype)), a.data(1), b.data(1), at->scale_a, at->scale_b, M, N, K,
+                           a.strides[0], b.strides[0], o.strides[0], at->out_dtype, nullptr);
+  if (rc) return rc;
+  return sync_default();
+}
+
+int lh_hip_payload_attention(void** args, int32_t nargs, const lh_attention_attrs* at) {
+  LH_REQUIRE(args && at, "lh_hip_payload_attention: null argument");
+  LH_REQUIRE(nargs == 4, "lh_hip_payload_attention: expected 4 arguments, got %d", nargs);
+  Memref m[4];
+  for (int i = 0; i < 4; ++i)
+    LH_REQUIRE(get_memref(args, i, 4, &m[i]), "lh_hip_payload_attention: bad memref descriptor %d", i);
+  for (int i = 1; i < 4; ++i)
+    for (int r = 0; r < 4; ++r)
+      LH_REQUIRE(m[i].sizes[r] == m[0].sizes[r], "lh_hip_payload_attention: shape mismatch in argument %d", i);
+  lh_strides3 st[4];
+  for (int i = 0; i < 4; ++i) {
+    LH_REQUIRE(m[i].strides[3] == 1, "lh_hip_payload_attention: innermost stride must be 1");
+    st[i] = lh_strides3{m[i].strides[0], m[i].strides[1], m[i].strides[2]};
+  }
+  const size_t e = dtype_size(at->dtype);
+  int rc = lh_hip_attention(m[0].data(e), m[1].data(e), m[2].data(e), m[3].data(e), m[0].sizes[0], m[0].sizes[1],
+                            m[0].sizes[2], m[0].sizes[3], st[0], st[1], st[2], st[3], at->scale, at->causal, at->dtype,
+                            nullptr);
+  if (rc) return rc;
+  return sync_default();
+}
+
+int lh_hip_payload_layer_norm(void** args, int32_t nargs, const lh_layer_norm_attrs* at) {
+  LH_REQUIRE(args && at, "lh_hip_payload_layer_norm: null argument");
+  LH_REQUIRE(nargs == 4, "lh_hip_payload_layer_norm: expected 4 arguments, got %d", nargs);
+  Memref o, x, g, b;
+  LH_REQUIRE(get_memref(args, 0, 2, &o) && get_memref(args, 1, 2, &x) && get_memref(args, 2, 1, &g) &&
+                 get_memref(args, 3, 1, &b),
+             "lh_hip_payload_layer_norm: bad memref descriptor");
+  const int64_t M = o.sizes[0], N = o.sizes[1];
+  LH_REQUIRE(x.sizes[0] == M && x.sizes[1] == N && g.sizes[0] == N && b.sizes[0] == N,
+             "lh_hip_payload_layer_norm: shape mismatch");
+  LH_REQUIRE(o.strides[1] == 1 && x.strides[1] == 1 && o.strides[0] == N && x.strides[0] == N && g.strides[0] == 1 &&
+                 b.strides[0] == 1,
+             "lh_hip_payload_layer_norm: buffers must be contiguous");
+  int rc = lh_hip_layer_norm(o.data(dtype_size(at->out_dtype)), x.data(dtype_size(at->x_dtype)),
+                             reinterpret_cast<const float*>(g.data(4)), reinterpret_cast<const float*>(b.data(4)), M, N,
+                             at->eps, at->x_dtype, at->out_dtype, nullptr);
+  if (rc) return rc;
+  return sync_default();
+}
+
+int lh_hip_payload_elementwise(void** args, int32_t nargs, const lh_elementwise_attrs* at) {
+  LH_REQUIRE(args && at, "lh_hip_payload_elementwise: null argument");
+  const int want = (at->kind == LH_EW_BIAS || at->kind == LH_EW_ADD) ? 3 : 2;
+  LH_REQUIRE(nargs == want, "lh_hip_payload_elementwise: expected %d arguments, got %d", want, nargs);
+  Memref o, x, y;
+  LH_REQUIRE(get_memref(args, 0, 2, &o) && get_memref(args, 1, 2, &x), "lh_hip_payload_elementwise: bad descriptor");
+  const int64_t M = o.sizes[0], N = o.sizes[1];
+  LH_REQUIRE(x.sizes[0] == M && x.sizes[1] == N, "lh_hip_payload_elementwise: shape mismatch");
+  LH_REQUIRE(o.strides[1] == 1 && x.strides[1] == 1 && o.strides[0] == N && x.strides[0] == N,
+             "lh_hip_payload_elementwise: buffers must be contiguous");
+  const size_t e = dtype_size(at->dtype);
+  int rc;
+  switch (at->kind) {
+    case LH_EW_SOFTMAX: rc = lh_hip_softmax(o.data(e), x.data(e), M, N, at->dtype, nullptr); break;
+    case LH_EW_GELU: rc = lh_hip_gelu_tanh(o.data(e), x.data(e), M * N, at->dtype, nullptr); break;
+    case LH_EW_BIAS:
+      LH_REQUIRE(get_memref(args, 2, 1, &y) && y.sizes[0] == N && y.strides[0] == 1,
+                 "lh_hip_payload_elementwise: bias must be contiguous [N]");
+      rc = lh_hip_bias_act(o.data(e), x.data(e), y.data(e), M, N, at->relu, at->dtype, nullptr);
+      break;
+    case LH_EW_ADD:
+      LH_REQUIRE(get_memref(args, 2, 2, &y) && y.sizes[0] == M && y.sizes[1] == N && y.strides[1] == 1 &&
+                     y.strides[0] == N,
+                 "lh_hip_payload_elementwise: second operand must be contiguous [M,N]");
+      rc = lh_hip_add(o.data(e), x.data(e), y.data(e), M * N, at->dtype, nullptr);
+      break;
+    case LH_EW_CAST:
+      rc = lh_hip_cast(o.data(dtype_size(at->dst_dtype)), x.data(e), M * N, at->dtype, at->dst_dtype, nullptr);
+      break;
+    default: return fail(LH_ERR_INVALID, "lh_hip_payload_elementwise: unknown kind %d", at->kind);
+  }
+  if (rc) return rc;
+  return sync_default();
+}
+
+int lh_hip_payload_nanogpt_block(void** args, int32_t nargs, const lh_nanogpt_block_attrs* at) {
+  LH_REQUIRE(args && at, "lh_hip_payload_nanogpt_block: null argument");
+  LH_REQUIRE(nargs == 15, "lh_hip_payload_nanogpt_block: expected 15 arguments, got %d", nargs);
+  Memref y, x, v[12], ws;
+  LH_REQUIRE(get_memref(args, 0, 2, &y) && get_memref(args, 1, 2, &x) && get_memref(args, 14, 1, &ws),
+             "lh_hip_payload_nanogpt_block: bad memref descriptor");
+  static const int ranks[12] = {1, 1, 2, 1, 2, 1, 1, 1, 2, 1, 2, 1};
+  for (int i = 0; i < 12; ++i)
+    LH_REQUIRE(get_memref(args, 2 + i, ranks[i], &v[i]), "lh_hip_payload_nanogpt_block: bad descriptor %d", 2 + i);
+  const int64_t rows = y.sizes[0], C = y.sizes[1];
+  LH_REQUIRE(rows == (int64_t)at->B * at->T && x.sizes[0] == rows && x.sizes[1] == C,
+             "lh_hip_payload_nanogpt_block: x / y shape does not match B*T x C");
+  LH_REQUIRE(y.strides[0] == C && y.strides[1] == 1 && x.strides[0] == C && x.strides[1] == 1,
+             "lh_hip_payload_nanogpt_block: x and y must be contiguous");
+  const int64_t want[12][2] = {{C, 0}, {C, 0}, {C, 3 * C}, {3 * C, 0}, {C, C}, {C, 0},
+                               {C, 0}, {C, 0}, {C, 4 * C}, {4 * C, 0}, {4 * C, C}, {C, 0}};
+  for (int i = 0; i < 12; ++i) {
+    LH_REQUIRE(v[i].sizes[0] == want[i][0] && (ranks[i] == 1 || v[i].sizes[1] == want[i][1]),
+               "lh_hip_payload_nanogpt_block: parameter %d has the wrong shape", 2 + i);
+    LH_REQUIRE(v[i].strides[ranks[i] - 1] == 1 && (ranks[i] == 1 || v[i].strides[0] == v[i].sizes[1]),
+               "lh_hip_payload_nanogpt_block: parameter %d must be contiguous", 2 + i);
+  }
+  const size_t e = dtype_size(at->dtype);
+  lh_nanogpt_block_params p;
+  p.ln1_g = (const float*)v[0].data(4); p.ln1_b = (const float*)v[1].data(4);
+  p.w_qkv = v[2].data(e); p.b_qkv = v[3].data(e);
+  p.w_o = v[4].data(e); p.b_o = v[5].data(e);
+  p.ln2_g = (const float*)v[6].data(4); p.ln2_b = (const float*)v[7].data(4);
+  p.w_fc = v[8].data(e); p.b_fc = v[9].data(e);
+  p.w_proj = v[10].data(e); p.b_proj = v[11].data(e);
+  int rc = lh_hip_nanogpt_block((float*)y.data(4), (const float*)x.data(4), &p, at->B, at->T, C, at->n_head, at->eps,
+                                at->dtype, ws.data(1), (size_t)ws.sizes[0], nullptr);
+  if (rc) return rc;
+  return sync_default();
+}
+
+int lh_hip_payload_benchmark(const char* payload, void** args, int32_t nargs, const void* attrs, double* host_times,
+                             int64_t nruns, int64_t nwarmup) {
+  LH_REQUIRE(payload && args && attrs, "lh_hip_payload_benchmark: null argument");
+  LH_REQUIRE(nruns >= 0 && nwarmup >= 0 && (nruns == 0 || host_times), "lh_hip_payload_benchmark: bad run counts");
+  int kind;
+  if (!std::strcmp(payload, "matmul")) kind = 0;
+  else if (!std::strcmp(payload, "matmul_fp8")) kind = 1;
+  else if (!std::strcmp(payload, "attention")) kind = 2;
+  else if (!std::strcmp(payload, "layer_norm")) kind = 3;
+  else if (!std::strcmp(payload, "elementwise")) kind = 4;
+  else if (!std::strcmp(payload, "nanogpt_block")) kind = 5;
+  else return fail(LH_ERR_INVALID, "lh_hip_payload_benchmark: unknown payload '%s'", payload);
+  auto call = [&]() -> int {
+    switch (kind) {
+      case 0: return lh_hip_payload_matmul(args, nargs, reinterpret_cast<const lh_matmul_attrs*>(attrs));
+      case 1: return lh_hip_payload_matmul_fp8(args, nargs, reinterpret_cast<const lh_matmul_fp8_attrs*>(attrs));
+      case 2: return lh_hip_payload_attention(args, nargs, reinterpret_cast<const lh_attention_attrs*>(attrs));
+      case 3: return lh_hip_payload_layer_norm(args, nargs, reinterpret_cast<const lh_layer_norm_attrs*>(attrs));
+      case 4: return lh_hip_payload_elementwise(args, nargs, reinterpret_cast<const lh_elementwise_attrs*>(attrs));
+      default: return lh_hip_payload_nanogpt_block(args, nargs, reinterpret_cast<const lh_nanogpt_block_attrs*>(attrs));
+    }
+  };
+  for (int64_t i = 0; i < nwarmup; ++i) {
+    int rc = call();
+    if (rc) return rc;
+  }
+  for (int64_t i = 0; i < nruns; ++i) {
+    auto t0 = std::chrono::steady_clock::now();
+    int rc = call();
+    auto t1 = std::chrono::steady_clock::now();
+    if (rc) return rc;
+    host_times[i] = std::chrono::duration<double>(t1 - t0).count();
+  }
+  return LH_OK;
+}
+
+}  // extern "C"

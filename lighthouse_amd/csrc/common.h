@@ -1,0 +1,149 @@
+// Shared declarations for the gfx950 kernels behind liblighthouse_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "lighthouse_hip.h"
+
+namespace lh {
+
+// ---- error reporting -------------------------------------------------------
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+
+#define LH_HIP_CHECK(expr)                                                                   \
+  do {                                                                                       \
+    hipError_t _e = (expr);                                                                  \
+    if (_e != hipSuccess)                                                                    \
+      return ::lh::fail(LH_ERR_RUNTIME, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), \
+                        __FILE__, __LINE__);                                                 \
+  } while (0)
+
+#define LH_REQUIRE(cond, ...)                                 \
+  do {                                                        \
+    if (!(cond)) return ::lh::fail(LH_ERR_INVALID, __VA_ARGS__); \
+  } while (0)
+
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(LH_ERR_RUNTIME, "launch of %s failed: %s", what, hipGetErrorString(e));
+  return LH_OK;
+}
+
+inline size_t dtype_size(int32_t dt) {
+  switch (dt) {
+    case LH_F32: return 4;
+    case LH_BF16: return 2;
+    case LH_F16: return 2;
+    case LH_F8E4M3: return 1;
+    case LH_F64: return 8;
+    case LH_I8: return 1;
+    case LH_I16: return 2;
+    case LH_I32: return 4;
+    case LH_I64: return 8;
+    default: return 0;
+  }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ---- vector types ------------------------------------------------------------
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+typedef int32_t i32x8 __attribute__((ext_vector_type(8)));
+
+// ---- scalar conversions (device) ----------------------------------------------
+// float -> bfloat16 bits, round to nearest even, quiet NaN (arith.truncf semantics).
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  uint32_t r = u + 0x7fffu + ((u >> 16) & 1u);
+  r = (f != f) ? (u | 0x00400000u) : r;
+  return (uint16_t)(r >> 16);
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
+  return __builtin_bit_cast(float, (uint32_t)h << 16);
+}
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+  _Float16 h = (_Float16)f;
+  return __builtin_bit_cast(uint16_t, h);
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t b) {
+  return (float)__builtin_bit_cast(_Float16, b);
+}
+
+// Pack two floats into one dword of two 16-bit values (lo = a, hi = b).
+template <int DT>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  if constexpr (DT == LH_BF16) {
+    return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+  } else {
+    return (uint32_t)f32_to_f16_bits(a) | ((uint32_t)f32_to_f16_bits(b) << 16);
+  }
+}
+template <int DT>
+__device__ __forceinline__ float unpack_lo(uint32_t w) {
+  if constexpr (DT == LH_BF16) return __builtin_bit_cast(float, w << 16);
+  else return f16_bits_to_f32((uint16_t)(w & 0xffffu));
+}
+template <int DT>
+__device__ __forceinline__ float unpack_hi(uint32_t w) {
+  if constexpr (DT == LH_BF16) return __builtin_bit_cast(float, w & 0xffff0000u);
+  else return f16_bits_to_f32((uint16_t)(w >> 16));
+}
+
+// Load / store one element of a run-time-typed buffer as float.
+template <int DT>
+__device__ __forceinline__ float load_as_f32(const void* p, int64_t i) {
+  if constexpr (DT == LH_F32) return reinterpret_cast<const float*>(p)[i];
+  else if constexpr (DT == LH_BF16) return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+  else return f16_bits_to_f32(reinterpret_cast<const uint16_t*>(p)[i]);
+}
+template <int DT>
+__device__ __forceinline__ void store_from_f32(void* p, int64_t i, float v) {
+  if constexpr (DT == LH_F32) reinterpret_cast<float*>(p)[i] = v;
+  else if constexpr (DT == LH_BF16) reinterpret_cast<uint16_t*>(p)[i] = f32_to_bf16_bits(v);
+  else reinterpret_cast<uint16_t*>(p)[i] = f32_to_f16_bits(v);
+}
+// Round a float to the named type and back (the rounding point of a conversion).
+template <int DT>
+__device__ __forceinline__ float round_through(float v) {
+  if constexpr (DT == LH_F32) return v;
+  else if constexpr (DT == LH_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(v));
+  else return f16_bits_to_f32(f32_to_f16_bits(v));
+}
+
+// arith.maximumf(x, 0): NaN propagates (lighthouse/ingress/mlir_gen/named.py:28-32).
+__device__ __forceinline__ float relu_nan(float v) { return (v != v) ? v : fmaxf(v, 0.0f); }
+
+// tanh-GELU, 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))), via one exp:
+// 0.5 (1 + tanh(u)) = 1 / (1 + exp(-2u)).
+__device__ __forceinline__ float gelu_tanh(float x) {
+  const float k = 0.7978845608028654f;
+  float u = k * (x + 0.044715f * x * x * x);
+  float e = __expf(-2.0f * u);
+  return x / (1.0f + e);
+}
+
+// Workgroup id -> tile id so that the workgroups resident on one XCD (ids congruent
+// modulo 8 are dispatched to the same XCD) cover a compact patch of tiles and share
+// their operand panels through that XCD's L2.
+__device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
+  const int nx = 8;
+  if (nblocks % nx != 0) return bid;
+  int per = nblocks / nx;
+  return (bid % nx) * per + bid / nx;
+}
+
+hipStream_t default_stream();
+
+}  // namespace lh

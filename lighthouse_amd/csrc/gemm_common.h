@@ -1,0 +1,90 @@
+// Argument block and register epilogue shared by the GEMM kernels.
+#pragma once
+
+#include "common.h"
+
+namespace lh {
+
+struct GemmArgs {
+  void* out;
+  const void* c;  // accumulator input for ACCUMULATE_C (out_dt typed; may alias out)
+  const void* a;
+  const void* b;
+  const void* bias;
+  int M, N, K;
+  int64_t lda, ldb, ldc;
+  uint32_t flags;
+  int out_dt;
+  int bias_dt;  // element type of bias
+  float alpha;  // accumulator scale applied first (1 for the unquantised payloads)
+};
+
+// Epilogue for 4 consecutive columns of one row.
+template <int DT>
+__device__ __forceinline__ void epilogue4(const GemmArgs& g, int m, int n, float v0, float v1, float v2, float v3) {
+  float v[4] = {v0 * g.alpha, v1 * g.alpha, v2 * g.alpha, v3 * g.alpha};
+  const int64_t off = (int64_t)m * g.ldc + n;
+  if (g.flags & LH_GEMM_ACCUMULATE_C) {
+    if (g.out_dt == LH_F32) {
+      f32x4 c = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.c) + off);
+      v[0] += c[0]; v[1] += c[1]; v[2] += c[2]; v[3] += c[3];
+    } else {
+      u32x2 c = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.c) + off);
+      v[0] += unpack_lo<DT>(c[0]); v[1] += unpack_hi<DT>(c[0]);
+      v[2] += unpack_lo<DT>(c[1]); v[3] += unpack_hi<DT>(c[1]);
+    }
+  }
+  if (g.flags & LH_GEMM_HAS_BIAS) {
+    if (g.bias_dt == LH_F32) {
+      f32x4 bb = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.bias) + n);
+      v[0] += bb[0]; v[1] += bb[1]; v[2] += bb[2]; v[3] += bb[3];
+    } else {
+      u32x2 bb = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.bias) + n);
+      v[0] += unpack_lo<DT>(bb[0]); v[1] += unpack_hi<DT>(bb[0]);
+      v[2] += unpack_lo<DT>(bb[1]); v[3] += unpack_hi<DT>(bb[1]);
+    }
+  }
+  if (g.flags & LH_GEMM_HAS_GELU) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
+  }
+  const bool relu = (g.flags & LH_GEMM_HAS_RELU) != 0;
+  if (g.out_dt == LH_F32) {
+    if (relu) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
+    }
+    f32x4 o = {v[0], v[1], v[2], v[3]};
+    *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(g.out) + off) = o;
+  } else {
+    if (relu) {
+      // ReLU is applied after the conversion (gpu_mlp_payload.py:147-151); max(x,0) and
+      // rounding commute for every input (0 is representable and rounding is monotone).
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
+    }
+    u32x2 o = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+    *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(g.out) + off) = o;
+  }
+}
+
+// One output element, any alignment (edge tiles and the generic kernels).
+template <int DT>
+__device__ __forceinline__ void epilogue1(const GemmArgs& g, int m, int n, float x) {
+  const int64_t off = (int64_t)m * g.ldc + n;
+  x *= g.alpha;
+  if (g.flags & LH_GEMM_ACCUMULATE_C)
+    x += (g.out_dt == LH_F32) ? reinterpret_cast<const float*>(g.c)[off] : load_as_f32<DT>(g.c, off);
+  if (g.flags & LH_GEMM_HAS_BIAS)
+    x += (g.bias_dt == LH_F32) ? reinterpret_cast<const float*>(g.bias)[n] : load_as_f32<DT>(g.bias, n);
+  if (g.flags & LH_GEMM_HAS_GELU) x = gelu_tanh(x);
+  if (g.flags & LH_GEMM_HAS_RELU) x = relu_nan(x);
+  if (g.out_dt == LH_F32) reinterpret_cast<float*>(g.out)[off] = x;
+  else store_from_f32<DT>(g.out, off, x);
+}
+
+int gemm16(const GemmArgs& g, int ab_dtype, hipStream_t s);
+int gemm32(const GemmArgs& g, hipStream_t s);
+int gemm8(const GemmArgs& g, hipStream_t s);
+
+}  // namespace lh

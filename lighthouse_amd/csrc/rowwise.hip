@@ -1,0 +1,297 @@
+// Bandwidth-bound row and elementwise kernels: LayerNorm, softmax, tanh-GELU, bias(+ReLU),
+// residual add, conversion.  One pass over HBM each: a row lives in registers between the
+// reduction passes, every global access is 8 or 16 bytes per lane and contiguous across the
+// wave.
+#include "common.h"
+
+namespace lh {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// 4 consecutive elements as floats.
+template <int DT>
+__device__ __forceinline__ f32x4 load4(const void* p, int64_t i) {
+  if constexpr (DT == LH_F32) {
+    return *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(p) + i);
+  } else {
+    u32x2 w = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(p) + i);
+    return f32x4{unpack_lo<DT>(w[0]), unpack_hi<DT>(w[0]), unpack_lo<DT>(w[1]), unpack_hi<DT>(w[1])};
+  }
+}
+template <int DT>
+__device__ __forceinline__ void store4(void* p, int64_t i, f32x4 v) {
+  if constexpr (DT == LH_F32) {
+    *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(p) + i) = v;
+  } else {
+    u32x2 w = {pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+    *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(p) + i) = w;
+  }
+}
+
+// LayerNorm, one wave per row, N = VPL * 256 exactly; the three loop nests of
+// emit_layer_norm_generics (lighthouse/ingress/mlir_gen/gpu_layer_norm_payload.py:15-87)
+// evaluated on the register-resident row: sum -> mean = sum * (1/N); sum of squared centred
+// values -> var = that * (1/N); (x - mean) * rsqrt(var + eps) * gamma + beta.
+template <int XDT, int ODT, int VPL>
+__global__ void __launch_bounds__(256) layer_norm_vec(void* out, const void* x, const float* gamma, const float* beta,
+                                                      int M, int N, float eps, float inv_n) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;
+  const int64_t base = (int64_t)row * N;
+  f32x4 v[VPL];
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    v[i] = load4<XDT>(x, base + (i * 64 + lane) * 4);
+    s += (v[i][0] + v[i][1]) + (v[i][2] + v[i][3]);
+  }
+  const float mean = wave_sum(s) * inv_n;
+  float q = 0.0f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float c = v[i][e] - mean;
+      q += c * c;
+    }
+  }
+  const float inv_std = rsqrtf(wave_sum(q) * inv_n + eps);
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    const int col = (i * 64 + lane) * 4;
+    f32x4 g = *reinterpret_cast<const f32x4*>(gamma + col);
+    f32x4 b = *reinterpret_cast<const f32x4*>(beta + col);
+    f32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = (v[i][e] - mean) * inv_std * g[e] + b[e];
+    store4<ODT>(out, base + col, o);
+  }
+}
+
+// Any N: one wave per row, three passes over the row (re-read from cache).
+template <int XDT, int ODT>
+__global__ void __launch_bounds__(256) layer_norm_generic(void* out, const void* x, const float* gamma,
+                                                          const float* beta, int M, int N, float eps, float inv_n) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;
+  const int64_t base = (int64_t)row * N;
+  float s = 0.0f;
+  for (int j = lane; j < N; j += 64) s += load_as_f32<XDT>(x, base + j);
+  const float mean = wave_sum(s) * inv_n;
+  float q = 0.0f;
+  for (int j = lane; j < N; j += 64) {
+    float c = load_as_f32<XDT>(x, base + j) - mean;
+    q += c * c;
+  }
+  const float inv_std = rsqrtf(wave_sum(q) * inv_n + eps);
+  for (int j = lane; j < N; j += 64)
+    store_from_f32<ODT>(out, base + j, (load_as_f32<XDT>(x, base + j) - mean) * inv_std * gamma[j] + beta[j]);
+}
+
+// Row softmax (lighthouse/ingress/mlir_gen/gpu_softmax_payload.py:46-55), one wave per row.
+template <int DT>
+__global__ void __launch_bounds__(256) softmax_rows(void* out, const void* x, int M, int N) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;
+  const int64_t base = (int64_t)row * N;
+  float mx = -INFINITY;
+  for (int j = lane; j < N; j += 64) mx = fmaxf(mx, load_as_f32<DT>(x, base + j));
+  mx = wave_max(mx);
+  float s = 0.0f;
+  for (int j = lane; j < N; j += 64) s += expf(load_as_f32<DT>(x, base + j) - mx);
+  s = wave_sum(s);
+  for (int j = lane; j < N; j += 64) store_from_f32<DT>(out, base + j, expf(load_as_f32<DT>(x, base + j) - mx) / s);
+}
+
+// Accurate tanh-GELU for the standalone kernel (the GEMM epilogue uses the single-exp form).
+__device__ __forceinline__ float gelu_tanh_ref(float x) {
+  const float k = 0.7978845608028654f;
+  float u = k * (x + 0.044715f * x * x * x);
+  return 0.5f * x * (1.0f + tanhf(u));
+}
+
+enum { EW_GELU = 0, EW_ADD = 1, EW_BIAS = 2, EW_BIAS_RELU = 3 };
+
+// n4 groups of 4 elements; `N` is the row length for the bias kinds.
+template <int DT, int KIND>
+__global__ void __launch_bounds__(256) elementwise4(void* out, const void* a, const void* b, int64_t n4, int N) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += stride) {
+    f32x4 x = load4<DT>(a, i * 4);
+    f32x4 o;
+    if constexpr (KIND == EW_GELU) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = gelu_tanh_ref(x[e]);
+    } else if constexpr (KIND == EW_ADD) {
+      f32x4 y = load4<DT>(b, i * 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = x[e] + y[e];
+    } else {
+      f32x4 y = load4<DT>(b, (i * 4) % N);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        o[e] = x[e] + y[e];
+        if constexpr (KIND == EW_BIAS_RELU) o[e] = relu_nan(o[e]);
+      }
+    }
+    store4<DT>(out, i * 4, o);
+  }
+}
+
+template <int DT, int KIND>
+__global__ void __launch_bounds__(256) elementwise1(void* out, const void* a, const void* b, int64_t n, int N) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    float x = load_as_f32<DT>(a, i), o;
+    if constexpr (KIND == EW_GELU) o = gelu_tanh_ref(x);
+    else if constexpr (KIND == EW_ADD) o = x + load_as_f32<DT>(b, i);
+    else {
+      o = x + load_as_f32<DT>(b, i % N);
+      if constexpr (KIND == EW_BIAS_RELU) o = relu_nan(o);
+    }
+    store_from_f32<DT>(out, i, o);
+  }
+}
+
+template <int SDT, int DDT>
+__global__ void __launch_bounds__(256) cast_kernel(void* out, const void* x, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  const int64_t n4 = n / 4;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n4; i += stride)
+    store4<DDT>(out, i * 4, load4<SDT>(x, i * 4));
+  for (int64_t i = n4 * 4 + (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+    store_from_f32<DDT>(out, i, load_as_f32<SDT>(x, i));
+}
+
+static inline unsigned ew_grid(int64_t work) {
+  int64_t b = (work + 255) / 256;
+  if (b < 1) b = 1;
+  const int64_t cap = 256 * 16;  // 16 workgroups per CU, grid-stride beyond that
+  return (unsigned)(b > cap ? cap : b);
+}
+
+template <int XDT, int ODT>
+static int layer_norm_launch(void* out, const void* x, const float* gamma, const float* beta, int M, int N, float eps,
+                             hipStream_t s) {
+  const float inv_n = (float)(1.0 / (double)N);
+  dim3 grid((M + 3) / 4), block(256);
+  const bool vec = N % 256 == 0 && aligned16(out) && aligned16(x) && aligned16(gamma) && aligned16(beta);
+#define LH_LN_CASE(V)                                                                                          \
+  case V:                                                                                                      \
+    hipLaunchKernelGGL((layer_norm_vec<XDT, ODT, V>), grid, block, 0, s, out, x, gamma, beta, M, N, eps, inv_n); \
+    return check_launch("layer_norm_vec");
+  if (vec) {
+    switch (N / 256) {
+      LH_LN_CASE(1) LH_LN_CASE(2) LH_LN_CASE(3) LH_LN_CASE(4) LH_LN_CASE(6) LH_LN_CASE(8) LH_LN_CASE(12) LH_LN_CASE(16)
+      default: break;
+    }
+  }
+#undef LH_LN_CASE
+  hipLaunchKernelGGL((layer_norm_generic<XDT, ODT>), grid, block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);
+  return check_launch("layer_norm_generic");
+}
+
+template <int DT, int KIND>
+static int ew_launch(void* out, const void* a, const void* b, int64_t n, int N, hipStream_t s) {
+  const bool vec = n % 4 == 0 && (KIND < EW_BIAS || N % 4 == 0) && aligned16(out) && aligned16(a) &&
+                   (b == nullptr || aligned16(b));
+  if (vec) hipLaunchKernelGGL((elementwise4<DT, KIND>), dim3(ew_grid(n / 4)), dim3(256), 0, s, out, a, b, n / 4, N);
+  else hipLaunchKernelGGL((elementwise1<DT, KIND>), dim3(ew_grid(n)), dim3(256), 0, s, out, a, b, n, N);
+  return check_launch("elementwise");
+}
+
+template <int KIND>
+static int ew_dispatch(void* out, const void* a, const void* b, int64_t n, int N, int dt, hipStream_t s) {
+  switch (dt) {
+    case LH_F32: return ew_launch<LH_F32, KIND>(out, a, b, n, N, s);
+    case LH_BF16: return ew_launch<LH_BF16, KIND>(out, a, b, n, N, s);
+    case LH_F16: return ew_launch<LH_F16, KIND>(out, a, b, n, N, s);
+    default: return fail(LH_ERR_UNSUPPORTED, "elementwise: unsupported dtype %d", dt);
+  }
+}
+
+}  // namespace lh
+
+using namespace lh;
+
+extern "C" {
+
+int lh_hip_layer_norm(void* out, const void* x, const float* gamma, const float* beta, int64_t M, int64_t N, float eps,
+                      int32_t x_dtype, int32_t out_dtype, void* stream) {
+  LH_REQUIRE(out && x && gamma && beta, "lh_hip_layer_norm: null pointer");
+  LH_REQUIRE(M > 0 && N > 0 && M < (1ll << 31) && N < (1ll << 31), "lh_hip_layer_norm: bad shape %lld x %lld",
+             (long long)M, (long long)N);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (x_dtype == LH_F32 && out_dtype == LH_F32)
+    return layer_norm_launch<LH_F32, LH_F32>(out, x, gamma, beta, (int)M, (int)N, eps, s);
+  if (x_dtype == LH_F32 && out_dtype == LH_BF16)
+    return layer_norm_launch<LH_F32, LH_BF16>(out, x, gamma, beta, (int)M, (int)N, eps, s);
+  if (x_dtype == LH_BF16 && out_dtype == LH_BF16)
+    return layer_norm_launch<LH_BF16, LH_BF16>(out, x, gamma, beta, (int)M, (int)N, eps, s);
+  if (x_dtype == LH_BF16 && out_dtype == LH_F32)
+    return layer_norm_launch<LH_BF16, LH_F32>(out, x, gamma, beta, (int)M, (int)N, eps, s);
+  return fail(LH_ERR_UNSUPPORTED, "lh_hip_layer_norm: unsupported dtypes x=%d out=%d", x_dtype, out_dtype);
+}
+
+int lh_hip_softmax(void* out, const void* x, int64_t M, int64_t N, int32_t dtype, void* stream) {
+  LH_REQUIRE(out && x, "lh_hip_softmax: null pointer");
+  LH_REQUIRE(M > 0 && N > 0 && M < (1ll << 31) && N < (1ll << 31), "lh_hip_softmax: bad shape");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  dim3 grid((unsigned)((M + 3) / 4)), block(256);
+  switch (dtype) {
+    case LH_F32: hipLaunchKernelGGL(softmax_rows<LH_F32>, grid, block, 0, s, out, x, (int)M, (int)N); break;
+    case LH_BF16: hipLaunchKernelGGL(softmax_rows<LH_BF16>, grid, block, 0, s, out, x, (int)M, (int)N); break;
+    case LH_F16: hipLaunchKernelGGL(softmax_rows<LH_F16>, grid, block, 0, s, out, x, (int)M, (int)N); break;
+    default: return fail(LH_ERR_UNSUPPORTED, "lh_hip_softmax: unsupported dtype %d", dtype);
+  }
+  return check_launch("softmax_rows");
+}
+
+int lh_hip_gelu_tanh(void* out, const void* x, int64_t n, int32_t dtype, void* stream) {
+  LH_REQUIRE(out && x && n > 0, "lh_hip_gelu_tanh: bad arguments");
+  return ew_dispatch<EW_GELU>(out, x, nullptr, n, 1, dtype, reinterpret_cast<hipStream_t>(stream));
+}
+
+int lh_hip_bias_act(void* out, const void* x, const void* bias, int64_t M, int64_t N, int32_t relu, int32_t dtype,
+                    void* stream) {
+  LH_REQUIRE(out && x && bias && M > 0 && N > 0 && N < (1ll << 31), "lh_hip_bias_act: bad arguments");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (relu) return ew_dispatch<EW_BIAS_RELU>(out, x, bias, M * N, (int)N, dtype, s);
+  return ew_dispatch<EW_BIAS>(out, x, bias, M * N, (int)N, dtype, s);
+}
+
+int lh_hip_add(void* out, const void* a, const void* b, int64_t n, int32_t dtype, void* stream) {
+  LH_REQUIRE(out && a && b && n > 0, "lh_hip_add: bad arguments");
+  return ew_dispatch<EW_ADD>(out, a, b, n, 1, dtype, reinterpret_cast<hipStream_t>(stream));
+}
+
+int lh_hip_cast(void* out, const void* x, int64_t n, int32_t src, int32_t dst, void* stream) {
+  LH_REQUIRE(out && x && n > 0, "lh_hip_cast: bad arguments");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const bool al = aligned16(out) && aligned16(x);
+  if (!al) return fail(LH_ERR_INVALID, "lh_hip_cast: buffers must be 16-byte aligned");
+  dim3 grid(ew_grid(n / 4 + 1)), block(256);
+#define LH_CAST(S, D)                                                         \
+  if (src == S && dst == D) {                                                 \
+    hipLaunchKernelGGL((cast_kernel<S, D>), grid, block, 0, s, out, x, n);    \
+    return check_launch("cast_kernel");                                       \
+  }
+  LH_CAST(LH_F32, LH_BF16) LH_CAST(LH_F32, LH_F16) LH_CAST(LH_BF16, LH_F32) LH_CAST(LH_F16, LH_F32)
+  LH_CAST(LH_F32, LH_F32) LH_CAST(LH_BF16, LH_BF16) LH_CAST(LH_F16, LH_F16)
+#undef LH_CAST
+  return fail(LH_ERR_UNSUPPORTED, "lh_hip_cast: unsupported conversion %d -> %d", src, dst);
+}
+
+}  // extern "C"

@@ -1,0 +1,121 @@
+"""Fused attention parity on the GPU vs the CPU oracle."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import lh_oracle as orc
+from tests.conftest import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(x, dtype):
+    return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to("cuda").to(dtype)
+
+
+def _host(t):
+    return t.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype,elt,rtol", [(torch.bfloat16, "bf16", 2e-2), (torch.float16, "f16", 2e-2),
+                                            (torch.float32, "f32", 1e-4)])
+@pytest.mark.parametrize("shape", [(1, 1, 128, 64), (2, 3, 256, 64), (1, 2, 512, 64)])
+def test_attention_vs_oracle(shape, dtype, elt, rtol, causal):
+    from lighthouse_amd import ops
+
+    rng = np.random.default_rng(42 + shape[2] + causal)
+    q, k, v = (orc.round_to(rng.standard_normal(shape).astype(np.float32), elt) for _ in range(3))
+    out = ops.attention(_dev(q, dtype), _dev(k, dtype), _dev(v, dtype), causal=causal)
+    ref = orc.attention(q, k, v, causal=causal)
+    assert_close(_host(out), ref, rtol, f"attention {shape} {elt} causal={causal}")
+
+
+def test_attention_reference_inputs():
+    """Inputs of the reference workload (examples/xegpu/fused_attention.py:145-154):
+    seed 42, uniform(-0.5, 0.5); checker tolerance rtol = atol = 1e-3 in f16."""
+    from lighthouse_amd import ops
+
+    shape = (2, 2, 256, 64)
+    np.random.seed(42)
+    q, k, v = (np.random.uniform(-0.5, 0.5, shape).astype(np.float16) for _ in range(3))
+    out = ops.attention(*(torch.from_numpy(t).cuda() for t in (q, k, v)))
+    ref = orc.attention(q.astype(np.float32), k.astype(np.float32), v.astype(np.float32))
+    assert np.allclose(_host(out), ref, rtol=1e-3, atol=1e-3)
+
+
+def test_attention_online_recurrence_matches_kernel_rounding():
+    """The kernel follows the tiled recurrence with P rounded to bf16 before P.V: it must agree
+    with the oracle's tiled restatement more tightly than with the unrounded one-shot form."""
+    from lighthouse_amd import ops
+
+    rng = np.random.default_rng(3)
+    q, k, v = (orc.round_bf16(rng.standard_normal((256, 64)).astype(np.float32)) for _ in range(3))
+    out = _host(ops.attention(*( _dev(t[None, None], torch.bfloat16) for t in (q, k, v)), causal=True))[0, 0]
+    tiled = orc.attention_online(q, k, v, tile=64, causal=True, elt="bf16")
+    assert_close(out, tiled, 1e-2, "attention vs tiled oracle")
+
+
+def test_attention_closed_forms():
+    from lighthouse_amd import ops
+
+    rng = np.random.default_rng(8)
+    shape = (1, 2, 256, 64)
+    q = _dev(rng.standard_normal(shape), torch.bfloat16)
+    k = _dev(rng.standard_normal(shape), torch.bfloat16)
+    v = _dev(rng.standard_normal(shape), torch.bfloat16)
+    # K = 0: uniform weights, O = mean of V over keys.
+    o = ops.attention(q, torch.zeros_like(k), v)
+    assert_close(_host(o), np.broadcast_to(_host(v).mean(2, keepdims=True), shape), 2e-2, "K=0")
+    # Constant V rows: O = that constant.
+    vc = torch.full_like(v, 0.75)
+    assert torch.equal(ops.attention(q, k, vc), vc)
+    # Causal row 0 sees only key 0.
+    oc = ops.attention(q, k, v, causal=True)
+    assert torch.equal(oc[:, :, 0], v[:, :, 0])
+    # Jointly permuting keys and values leaves the non-causal output unchanged (up to summation order).
+    perm = torch.randperm(shape[2], device="cuda")
+    assert_close(_host(ops.attention(q, k[:, :, perm], v[:, :, perm])), _host(ops.attention(q, k, v)), 2e-2, "perm")
+
+
+def test_attention_strided_views():
+    """(T, H*d) projection buffers viewed as (H, T, d) without a copy
+    (examples/xegpu/nanoGPT_payload.py:198-217)."""
+    from lighthouse_amd import ops
+
+    B, T, H, d = 2, 256, 3, 64
+    rng = np.random.default_rng(21)
+    qkv = _dev(rng.standard_normal((B, T, 3 * H * d)), torch.bfloat16)
+    q, k, v = (qkv[:, :, i * H * d:(i + 1) * H * d].view(B, T, H, d).permute(0, 2, 1, 3) for i in range(3))
+    out_buf = torch.empty(B, T, H * d, device="cuda", dtype=torch.bfloat16)
+    out = out_buf.view(B, T, H, d).permute(0, 2, 1, 3)
+    ops.attention(q, k, v, causal=True, out=out)
+    ref = ops.attention(q.contiguous(), k.contiguous(), v.contiguous(), causal=True)
+    assert torch.equal(out.contiguous(), ref)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_benchmark_size(causal):
+    """[4,16,2048,64] bf16: sampled (batch, head) pairs against the oracle."""
+    from lighthouse_amd import ops
+
+    g = torch.Generator(device="cuda").manual_seed(77)
+    shape = (4, 16, 2048, 64)
+    q, k, v = (torch.randn(shape, device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
+    out = ops.attention(q, k, v, causal=causal)
+    assert torch.isfinite(out.float()).all()
+    for z, h in [(0, 0), (3, 15), (1, 7)]:
+        ref = orc.attention(_host(q[z, h]), _host(k[z, h]), _host(v[z, h]), causal=causal)
+        assert_close(_host(out[z, h]), ref, 2e-2, f"attention bench size z={z} h={h} causal={causal}")
+
+
+def test_attention_errors():
+    from lighthouse_amd import ops
+
+    x = torch.zeros(1, 1, 128, 32, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.attention(x, x, x)
+    y = torch.zeros(1, 1, 100, 64, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.attention(y, y, y)

@@ -1,0 +1,142 @@
+"""nanoGPT block parity and the Runner boundary on the GPU."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import lh_oracle as orc
+from tests.conftest import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def make_block_params(C, rng, std=0.02, bias_std=0.0):
+    def w(*s):
+        return (rng.standard_normal(s) * std).astype(np.float32)
+
+    def bvec(n):
+        return (rng.standard_normal(n) * bias_std).astype(np.float32)
+
+    return {
+        "ln1_g": np.ones(C, np.float32), "ln1_b": np.zeros(C, np.float32),
+        "w_qkv": w(C, 3 * C), "b_qkv": bvec(3 * C), "w_o": w(C, C), "b_o": bvec(C),
+        "ln2_g": np.ones(C, np.float32), "ln2_b": np.zeros(C, np.float32),
+        "w_fc": w(C, 4 * C), "b_fc": bvec(4 * C), "w_proj": w(4 * C, C), "b_proj": bvec(C),
+    }
+
+
+def to_device(params, dtype):
+    out = {}
+    for k, v in params.items():
+        t = torch.from_numpy(v).cuda()
+        out[k] = t if k.startswith("ln") else t.to(dtype)
+    return out
+
+
+@pytest.mark.parametrize("mode,dtype,rtol", [("f32", torch.float32, 1e-4), ("bf16", torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("bias_std", [0.0, 0.02])
+def test_nanogpt_block_small(mode, dtype, rtol, bias_std):
+    from lighthouse_amd import ops
+
+    B, T, C, H = 2, 128, 256, 4
+    rng = np.random.default_rng(0xB10C)
+    p = make_block_params(C, rng, bias_std=bias_std)
+    p["ln1_g"] = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    p["ln2_b"] = rng.uniform(-0.1, 0.1, C).astype(np.float32)
+    x = rng.standard_normal((B, T, C)).astype(np.float32)
+    y = ops.nanogpt_block(torch.from_numpy(x).cuda(), to_device(p, dtype), H)
+    ref = orc.nanogpt_block(x, p, H, mode=mode)
+    assert_close(y.cpu().numpy(), ref, rtol, f"nanoGPT block {mode}")
+
+
+@pytest.mark.parametrize("mode,dtype,rtol", [("f32", torch.float32, 1e-4), ("bf16", torch.bfloat16, 2e-2)])
+def test_nanogpt_block_benchmark_shape(mode, dtype, rtol):
+    """n_embd 768, 12 heads, T 1024 (batch 2 of the 8 for the oracle's sake; the batch entries
+    are independent, and the full batch is checked for equality of repeated entries)."""
+    from lighthouse_amd import ops
+
+    B, T, C, H = 2, 1024, 768, 12
+    rng = np.random.default_rng(0x6E616E6F)
+    p = make_block_params(C, rng)
+    x = rng.standard_normal((B, T, C)).astype(np.float32)
+    dp = to_device(p, dtype)
+    y = ops.nanogpt_block(torch.from_numpy(x).cuda(), dp, H)
+    ref = orc.nanogpt_block(x, p, H, mode=mode)
+    assert_close(y.cpu().numpy(), ref, rtol, f"nanoGPT block {mode} 768/12/1024")
+    x8 = torch.from_numpy(x).cuda().repeat(4, 1, 1)
+    y8 = ops.nanogpt_block(x8, dp, H)
+    assert torch.equal(y8[:2], y) and torch.equal(y8[6:], y)
+
+
+def test_runner_matmul_golden():
+    """lh-run's known-answer test (test/run/pipeline-check.mlir:1,16-31) through the Runner."""
+    from lighthouse_amd.execution import KernelArgumentParser, Runner
+    from lighthouse_amd.ingress import generate_gpu_matmul_payload
+    import json
+    from pathlib import Path
+
+    golden = json.loads((Path(__file__).parent / "golden" / "lh_run_pipeline_check.json").read_text())
+    np.random.seed(golden["seed"])
+    a, b, c = (arg.arg for arg in KernelArgumentParser.parse_all(golden["input_shape"]))
+    module = generate_gpu_matmul_payload("main", 16, 32, 64, "f32", "f32")
+    runner = Runner(module)
+    runner.execute("main", [c, a, b])
+    np.testing.assert_allclose(c[:, 0], np.array(golden["row_values"], dtype=np.float32), rtol=2e-6)
+    assert (c == c[:, :1]).all()
+    times = runner.benchmark([c, a, b])
+    assert times.shape == (100,) and (times > 0).all()
+
+
+def test_runner_memory_managers():
+    from lighthouse_amd.execution import GPUMemoryManager, Runner, TorchMemoryManager
+    from lighthouse_amd.ingress import generate_gpu_matmul_payload
+    from lighthouse_amd.utils.numpy import bf16_to_f32, f32_to_bf16
+
+    M, N, K = 256, 128, 64
+    rng = np.random.default_rng(2)
+    a = f32_to_bf16(rng.standard_normal((M, K)))
+    b = f32_to_bf16(rng.standard_normal((K, N)))
+    bias = f32_to_bf16(rng.standard_normal(N))
+    c = f32_to_bf16(np.zeros((M, N)))
+    module = generate_gpu_matmul_payload("payload", M, N, K, "bf16", "f32", has_bias=True, has_relu=True,
+                                         result_type="bf16")
+    ref = orc.matmul(bf16_to_f32(a), bf16_to_f32(b), bias=bf16_to_f32(bias), relu=True, result_type="bf16")
+    runner = Runner(module, mem_manager_cls=GPUMemoryManager)
+    host_out = np.zeros_like(c)
+    runner.execute("payload", [c, a, b, bias], Runner.get_gpu_argument_access_callback(host_out))
+    assert_close(bf16_to_f32(host_out), ref, 2e-2, "runner GPUMemoryManager")
+    times = runner.benchmark([c, a, b, bias], nruns=5, nwarmup=2)
+    assert times.shape == (5,) and (times > 0).all()
+    # Pass-through manager with torch tensors.
+    tr = Runner(module, mem_manager_cls=TorchMemoryManager)
+    tens = [torch.from_numpy(np.asarray(t).view(np.int16)).cuda().view(torch.bfloat16) for t in (c, a, b, bias)]
+    tr.execute("payload", tens)
+    assert_close(tens[0].float().cpu().numpy(), ref, 2e-2, "runner TorchMemoryManager")
+    with pytest.raises(ValueError):
+        Runner(module, mem_manager_cls=dict).execute("payload", [c, a, b, bias])
+    with pytest.raises(ValueError):
+        runner.execute("payload", [c, a, b])
+    with pytest.raises(ValueError):
+        runner.execute("payload", [c, a, b[:, :-1], bias])
+
+
+def test_runner_attention_and_layer_norm_payloads():
+    from lighthouse_amd.execution import GPUMemoryManager, Runner
+    from lighthouse_amd.ingress import generate_gpu_attention_payload, generate_gpu_layer_norm_payload
+
+    shape = (1, 2, 128, 64)
+    np.random.seed(42)
+    q, k, v = (np.random.uniform(-0.5, 0.5, shape).astype(np.float16) for _ in range(3))
+    out = np.zeros(shape, np.float16)
+    runner = Runner(generate_gpu_attention_payload("payload", *shape, "f16"), mem_manager_cls=GPUMemoryManager)
+    runner.execute("payload", [out, q, k, v], Runner.get_gpu_argument_access_callback(out))
+    ref = orc.attention(q.astype(np.float32), k.astype(np.float32), v.astype(np.float32))
+    assert np.allclose(out.astype(np.float32), ref, rtol=1e-3, atol=1e-3)
+
+    M, N = 64, 768
+    x = np.random.uniform(-1, 1, (M, N)).astype(np.float32)
+    g = np.random.uniform(0.5, 1.5, N).astype(np.float32)
+    b = np.random.uniform(-0.1, 0.1, N).astype(np.float32)
+    o = np.zeros((M, N), np.float32)
+    Runner(generate_gpu_layer_norm_payload("payload", M, N, "f32")).execute("payload", [o, x, g, b])
+    assert np.allclose(o, orc.layer_norm(x, g, b), rtol=1e-3, atol=1e-4)

@@ -1,0 +1,190 @@
+"""GEMM parity on the GPU: HIP kernels (through the C ABI) vs the CPU oracle."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import lh_oracle as orc
+from tests.conftest import assert_close
+
+pytestmark = pytest.mark.gpu
+
+F32_RTOL = 1e-4   # benchmark definition: f32 within rtol 1e-4
+BF16_RTOL = 2e-2  # bf16 within rtol 2e-2 of the f32 reference
+
+
+def _dev(x, dtype):
+    return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to("cuda").to(dtype)
+
+
+def _host(t):
+    return t.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("shape", [(64, 64, 32), (128, 128, 64), (256, 192, 96), (1024, 1024, 1024), (100, 70, 50),
+                                   (1, 1, 1), (33, 65, 17)])
+@pytest.mark.parametrize("epi", ["none", "bias_relu"])
+def test_gemm_f32(shape, epi):
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(0xC0FFEE + M + N + K)
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (N,)).astype(np.float32)
+    has = epi == "bias_relu"
+    out = ops.gemm(_dev(a, torch.float32), _dev(b, torch.float32), _dev(bias, torch.float32) if has else None, relu=has)
+    ref = orc.matmul(a, b, bias=bias if has else None, relu=has)
+    assert_close(_host(out), ref, F32_RTOL, f"f32 gemm {shape} {epi}")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(128, 128, 64), (256, 256, 128), (512, 768, 256), (1024, 1024, 512),
+                                   (2048, 2048, 256), (100, 70, 50), (1, 1, 1), (130, 257, 66)])
+@pytest.mark.parametrize("epi", ["none", "bias_relu", "bias_gelu", "f32out", "acc"])
+def test_gemm_16bit(dtype, shape, epi):
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    elt = "bf16" if dtype == torch.bfloat16 else "f16"
+    rng = np.random.default_rng(7 + M + 3 * N + 5 * K)
+    a = orc.round_to(rng.standard_normal((M, K)).astype(np.float32), elt)
+    b = orc.round_to(rng.standard_normal((K, N)).astype(np.float32), elt)
+    bias = orc.round_to(rng.standard_normal((N,)).astype(np.float32), elt)
+    da, db = _dev(a, dtype), _dev(b, dtype)
+    if epi == "none":
+        out = ops.gemm(da, db)
+        ref = orc.matmul(a, b, result_type=elt)
+    elif epi == "bias_relu":
+        out = ops.gemm(da, db, _dev(bias, dtype), relu=True)
+        ref = orc.matmul(a, b, bias=bias, relu=True, result_type=elt)
+    elif epi == "bias_gelu":
+        out = ops.gemm(da, db, _dev(bias, dtype), gelu=True)
+        ref = orc.matmul(a, b, bias=bias, gelu=True, result_type=elt)
+    elif epi == "f32out":
+        out = ops.gemm(da, db, out_dtype=torch.float32)
+        ref = orc.matmul(a, b, result_type="f32")
+    else:
+        c = rng.standard_normal((M, N)).astype(np.float32)
+        out = _dev(c, torch.float32)
+        ops.gemm(da, db, out=out, accumulate_c=True)
+        ref = orc.matmul(a, b, c=c, accumulate_c=True, result_type="f32")
+    rtol = F32_RTOL if epi in ("f32out", "acc") else BF16_RTOL
+    assert_close(_host(out), ref, rtol, f"{elt} gemm {shape} {epi}")
+
+
+@pytest.mark.parametrize("ta,tb", [(True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_gemm_transposed(dtype, ta, tb):
+    from lighthouse_amd import ops
+
+    M, N, K = 256, 128, 192
+    elt = "bf16" if dtype == torch.bfloat16 else "f32"
+    rng = np.random.default_rng(99)
+    a = orc.round_to(rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32), elt)
+    b = orc.round_to(rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32), elt)
+    out = ops.gemm(_dev(a, dtype), _dev(b, dtype), out_dtype=torch.float32, transpose_a=ta, transpose_b=tb)
+    ref = orc.matmul(a, b, transpose_a=ta, transpose_b=tb)
+    assert_close(_host(out), ref, F32_RTOL, f"transposed gemm ta={ta} tb={tb} {elt}")
+
+
+def test_gemm_integer_inputs_exact():
+    """Integer inputs in [-3, 3] (examples/xegpu/matmul.py:143-152) are exact in bf16 and f32."""
+    from lighthouse_amd import ops
+
+    rng = np.random.default_rng(2)
+    a = rng.integers(-3, 4, (512, 256)).astype(np.float32)
+    b = rng.integers(-3, 4, (256, 384)).astype(np.float32)
+    out = ops.gemm(_dev(a, torch.bfloat16), _dev(b, torch.bfloat16), out_dtype=torch.float32)
+    np.testing.assert_array_equal(_host(out), a @ b)
+
+
+def test_gemm_identity_and_ones():
+    """B = I gives C == A bit for bit; B = 1 gives row sums (the lh-run golden's structure)."""
+    from lighthouse_amd import ops
+
+    rng = np.random.default_rng(5)
+    a = orc.round_bf16(rng.standard_normal((256, 256)).astype(np.float32))
+    out = ops.gemm(_dev(a, torch.bfloat16), torch.eye(256, device="cuda", dtype=torch.bfloat16))
+    np.testing.assert_array_equal(_host(out), a)
+    a32 = rng.uniform(0, 1, (128, 64)).astype(np.float32)
+    out = ops.gemm(_dev(a32, torch.float32), torch.ones(64, 128, device="cuda"))
+    assert_close(_host(out), np.repeat(a32.astype(np.float64).sum(1, keepdims=True), 128, 1), F32_RTOL, "ones")
+
+
+def test_gemm_bf16_4096_properties():
+    """Benchmark size (4096^3): checked against the oracle on a sampled set of rows/columns and
+    through linearity: (A1 + A2) B == A1 B + A2 B when all three are exact in f32 output."""
+    from lighthouse_amd import ops
+
+    n = 4096
+    g = torch.Generator(device="cuda").manual_seed(1234)
+    a = torch.randn(n, n, device="cuda", generator=g).to(torch.bfloat16)
+    b = torch.randn(n, n, device="cuda", generator=g).to(torch.bfloat16)
+    bias = torch.randn(n, device="cuda", generator=g).to(torch.bfloat16)
+    out = ops.gemm(a, b)
+    out_epi = ops.gemm(a, b, bias, relu=True)
+    rows = np.array([0, 1, 255, 256, 1023, 2048, 3071, 4095])
+    cols = np.array([0, 31, 32, 63, 64, 2047, 4000, 4095])
+    a_h = a[rows].float().cpu().numpy()
+    b_h = b[:, cols].float().cpu().numpy()
+    ref = orc.matmul(a_h, b_h, result_type="bf16")
+    assert_close(_host(out[rows][:, cols]), ref, BF16_RTOL, "bf16 4096 sample")
+    ref_epi = orc.matmul(a_h, b_h, bias=bias[cols].float().cpu().numpy(), relu=True, result_type="bf16")
+    assert_close(_host(out_epi[rows][:, cols]), ref_epi, BF16_RTOL, "bf16 4096 epilogue sample")
+    # Small-integer matrices: every partial sum is exact, so linearity must hold bit for bit.
+    a1 = torch.randint(-2, 3, (n, n), device="cuda", generator=g).to(torch.bfloat16)
+    a2 = torch.randint(-2, 3, (n, n), device="cuda", generator=g).to(torch.bfloat16)
+    bi = torch.randint(-2, 3, (n, n), device="cuda", generator=g).to(torch.bfloat16)
+    lhs = ops.gemm(a1 + a2, bi, out_dtype=torch.float32)
+    rhs = ops.gemm(a1, bi, out_dtype=torch.float32) + ops.gemm(a2, bi, out_dtype=torch.float32)
+    assert torch.equal(lhs, rhs)
+
+
+def test_gemm_errors():
+    from lighthouse_amd import ops
+
+    a = torch.zeros(8, 8, device="cuda")
+    with pytest.raises(ValueError):
+        ops.gemm(a, torch.zeros(8, 8, device="cuda", dtype=torch.bfloat16))
+    with pytest.raises(ValueError):
+        ops.gemm(a.to(torch.float64), a.to(torch.float64))
+    with pytest.raises(ValueError):
+        ops.gemm(a, a, relu=True, gelu=True)
+
+
+@pytest.mark.parametrize("shape", [(128, 128, 128), (256, 256, 512), (96, 80, 200), (16, 256, 1024), (5, 128, 256)])
+def test_gemm_fp8(shape):
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(11 + M + N + K)
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    b = rng.standard_normal((K, N)).astype(np.float32)
+    aq, sa = orc.quantize_per_tensor_e4m3(a)
+    bq, sb = orc.quantize_per_tensor_e4m3(b)
+    da = torch.from_numpy(aq).to("cuda").view(torch.float8_e4m3fn)
+    db = torch.from_numpy(bq).to("cuda").view(torch.float8_e4m3fn)
+    out = ops.gemm_fp8(da, db, float(sa), float(sb))
+    ref = orc.matmul_fp8(aq, bq, sa, sb)
+    assert_close(_host(out), ref, 5e-2, f"fp8 gemm {shape}")
+    # Against the dequantised float reference, as the benchmark defines the tolerance.
+    deq = (orc.e4m3_dequant(aq).astype(np.float64) * sa) @ (orc.e4m3_dequant(bq).astype(np.float64) * sb)
+    assert_close(_host(out), deq, 5e-2, f"fp8 gemm vs dequantised {shape}")
+
+
+def test_gemm_fp8_all_codes():
+    """Every finite e4m3 code against every other: a 256 x 256 outer-product table (K padded with zeros)."""
+    from lighthouse_amd import ops
+
+    table = orc.e4m3_decode_table()
+    codes = np.array([c for c in range(256) if np.isfinite(table[c])], dtype=np.uint8)
+    n = 256
+    a = np.zeros((n, 128), np.uint8)
+    b = np.zeros((128, n), np.uint8)
+    a[: len(codes), 0] = codes
+    b[0, : len(codes)] = codes
+    out = ops.gemm_fp8(torch.from_numpy(a).cuda().view(torch.float8_e4m3fn),
+                       torch.from_numpy(b).cuda().view(torch.float8_e4m3fn), 1.0, 1.0, out_dtype=torch.float32)
+    ref = np.outer(table[a[:, 0]].astype(np.float64), table[b[0, :]].astype(np.float64))
+    np.testing.assert_array_equal(_host(out), ref.astype(np.float32))
