@@ -115,11 +115,12 @@ __global__ void __launch_bounds__(256) softmax_rows(void* out, const void* x, in
   for (int j = lane; j < N; j += 64) store_from_f32<DT>(out, base + j, expf(load_as_f32<DT>(x, base + j) - mx) / s);
 }
 
-// Accurate tanh-GELU for the standalone kernel (the GEMM epilogue uses the single-exp form).
+// tanh-GELU as x / (1 + exp(-2u)), u = sqrt(2/pi) (x + 0.044715 x^3): identical to
+// 0.5 x (1 + tanh u) but without the cancellation of 1 + tanh(u) in the negative tail.
 __device__ __forceinline__ float gelu_tanh_ref(float x) {
   const float k = 0.7978845608028654f;
   float u = k * (x + 0.044715f * x * x * x);
-  return 0.5f * x * (1.0f + tanhf(u));
+  return x / (1.0f + expf(-2.0f * u));
 }
 
 enum { EW_GELU = 0, EW_ADD = 1, EW_BIAS = 2, EW_BIAS_RELU = 3 };

@@ -48,12 +48,13 @@ def test_layer_norm_bf16_out_and_in():
 def test_layer_norm_special_cases():
     from lighthouse_amd import ops
 
-    n = 768
-    ones, zeros = torch.ones(n, device="cuda"), torch.zeros(n, device="cuda")
-    # Constant rows normalise to beta exactly.
+    # Constant rows normalise to beta exactly when the row sum and 1/N are exact (N a power of two).
+    n = 1024
     x = torch.full((16, n), 3.25, device="cuda")
     beta = torch.linspace(-1, 1, n, device="cuda")
-    assert torch.equal(ops.layer_norm(x, ones, beta), beta.expand(16, n))
+    assert torch.equal(ops.layer_norm(x, torch.ones(n, device="cuda"), beta), beta.expand(16, n))
+    n = 768
+    ones, zeros = torch.ones(n, device="cuda"), torch.zeros(n, device="cuda")
     # gamma = 1, beta = 0: zero mean, unit variance rows.
     y = ops.layer_norm(torch.randn(64, n, device="cuda") * 5 + 2, ones, zeros)
     assert y.mean(1).abs().max() < 1e-5
