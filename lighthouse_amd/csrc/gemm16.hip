@@ -192,6 +192,324 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm16_fast(GemmArgs g)
                       acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
 }
 
+
+// ---- direct-to-LDS kernel ---------------------------------------------------------------
+// 256 x 256 workgroup tile, 8 waves (2 x 4, 128 x 64 per wave).  Both panels go global -> LDS
+// with global_load_lds_dwordx4 (no register staging, no LDS store instructions) in their
+// GLOBAL orientation.  The k-contiguous A fragment is one 16-byte LDS read; the n-contiguous B
+// panel is read with ds_read_b64_tr_b16, which hands each lane 4 k-values of one column, i.e.
+// the MFMA operand layout, transposing in the LDS crossbar.
+//
+// LDS rings: A in 2 stages of 64 k (256 rows x 128 bytes: every global request is a full
+// 128-byte line), B in 4 stages of 32 k (32 rows x 512 bytes).  The main loop advances 32 k per
+// step; the barrier sits in the MIDDLE of a step, after the LDS reads of the step's second
+// k-half have been issued, so fragment reads always overlap MFMAs of the previous k-half and
+// the buffer a step has finished reading is refilled right away (B: 3 stages ahead, A: on odd
+// steps, one 64-k stage ahead).
+//
+// A wave-wide global_load_lds writes 64 x 16 contiguous LDS bytes, so rows cannot be padded;
+// bank conflicts are avoided by XOR-swizzling which 16-byte chunk of a row each lane fetches
+// (A: chunk ^ ((row / 2) % 8); B: chunk ^ 4 (k % 4)).
+constexpr int kDirectABytes = 256 * 64 * 2;   // one A stage: 32 KiB
+constexpr int kDirectBBytes = 32 * 256 * 2;   // one B stage: 16 KiB
+constexpr int kDirectBBase = 2 * kDirectABytes;
+constexpr int kDirectRingBytes = kDirectBBase + 4 * kDirectBBytes;  // 128 KiB
+constexpr int kDirectLdsBytes = 8 * 128 * 136;  // output staging (139264) >= the rings
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void async_copy16(const void* gsrc, uint8_t* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(gsrc, (lds_void_t*)lds_wave_base, 16, 0, 0);
+}
+
+struct DirectCtx {
+  const uint16_t* a_src[4];  // lane's source of A load i at k = 0
+  const uint16_t* b_src[2];
+  int a_off[4];              // byte offset of the lane's A row in a stage, per m-subtile
+  int a_swz[4];
+  int64_t ldb;
+  int wave, h, b_off, b_chunk, b_swz;
+};
+
+struct DirectFrags {
+  u32x4 a[4];
+  u32x4 b[2];
+};
+
+// A stage `sa` (k = 64 sa .. +64): 4 loads per lane.
+__device__ __forceinline__ void direct_load_a(const DirectCtx& c, int sa, uint8_t* __restrict__ abuf) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) async_copy16(c.a_src[i] + sa * 64, abuf + (8 * i + c.wave) * 1024);
+}
+// B stage `sb` (k = 32 sb .. +32): 2 loads per lane.
+__device__ __forceinline__ void direct_load_b(const DirectCtx& c, int sb, uint8_t* __restrict__ bbuf) {
+#pragma unroll
+  for (int i = 0; i < 2; ++i) async_copy16(c.b_src[i] + (int64_t)(sb * 32) * c.ldb, bbuf + (8 * i + c.wave) * 1024);
+}
+
+// Fragments of 16 k: A chunk pair `kc` (0..3: which 16 of the stage's 64 k), B k-step `ks`
+// (0..1: which 16 of the stage's 32 k).
+__device__ __forceinline__ void direct_read_frags(const DirectCtx& c, const uint8_t* __restrict__ as,
+                                                  const uint8_t* __restrict__ bs, int kc, int ks, DirectFrags& f) {
+#ifdef LH_EXP_NO_READS
+  if (ks >= 0) return;
+#endif
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    f.a[j] = *reinterpret_cast<const u32x4*>(as + c.a_off[j] + (((2 * kc + c.h) ^ c.a_swz[j]) << 4));
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int p = (c.b_chunk + 4 * i) ^ c.b_swz;
+    const uint8_t* p0 = bs + ks * 16 * 512 + c.b_off + p * 16;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p0);
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p0 + 4 * 512));
+    u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+    f.b[i] = u32x4{l2[0], l2[1], h2[0], h2[1]};
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void direct_mfma(f32x16 (&acc)[2][4], const DirectFrags& f) {
+#ifdef LH_EXP_NO_MFMA
+#pragma unroll
+  for (int j = 0; j < 4; ++j) asm volatile("" ::"v"(f.a[j]));
+#pragma unroll
+  for (int i = 0; i < 2; ++i) asm volatile("" ::"v"(f.b[i]));
+  return;
+#endif
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = Mfma16<DT>::mma(f.b[i], f.a[j], acc[i][j]);
+}
+
+// Ask the scheduler to put one LDS read of the next k-half after each MFMA of the current one.
+__device__ __forceinline__ void direct_interleave_hint() {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+  }
+}
+
+#ifdef LH_EXP_NO_BARRIER
+#define LH_BAR ""
+#else
+#define LH_BAR "\n\ts_barrier"
+#endif
+
+// Wait until at most `allowed` of this wave's loads are still in flight and all its LDS reads
+// have returned, then barrier.  One asm block: a __syncthreads() would add a release fence,
+// i.e. a wait for ALL outstanding loads, and drain the rings.
+__device__ __forceinline__ void direct_wait_barrier(int allowed) {
+  if (allowed >= 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" LH_BAR ::: "memory");
+  else if (allowed >= 4) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" LH_BAR ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" LH_BAR ::: "memory");
+}
+
+// Steps kt (even) and kt + 1 of the main loop; both have a successor step.  On entry f0 holds
+// the fragments of (step kt, first k-half).  a_cur = A stage kt / 2, a_nxt = the next A stage,
+// b0 / b1 / b2 = B stages kt, kt + 1, kt + 2.  The refill pointers alias a_cur, b0 and b1: every
+// read of a buffer precedes the barrier after which it is refilled.  They are separate restrict
+// parameters so that the compiler does not make LDS reads wait for the asynchronous writes.
+//
+// In-flight loads, oldest first, when a barrier is reached (steady state):
+//   even step: [A(kt/2) B(kt+1)] [B(kt+2)] [A(kt/2+1) B(kt+3)]  -> B(kt+1) needed: 8 may remain
+//   odd step : [B(kt+1)] [A((kt+1)/2) B(kt+2)] [B(kt+3)]        -> A needed: 4 may remain
+// Near the end loads are no longer issued and the waits become full waits.
+template <int DT>
+__device__ __forceinline__ void direct_step_pair(const DirectCtx& c, f32x16 (&acc)[2][4], DirectFrags& f0,
+                                                 const uint8_t* __restrict__ a_cur, const uint8_t* __restrict__ a_nxt,
+                                                 const uint8_t* __restrict__ b0, const uint8_t* __restrict__ b1,
+                                                 const uint8_t* __restrict__ b2, uint8_t* __restrict__ a_refill,
+                                                 uint8_t* __restrict__ b_refill0, uint8_t* __restrict__ b_refill1,
+                                                 int kt, int nk) {
+  DirectFrags f1;
+  const bool steady = kt + 6 < nk;  // all loads of both steps are real
+  // ---- even step kt
+  direct_read_frags(c, a_cur, b0, 1, 1, f1);
+  direct_mfma<DT>(acc, f0);
+  direct_interleave_hint();
+  direct_wait_barrier(steady ? 8 : 0);
+#ifndef LH_EXP_NO_LOADS
+  if (kt + 4 < nk) direct_load_b(c, kt + 4, b_refill0);
+#endif
+  direct_read_frags(c, a_cur, b1, 2, 0, f0);
+  direct_mfma<DT>(acc, f1);
+  direct_interleave_hint();
+  // ---- odd step kt + 1
+  direct_read_frags(c, a_cur, b1, 3, 1, f1);
+  direct_mfma<DT>(acc, f0);
+  direct_interleave_hint();
+  direct_wait_barrier(steady ? 4 : 0);
+#ifndef LH_EXP_NO_LOADS
+  if (kt + 4 < nk) direct_load_a(c, kt / 2 + 2, a_refill);
+  if (kt + 5 < nk) direct_load_b(c, kt + 5, b_refill1);
+#endif
+  direct_read_frags(c, a_nxt, b2, 0, 0, f0);
+  direct_mfma<DT>(acc, f1);
+  direct_interleave_hint();
+}
+
+template <int DT>
+__global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
+  constexpr int BM = 256, BN = 256, TM = 4, TN = 2, WN = 4, WTN = 64;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_d[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave / WN) * 128, wn0 = (wave % WN) * WTN;
+
+  const int tiles_m = g.M / BM, tiles_n = g.N / BN;
+  int id = xcd_remap(blockIdx.x, gridDim.x);
+  constexpr int GROUP_M = 4;
+  const int group_size = GROUP_M * tiles_n;
+  const int first_m = (id / group_size) * GROUP_M;
+  const int gm = min(tiles_m - first_m, GROUP_M);
+  const int m0 = (first_m + (id % group_size) % gm) * BM;
+  const int n0 = ((id % group_size) / gm) * BN;
+
+  const uint16_t* A = reinterpret_cast<const uint16_t*>(g.a);
+  const uint16_t* B = reinterpret_cast<const uint16_t*>(g.b);
+
+  DirectCtx c;
+  c.ldb = g.ldb;
+  c.wave = wave;
+  const int r32 = lane & 31, h = lane >> 5;
+  c.h = h;
+  // Loader addressing.  A: load i of wave w fills rows (8 i + w) 8 .. +8 (1024 bytes); lane ->
+  // row += lane / 8, LDS chunk p = lane % 8 holds global chunk p ^ ((row / 2) % 8).
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int ar = (8 * i + wave) * 8 + (lane >> 3);
+    const int ac = (lane & 7) ^ ((ar >> 1) & 7);
+    c.a_src[i] = A + (int64_t)(m0 + ar) * g.lda + ac * 8;
+  }
+  // B: load i of wave w fills k rows (8 i + w) 2 .. +2; lane -> row += lane / 32, LDS chunk
+  // p = lane % 32 holds global chunk p ^ 4 (k % 4).
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int bk = (8 * i + wave) * 2 + (lane >> 5);
+    const int bc = (lane & 31) ^ (4 * (bk & 3));
+    c.b_src[i] = B + (int64_t)bk * g.ldb + n0 + bc * 8;
+  }
+  // A fragment (second MFMA operand): row wm0 + 32 j + r32, logical chunk 2 kc + h.
+#pragma unroll
+  for (int j = 0; j < TM; ++j) {
+    const int r = wm0 + 32 * j + r32;
+    c.a_off[j] = r * 128;
+    c.a_swz[j] = (r >> 1) & 7;
+  }
+  // B fragment (first MFMA operand) through the transposing read: lane (grp = lane / 16,
+  // j = lane % 16) addresses k row 16 ks + 8 h + j / 4 (+4 for the second read), columns
+  // wn0 + 32 i + 16 (grp % 2) + 4 (j % 4) .. +4.
+  {
+    const int j16 = lane & 15, grp = lane >> 4;
+    const int krow = 8 * h + (j16 >> 2);
+    const int col = wn0 + 16 * (grp & 1) + 4 * (j16 & 3);
+    c.b_chunk = col >> 3;
+    c.b_swz = 4 * (krow & 3);
+    c.b_off = krow * 512 + 8 * ((col >> 2) & 1);
+  }
+
+  f32x16 acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  const int nk = g.K / 32;  // even: K is a multiple of 64
+  uint8_t* const abuf = smem_d;
+  uint8_t* const bbuf = smem_d + kDirectBBase;
+  // Prologue: A stages 0, 1 and B stages 0 .. 3.
+  direct_load_a(c, 0, abuf);
+  if (nk > 2) direct_load_a(c, 1, abuf + kDirectABytes);
+#pragma unroll
+  for (int st = 0; st < 4; ++st)
+    if (st < nk) direct_load_b(c, st, bbuf + st * kDirectBBytes);
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  DirectFrags f0;
+  direct_read_frags(c, abuf, bbuf, 0, 0, f0);
+  int kt = 0;
+  for (; kt + 2 < nk; kt += 2) {
+    uint8_t* a_cur = abuf + ((kt >> 1) & 1) * kDirectABytes;
+    uint8_t* a_nxt = abuf + (((kt >> 1) + 1) & 1) * kDirectABytes;
+    uint8_t* b0 = bbuf + (kt & 3) * kDirectBBytes;
+    uint8_t* b1 = bbuf + ((kt + 1) & 3) * kDirectBBytes;
+    uint8_t* b2 = bbuf + ((kt + 2) & 3) * kDirectBBytes;
+    direct_step_pair<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
+  }
+  {
+    // Last two steps: nothing left to load; stage nk - 1 of B must have landed.
+    const uint8_t* a_cur = abuf + ((kt >> 1) & 1) * kDirectABytes;
+    const uint8_t* b0 = bbuf + (kt & 3) * kDirectBBytes;
+    const uint8_t* b1 = bbuf + ((kt + 1) & 3) * kDirectBBytes;
+    DirectFrags f1;
+    direct_read_frags(c, a_cur, b0, 1, 1, f1);
+    direct_mfma<DT>(acc, f0);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" LH_BAR ::: "memory");
+    direct_read_frags(c, a_cur, b1, 2, 0, f0);
+    direct_mfma<DT>(acc, f1);
+    direct_read_frags(c, a_cur, b1, 3, 1, f1);
+    direct_mfma<DT>(acc, f0);
+    direct_mfma<DT>(acc, f1);
+  }
+
+  const int m_base = m0 + wm0 + r32;
+  const int n_base = n0 + wn0 + 4 * h;
+  if (g.out_dt != LH_F32 && !(g.flags & LH_GEMM_ACCUMULATE_C)) {
+    // 16-bit output: stage the wave's 128 x 64 sub-tile in LDS (row stride 136 bytes keeps the
+    // 8-byte writes of 32 rows on distinct banks) and store full 128-byte row segments.
+    constexpr int cstride = WTN * 2 + 8;
+    static_assert(8 * 128 * cstride <= kDirectLdsBytes, "output staging must fit");
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the rings
+    uint8_t* cw = smem_d + wave * (128 * cstride);
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          u32x2 w = epilogue4_pack<DT>(g, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                                       acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+          *reinterpret_cast<u32x2*>(cw + (32 * j + r32) * cstride + (32 * i + 8 * q + 4 * h) * 2) = w;
+        }
+    uint16_t* outp = reinterpret_cast<uint16_t*>(g.out);
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      const int row = 8 * t + (lane >> 3), ch = lane & 7;
+      u32x4 w = *reinterpret_cast<const u32x4*>(cw + row * cstride + ch * 16);
+      *reinterpret_cast<u32x4*>(outp + (int64_t)(m0 + wm0 + row) * g.ldc + n0 + wn0 + ch * 8) = w;
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        epilogue4<DT>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                      acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+}
+
+template <int DT>
+static int launch_direct(const GemmArgs& g, hipStream_t s) {
+  auto kern = gemm16_direct<DT>;
+  constexpr size_t lds = kDirectLdsBytes;
+  static_assert(kDirectLdsBytes >= kDirectRingBytes, "rings must fit");
+  static bool configured = false;
+  if (!configured) {
+    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)lds));
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((g.M / 256) * (g.N / 256)), dim3(512), lds, s, g);
+  return check_launch("gemm16_direct");
+}
+
 // Any shape / stride / transpose; 64 x 64 x 32 tiles, 256 threads, bounds-checked.
 template <int DT>
 __global__ void __launch_bounds__(256) gemm16_generic(GemmArgs g) {
@@ -268,6 +586,7 @@ static int gemm16_dispatch(const GemmArgs& g, hipStream_t s) {
   if (vec_ok) {
     const int cus = 256;
     const bool big = g.M % 256 == 0 && g.N % 256 == 0 && (int64_t)(g.M / 256) * (g.N / 256) >= cus;
+    if (big && !tb && g.ldc % 8 == 0) return launch_direct<DT>(g, s);
     if (big) {
       return tb ? launch_fast<DT, 256, 256, 2, 4, true>(g, s) : launch_fast<DT, 256, 256, 2, 4, false>(g, s);
     }

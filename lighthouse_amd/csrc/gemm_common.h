@@ -68,6 +68,32 @@ __device__ __forceinline__ void epilogue4(const GemmArgs& g, int m, int n, float
   }
 }
 
+// Bias / activation / conversion for 4 consecutive columns of a 16-bit output, returned as two
+// packed dwords (no accumulator input); same order of operations as epilogue4.
+template <int DT>
+__device__ __forceinline__ u32x2 epilogue4_pack(const GemmArgs& g, int n, float v0, float v1, float v2, float v3) {
+  float v[4] = {v0 * g.alpha, v1 * g.alpha, v2 * g.alpha, v3 * g.alpha};
+  if (g.flags & LH_GEMM_HAS_BIAS) {
+    if (g.bias_dt == LH_F32) {
+      f32x4 bb = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.bias) + n);
+      v[0] += bb[0]; v[1] += bb[1]; v[2] += bb[2]; v[3] += bb[3];
+    } else {
+      u32x2 bb = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.bias) + n);
+      v[0] += unpack_lo<DT>(bb[0]); v[1] += unpack_hi<DT>(bb[0]);
+      v[2] += unpack_lo<DT>(bb[1]); v[3] += unpack_hi<DT>(bb[1]);
+    }
+  }
+  if (g.flags & LH_GEMM_HAS_GELU) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
+  }
+  if (g.flags & LH_GEMM_HAS_RELU) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
+  }
+  return u32x2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+}
+
 // One output element, any alignment (edge tiles and the generic kernels).
 template <int DT>
 __device__ __forceinline__ void epilogue1(const GemmArgs& g, int m, int n, float x) {
