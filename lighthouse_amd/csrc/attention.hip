@@ -5,18 +5,18 @@
 // accumulator live in f32; P is rounded to the element type before P.V; the row sum uses
 // the unrounded P; the output is acc / l rounded to the element type.
 //
-// Work split: a workgroup owns 128 query rows of one (batch, head); each of its 4 waves owns
-// 32 rows.  K/V tiles of 64 keys are staged through LDS (double buffered, one barrier per
-// tile) and shared by the 4 waves.
+// Work split (16-bit kernel): a workgroup owns 256 query rows of one (batch, head); each of its
+// 4 waves owns 64 rows.  K/V tiles of 64 keys are staged through a 4-deep LDS ring with
+// asynchronous global -> LDS loads and shared by the 4 waves, one barrier per tile.
 //
 // Both products are computed TRANSPOSED on the matrix cores: S^T = K Q^T and O^T = V^T P^T.
 // With the 32x32 MFMA accumulator layout a lane then owns ONE query row (column of S^T) and
 // 16 of its keys per tile, so the row max / row sum are register reductions plus a single
 // exchange between the two half-waves, the softmax state (m, l, alpha) is one scalar per
 // lane, and the S^T accumulator registers, converted to 16 bit, ARE the second operand of
-// the V^T P^T product (no LDS round trip or cross-lane shuffle for P).  V is transposed in
-// registers on its way into LDS, with the keys of every group of 16 stored in the order the
-// accumulator layout produces them.
+// the V^T P^T product (no LDS round trip or cross-lane shuffle for P).  V^T fragments are read
+// from the row-major V tile with the transposing LDS read, in the key order the accumulator
+// layout produces.
 #include "common.h"
 
 namespace lh {
@@ -45,170 +45,260 @@ __device__ __forceinline__ f32x16 mfma16(u32x4 a, u32x4 b, f32x16 c) {
 
 constexpr int kHeadDim = 64;
 constexpr int kKvTile = 64;
-constexpr int kQBlock = 128;
-constexpr int kAttnStride = 72;  // 16-bit elements per LDS row (64 + 8 pad)
+constexpr int kQBlock = 128;        // query rows per workgroup of the f32 kernel
+constexpr int kQBlock16 = 256;      // query rows per workgroup of the 16-bit kernel (4 waves x 64)
+constexpr int kAttnStages = 4;      // K/V ring depth
+constexpr int kAttnStageBytes = 2 * kKvTile * kHeadDim * 2;  // K tile + V tile, 16 KiB
 
+typedef __attribute__((address_space(3))) void attn_lds_void_t;
+typedef short attn_s16x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// v_permlane32_swap exchanges lanes 32..63 of its first operand with lanes 0..31 of its second.
+// Fed the same value twice it leaves (low half, low half) in the first and (high half, high
+// half) in the second register, so combining the two gives every lane f(x[lane], x[lane ^ 32]).
+// Written as inline asm (with the wait states the instruction needs after a VALU write of its
+// operands): the compiler builtin mis-assigns the second result register.
+__device__ __forceinline__ void halfwave_swap(float& lo, float& hi) {
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+}
+__device__ __forceinline__ float halfwave_max(float x) {
+  float a = x, b = x;
+  halfwave_swap(a, b);
+  return fmaxf(a, b);
+}
+__device__ __forceinline__ float halfwave_sum(float x) {
+  float a = x, b = x;
+  halfwave_swap(a, b);
+  return a + b;
+}
+
+struct AttnCtx {
+  const uint16_t* k_src[2];  // lane's source of K load i at key 0
+  const uint16_t* v_src[2];
+  int64_t k_step, v_step;    // elements per key tile
+  int wave, r32, h;
+  int k_off[2], k_swz[2];    // K fragment: byte offset of the lane's row, its swizzle, per key sub-tile
+  int v_off, v_swz;          // V fragment through the transposing read
+};
+
+__device__ __forceinline__ void attn_issue_loads(const AttnCtx& c, int jt, uint8_t* __restrict__ stage) {
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    __builtin_amdgcn_global_load_lds(c.k_src[i] + jt * c.k_step, (attn_lds_void_t*)(stage + (4 * i + c.wave) * 1024),
+                                     16, 0, 0);
+    __builtin_amdgcn_global_load_lds(c.v_src[i] + jt * c.v_step,
+                                     (attn_lds_void_t*)(stage + 8192 + (4 * i + c.wave) * 1024), 16, 0, 0);
+  }
+}
+
+// One key tile (64 keys) for the wave's two 32-row query sub-tiles.  `rd` holds the tile, `wr`
+// is the ring slot that receives a later tile meanwhile (separate restrict pointers so that LDS
+// reads do not wait for the asynchronous writes).
 template <int DT>
-__global__ void __launch_bounds__(256) attention16_kernel(AttnArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][kKvTile * kAttnStride];   // [key][d]
-  __shared__ __attribute__((aligned(16))) uint16_t Vts[2][kHeadDim * kAttnStride];  // [d][key slot]
+__device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, const u32x4 (&qf)[2][4],
+                                          f32x16 (&acc_o)[2][2], float (&m_run)[2], float (&l_run)[2],
+                                          const uint8_t* __restrict__ rd, uint8_t* __restrict__ wr, int next_jt,
+                                          bool prefetch, int j0, int wq0, bool active, bool need_mask) {
+  if (prefetch) attn_issue_loads(c, next_jt, wr);
+  if (!active) return;
+  const uint8_t* ks = rd;
+  const uint8_t* vs = rd + 8192;
+  // S^T = K Q^T: key sub-tile i (32 keys) x query sub-tile qt (32 rows).
+  f32x16 s_acc[2][2];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s_acc[qt][i][v] = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int sd = 0; sd < 4; ++sd) {
+      u32x4 kf = *reinterpret_cast<const u32x4*>(ks + c.k_off[i] + (((2 * sd + c.h) ^ c.k_swz[i]) << 4));
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) s_acc[qt][i] = mfma16<DT>(kf, qf[qt][sd], s_acc[qt][i]);
+    }
+  // s_acc[qt][i][v] = S[q = wq0 + 32 qt + r32][key = j0 + 32 i + 8 (v/4) + 4 h + v%4] (unscaled)
+  u32x4 pf[2][2][2];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    if (need_mask) {
+      const int qrow = wq0 + 32 * qt + c.r32;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          int key = j0 + 32 * i + 8 * (v >> 2) + 4 * c.h + (v & 3);
+          if (key > qrow) s_acc[qt][i][v] = -INFINITY;
+        }
+    }
+    float mx = fmaxf(s_acc[qt][0][0], s_acc[qt][1][0]);
+#pragma unroll
+    for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[qt][0][v]), s_acc[qt][1][v]);
+    mx = halfwave_max(mx);
+    const float m_new = fmaxf(m_run[qt], mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+    const float mc = m_safe * a.scale_log2e;
+    const float alpha = exp2_fast(m_run[qt] * a.scale_log2e - mc);
+    float l_tile = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      float p[16];
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        p[v] = exp2_fast(s_acc[qt][i][v] * a.scale_log2e - mc);
+        l_tile += p[v];
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int d = 0; d < 4; ++d) pf[qt][i][u][d] = pack2<DT>(p[8 * u + 2 * d], p[8 * u + 2 * d + 1]);
+    }
+    l_run[qt] = l_run[qt] * alpha + l_tile;
+    m_run[qt] = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc_o[qt][j][v] *= alpha;
+    }
+  }
+  // O^T += V^T P^T: head-dim sub-tile j (32 of d) x query sub-tile qt, over 4 k-steps of 16 keys.
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const uint8_t* p0 = vs + (32 * i + 16 * u) * 128 + c.v_off + (((4 * j) ^ c.v_swz) << 4);
+        attn_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) attn_s16x4*)p0);
+        attn_s16x4 hi =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) attn_s16x4*)(p0 + 8 * 128));
+        u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        u32x4 vf = {l2[0], l2[1], h2[0], h2[1]};
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) acc_o[qt][j] = mfma16<DT>(vf, pf[qt][i][u], acc_o[qt][j]);
+      }
+}
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+// 16-bit kernel.  A workgroup owns 256 query rows of one (batch, head): 4 waves x 64 rows (two
+// 32-row sub-tiles per wave share every K and V fragment).  K/V tiles of 64 keys go global ->
+// LDS with global_load_lds_dwordx4 through a ring of 4 stages; K fragments are 16-byte LDS
+// reads, V^T fragments come from ds_read_b64_tr_b16 on the row-major V tile.  Rows of a tile
+// are 128 bytes and cannot be padded (a wave-wide load writes 1 KiB contiguous), so the
+// 16-byte chunk a lane fetches is XOR-swizzled: K chunk ^ ((key / 2) % 8), V chunk ^ 4 ((key / 2) % 2).
+template <int DT>
+__global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, h = lane >> 5;
-  const int nqb = a.T / kQBlock;
+  const int nqb = (a.T + kQBlock16 - 1) / kQBlock16;
   // Causal: the last query blocks have the most key tiles; start them first.
   const int qb = a.causal ? (nqb - 1 - (int)blockIdx.x) : (int)blockIdx.x;
   const int bh = blockIdx.y;
   const int z = bh / a.H, hd = bh % a.H;
-  const int q0 = qb * kQBlock;
-  const int wq0 = q0 + wave * 32;
+  const int q0 = qb * kQBlock16;
+  const int wq0 = q0 + wave * 64;
+  // T is a multiple of 64: a wave's 64 rows are all inside the sequence or all outside (last
+  // workgroup only); an outside wave still takes part in the loads and barriers.
+  const bool wave_valid = wq0 < a.T;
+  const int wq_load = wave_valid ? wq0 : 0;
 
   const uint16_t* Q = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)z * a.sq.z + (int64_t)hd * a.sq.h;
   const uint16_t* K = reinterpret_cast<const uint16_t*>(a.k) + (int64_t)z * a.sk.z + (int64_t)hd * a.sk.h;
   const uint16_t* V = reinterpret_cast<const uint16_t*>(a.v) + (int64_t)z * a.sv.z + (int64_t)hd * a.sv.h;
   uint16_t* O = reinterpret_cast<uint16_t*>(a.out) + (int64_t)z * a.so.z + (int64_t)hd * a.so.h;
 
-  // Q fragment: second MFMA operand of S^T = K Q^T; lane (q = r32, half h) holds
-  // Q[q][16s + 8h .. +8] for the 4 k-steps s over the head dimension.
-  u32x4 qf[4];
+  AttnCtx c;
+  c.wave = wave; c.r32 = r32; c.h = h;
+  c.k_step = (int64_t)kKvTile * a.sk.t;
+  c.v_step = (int64_t)kKvTile * a.sv.t;
+  // Loader: load i of wave w fills keys (4 i + w) 8 .. +8 of the tile; lane -> key += lane / 8,
+  // LDS chunk p = lane % 8 holds global chunk p ^ swizzle(key).
 #pragma unroll
-  for (int s = 0; s < 4; ++s)
-    qf[s] = *reinterpret_cast<const u32x4*>(Q + (int64_t)(wq0 + r32) * a.sq.t + 16 * s + 8 * h);
+  for (int i = 0; i < 2; ++i) {
+    const int key = (4 * i + wave) * 8 + (lane >> 3);
+    const int p = lane & 7;
+    c.k_src[i] = K + (int64_t)key * a.sk.t + ((p ^ ((key >> 1) & 7)) << 3);
+    c.v_src[i] = V + (int64_t)key * a.sv.t + ((p ^ (4 * ((key >> 1) & 1))) << 3);
+  }
+  // K fragment (first MFMA operand of S^T): key 32 i + r32, logical chunk 2 sd + h.
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int key = 32 * i + r32;
+    c.k_off[i] = key * 128;
+    c.k_swz[i] = (key >> 1) & 7;
+  }
+  // V^T fragment (first MFMA operand of O^T) through the transposing read.  Lane (grp = lane/16,
+  // j16 = lane % 16) addresses key row 4 h + j16 / 4 of the k-step (+8 for the second read),
+  // head-dim columns 32 j + 16 (grp % 2) + 4 (j16 % 4) .. +4.  The slot order of the 8 values a
+  // lane receives (keys 4h..4h+3, then 8+4h..8+4h+3) is exactly the key order of the packed
+  // S^T accumulator registers it is multiplied with.
+  {
+    const int j16 = lane & 15, grp = lane >> 4;
+    const int krow = 4 * h + (j16 >> 2);
+    const int col = 16 * (grp & 1) + 4 * (j16 & 3);
+    c.v_swz = 4 * ((krow >> 1) & 1);  // unchanged by + 8, + 16 u, + 32 i
+    c.v_off = krow * 128 + 8 * ((col >> 2) & 1) + (((col >> 3) ^ 0) << 4);
+  }
+  // Q fragments: second MFMA operand of S^T = K Q^T; lane (q = r32, half h) holds
+  // Q[q][16 sd + 8 h .. +8] for the 4 k-steps over the head dimension, for both sub-tiles.
+  u32x4 qf[2][4];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+    for (int sd = 0; sd < 4; ++sd)
+      qf[qt][sd] = *reinterpret_cast<const u32x4*>(Q + (int64_t)(wq_load + 32 * qt + r32) * a.sq.t + 16 * sd + 8 * h);
 
-  // Global -> register staging of one K/V tile.
-  u32x4 rk[2];
-  u32x2 rv[4];
-  const int k_row = tid >> 3, k_chunk = tid & 7;  // + 32 rows for the second chunk
-  const int v_dgrp = tid & 15, v_kq = tid >> 4;   // 4 keys x 4 d per thread
-  auto load_tile = [&](int j0) {
+  f32x16 acc_o[2][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      rk[i] = *reinterpret_cast<const u32x4*>(K + (int64_t)(j0 + k_row + 32 * i) * a.sk.t + k_chunk * 8);
+  for (int qt = 0; qt < 2; ++qt)
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      rv[r] = *reinterpret_cast<const u32x2*>(V + (int64_t)(j0 + 4 * v_kq + r) * a.sv.t + v_dgrp * 4);
-  };
-  auto store_tile = [&](int buf) {
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      *reinterpret_cast<u32x4*>(&Ks[buf][(k_row + 32 * i) * kAttnStride + k_chunk * 8]) = rk[i];
-    // Keys 4*kq .. 4*kq+3 of this thread go to slot 16*(kq/4) + 8*(kq%2) + 4*((kq%4)/2) + r:
-    // within each group of 16 keys the order is the one the S^T accumulator produces.
-    const int slot = 16 * (v_kq >> 2) + 8 * (v_kq & 1) + 4 * ((v_kq & 3) >> 1);
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
-      u32x2 w;
-      w[0] = __builtin_amdgcn_perm(rv[1][c >> 1], rv[0][c >> 1], sel);
-      w[1] = __builtin_amdgcn_perm(rv[3][c >> 1], rv[2][c >> 1], sel);
-      *reinterpret_cast<u32x2*>(&Vts[buf][(v_dgrp * 4 + c) * kAttnStride + slot]) = w;
-    }
-  };
+      for (int v = 0; v < 16; ++v) acc_o[qt][j][v] = 0.0f;
+  float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.0f, 0.0f};
 
-  f32x16 acc_o[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc_o[j][v] = 0.0f;
-  float m_run = -INFINITY, l_run = 0.0f;
-
-  const int kv_end = a.causal ? min(a.T, q0 + kQBlock) : a.T;
+  const int kv_end = a.causal ? min(a.T, q0 + kQBlock16) : a.T;
   const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
+#pragma unroll
+  for (int st = 0; st < kAttnStages - 1; ++st)
+    if (st < ntiles) attn_issue_loads(c, st, smem_attn + st * kAttnStageBytes);
 
   for (int jt = 0; jt < ntiles; ++jt) {
-    const int buf = jt & 1;
+    // 4 loads per lane and stage; the 2 younger stages may stay in flight.  One asm block: a
+    // __syncthreads() would add a fence that waits for ALL outstanding loads.
+    const int younger = min(ntiles - 1 - jt, kAttnStages - 2);
+    if (younger >= 2) asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+    else if (younger == 1) asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     const int j0 = jt * kKvTile;
-    if (jt + 1 < ntiles) load_tile(j0 + kKvTile);
-
-    // A wave whose 32 rows all precede this tile has nothing to do in it (causal only).
-    const bool active = !a.causal || (j0 <= wq0 + 31);
-    if (active) {
-      f32x16 s_acc[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-#pragma unroll
-        for (int v = 0; v < 16; ++v) s_acc[i][v] = 0.0f;
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          u32x4 kf = *reinterpret_cast<const u32x4*>(&Ks[buf][(32 * i + r32) * kAttnStride + 16 * s + 8 * h]);
-          s_acc[i] = mfma16<DT>(kf, qf[s], s_acc[i]);
-        }
-      }
-      // s_acc[i][v] = S[q = wq0 + r32][key = j0 + 32 i + 8 (v/4) + 4 h + v%4] (unscaled)
-      if (a.causal && (j0 + kKvTile - 1 > wq0)) {
-        const int qrow = wq0 + r32;
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            int key = j0 + 32 * i + 8 * (v >> 2) + 4 * h + (v & 3);
-            if (key > qrow) s_acc[i][v] = -INFINITY;
-          }
-      }
-      float mx = s_acc[0][0];
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s_acc[i][v]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run, mx);
-      const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-      const float mc = m_safe * a.scale_log2e;
-      const float alpha = exp2f(m_run * a.scale_log2e - mc);
-      float l_tile = 0.0f;
-      u32x4 pf[2][2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        float p[16];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          p[v] = exp2f(s_acc[i][v] * a.scale_log2e - mc);
-          l_tile += p[v];
-        }
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-          for (int d = 0; d < 4; ++d) pf[i][u][d] = pack2<DT>(p[8 * u + 2 * d], p[8 * u + 2 * d + 1]);
-      }
-      l_run = l_run * alpha + l_tile;
-      m_run = m_new;
-      if (alpha != 1.0f) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) acc_o[j][v] *= alpha;
-      }
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            u32x4 vf =
-                *reinterpret_cast<const u32x4*>(&Vts[buf][(32 * j + r32) * kAttnStride + 32 * i + 16 * u + 8 * h]);
-            acc_o[j] = mfma16<DT>(vf, pf[i][u], acc_o[j]);
-          }
-    }
-
-    if (jt + 1 < ntiles) store_tile(buf ^ 1);
-    __syncthreads();
+    const bool active = wave_valid && (!a.causal || (j0 <= wq0 + 63));
+    const bool need_mask = a.causal && (j0 + kKvTile - 1 > wq0);
+    const int nxt = jt + kAttnStages - 1;
+    attn_tile<DT>(c, a, qf, acc_o, m_run, l_run, smem_attn + (jt % kAttnStages) * kAttnStageBytes,
+                  smem_attn + (nxt % kAttnStages) * kAttnStageBytes, nxt, nxt < ntiles, j0, wq0, active, need_mask);
   }
 
-  // acc_o[j][v] = O[q = wq0 + r32][d = 32 j + 8 (v/4) + 4 h + v%4] * l
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-  const float inv_l = 1.0f / l_tot;
-  uint16_t* orow = O + (int64_t)(wq0 + r32) * a.so.t;
+  // acc_o[qt][j][v] = O[q = wq0 + 32 qt + r32][d = 32 j + 8 (v/4) + 4 h + v%4] * l
+  if (!wave_valid) return;
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int qt = 0; qt < 2; ++qt) {
+    const float inv_l = 1.0f / halfwave_sum(l_run[qt]);
+    uint16_t* orow = O + (int64_t)(wq0 + 32 * qt + r32) * a.so.t;
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      u32x2 w = {pack2<DT>(acc_o[j][4 * g] * inv_l, acc_o[j][4 * g + 1] * inv_l),
-                 pack2<DT>(acc_o[j][4 * g + 2] * inv_l, acc_o[j][4 * g + 3] * inv_l)};
-      *reinterpret_cast<u32x2*>(orow + 32 * j + 8 * g + 4 * h) = w;
-    }
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w = {pack2<DT>(acc_o[qt][j][4 * g] * inv_l, acc_o[qt][j][4 * g + 1] * inv_l),
+                   pack2<DT>(acc_o[qt][j][4 * g + 2] * inv_l, acc_o[qt][j][4 * g + 3] * inv_l)};
+        *reinterpret_cast<u32x2*>(orow + 32 * j + 8 * g + 4 * h) = w;
+      }
+  }
 }
 
 // f32 variant (all tensors f32, f32 MFMA): same structure; P stays f32, K and V tiles keep
@@ -329,12 +419,25 @@ __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
     }
 }
 
+template <int DT>
+static int attention16_launch(const AttnArgs& a, hipStream_t s) {
+  auto kern = attention16_kernel<DT>;
+  constexpr size_t lds = (size_t)kAttnStages * kAttnStageBytes;
+  static bool configured = false;
+  if (!configured) {
+    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)lds));
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((a.T + kQBlock16 - 1) / kQBlock16, a.Z * a.H), dim3(256), lds, s, a);
+  return check_launch("attention16");
+}
+
 int attention_launch(const AttnArgs& a, int dtype, hipStream_t s) {
-  dim3 grid(a.T / kQBlock, a.Z * a.H);
-  if (dtype == LH_BF16) hipLaunchKernelGGL(attention16_kernel<LH_BF16>, grid, dim3(256), 0, s, a);
-  else if (dtype == LH_F16) hipLaunchKernelGGL(attention16_kernel<LH_F16>, grid, dim3(256), 0, s, a);
-  else hipLaunchKernelGGL(attention32_kernel, grid, dim3(256), 0, s, a);
-  return check_launch("attention");
+  if (dtype == LH_BF16) return attention16_launch<LH_BF16>(a, s);
+  if (dtype == LH_F16) return attention16_launch<LH_F16>(a, s);
+  hipLaunchKernelGGL(attention32_kernel, dim3(a.T / kQBlock, a.Z * a.H), dim3(256), 0, s, a);
+  return check_launch("attention32");
 }
 
 }  // namespace lh
@@ -349,8 +452,9 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   LH_REQUIRE(Z > 0 && H > 0 && T > 0, "lh_hip_attention: empty problem Z=%lld H=%lld T=%lld", (long long)Z,
              (long long)H, (long long)T);
   if (d != kHeadDim) return fail(LH_ERR_UNSUPPORTED, "lh_hip_attention: head_dim %lld not supported (only 64)", (long long)d);
-  if (T % kQBlock != 0)
-    return fail(LH_ERR_UNSUPPORTED, "lh_hip_attention: seq_len %lld must be a multiple of %d", (long long)T, kQBlock);
+  const int qblock = (dtype == LH_F32) ? kQBlock : kKvTile;
+  if (T % qblock != 0)
+    return fail(LH_ERR_UNSUPPORTED, "lh_hip_attention: seq_len %lld must be a multiple of %d", (long long)T, qblock);
   LH_REQUIRE(Z * H <= 65535 && T < (1 << 30), "lh_hip_attention: problem too large");
   const int vec = (dtype == LH_F32) ? 4 : 8;  // elements per 16-byte access
   const lh_strides3* ss[4] = {&so, &sq, &sk, &sv};

@@ -65,10 +65,7 @@ typedef int32_t i32x8 __attribute__((ext_vector_type(8)));
 // ---- scalar conversions (device) ----------------------------------------------
 // float -> bfloat16 bits, round to nearest even, quiet NaN (arith.truncf semantics).
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  uint32_t r = u + 0x7fffu + ((u >> 16) & 1u);
-  r = (f != f) ? (u | 0x00400000u) : r;
-  return (uint16_t)(r >> 16);
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
 }
 __device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) {
   return __builtin_bit_cast(float, (uint32_t)h << 16);
@@ -81,13 +78,17 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t b) {
   return (float)__builtin_bit_cast(_Float16, b);
 }
 
-// Pack two floats into one dword of two 16-bit values (lo = a, hi = b).
+// Pack two floats into one dword of two 16-bit values (lo = a, hi = b), round to nearest
+// even; one v_cvt_pk_bf16_f32 for bf16.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 template <int DT>
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
+  f32x2 v = {a, b};
   if constexpr (DT == LH_BF16) {
-    return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
   } else {
-    return (uint32_t)f32_to_f16_bits(a) | ((uint32_t)f32_to_f16_bits(b) << 16);
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
   }
 }
 template <int DT>
