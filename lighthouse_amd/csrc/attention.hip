@@ -35,6 +35,11 @@ struct AttnArgs {
 
 template <int DT>
 __device__ __forceinline__ f32x16 mfma16(u32x4 a, u32x4 b, f32x16 c) {
+#ifdef LH_AEXP_NO_MFMA
+  asm volatile("" ::"v"(a), "v"(b));
+  c[0] += __builtin_bit_cast(float, a[0]);
+  return c;
+#endif
   if constexpr (DT == LH_BF16)
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
                                                    0, 0);
@@ -135,14 +140,38 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
           if (key > qrow) s_acc[qt][i][v] = -INFINITY;
         }
     }
+#ifdef LH_AEXP_NO_SOFTMAX
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          pf[qt][i][u][d] = __builtin_bit_cast(uint32_t, s_acc[qt][i][8 * u + 2 * d]) ^
+                            __builtin_bit_cast(uint32_t, s_acc[qt][i][8 * u + 2 * d + 1]);
+    continue;
+#endif
     float mx = fmaxf(s_acc[qt][0][0], s_acc[qt][1][0]);
 #pragma unroll
     for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[qt][0][v]), s_acc[qt][1][v]);
     mx = halfwave_max(mx);
-    const float m_new = fmaxf(m_run[qt], mx);
-    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-    const float mc = m_safe * a.scale_log2e;
-    const float alpha = exp2_fast(m_run[qt] * a.scale_log2e - mc);
+    // Deferred rescaling: m_run is the offset in use, not necessarily the running maximum.  It
+    // is raised (and l, acc rescaled by alpha) only when some row of the wave has grown past it
+    // by more than 2^8 after scaling; until then P = exp(S - m_run) stays below 256, exactly as
+    // accurate in 16 bit as values below 1, and softmax does not depend on the offset.
+    const bool grow = (mx - m_run[qt]) * a.scale_log2e > 8.0f;
+    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
+      const float m_new = fmaxf(m_run[qt], mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+      const float alpha = exp2_fast((m_run[qt] - m_safe) * a.scale_log2e);
+      l_run[qt] *= alpha;
+      m_run[qt] = m_new;
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc_o[qt][j][v] *= alpha;
+    }
+    const float mc = ((m_run[qt] == -INFINITY) ? 0.0f : m_run[qt]) * a.scale_log2e;
     float l_tile = 0.0f;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -157,14 +186,7 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
 #pragma unroll
         for (int d = 0; d < 4; ++d) pf[qt][i][u][d] = pack2<DT>(p[8 * u + 2 * d], p[8 * u + 2 * d + 1]);
     }
-    l_run[qt] = l_run[qt] * alpha + l_tile;
-    m_run[qt] = m_new;
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc_o[qt][j][v] *= alpha;
-    }
+    l_run[qt] += l_tile;
   }
   // O^T += V^T P^T: head-dim sub-tile j (32 of d) x query sub-tile qt, over 4 k-steps of 16 keys.
 #pragma unroll

@@ -119,6 +119,8 @@ class Runner:
         if len(buffers) != len(fn.args):
             raise ValueError(f"function '{fn.name}' takes {len(fn.args)} buffers, got {len(buffers)}")
         for i, (spec, buf) in enumerate(zip(fn.args, buffers)):
+            if not hasattr(buf, "shape") or not hasattr(buf, "dtype"):
+                raise ValueError(f"argument {i} of '{fn.name}' is not an array or tensor: {type(buf).__name__}")
             shape = tuple(buf.shape)
             if shape != tuple(spec.shape):
                 raise ValueError(f"argument {i} of '{fn.name}' has shape {shape}, expected {tuple(spec.shape)}")
