@@ -86,6 +86,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--only", choices=["gemm_bf16", "attention", "copy"], default=None,
+                    help="profiling aid: run just this kernel --steps times and exit (no JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (one MI355X per box); use --gpus 1",
@@ -97,6 +99,24 @@ def main() -> int:
     from lighthouse_amd import ops
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if args.only == "copy":
+        # Calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain copy of 256 MiB
+        # (lh_hip_cast f32 -> f32 reads and writes every byte exactly once).
+        src = torch.ones(64 * 1024 * 1024, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(args.steps):
+            ops.cast(src, torch.float32, out=dst)
+        torch.cuda.synchronize()
+        return 0
+    if args.only == "attention":
+        g = torch.Generator(device="cuda").manual_seed(3)
+        q, k, v = (torch.randn((4, 16, 2048, 64), device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
+        o = torch.empty_like(q)
+        for _ in range(args.steps):
+            ops.attention(q, k, v, out=o)
+            ops.attention(q, k, v, causal=True, out=o)
+        torch.cuda.synchronize()
+        return 0
     n = 4096
     g = torch.Generator(device="cuda").manual_seed(0xC0FFEE + 2)
     a = torch.randn(n, n, device="cuda", generator=g).to(torch.bfloat16)
@@ -104,6 +124,11 @@ def main() -> int:
     bias = torch.randn(n, device="cuda", generator=g).to(torch.bfloat16)
     out = torch.empty(n, n, device="cuda", dtype=torch.bfloat16)
 
+    if args.only == "gemm_bf16":
+        for _ in range(args.steps):
+            ops.gemm(a, b, out=out)
+        torch.cuda.synchronize()
+        return 0
     flops = 2.0 * n * n * n
     wall, ev = time_region(lambda: ops.gemm(a, b, out=out), args.steps, args.warmup)
     value = flops * args.steps / wall / 1e12
