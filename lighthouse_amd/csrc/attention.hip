@@ -35,11 +35,6 @@ struct AttnArgs {
 
 template <int DT>
 __device__ __forceinline__ f32x16 mfma16(u32x4 a, u32x4 b, f32x16 c) {
-#ifdef LH_AEXP_NO_MFMA
-  asm volatile("" ::"v"(a), "v"(b));
-  c[0] += __builtin_bit_cast(float, a[0]);
-  return c;
-#endif
   if constexpr (DT == LH_BF16)
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
                                                    0, 0);
@@ -140,17 +135,6 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
           if (key > qrow) s_acc[qt][i][v] = -INFINITY;
         }
     }
-#ifdef LH_AEXP_NO_SOFTMAX
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int d = 0; d < 4; ++d)
-          pf[qt][i][u][d] = __builtin_bit_cast(uint32_t, s_acc[qt][i][8 * u + 2 * d]) ^
-                            __builtin_bit_cast(uint32_t, s_acc[qt][i][8 * u + 2 * d + 1]);
-    continue;
-#endif
     float mx = fmaxf(s_acc[qt][0][0], s_acc[qt][1][0]);
 #pragma unroll
     for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[qt][0][v]), s_acc[qt][1][v]);
@@ -219,9 +203,26 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, h = lane >> 5;
   const int nqb = (a.T + kQBlock16 - 1) / kQBlock16;
-  // Causal: the last query blocks have the most key tiles; start them first.
-  const int qb = a.causal ? (nqb - 1 - (int)blockIdx.x) : (int)blockIdx.x;
-  const int bh = blockIdx.y;
+  int qb, bh;
+  if (a.causal) {
+    // Causal work grows with the query block index.  The 1-D grid lists the heavier half of the
+    // query blocks first (heaviest first), then the lighter half lightest first, so that
+    // workgroup L and workgroup L + gridDim/2 -- which share a CU when the whole grid is
+    // resident at two workgroups per CU -- always add up to the same number of key tiles.
+    const int bhn = a.Z * a.H;
+    const int L = blockIdx.x;
+    const int heavy = (nqb / 2) * bhn;  // workgroups in the heavy half
+    if (L < heavy) {
+      qb = nqb - 1 - L / bhn;
+      bh = L % bhn;
+    } else {
+      qb = (L - heavy) / bhn;
+      bh = (L - heavy) % bhn;
+    }
+  } else {
+    qb = blockIdx.x;
+    bh = blockIdx.y;
+  }
   const int z = bh / a.H, hd = bh % a.H;
   const int q0 = qb * kQBlock16;
   const int wq0 = q0 + wave * 64;
@@ -451,7 +452,9 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
                                      (int)lds));
     configured = true;
   }
-  hipLaunchKernelGGL(kern, dim3((a.T + kQBlock16 - 1) / kQBlock16, a.Z * a.H), dim3(256), lds, s, a);
+  const int nqb = (a.T + kQBlock16 - 1) / kQBlock16;
+  const dim3 grid = a.causal ? dim3(nqb * a.Z * a.H) : dim3(nqb, a.Z * a.H);
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, a);
   return check_launch("attention16");
 }
 

@@ -252,9 +252,6 @@ __device__ __forceinline__ void direct_load_b(const DirectCtx& c, int sb, uint8_
 // (0..1: which 16 of the stage's 32 k).
 __device__ __forceinline__ void direct_read_frags(const DirectCtx& c, const uint8_t* __restrict__ as,
                                                   const uint8_t* __restrict__ bs, int kc, int ks, DirectFrags& f) {
-#ifdef LH_EXP_NO_READS
-  if (ks >= 0) return;
-#endif
 #pragma unroll
   for (int j = 0; j < 4; ++j)
     f.a[j] = *reinterpret_cast<const u32x4*>(as + c.a_off[j] + (((2 * kc + c.h) ^ c.a_swz[j]) << 4));
@@ -271,20 +268,14 @@ __device__ __forceinline__ void direct_read_frags(const DirectCtx& c, const uint
 
 template <int DT>
 __device__ __forceinline__ void direct_mfma(f32x16 (&acc)[2][4], const DirectFrags& f) {
-#ifdef LH_EXP_NO_MFMA
-#pragma unroll
-  for (int j = 0; j < 4; ++j) asm volatile("" ::"v"(f.a[j]));
-#pragma unroll
-  for (int i = 0; i < 2; ++i) asm volatile("" ::"v"(f.b[i]));
-  return;
-#endif
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = Mfma16<DT>::mma(f.b[i], f.a[j], acc[i][j]);
 }
 
-// Ask the scheduler to put one LDS read of the next k-half after each MFMA of the current one.
+// Scheduling hint for one k-half: where the 8 LDS reads of the NEXT k-half go relative to the 8
+// MFMAs of the current one.
 __device__ __forceinline__ void direct_interleave_hint() {
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -293,19 +284,14 @@ __device__ __forceinline__ void direct_interleave_hint() {
   }
 }
 
-#ifdef LH_EXP_NO_BARRIER
-#define LH_BAR ""
-#else
-#define LH_BAR "\n\ts_barrier"
-#endif
 
 // Wait until at most `allowed` of this wave's loads are still in flight and all its LDS reads
 // have returned, then barrier.  One asm block: a __syncthreads() would add a release fence,
 // i.e. a wait for ALL outstanding loads, and drain the rings.
 __device__ __forceinline__ void direct_wait_barrier(int allowed) {
-  if (allowed >= 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" LH_BAR ::: "memory");
-  else if (allowed >= 4) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" LH_BAR ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" LH_BAR ::: "memory");
+  if (allowed >= 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  else if (allowed >= 4) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
 // Steps kt (even) and kt + 1 of the main loop; both have a successor step.  On entry f0 holds
@@ -332,9 +318,7 @@ __device__ __forceinline__ void direct_step_pair(const DirectCtx& c, f32x16 (&ac
   direct_mfma<DT>(acc, f0);
   direct_interleave_hint();
   direct_wait_barrier(steady ? 8 : 0);
-#ifndef LH_EXP_NO_LOADS
   if (kt + 4 < nk) direct_load_b(c, kt + 4, b_refill0);
-#endif
   direct_read_frags(c, a_cur, b1, 2, 0, f0);
   direct_mfma<DT>(acc, f1);
   direct_interleave_hint();
@@ -343,10 +327,8 @@ __device__ __forceinline__ void direct_step_pair(const DirectCtx& c, f32x16 (&ac
   direct_mfma<DT>(acc, f0);
   direct_interleave_hint();
   direct_wait_barrier(steady ? 4 : 0);
-#ifndef LH_EXP_NO_LOADS
   if (kt + 4 < nk) direct_load_a(c, kt / 2 + 2, a_refill);
   if (kt + 5 < nk) direct_load_b(c, kt + 5, b_refill1);
-#endif
   direct_read_frags(c, a_nxt, b2, 0, 0, f0);
   direct_mfma<DT>(acc, f1);
   direct_interleave_hint();
@@ -449,7 +431,7 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
     DirectFrags f1;
     direct_read_frags(c, a_cur, b0, 1, 1, f1);
     direct_mfma<DT>(acc, f0);
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" LH_BAR ::: "memory");
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     direct_read_frags(c, a_cur, b1, 2, 0, f0);
     direct_mfma<DT>(acc, f1);
     direct_read_frags(c, a_cur, b1, 3, 1, f1);

@@ -151,6 +151,259 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm8_fast(GemmArgs g) 
                            acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
 }
 
+// ---- direct-to-LDS kernel ---------------------------------------------------------------
+// Same structure as the 16-bit direct kernel: 256 x 256 workgroup tile, 8 waves (2 x 4, 128 x 64
+// per wave), panels global -> LDS with global_load_lds_dwordx4 in their global orientation, A ring
+// 2 stages x 128 k (256 rows x 128 bytes), B ring 4 stages x 64 k (64 rows x 256 bytes), one
+// v_mfma_f32_32x32x64_f8f6f4 k-step (64 k) per main-loop step with the barrier in the middle.
+// The k-contiguous A fragment (32 bytes per lane) is two 16-byte LDS reads; the n-contiguous B
+// panel is read with ds_read_b64_tr_b8, which hands a lane 8 k-values of one column (16 lanes
+// cover 8 k-rows x 16 columns), four reads per fragment.  Swizzles: A chunk ^ ((row / 2) % 8),
+// B chunk ^ 2 (k % 8).
+constexpr int kD8ABytes = 256 * 128;   // one A stage (128 k): 32 KiB
+constexpr int kD8BBytes = 64 * 256;    // one B stage (64 k): 16 KiB
+constexpr int kD8BBase = 2 * kD8ABytes;
+constexpr int kD8RingBytes = kD8BBase + 4 * kD8BBytes;  // 128 KiB
+constexpr int kD8LdsBytes = 8 * 128 * 136;              // bf16 output staging (139264) >= rings
+
+typedef __attribute__((address_space(3))) void lds8_void_t;
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ void async8_copy16(const void* gsrc, uint8_t* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(gsrc, (lds8_void_t*)lds_wave_base, 16, 0, 0);
+}
+
+struct D8Ctx {
+  const uint8_t* a_src[4];
+  const uint8_t* b_src[2];
+  int a_off[4], a_swz[4];
+  int64_t ldb;
+  int wave, h, b_off, b_chunk, b_swz;
+};
+
+struct D8Frags {
+  i32x8 a[4];
+  i32x8 b[2];
+};
+
+__device__ __forceinline__ void d8_load_a(const D8Ctx& c, int sa, uint8_t* __restrict__ abuf) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) async8_copy16(c.a_src[i] + sa * 128, abuf + (8 * i + c.wave) * 1024);
+}
+__device__ __forceinline__ void d8_load_b(const D8Ctx& c, int sb, uint8_t* __restrict__ bbuf) {
+#pragma unroll
+  for (int i = 0; i < 2; ++i) async8_copy16(c.b_src[i] + (int64_t)(sb * 64) * c.ldb, bbuf + (8 * i + c.wave) * 1024);
+}
+
+// Fragments of one 64-k step: A bytes 64 kb .. +64 of the stage's rows (kb = 0 / 1), B stage bs.
+__device__ __forceinline__ void d8_read_frags(const D8Ctx& c, const uint8_t* __restrict__ as,
+                                              const uint8_t* __restrict__ bs, int kb, D8Frags& f) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int c0 = 4 * kb + 2 * c.h;
+    i32x4 lo = *reinterpret_cast<const i32x4*>(as + c.a_off[j] + ((c0 ^ c.a_swz[j]) << 4));
+    i32x4 hi = *reinterpret_cast<const i32x4*>(as + c.a_off[j] + (((c0 + 1) ^ c.a_swz[j]) << 4));
+    f.a[j] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const uint8_t* p0 = bs + c.b_off + (((c.b_chunk + 2 * i) ^ c.b_swz) << 4);
+    i32x2 r[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      r[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(p0 + q * 8 * 256));
+    f.b[i] = i32x8{r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]};
+  }
+}
+
+__device__ __forceinline__ void d8_mfma(f32x16 (&acc)[2][4], const D8Frags& f) {
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = mfma_f8_32(f.b[i], f.a[j], acc[i][j]);
+}
+
+// 16 LDS reads of the next step spread over the 8 MFMAs of the current one.
+__device__ __forceinline__ void d8_interleave_hint() {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+  }
+}
+
+__device__ __forceinline__ void d8_wait_barrier(int allowed) {
+  if (allowed >= 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  else if (allowed >= 4) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+// Steps kt (even) and kt + 1.  f holds the fragments of step kt on entry and of step kt + 2 on
+// exit.  Unlike the 16-bit kernel a step is a single MFMA k-step, so the fragments of the next
+// step are read (into g) while the current ones are multiplied; the barrier that makes the next
+// B stage visible therefore comes BEFORE the step's MFMAs:
+//   barrier(kt): B(kt+1) landed (and A for odd -> even transitions); refill B slot of kt-1...
+// To keep the LDS-DMA accounting identical to the 16-bit kernel the refills are issued for the
+// stage that was finished one step earlier (its reads completed before this barrier).
+__device__ __forceinline__ void d8_step_pair(const D8Ctx& c, f32x16 (&acc)[2][4], D8Frags& f,
+                                             const uint8_t* __restrict__ a_cur, const uint8_t* __restrict__ a_nxt,
+                                             const uint8_t* __restrict__ b1, const uint8_t* __restrict__ b2,
+                                             uint8_t* __restrict__ a_refill, uint8_t* __restrict__ b_refill0,
+                                             uint8_t* __restrict__ b_refill1, int kt, int nk) {
+  D8Frags g;
+  const bool steady = kt + 6 < nk;
+  // ---- even step kt: fragments f (read earlier).  Stage kt of B and the first half of a_cur are
+  // no longer needed by this wave once f is in registers.
+  d8_wait_barrier(steady ? 8 : 0);   // B(kt+1) landed for everyone; everyone holds step kt in registers
+  if (kt + 4 < nk) d8_load_b(c, kt + 4, b_refill0);
+  d8_read_frags(c, a_cur, b1, 1, g);  // step kt + 1
+  d8_mfma(acc, f);
+  d8_interleave_hint();
+  // ---- odd step kt + 1: fragments g.
+  d8_wait_barrier(steady ? 4 : 0);   // A stage kt/2 + 1 and B(kt+2) landed; a_cur and B(kt+1) are free
+  if (kt + 4 < nk) d8_load_a(c, kt / 2 + 2, a_refill);
+  if (kt + 5 < nk) d8_load_b(c, kt + 5, b_refill1);
+  d8_read_frags(c, a_nxt, b2, 0, f);  // step kt + 2
+  d8_mfma(acc, g);
+  d8_interleave_hint();
+}
+
+__global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
+  constexpr int BM = 256, BN = 256, TM = 4, TN = 2, WN = 4, WTN = 64;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_8[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave / WN) * 128, wn0 = (wave % WN) * WTN;
+  const int tiles_m = g.M / BM, tiles_n = g.N / BN;
+  int id = xcd_remap(blockIdx.x, gridDim.x);
+  constexpr int GROUP_M = 4;
+  const int group_size = GROUP_M * tiles_n;
+  const int first_m = (id / group_size) * GROUP_M;
+  const int gm = min(tiles_m - first_m, GROUP_M);
+  const int m0 = (first_m + (id % group_size) % gm) * BM;
+  const int n0 = ((id % group_size) / gm) * BN;
+  const uint8_t* A = reinterpret_cast<const uint8_t*>(g.a);
+  const uint8_t* B = reinterpret_cast<const uint8_t*>(g.b);
+
+  D8Ctx c;
+  c.ldb = g.ldb;
+  c.wave = wave;
+  const int r32 = lane & 31, h = lane >> 5;
+  c.h = h;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int ar = (8 * i + wave) * 8 + (lane >> 3);
+    const int ac = (lane & 7) ^ ((ar >> 1) & 7);
+    c.a_src[i] = A + (int64_t)(m0 + ar) * g.lda + ac * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int bk = (8 * i + wave) * 4 + (lane >> 4);
+    const int bc = (lane & 15) ^ (2 * (bk & 7));
+    c.b_src[i] = B + (int64_t)bk * g.ldb + n0 + bc * 16;
+  }
+#pragma unroll
+  for (int j = 0; j < TM; ++j) {
+    const int r = wm0 + 32 * j + r32;
+    c.a_off[j] = r * 128;
+    c.a_swz[j] = (r >> 1) & 7;
+  }
+  {
+    // Lane (grp = lane / 16, j = lane % 16) addresses k row 32 h + 8 q + j / 2 (q = 0..3), columns
+    // wn0 + 32 i + 16 (grp % 2) + 8 (j % 2) .. +8.
+    const int j16 = lane & 15, grp = lane >> 4;
+    const int krow = 32 * h + (j16 >> 1);
+    const int col = wn0 + 16 * (grp & 1) + 8 * (j16 & 1);
+    c.b_chunk = col >> 4;
+    c.b_swz = 2 * (krow & 7);
+    c.b_off = krow * 256 + (col & 8);
+  }
+
+  f32x16 acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  const int nk = g.K / 64;  // even: K is a multiple of 128
+  uint8_t* const abuf = smem_8;
+  uint8_t* const bbuf = smem_8 + kD8BBase;
+  d8_load_a(c, 0, abuf);
+  if (nk > 2) d8_load_a(c, 1, abuf + kD8ABytes);
+#pragma unroll
+  for (int st = 0; st < 4; ++st)
+    if (st < nk) d8_load_b(c, st, bbuf + st * kD8BBytes);
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  D8Frags f;
+  d8_read_frags(c, abuf, bbuf, 0, f);
+  int kt = 0;
+  for (; kt + 2 < nk; kt += 2) {
+    uint8_t* a_cur = abuf + ((kt >> 1) & 1) * kD8ABytes;
+    uint8_t* a_nxt = abuf + (((kt >> 1) + 1) & 1) * kD8ABytes;
+    uint8_t* b0 = bbuf + (kt & 3) * kD8BBytes;
+    uint8_t* b1 = bbuf + ((kt + 1) & 3) * kD8BBytes;
+    uint8_t* b2 = bbuf + ((kt + 2) & 3) * kD8BBytes;
+    d8_step_pair(c, acc, f, a_cur, a_nxt, b1, b2, a_cur, b0, b1, kt, nk);
+  }
+  {
+    const uint8_t* a_cur = abuf + ((kt >> 1) & 1) * kD8ABytes;
+    const uint8_t* b1 = bbuf + ((kt + 1) & 3) * kD8BBytes;
+    D8Frags gfr;
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    d8_read_frags(c, a_cur, b1, 1, gfr);
+    d8_mfma(acc, f);
+    d8_mfma(acc, gfr);
+  }
+
+  const int m_base = m0 + wm0 + r32;
+  const int n_base = n0 + wn0 + 4 * h;
+  if (g.out_dt != LH_F32) {
+    constexpr int cstride = WTN * 2 + 8;
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    uint8_t* cw = smem_8 + wave * (128 * cstride);
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          u32x2 w = epilogue4_pack<LH_BF16>(g, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                                            acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+          *reinterpret_cast<u32x2*>(cw + (32 * j + r32) * cstride + (32 * i + 8 * q + 4 * h) * 2) = w;
+        }
+    uint16_t* outp = reinterpret_cast<uint16_t*>(g.out);
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      const int row = 8 * t + (lane >> 3), ch = lane & 7;
+      u32x4 w = *reinterpret_cast<const u32x4*>(cw + row * cstride + ch * 16);
+      *reinterpret_cast<u32x4*>(outp + (int64_t)(m0 + wm0 + row) * g.ldc + n0 + wn0 + ch * 8) = w;
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        epilogue4<LH_BF16>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                           acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+}
+
+static int launch_direct8(const GemmArgs& g, hipStream_t s) {
+  static_assert(kD8LdsBytes >= kD8RingBytes, "rings must fit");
+  static bool configured = false;
+  if (!configured) {
+    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_direct),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kD8LdsBytes));
+    configured = true;
+  }
+  hipLaunchKernelGGL(gemm8_direct, dim3((g.M / 256) * (g.N / 256)), dim3(512), kD8LdsBytes, s, g);
+  return check_launch("gemm8_direct");
+}
+
 // Any shape: 32 x 32 x 64 tile per wave, one wave per workgroup tile of 32 x 32,
 // bounds-checked byte loads (zero padding: code 0 is +0).
 __global__ void __launch_bounds__(64) gemm8_generic(GemmArgs g) {
@@ -315,8 +568,10 @@ int gemm8(const GemmArgs& g, hipStream_t s) {
                        splits);
     return check_launch("gemm8_skinny_reduce");
   }
-  if (vec_ok && g.M % 256 == 0 && g.N % 256 == 0 && (int64_t)(g.M / 256) * (g.N / 256) >= 128)
+  if (vec_ok && g.M % 256 == 0 && g.N % 256 == 0 && (int64_t)(g.M / 256) * (g.N / 256) >= 128) {
+    if (g.ldb % 16 == 0 && g.ldc % 8 == 0) return launch_direct8(g, s);
     return launch_fast8<256, 256, 2, 4>(g, s);
+  }
   if (vec_ok && g.M % 128 == 0 && g.N % 128 == 0) return launch_fast8<128, 128, 2, 2>(g, s);
   dim3 grid((g.N + 31) / 32, (g.M + 31) / 32);
   hipLaunchKernelGGL(gemm8_generic, grid, dim3(64), 0, s, g);
