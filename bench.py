@@ -23,6 +23,10 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0
 PEAK_F32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM bytes one launch of the headline kernel moves, from two rocprofv3 --pmc runs of
+# `bench.py --only gemm_bf16` (FETCH_SIZE 98560.8 KiB x 2.0, the factor a plain copy of known size
+# gives for that counter, plus WRITE_SIZE 32768 KiB x 1.0); algorithmic minimum 100.7 MB.
+GEMM_BF16_4096_TRAFFIC_BYTES = 235.4e6
 
 
 def time_region(fn, steps, warmup):
@@ -82,8 +86,8 @@ def cpu_baseline_gemm_bf16(n: int, target_seconds: float = 12.0):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--only", choices=["gemm_bf16", "attention", "copy"], default=None,
@@ -206,9 +210,9 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "bf16 GEMM M=N=K=4096, A,B ~ N(0,1), f32 accumulation, bf16 output, no epilogue",
-                   "kernel": "gemm16_fast<bf16,256,256,2,4>"},
+                   "kernel": "gemm16_direct<bf16> (256x256 tile, 8 waves, direct-to-LDS rings)"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None},
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": GEMM_BF16_4096_TRAFFIC_BYTES},
         "cpu_baseline": cpu,
         "pct_of_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
         "speedup_vs_cpu": (value / cpu["value"]) if cpu else None,
