@@ -65,6 +65,16 @@ typedef enum lh_dtype {
 #define LH_GEMM_TRANSPOSE_A 8u
 #define LH_GEMM_TRANSPOSE_B 16u
 #define LH_GEMM_HAS_GELU 32u /* tanh-GELU on the accumulator instead of ReLU (nanoGPT MLP) */
+/* Workgroup-tile request for the 16-bit GEMM, the counterpart of the wg_m / wg_n schedule
+ * parameters (lighthouse/schedule/xegpu/mlp_schedule.py:72-78,142).  AUTO lets the library pick by
+ * shape; an explicit tile must divide M and N and needs untransposed operands, K % 64 == 0 and
+ * 16-byte aligned rows, otherwise the call fails with LH_ERR_INVALID. */
+#define LH_GEMM_TILE_MASK 0x700u
+#define LH_GEMM_TILE_AUTO 0x000u
+#define LH_GEMM_TILE_256x256 0x100u
+#define LH_GEMM_TILE_256x128 0x200u
+#define LH_GEMM_TILE_128x256 0x300u
+#define LH_GEMM_TILE_128x128 0x400u
 
 /* ---------------------------------------------------------------- runtime ---- */
 

@@ -23,6 +23,8 @@ GEMM_ACCUMULATE_C = 4
 GEMM_TRANSPOSE_A = 8
 GEMM_TRANSPOSE_B = 16
 GEMM_HAS_GELU = 32
+GEMM_TILE_AUTO = 0
+GEMM_TILES = {(256, 256): 0x100, (256, 128): 0x200, (128, 256): 0x300, (128, 128): 0x400}
 
 # lh_elementwise_kind
 EW_SOFTMAX, EW_GELU, EW_BIAS, EW_ADD, EW_CAST = range(5)

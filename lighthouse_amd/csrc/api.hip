@@ -20,8 +20,10 @@ static int gemm_common_checks(const char* who, const void* out, const void* a, c
   LH_REQUIRE(!(flags & LH_GEMM_HAS_BIAS) || bias != nullptr, "%s: HAS_BIAS set but bias is null", who);
   LH_REQUIRE(!((flags & LH_GEMM_HAS_RELU) && (flags & LH_GEMM_HAS_GELU)), "%s: RELU and GELU are exclusive", who);
   const uint32_t known = LH_GEMM_HAS_BIAS | LH_GEMM_HAS_RELU | LH_GEMM_ACCUMULATE_C | LH_GEMM_TRANSPOSE_A |
-                         LH_GEMM_TRANSPOSE_B | LH_GEMM_HAS_GELU;
+                         LH_GEMM_TRANSPOSE_B | LH_GEMM_HAS_GELU | LH_GEMM_TILE_MASK;
   LH_REQUIRE((flags & ~known) == 0, "%s: unknown flag bits 0x%x", who, flags & ~known);
+  LH_REQUIRE((flags & LH_GEMM_TILE_MASK) <= LH_GEMM_TILE_128x128, "%s: unknown tile request 0x%x", who,
+             flags & LH_GEMM_TILE_MASK);
   return LH_OK;
 }
 
@@ -34,7 +36,10 @@ int gemm_run(void* out, const void* c, const void* a, const void* b, const void*
   g.M = (int)M; g.N = (int)N; g.K = (int)K;
   g.lda = lda; g.ldb = ldb; g.ldc = ldc;
   g.flags = flags; g.out_dt = out_dtype; g.bias_dt = bias_dtype; g.alpha = 1.0f;
-  if (ab_dtype == LH_F32) return gemm32(g, s);
+  if (ab_dtype == LH_F32) {
+    LH_REQUIRE((flags & LH_GEMM_TILE_MASK) == LH_GEMM_TILE_AUTO, "gemm: tile requests apply to 16-bit inputs only");
+    return gemm32(g, s);
+  }
   return gemm16(g, ab_dtype, s);
 }
 

@@ -193,28 +193,42 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm16_fast(GemmArgs g)
 }
 
 
-// ---- direct-to-LDS kernel ---------------------------------------------------------------
-// 256 x 256 workgroup tile, 8 waves (2 x 4, 128 x 64 per wave).  Both panels go global -> LDS
-// with global_load_lds_dwordx4 (no register staging, no LDS store instructions) in their
-// GLOBAL orientation.  The k-contiguous A fragment is one 16-byte LDS read; the n-contiguous B
-// panel is read with ds_read_b64_tr_b16, which hands each lane 4 k-values of one column, i.e.
-// the MFMA operand layout, transposing in the LDS crossbar.
+// ---- direct-to-LDS kernels --------------------------------------------------------------
+// Workgroup tile (64 TM) x (128 TN), 8 waves as 2 x 4, (32 TM) x (32 TN) per wave; TM x TN is
+// 4 x 2 (256 x 256), 4 x 1 (256 x 128), 2 x 2 (128 x 256) or 2 x 1 (128 x 128).  Both panels go
+// global -> LDS with global_load_lds_dwordx4 (no register staging, no LDS store instructions) in
+// their GLOBAL orientation.  The k-contiguous A fragment is one 16-byte LDS read; the
+// n-contiguous B panel is read with ds_read_b64_tr_b16, which hands each lane 4 k-values of one
+// column, i.e. the MFMA operand layout, transposing in the LDS crossbar.
 //
-// LDS rings: A in 2 stages of 64 k (256 rows x 128 bytes: every global request is a full
-// 128-byte line), B in 4 stages of 32 k (32 rows x 512 bytes).  The main loop advances 32 k per
-// step; the barrier sits in the MIDDLE of a step, after the LDS reads of the step's second
-// k-half have been issued, so fragment reads always overlap MFMAs of the previous k-half and
-// the buffer a step has finished reading is refilled right away (B: 3 stages ahead, A: on odd
-// steps, one 64-k stage ahead).
+// LDS rings: A in 2 stages of 64 k (rows of 128 bytes: every global request is a full 128-byte
+// line), B in 4 stages of 32 k.  The main loop advances 32 k per step; the barrier sits in the
+// MIDDLE of a step, after the LDS reads of the step's second k-half have been issued, so
+// fragment reads always overlap MFMAs of the previous k-half and the buffer a step has finished
+// reading is refilled right away (B: 3 stages ahead, A: on odd steps, one 64-k stage ahead).
 //
 // A wave-wide global_load_lds writes 64 x 16 contiguous LDS bytes, so rows cannot be padded;
 // bank conflicts are avoided by XOR-swizzling which 16-byte chunk of a row each lane fetches
 // (A: chunk ^ ((row / 2) % 8); B: chunk ^ 4 (k % 4)).
-constexpr int kDirectABytes = 256 * 64 * 2;   // one A stage: 32 KiB
-constexpr int kDirectBBytes = 32 * 256 * 2;   // one B stage: 16 KiB
-constexpr int kDirectBBase = 2 * kDirectABytes;
-constexpr int kDirectRingBytes = kDirectBBase + 4 * kDirectBBytes;  // 128 KiB
-constexpr int kDirectLdsBytes = 8 * 128 * 136;  // output staging (139264) >= the rings
+template <int TM, int TN>
+struct DirectCfg {
+  static constexpr int BM = 64 * TM, BN = 128 * TN;
+  static constexpr int WTM = 32 * TM, WTN = 32 * TN;      // per-wave sub-tile
+  static constexpr int kABytes = BM * 64 * 2;             // one A stage (64 k)
+  static constexpr int kBRow = BN * 2;                    // bytes of one k row of a B stage
+  static constexpr int kBBytes = 32 * kBRow;              // one B stage (32 k)
+  static constexpr int kBBase = 2 * kABytes;
+  static constexpr int kRingBytes = kBBase + 4 * kBBytes;
+  static constexpr int kCStride = WTN * 2 + 8;            // staged output row: +8 bytes keeps the
+                                                          // 8-byte writes of 32 rows on distinct banks
+  static constexpr int kStageBytes = 8 * WTM * kCStride;
+  static constexpr int kLdsBytes = kRingBytes > kStageBytes ? kRingBytes : kStageBytes;
+  static constexpr int kBChunks = kBRow / 16;             // 16-byte chunks per B row
+  static constexpr int kBRowsPerLoad = 1024 / kBRow;      // k rows one wave-wide load covers
+  // Loads a lane has in flight per stage, hence the s_waitcnt immediates of the main loop.
+  static constexpr int kWaitEven = TM + 2 * TN;
+  static constexpr int kWaitOdd = 2 * TN;
+};
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -223,75 +237,83 @@ __device__ __forceinline__ void async_copy16(const void* gsrc, uint8_t* lds_wave
   __builtin_amdgcn_global_load_lds(gsrc, (lds_void_t*)lds_wave_base, 16, 0, 0);
 }
 
+template <int TM, int TN>
 struct DirectCtx {
-  const uint16_t* a_src[4];  // lane's source of A load i at k = 0
-  const uint16_t* b_src[2];
-  int a_off[4];              // byte offset of the lane's A row in a stage, per m-subtile
-  int a_swz[4];
+  const uint16_t* a_src[TM];  // lane's source of A load i at k = 0
+  const uint16_t* b_src[TN];
+  int a_off[TM];              // byte offset of the lane's A row in a stage, per m-subtile
+  int a_swz[TM];
   int64_t ldb;
   int wave, h, b_off, b_chunk, b_swz;
 };
 
+template <int TM, int TN>
 struct DirectFrags {
-  u32x4 a[4];
-  u32x4 b[2];
+  u32x4 a[TM];
+  u32x4 b[TN];
 };
 
-// A stage `sa` (k = 64 sa .. +64): 4 loads per lane.
-__device__ __forceinline__ void direct_load_a(const DirectCtx& c, int sa, uint8_t* __restrict__ abuf) {
+// A stage `sa` (k = 64 sa .. +64): TM loads per lane.
+template <int TM, int TN>
+__device__ __forceinline__ void direct_load_a(const DirectCtx<TM, TN>& c, int sa, uint8_t* __restrict__ abuf) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) async_copy16(c.a_src[i] + sa * 64, abuf + (8 * i + c.wave) * 1024);
+  for (int i = 0; i < TM; ++i) async_copy16(c.a_src[i] + sa * 64, abuf + (8 * i + c.wave) * 1024);
 }
-// B stage `sb` (k = 32 sb .. +32): 2 loads per lane.
-__device__ __forceinline__ void direct_load_b(const DirectCtx& c, int sb, uint8_t* __restrict__ bbuf) {
+// B stage `sb` (k = 32 sb .. +32): TN loads per lane.
+template <int TM, int TN>
+__device__ __forceinline__ void direct_load_b(const DirectCtx<TM, TN>& c, int sb, uint8_t* __restrict__ bbuf) {
 #pragma unroll
-  for (int i = 0; i < 2; ++i) async_copy16(c.b_src[i] + (int64_t)(sb * 32) * c.ldb, bbuf + (8 * i + c.wave) * 1024);
+  for (int i = 0; i < TN; ++i) async_copy16(c.b_src[i] + (int64_t)(sb * 32) * c.ldb, bbuf + (8 * i + c.wave) * 1024);
 }
 
 // Fragments of 16 k: A chunk pair `kc` (0..3: which 16 of the stage's 64 k), B k-step `ks`
 // (0..1: which 16 of the stage's 32 k).
-__device__ __forceinline__ void direct_read_frags(const DirectCtx& c, const uint8_t* __restrict__ as,
-                                                  const uint8_t* __restrict__ bs, int kc, int ks, DirectFrags& f) {
+template <int TM, int TN>
+__device__ __forceinline__ void direct_read_frags(const DirectCtx<TM, TN>& c, const uint8_t* __restrict__ as,
+                                                  const uint8_t* __restrict__ bs, int kc, int ks,
+                                                  DirectFrags<TM, TN>& f) {
+  constexpr int row = DirectCfg<TM, TN>::kBRow;
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+  for (int j = 0; j < TM; ++j)
     f.a[j] = *reinterpret_cast<const u32x4*>(as + c.a_off[j] + (((2 * kc + c.h) ^ c.a_swz[j]) << 4));
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < TN; ++i) {
     const int p = (c.b_chunk + 4 * i) ^ c.b_swz;
-    const uint8_t* p0 = bs + ks * 16 * 512 + c.b_off + p * 16;
+    const uint8_t* p0 = bs + ks * 16 * row + c.b_off + p * 16;
     s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p0);
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p0 + 4 * 512));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p0 + 4 * row));
     u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
     f.b[i] = u32x4{l2[0], l2[1], h2[0], h2[1]};
   }
 }
 
-template <int DT>
-__device__ __forceinline__ void direct_mfma(f32x16 (&acc)[2][4], const DirectFrags& f) {
+template <int DT, int TM, int TN>
+__device__ __forceinline__ void direct_mfma(f32x16 (&acc)[TN][TM], const DirectFrags<TM, TN>& f) {
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TN; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = Mfma16<DT>::mma(f.b[i], f.a[j], acc[i][j]);
+    for (int j = 0; j < TM; ++j) acc[i][j] = Mfma16<DT>::mma(f.b[i], f.a[j], acc[i][j]);
 }
 
-// Scheduling hint for one k-half: where the 8 LDS reads of the NEXT k-half go relative to the 8
-// MFMAs of the current one.
+// Scheduling hint for one k-half: spread the TM + 2 TN LDS reads of the NEXT k-half evenly
+// between the TM TN MFMAs of the current one.
+template <int I, int NM, int NR>
+__device__ __forceinline__ void direct_interleave_step() {
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                // MFMA
+  __builtin_amdgcn_sched_group_barrier(0x100, (I + 1) * NR / NM - I * NR / NM, 0);  // DS reads
+  if constexpr (I + 1 < NM) direct_interleave_step<I + 1, NM, NR>();
+}
+template <int TM, int TN>
 __device__ __forceinline__ void direct_interleave_hint() {
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-  }
+  direct_interleave_step<0, TM * TN, TM + 2 * TN>();
 }
 
-
-// Wait until at most `allowed` of this wave's loads are still in flight and all its LDS reads
-// have returned, then barrier.  One asm block: a __syncthreads() would add a release fence,
-// i.e. a wait for ALL outstanding loads, and drain the rings.
-__device__ __forceinline__ void direct_wait_barrier(int allowed) {
-  if (allowed >= 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  else if (allowed >= 4) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+// Wait until at most N of this wave's loads are still in flight and all its LDS reads have
+// returned, then barrier.  One asm block: a __syncthreads() would add a release fence, i.e. a
+// wait for ALL outstanding loads, and drain the rings.
+template <int N>
+__device__ __forceinline__ void direct_wait_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
 // Steps kt (even) and kt + 1 of the main loop; both have a successor step.  On entry f0 holds
@@ -301,46 +323,50 @@ __device__ __forceinline__ void direct_wait_barrier(int allowed) {
 // parameters so that the compiler does not make LDS reads wait for the asynchronous writes.
 //
 // In-flight loads, oldest first, when a barrier is reached (steady state):
-//   even step: [A(kt/2) B(kt+1)] [B(kt+2)] [A(kt/2+1) B(kt+3)]  -> B(kt+1) needed: 8 may remain
-//   odd step : [B(kt+1)] [A((kt+1)/2) B(kt+2)] [B(kt+3)]        -> A needed: 4 may remain
+//   even step: [A(kt/2) B(kt+1)] [B(kt+2)] [A(kt/2+1) B(kt+3)]  -> B(kt+1) needed: TM + 2 TN may remain
+//   odd step : [B(kt+1)] [A((kt+1)/2) B(kt+2)] [B(kt+3)]        -> A needed: 2 TN may remain
 // Near the end loads are no longer issued and the waits become full waits.
-template <int DT>
-__device__ __forceinline__ void direct_step_pair(const DirectCtx& c, f32x16 (&acc)[2][4], DirectFrags& f0,
-                                                 const uint8_t* __restrict__ a_cur, const uint8_t* __restrict__ a_nxt,
-                                                 const uint8_t* __restrict__ b0, const uint8_t* __restrict__ b1,
-                                                 const uint8_t* __restrict__ b2, uint8_t* __restrict__ a_refill,
-                                                 uint8_t* __restrict__ b_refill0, uint8_t* __restrict__ b_refill1,
-                                                 int kt, int nk) {
-  DirectFrags f1;
+template <int DT, int TM, int TN>
+__device__ __forceinline__ void direct_step_pair(const DirectCtx<TM, TN>& c, f32x16 (&acc)[TN][TM],
+                                                 DirectFrags<TM, TN>& f0, const uint8_t* __restrict__ a_cur,
+                                                 const uint8_t* __restrict__ a_nxt, const uint8_t* __restrict__ b0,
+                                                 const uint8_t* __restrict__ b1, const uint8_t* __restrict__ b2,
+                                                 uint8_t* __restrict__ a_refill, uint8_t* __restrict__ b_refill0,
+                                                 uint8_t* __restrict__ b_refill1, int kt, int nk) {
+  using Cfg = DirectCfg<TM, TN>;
+  DirectFrags<TM, TN> f1;
   const bool steady = kt + 6 < nk;  // all loads of both steps are real
   // ---- even step kt
   direct_read_frags(c, a_cur, b0, 1, 1, f1);
   direct_mfma<DT>(acc, f0);
-  direct_interleave_hint();
-  direct_wait_barrier(steady ? 8 : 0);
+  direct_interleave_hint<TM, TN>();
+  if (steady) direct_wait_barrier<Cfg::kWaitEven>();
+  else direct_wait_barrier<0>();
   if (kt + 4 < nk) direct_load_b(c, kt + 4, b_refill0);
   direct_read_frags(c, a_cur, b1, 2, 0, f0);
   direct_mfma<DT>(acc, f1);
-  direct_interleave_hint();
+  direct_interleave_hint<TM, TN>();
   // ---- odd step kt + 1
   direct_read_frags(c, a_cur, b1, 3, 1, f1);
   direct_mfma<DT>(acc, f0);
-  direct_interleave_hint();
-  direct_wait_barrier(steady ? 4 : 0);
+  direct_interleave_hint<TM, TN>();
+  if (steady) direct_wait_barrier<Cfg::kWaitOdd>();
+  else direct_wait_barrier<0>();
   if (kt + 4 < nk) direct_load_a(c, kt / 2 + 2, a_refill);
   if (kt + 5 < nk) direct_load_b(c, kt + 5, b_refill1);
   direct_read_frags(c, a_nxt, b2, 0, 0, f0);
   direct_mfma<DT>(acc, f1);
-  direct_interleave_hint();
+  direct_interleave_hint<TM, TN>();
 }
 
-template <int DT>
+template <int DT, int TM, int TN>
 __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
-  constexpr int BM = 256, BN = 256, TM = 4, TN = 2, WN = 4, WTN = 64;
+  using Cfg = DirectCfg<TM, TN>;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, WN = 4, WTM = Cfg::WTM, WTN = Cfg::WTN;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_d[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm0 = (wave / WN) * 128, wn0 = (wave % WN) * WTN;
+  const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
 
   const int tiles_m = g.M / BM, tiles_n = g.N / BN;
   int id = xcd_remap(blockIdx.x, gridDim.x);
@@ -354,7 +380,7 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
   const uint16_t* A = reinterpret_cast<const uint16_t*>(g.a);
   const uint16_t* B = reinterpret_cast<const uint16_t*>(g.b);
 
-  DirectCtx c;
+  DirectCtx<TM, TN> c;
   c.ldb = g.ldb;
   c.wave = wave;
   const int r32 = lane & 31, h = lane >> 5;
@@ -362,17 +388,17 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
   // Loader addressing.  A: load i of wave w fills rows (8 i + w) 8 .. +8 (1024 bytes); lane ->
   // row += lane / 8, LDS chunk p = lane % 8 holds global chunk p ^ ((row / 2) % 8).
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < TM; ++i) {
     const int ar = (8 * i + wave) * 8 + (lane >> 3);
     const int ac = (lane & 7) ^ ((ar >> 1) & 7);
     c.a_src[i] = A + (int64_t)(m0 + ar) * g.lda + ac * 8;
   }
-  // B: load i of wave w fills k rows (8 i + w) 2 .. +2; lane -> row += lane / 32, LDS chunk
-  // p = lane % 32 holds global chunk p ^ 4 (k % 4).
+  // B: load i of wave w fills k rows (8 i + w) R .. +R with R = 1024 / row bytes; lane ->
+  // row += lane / chunks-per-row, LDS chunk p holds global chunk p ^ 4 (k % 4).
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int bk = (8 * i + wave) * 2 + (lane >> 5);
-    const int bc = (lane & 31) ^ (4 * (bk & 3));
+  for (int i = 0; i < TN; ++i) {
+    const int bk = (8 * i + wave) * Cfg::kBRowsPerLoad + lane / Cfg::kBChunks;
+    const int bc = (lane % Cfg::kBChunks) ^ (4 * (bk & 3));
     c.b_src[i] = B + (int64_t)bk * g.ldb + n0 + bc * 8;
   }
   // A fragment (second MFMA operand): row wm0 + 32 j + r32, logical chunk 2 kc + h.
@@ -391,7 +417,7 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
     const int col = wn0 + 16 * (grp & 1) + 4 * (j16 & 3);
     c.b_chunk = col >> 3;
     c.b_swz = 4 * (krow & 3);
-    c.b_off = krow * 512 + 8 * ((col >> 2) & 1);
+    c.b_off = krow * Cfg::kBRow + 8 * ((col >> 2) & 1);
   }
 
   f32x16 acc[TN][TM];
@@ -404,34 +430,34 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
 
   const int nk = g.K / 32;  // even: K is a multiple of 64
   uint8_t* const abuf = smem_d;
-  uint8_t* const bbuf = smem_d + kDirectBBase;
+  uint8_t* const bbuf = smem_d + Cfg::kBBase;
   // Prologue: A stages 0, 1 and B stages 0 .. 3.
   direct_load_a(c, 0, abuf);
-  if (nk > 2) direct_load_a(c, 1, abuf + kDirectABytes);
+  if (nk > 2) direct_load_a(c, 1, abuf + Cfg::kABytes);
 #pragma unroll
   for (int st = 0; st < 4; ++st)
-    if (st < nk) direct_load_b(c, st, bbuf + st * kDirectBBytes);
+    if (st < nk) direct_load_b(c, st, bbuf + st * Cfg::kBBytes);
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-  DirectFrags f0;
+  DirectFrags<TM, TN> f0;
   direct_read_frags(c, abuf, bbuf, 0, 0, f0);
   int kt = 0;
   for (; kt + 2 < nk; kt += 2) {
-    uint8_t* a_cur = abuf + ((kt >> 1) & 1) * kDirectABytes;
-    uint8_t* a_nxt = abuf + (((kt >> 1) + 1) & 1) * kDirectABytes;
-    uint8_t* b0 = bbuf + (kt & 3) * kDirectBBytes;
-    uint8_t* b1 = bbuf + ((kt + 1) & 3) * kDirectBBytes;
-    uint8_t* b2 = bbuf + ((kt + 2) & 3) * kDirectBBytes;
+    uint8_t* a_cur = abuf + ((kt >> 1) & 1) * Cfg::kABytes;
+    uint8_t* a_nxt = abuf + (((kt >> 1) + 1) & 1) * Cfg::kABytes;
+    uint8_t* b0 = bbuf + (kt & 3) * Cfg::kBBytes;
+    uint8_t* b1 = bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
+    uint8_t* b2 = bbuf + ((kt + 2) & 3) * Cfg::kBBytes;
     direct_step_pair<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
   }
   {
     // Last two steps: nothing left to load; stage nk - 1 of B must have landed.
-    const uint8_t* a_cur = abuf + ((kt >> 1) & 1) * kDirectABytes;
-    const uint8_t* b0 = bbuf + (kt & 3) * kDirectBBytes;
-    const uint8_t* b1 = bbuf + ((kt + 1) & 3) * kDirectBBytes;
-    DirectFrags f1;
+    const uint8_t* a_cur = abuf + ((kt >> 1) & 1) * Cfg::kABytes;
+    const uint8_t* b0 = bbuf + (kt & 3) * Cfg::kBBytes;
+    const uint8_t* b1 = bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
+    DirectFrags<TM, TN> f1;
     direct_read_frags(c, a_cur, b0, 1, 1, f1);
     direct_mfma<DT>(acc, f0);
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    direct_wait_barrier<0>();
     direct_read_frags(c, a_cur, b1, 2, 0, f0);
     direct_mfma<DT>(acc, f1);
     direct_read_frags(c, a_cur, b1, 3, 1, f1);
@@ -442,12 +468,13 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
   const int m_base = m0 + wm0 + r32;
   const int n_base = n0 + wn0 + 4 * h;
   if (g.out_dt != LH_F32 && !(g.flags & LH_GEMM_ACCUMULATE_C)) {
-    // 16-bit output: stage the wave's 128 x 64 sub-tile in LDS (row stride 136 bytes keeps the
-    // 8-byte writes of 32 rows on distinct banks) and store full 128-byte row segments.
-    constexpr int cstride = WTN * 2 + 8;
-    static_assert(8 * 128 * cstride <= kDirectLdsBytes, "output staging must fit");
+    // 16-bit output: stage the wave's sub-tile in LDS and store full row segments of the
+    // sub-tile (128 or 64 bytes) with 16 bytes per lane.
+    constexpr int cstride = Cfg::kCStride;
+    constexpr int chunks = WTN * 2 / 16;       // 16-byte chunks per staged row
+    constexpr int rows_per_pass = 64 / chunks;
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the rings
-    uint8_t* cw = smem_d + wave * (128 * cstride);
+    uint8_t* cw = smem_d + wave * (WTM * cstride);
 #pragma unroll
     for (int i = 0; i < TN; ++i)
 #pragma unroll
@@ -460,8 +487,8 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
         }
     uint16_t* outp = reinterpret_cast<uint16_t*>(g.out);
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-      const int row = 8 * t + (lane >> 3), ch = lane & 7;
+    for (int t = 0; t < WTM / rows_per_pass; ++t) {
+      const int row = rows_per_pass * t + lane / chunks, ch = lane % chunks;
       u32x4 w = *reinterpret_cast<const u32x4*>(cw + row * cstride + ch * 16);
       *reinterpret_cast<u32x4*>(outp + (int64_t)(m0 + wm0 + row) * g.ldc + n0 + wn0 + ch * 8) = w;
     }
@@ -477,18 +504,18 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
                       acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
 }
 
-template <int DT>
+template <int DT, int TM, int TN>
 static int launch_direct(const GemmArgs& g, hipStream_t s) {
-  auto kern = gemm16_direct<DT>;
-  constexpr size_t lds = kDirectLdsBytes;
-  static_assert(kDirectLdsBytes >= kDirectRingBytes, "rings must fit");
+  using Cfg = DirectCfg<TM, TN>;
+  auto kern = gemm16_direct<DT, TM, TN>;
+  constexpr size_t lds = Cfg::kLdsBytes;
   static bool configured = false;
   if (!configured) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds));
     configured = true;
   }
-  hipLaunchKernelGGL(kern, dim3((g.M / 256) * (g.N / 256)), dim3(512), lds, s, g);
+  hipLaunchKernelGGL(kern, dim3((g.M / Cfg::BM) * (g.N / Cfg::BN)), dim3(512), lds, s, g);
   return check_launch("gemm16_direct");
 }
 
@@ -559,16 +586,51 @@ static int launch_fast(const GemmArgs& g, hipStream_t s) {
   return check_launch("gemm16_fast");
 }
 
+// Tile choice for the direct kernels: 0 = 256 x 256, 1 = 256 x 128, 2 = 128 x 256, 3 = 128 x 128,
+// -1 = none fits.  Cost model: rounds of 256 workgroups (one per CU) times the tile area, with a
+// penalty for the smaller tiles' extra operand traffic per flop.
+static int direct_variant(int M, int N) {
+  static const int bm[4] = {256, 256, 128, 128}, bn[4] = {256, 128, 256, 128};
+  static const double penalty[4] = {1.0, 1.1, 1.1, 1.25};
+  int best = -1;
+  double best_cost = 0.0;
+  for (int v = 0; v < 4; ++v) {
+    if (M % bm[v] || N % bn[v]) continue;
+    const int64_t tiles = (int64_t)(M / bm[v]) * (N / bn[v]);
+    const double cost = (double)((tiles + 255) / 256) * bm[v] * bn[v] * penalty[v];
+    if (best < 0 || cost < best_cost) {
+      best = v;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+
 template <int DT>
 static int gemm16_dispatch(const GemmArgs& g, hipStream_t s) {
   const bool ta = g.flags & LH_GEMM_TRANSPOSE_A, tb = g.flags & LH_GEMM_TRANSPOSE_B;
   const bool vec_ok = !ta && g.K % kBK == 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 && g.ldc % 4 == 0 &&
                       aligned16(g.a) && aligned16(g.b) && aligned16(g.out) &&
                       (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias));
+  const uint32_t tile = g.flags & LH_GEMM_TILE_MASK;
+  if (tile != LH_GEMM_TILE_AUTO) {
+    static const int bm[4] = {256, 256, 128, 128}, bn[4] = {256, 128, 256, 128};
+    const int v = (int)(tile >> 8) - 1;
+    LH_REQUIRE(vec_ok && !tb && g.ldc % 8 == 0 && g.M % bm[v] == 0 && g.N % bn[v] == 0,
+               "gemm: the requested %d x %d tile needs untransposed operands, M %% %d == 0, N %% %d == 0, "
+               "K %% 64 == 0 and 16-byte aligned rows (M=%d N=%d K=%d)",
+               bm[v], bn[v], bm[v], bn[v], g.M, g.N, g.K);
+  }
   if (vec_ok) {
+    if (!tb && g.ldc % 8 == 0) {
+      const int v = tile != LH_GEMM_TILE_AUTO ? (int)(tile >> 8) - 1 : direct_variant(g.M, g.N);
+      if (v == 0) return launch_direct<DT, 4, 2>(g, s);
+      if (v == 1) return launch_direct<DT, 4, 1>(g, s);
+      if (v == 2) return launch_direct<DT, 2, 2>(g, s);
+      if (v == 3) return launch_direct<DT, 2, 1>(g, s);
+    }
     const int cus = 256;
     const bool big = g.M % 256 == 0 && g.N % 256 == 0 && (int64_t)(g.M / 256) * (g.N / 256) >= cus;
-    if (big && !tb && g.ldc % 8 == 0) return launch_direct<DT>(g, s);
     if (big) {
       return tb ? launch_fast<DT, 256, 256, 2, 4, true>(g, s) : launch_fast<DT, 256, 256, 2, 4, false>(g, s);
     }

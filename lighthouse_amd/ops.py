@@ -36,8 +36,8 @@ def device_info() -> dict:
 
 
 def gemm(a, b, bias=None, *, out=None, out_dtype=None, relu=False, gelu=False, accumulate_c=False,
-         transpose_a=False, transpose_b=False):
-    """out = epilogue(A @ B); see lh_hip_gemm."""
+         transpose_a=False, transpose_b=False, tile=None):
+    """out = epilogue(A @ B); see lh_hip_gemm.  `tile=(bm, bn)` requests a workgroup tile."""
     _need_cuda(a, b, bias, out)
     if a.dim() != 2 or b.dim() != 2:
         raise ValueError("gemm expects 2-D tensors")
@@ -52,6 +52,10 @@ def gemm(a, b, bias=None, *, out=None, out_dtype=None, relu=False, gelu=False, a
     flags = ((_lib.GEMM_HAS_BIAS if bias is not None else 0) | (_lib.GEMM_HAS_RELU if relu else 0)
              | (_lib.GEMM_HAS_GELU if gelu else 0) | (_lib.GEMM_ACCUMULATE_C if accumulate_c else 0)
              | (_lib.GEMM_TRANSPOSE_A if transpose_a else 0) | (_lib.GEMM_TRANSPOSE_B if transpose_b else 0))
+    if tile is not None:
+        if tuple(tile) not in _lib.GEMM_TILES:
+            raise ValueError(f"unsupported tile {tile}; choose from {sorted(_lib.GEMM_TILES)}")
+        flags |= _lib.GEMM_TILES[tuple(tile)]
     if bias is not None and bias.dtype != out.dtype:
         raise ValueError("bias must have the output dtype")
     if a.dtype != b.dtype:

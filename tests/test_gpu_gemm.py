@@ -73,6 +73,49 @@ def test_gemm_16bit(dtype, shape, epi):
     assert_close(_host(out), ref, rtol, f"{elt} gemm {shape} {epi}")
 
 
+@pytest.mark.parametrize("tile", [(256, 256), (256, 128), (128, 256), (128, 128)])
+@pytest.mark.parametrize("K", [64, 128, 192, 448])
+@pytest.mark.parametrize("epi", ["none", "bias_gelu", "f32out_acc"])
+def test_gemm_16bit_requested_tile(tile, K, epi):
+    """Every workgroup tile of the direct-to-LDS kernel, on a grid of 2 x 3 tiles, with K spanning
+    the pipeline's prologue-only, one-pair and multi-pair paths."""
+    from lighthouse_amd import ops
+
+    M, N = 2 * tile[0], 3 * tile[1]
+    rng = np.random.default_rng(K + tile[0] + 7 * tile[1])
+    a = orc.round_to(rng.standard_normal((M, K)).astype(np.float32), "bf16")
+    b = orc.round_to(rng.standard_normal((K, N)).astype(np.float32), "bf16")
+    da, db = _dev(a, torch.bfloat16), _dev(b, torch.bfloat16)
+    if epi == "none":
+        out = ops.gemm(da, db, tile=tile)
+        ref = orc.matmul(a, b, result_type="bf16")
+    elif epi == "bias_gelu":
+        bias = orc.round_to(rng.standard_normal((N,)).astype(np.float32), "bf16")
+        out = ops.gemm(da, db, _dev(bias, torch.bfloat16), gelu=True, tile=tile)
+        ref = orc.matmul(a, b, bias=bias, gelu=True, result_type="bf16")
+    else:
+        c = rng.standard_normal((M, N)).astype(np.float32)
+        out = _dev(c, torch.float32)
+        ops.gemm(da, db, out=out, accumulate_c=True, tile=tile)
+        ref = orc.matmul(a, b, c=c, accumulate_c=True, result_type="f32")
+    rtol = F32_RTOL if epi == "f32out_acc" else BF16_RTOL
+    assert_close(_host(out), ref, rtol, f"bf16 gemm tile {tile} K={K} {epi}")
+
+
+def test_gemm_tile_request_errors():
+    from lighthouse_amd import ops
+
+    a = torch.zeros(256, 64, device="cuda", dtype=torch.bfloat16)
+    b = torch.zeros(64, 384, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.gemm(a, b, tile=(256, 256))  # N = 384 is not a multiple of 256
+    with pytest.raises(ValueError):
+        ops.gemm(a, b, tile=(64, 64))
+    with pytest.raises(ValueError):
+        ops.gemm(a.float(), b.float(), tile=(128, 128))
+    ops.gemm(a, b, tile=(256, 128))
+
+
 @pytest.mark.parametrize("ta,tb", [(True, False), (False, True), (True, True)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_gemm_transposed(dtype, ta, tb):
@@ -153,7 +196,8 @@ def test_gemm_errors():
         ops.gemm(a, a, relu=True, gelu=True)
 
 
-@pytest.mark.parametrize("shape", [(128, 128, 128), (256, 256, 512), (96, 80, 200), (16, 256, 1024), (5, 128, 256)])
+@pytest.mark.parametrize("shape", [(128, 128, 128), (256, 256, 512), (96, 80, 200), (16, 256, 1024), (5, 128, 256),
+                                   (2048, 4096, 128), (4096, 2048, 384)])  # the last two: direct-to-LDS kernel
 def test_gemm_fp8(shape):
     from lighthouse_amd import ops
 
