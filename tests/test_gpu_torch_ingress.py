@@ -1,0 +1,107 @@
+"""torch.compile models through the HIP backend, checked against the oracle."""
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from tests.conftest import assert_close
+from oracle import lh_oracle as orc
+from tests.test_torch_ingress import Block
+
+pytestmark = pytest.mark.gpu
+
+
+def _np(t):
+    return t.detach().float().cpu().numpy()
+
+
+def test_compiled_mlp_f32():
+    """Linear+ReLU, Linear: the shape of examples/ingress/torch/compile_model.py's MLP."""
+    from lighthouse_amd.ingress.torch import gpu_backend
+
+    torch.manual_seed(0)
+    model = nn.Sequential(nn.Linear(256, 512), nn.ReLU(), nn.Linear(512, 128)).cuda()
+    x = torch.randn(64, 256, device="cuda")
+    backend = gpu_backend()
+    compiled = torch.compile(model, backend=backend, dynamic=False)
+    with torch.no_grad():
+        y = compiled(x)
+    h = orc.matmul(_np(x), _np(model[0].weight).T, bias=_np(model[0].bias), relu=True)
+    ref = orc.matmul(h, _np(model[2].weight).T, bias=_np(model[2].bias))
+    assert_close(_np(y), ref, 1e-4, "compiled MLP f32")
+    assert backend.last_jit_function.kinds == ["hip.gemm", "hip.gemm"]
+
+
+def _block_params(m: Block):
+    t = lambda w: _np(w).T.copy()  # noqa: E731  Linear stores [out, in]; the oracle takes [in, out]
+    return {
+        "ln1_g": _np(m.ln_1.weight), "ln1_b": _np(m.ln_1.bias), "w_qkv": t(m.c_attn.weight), "b_qkv": _np(m.c_attn.bias),
+        "w_o": t(m.c_proj.weight), "b_o": _np(m.c_proj.bias), "ln2_g": _np(m.ln_2.weight), "ln2_b": _np(m.ln_2.bias),
+        "w_fc": t(m.c_fc.weight), "b_fc": _np(m.c_fc.bias), "w_proj": t(m.mlp_proj.weight), "b_proj": _np(m.mlp_proj.bias),
+    }
+
+
+def test_compiled_block_f32():
+    from lighthouse_amd.ingress.torch import gpu_backend
+
+    torch.manual_seed(1)
+    B, T, C, H = 2, 128, 256, 4
+    model = Block(C, H).cuda()
+    with torch.no_grad():
+        model.ln_1.weight.uniform_(0.5, 1.5)
+        model.ln_2.bias.uniform_(-0.1, 0.1)
+    x = torch.randn(B, T, C, device="cuda")
+    backend = gpu_backend()
+    compiled = torch.compile(model, backend=backend, dynamic=False)
+    with torch.no_grad():
+        y = compiled(x)
+    ref = orc.nanogpt_block(_np(x), _block_params(model), H, mode="f32")
+    assert_close(_np(y), ref, 1e-4, "compiled nanoGPT block f32")
+    assert backend.last_jit_function.kinds.count("hip.gemm") == 4
+    # second call reuses the cached transposed weights and gives the same result
+    with torch.no_grad():
+        assert torch.equal(compiled(x), y)
+
+
+def test_compiled_block_bf16():
+    """A bfloat16 module: every tensor bf16 (residual stream included), statistics and accumulators
+    f32.  Reference: the oracle's operators chained with the same rounding points."""
+    from lighthouse_amd.ingress.torch import gpu_backend
+
+    torch.manual_seed(2)
+    B, T, C, H = 2, 128, 256, 4
+    model = Block(C, H).cuda().bfloat16()
+    x = torch.randn(B, T, C, device="cuda").bfloat16()
+    compiled = torch.compile(model, backend=gpu_backend(), dynamic=False)
+    with torch.no_grad():
+        y = compiled(x)
+    assert y.dtype == torch.bfloat16
+    p = _block_params(model)
+    r = orc.round_bf16
+    x2 = _np(x).reshape(B * T, C)
+    ln1 = orc.layer_norm(x2, p["ln1_g"], p["ln1_b"], 1e-5, "bf16")
+    qkv = orc.matmul(ln1, p["w_qkv"], bias=p["b_qkv"], result_type="bf16").reshape(B, T, 3, H, C // H)
+    q, k, v = (qkv[:, :, i].transpose(0, 2, 1, 3) for i in range(3))
+    att = orc.attention(q, k, v, causal=True, result_type="bf16")
+    att = att.transpose(0, 2, 1, 3).reshape(B * T, C)
+    a = r(x2 + orc.matmul(att, p["w_o"], bias=p["b_o"], result_type="bf16"))
+    ln2 = orc.layer_norm(a, p["ln2_g"], p["ln2_b"], 1e-5, "bf16")
+    h = orc.matmul(ln2, p["w_fc"], bias=p["b_fc"], gelu=True, result_type="bf16")
+    ref = r(a + orc.matmul(h, p["w_proj"], bias=p["b_proj"], result_type="bf16")).reshape(B, T, C)
+    assert_close(_np(y), ref, 2e-2, "compiled nanoGPT block bf16")
+
+
+def test_jit_function_benchmark_protocol():
+    from lighthouse_amd.ingress.torch import gpu_backend
+
+    model = nn.Sequential(nn.Linear(128, 128), nn.ReLU()).cuda()
+    x = torch.randn(128, 128, device="cuda")
+    backend = gpu_backend()
+    jit = backend(torch.fx.symbolic_trace(model), [x])
+    out = jit(x)
+    assert isinstance(out, list) and len(out) == 1 and out[0].shape == (128, 128)
+    times = jit.benchmark(x, nruns=5, nwarmup=2)
+    assert times.shape == (5,) and times.dtype == np.float64 and (times > 0).all()
+    with pytest.raises(ValueError):
+        jit(x.cpu())

@@ -1,0 +1,98 @@
+"""Lowering of FX graphs to HIP kernel plans (no GPU needed: plans are built, not run).
+
+Contract mirrored: lighthouse/ingress/torch/compile.py:154-496 (backend callable, static shapes,
+JITFunction) and examples/ingress/torch/compile_model.py:60-140 (how the backend is driven).
+"""
+
+import pytest
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from lighthouse_amd.ingress.torch import JITFunction, gpu_backend
+
+
+class Block(nn.Module):
+    """GPT-2 block written the nanoGPT way (fused QKV Linear, SDPA, tanh-GELU MLP)."""
+
+    def __init__(self, C=64, H=4):
+        super().__init__()
+        self.ln_1, self.ln_2 = nn.LayerNorm(C), nn.LayerNorm(C)
+        self.c_attn, self.c_proj = nn.Linear(C, 3 * C), nn.Linear(C, C)
+        self.c_fc, self.mlp_proj = nn.Linear(C, 4 * C), nn.Linear(4 * C, C)
+        self.H = H
+
+    def forward(self, x):
+        B, T, C = x.size()
+        q, k, v = self.c_attn(self.ln_1(x)).split(C, dim=2)
+        q, k, v = (t.view(B, T, self.H, C // self.H).transpose(1, 2) for t in (q, k, v))
+        y = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+        x = x + self.c_proj(y.transpose(1, 2).contiguous().view(B, T, C))
+        return x + self.mlp_proj(F.gelu(self.c_fc(self.ln_2(x)), approximate="tanh"))
+
+
+def test_mlp_plan_fuses_activations():
+    model = nn.Sequential(nn.Linear(8, 16), nn.ReLU(), nn.Linear(16, 4), nn.GELU(approximate="tanh"))
+    jit = gpu_backend()(torch.fx.symbolic_trace(model), [torch.randn(2, 8)])
+    assert isinstance(jit, JITFunction)
+    assert jit.kinds == ["hip.gemm", "hip.gemm"]
+    gemms = [s for s in jit.plan if s.kind == "hip.gemm"]
+    assert [g.detail["activation"] for g in gemms] == ["relu", "gelu"]
+    assert all(g.detail["bias"] for g in gemms)
+
+
+def test_activation_with_second_user_is_not_fused():
+    class M(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc = nn.Linear(8, 8)
+
+        def forward(self, x):
+            h = self.fc(x)
+            return F.relu(h) + h
+
+    jit = gpu_backend()(torch.fx.symbolic_trace(M()), [torch.randn(2, 8)])
+    assert jit.kinds == ["hip.gemm", "hip.relu", "hip.add"]
+
+
+def test_block_plan_through_dynamo():
+    backend = gpu_backend()
+    compiled = torch.compile(Block(), backend=backend, dynamic=False)
+    with pytest.raises(ValueError, match="compiled for cuda"):  # the plan exists; running needs the GPU
+        with torch.no_grad():
+            compiled(torch.randn(2, 8, 64))
+    assert backend.last_jit_function.kinds == [
+        "hip.layer_norm", "hip.gemm", "hip.attention", "hip.gemm", "hip.add",
+        "hip.layer_norm", "hip.gemm", "hip.gemm", "hip.add"]
+    attn = next(s for s in backend.last_jit_function.plan if s.kind == "hip.attention")
+    assert attn.detail["causal"] is True
+
+
+def test_unsupported_compute_node_is_an_error():
+    model = nn.Sequential(nn.Linear(8, 16), nn.Sigmoid())
+    with pytest.raises(ValueError, match="no HIP kernel"):
+        gpu_backend()(torch.fx.symbolic_trace(model), [torch.randn(2, 8)])
+    jit = gpu_backend(allow_torch_fallback=True)(torch.fx.symbolic_trace(model), [torch.randn(2, 8)])
+    assert jit.kinds == ["hip.gemm", "torch.Sigmoid"]
+
+
+def test_unsupported_attention_arguments():
+    class M(nn.Module):
+        def forward(self, q, k, v, m):
+            return F.scaled_dot_product_attention(q, k, v, attn_mask=m)
+
+    with pytest.raises(ValueError, match="masks"):
+        gpu_backend()(torch.fx.symbolic_trace(M()), [torch.randn(1, 1, 4, 4)] * 4)
+
+
+def test_fn_compile_hook_and_device_check():
+    seen = []
+
+    def fn_compile(plan):
+        seen.extend(s.kind for s in plan)
+        return plan
+
+    gpu_backend(fn_compile)(torch.fx.symbolic_trace(nn.Linear(4, 4)), [torch.randn(1, 4)])
+    assert "hip.gemm" in seen
+    with pytest.raises(AssertionError):
+        gpu_backend(device="cpu")
