@@ -165,7 +165,7 @@ class Runner:
             for i, (spec, m) in enumerate(zip(fn.args, inputs)):
                 if memref_shape(m) != tuple(spec.shape):
                     raise ValueError(f"argument {i}: descriptor shape {memref_shape(m)} != {tuple(spec.shape)}")
-            args = to_packed_args(inputs)
+            args = to_packed_args(inputs if fn.arg_order is None else [inputs[i] for i in fn.arg_order])
             if benchmark:
                 time_array = np.zeros((nruns,), dtype=np.float64)
                 self.engine.lookup_benchmark(payload_function_name)(args, time_array, nruns, nwarmup)

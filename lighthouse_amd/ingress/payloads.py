@@ -31,9 +31,13 @@ class PayloadFunction:
     name: str
     entry: str                      # C entry point suffix: lh_hip_payload_<entry>
     attrs: ctypes.Structure
-    args: list[ArgSpec]
+    args: list[ArgSpec]             # in the order the caller passes buffers
     flops: int = 0
     bytes_moved: int = 0
+    # For each argument of the C entry point (output first), its position in `args`; None when the
+    # function already has the entry point's order.  Set for functions read from MLIR text, whose
+    # signature fixes the caller's order.
+    arg_order: list[int] | None = None
 
     @property
     def outputs(self) -> list[int]:

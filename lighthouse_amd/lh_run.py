@@ -1,0 +1,116 @@
+"""``lh-run`` for the HIP target: run or benchmark a payload function on the GPU.
+
+Same command line as lighthouse/lh_run.py:14-145 (``payload_module --entry-point F
+--input-shape SPECS --stage S... [--seed N] [-O n] [--benchmark] [--print-tensor N]
+[--print-optimized-module] [--print-mlir-after-all]``), same output lines (``N runs: T seconds``,
+``Output: <array>``) and exit codes (1 on FileNotFoundError / OSError / ValueError, 130 on
+Ctrl-C).  The payload module is MLIR text of one of the matmul forms this target has a kernel for
+(see ingress/mlir_text.py).  A ``--stage`` that names a pipeline descriptor with a ``kernel:`` stage
+(descriptors/gfx950/<pipeline>/<dtype>.yaml) selects that kernel's parameters; MLIR pass /
+transform stages have no counterpart here (the kernels are already lowered) and are skipped with a
+note on stderr, so the reference's own RUN lines work unchanged.
+"""
+
+from __future__ import annotations
+
+import argparse
+import sys
+from datetime import datetime
+
+import numpy as np
+
+from . import _lib
+from .execution.init import KernelArgumentParser
+from .execution.runner import Runner
+from .ingress.mlir_text import load_payload_module
+from .ingress.payloads import PayloadModule
+from .pipeline.descriptor import Descriptor, PipelineDescriptor
+
+
+def apply_stage(module: PayloadModule, stage: str, notes: list[str]) -> None:
+    """Apply one ``--stage`` to every function of the module."""
+    desc = Descriptor(stage)
+    if desc.is_include():
+        stages = PipelineDescriptor(desc).get_stages()
+    else:
+        stages = [desc]
+    for st in stages:
+        if not st.is_kernel():
+            notes.append(f"stage '{st}': MLIR {st.type or 'pass'} stage skipped (the HIP kernels are already lowered)")
+            continue
+        params = {**st.args, **st.opts}
+        matched = False
+        for fn in module.functions.values():
+            if fn.entry != st.basename:
+                continue
+            matched = True
+            tile = (params.get("tile_m"), params.get("tile_n"))
+            if fn.entry == "matmul" and tuple(tile) in _lib.GEMM_TILES:
+                out_shape = fn.args[fn.arg_order[0] if fn.arg_order else 0].shape
+                if out_shape[0] % tile[0] == 0 and out_shape[1] % tile[1] == 0 and fn.attrs.ab_dtype != _lib.F32:
+                    fn.attrs.flags = (fn.attrs.flags & ~0x700) | _lib.GEMM_TILES[tuple(tile)]
+                else:
+                    notes.append(f"stage '{st.basename}': tile {tile[0]}x{tile[1]} does not apply to @{fn.name} "
+                                 f"({out_shape[0]}x{out_shape[1]}); the library chooses")
+        if not matched:
+            notes.append(f"stage '{st.basename}': no function of this kind in the module")
+
+
+def main(argv: list[str] | None = None) -> int:
+    try:
+        parser = argparse.ArgumentParser(
+            prog="lh-run",
+            description="Lighthouse runner, HIP target: runs a payload function of an MLIR module on the GPU.")
+        parser.add_argument("payload_module", type=str, help="Path to the payload MLIR module.")
+        parser.add_argument("--entry-point", type=str, required=True,
+                            help="Name of the entrypoint function in the payload MLIR module.")
+        parser.add_argument("--input-shape", required=True,
+                            help="Shape of the input tensors in format: DIMS(MxNx...)xTYPE(f16/f32/f64/bf16/i8)"
+                                 "xINIT(0/1/rnd/id). For multiple inputs, separate by comma.")
+        parser.add_argument("--seed", type=int, default=0, help="Random seed for initializing input tensors.")
+        parser.add_argument("--stage", action="append", required=True,
+                            help="Pipeline descriptors / stages to apply to the input module.")
+        parser.add_argument("-O", type=int, default=3, help="Optimization level (accepted, unused).")
+        parser.add_argument("--benchmark", action=argparse.BooleanOptionalAction,
+                            help="Whether to run the benchmark. Default is False.")
+        parser.add_argument("--print-optimized-module", action=argparse.BooleanOptionalAction,
+                            help="Whether to print the module after all stages. Default is False.")
+        parser.add_argument("--print-tensor", type=int, default=0, help="Print the Nth tensor. Default is 0 (no print).")
+        parser.add_argument("--print-mlir-after-all", action=argparse.BooleanOptionalAction,
+                            help="Whether to print the module after every stage. Default is False.")
+        args = parser.parse_args(argv)
+
+        np.random.seed(args.seed if args.seed else int(datetime.now().timestamp()))
+
+        module = load_payload_module(args.payload_module, [args.entry_point])
+        notes: list[str] = []
+        for stage in args.stage:
+            apply_stage(module, stage, notes)
+            if args.print_mlir_after_all:
+                print(f"// -----// after stage {stage} //----- //\n{module}")
+        for note in notes:
+            print(f"lh-run: {note}", file=sys.stderr)
+        if args.print_optimized_module:
+            print(module)
+
+        buffers = [arg.arg for arg in KernelArgumentParser.parse_all(args.input_shape)]
+        runner = Runner(module, opt_level=args.O)
+        if args.benchmark:
+            time_array = runner.benchmark(host_input_buffers=buffers, payload_function_name=args.entry_point)
+            print(f"{len(time_array)} runs: {np.mean(time_array)} seconds")
+        else:
+            runner.execute(payload_function_name=args.entry_point, host_input_buffers=buffers)
+
+        if args.print_tensor > 0:
+            print(f"Output: {buffers[args.print_tensor - 1]}")
+        return 0
+    except KeyboardInterrupt:
+        print("\nInterrupted", file=sys.stderr)
+        return 130
+    except (FileNotFoundError, OSError, ValueError) as exc:
+        print(f"Error: {exc}", file=sys.stderr)
+        return 1
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -140,3 +140,33 @@ def test_runner_attention_and_layer_norm_payloads():
     o = np.zeros((M, N), np.float32)
     Runner(generate_gpu_layer_norm_payload("payload", M, N, "f32")).execute("payload", [o, x, g, b])
     assert np.allclose(o, orc.layer_norm(x, g, b), rtol=1e-3, atol=1e-4)
+
+
+def test_lh_run_cli_golden(tmp_path, capsys):
+    """The command line of test/run/pipeline-check.mlir:1-2 on a module of the same form: seed 123,
+    uniform A, all-ones B, zero C; prints buffer 3 and, with --benchmark, '100 runs: T seconds'."""
+    import json
+    import re
+    from pathlib import Path
+
+    from lighthouse_amd.lh_run import main
+
+    golden = json.loads((Path(__file__).parent / "golden" / "lh_run_pipeline_check.json").read_text())
+    mlir = tmp_path / "payload.mlir"
+    mlir.write_text("""
+module {
+  func.func @main(%lhs: tensor<16x64xf32>, %rhs: tensor<64x32xf32>, %acc: tensor<16x32xf32>) {
+    %r = linalg.matmul ins(%lhs, %rhs : tensor<16x64xf32>, tensor<64x32xf32>) outs(%acc : tensor<16x32xf32>) -> tensor<16x32xf32>
+    return
+  }
+}
+""")
+    common = [str(mlir), "--entry-point=main", f"--input-shape={golden['input_shape']}", "--stage=canonicalize"]
+    assert main(common + ["--print-tensor=3", f"--seed={golden['seed']}"]) == 0
+    out = capsys.readouterr().out
+    assert out.startswith("Output: [[")
+    rows = [[float(v) for v in re.findall(r"[-+]?\d+\.\d+(?:e[-+]?\d+)?", line)] for line in out.splitlines() if "[" in line]
+    first_values = np.array([r[0] for r in rows if r], dtype=np.float32)
+    np.testing.assert_allclose(first_values, np.array(golden["row_values"], dtype=np.float32), rtol=2e-6)
+    assert main(common + ["--benchmark"]) == 0
+    assert re.match(r"100 runs: [0-9.e-]+ seconds", capsys.readouterr().out)

@@ -1,0 +1,123 @@
+"""MLIR-text ingress and the lh-run command line (host side; no GPU needed).
+
+Forms covered are those of the reference's fixtures: the named-op module of
+test/run/pipeline-check.mlir:8-14 and the linalg.generic chain of test/opt/pipeline-check.mlir:27-46
+(re-typed here with other shapes and names, not copied).
+"""
+
+import pytest
+
+from lighthouse_amd import _lib
+from lighthouse_amd.ingress.mlir_text import parse_payload_module
+from lighthouse_amd.lh_run import apply_stage, main
+
+NAMED = """
+module {
+  func.func @mm(%a: tensor<8x24xf32>, %b: tensor<24x16xf32>, %c: tensor<8x16xf32>) {
+    %zero = arith.constant 0.000000e+00 : f32
+    %unused = linalg.fill ins(%zero : f32) outs(%c : tensor<8x16xf32>) -> tensor<8x16xf32>
+    %r = linalg.matmul ins(%a, %b : tensor<8x24xf32>, tensor<24x16xf32>) outs(%c : tensor<8x16xf32>) -> tensor<8x16xf32>
+    return
+  }
+}
+"""
+
+NAMED_ZERO_INIT = NAMED.replace("outs(%c : tensor<8x16xf32>) -> tensor<8x16xf32>\n    return",
+                                "outs(%unused : tensor<8x16xf32>) -> tensor<8x16xf32>\n    return")
+
+GENERIC = """
+#mk = affine_map<(d0, d1, d2) -> (d0, d2)>
+#kn = affine_map<(d0, d1, d2) -> (d2, d1)>
+#mn = affine_map<(d0, d1, d2) -> (d0, d1)>
+#row = affine_map<(d0, d1) -> (d1)>
+#id = affine_map<(d0, d1) -> (d0, d1)>
+module {
+  func.func @layer(%x: tensor<32x64xbf16>, %w: tensor<64x128xbf16>, %bias: tensor<128xbf16>, %y: tensor<32x128xbf16>) -> tensor<32x128xbf16> {
+    %0 = linalg.generic {indexing_maps = [#mk, #kn, #mn], iterator_types = ["parallel", "parallel", "reduction"]} ins(%x, %w : tensor<32x64xbf16>, tensor<64x128xbf16>) outs(%y : tensor<32x128xbf16>) {
+    ^bb0(%in: bf16, %in_0: bf16, %out: bf16):
+      %5 = arith.mulf %in, %in_0 : bf16
+      %6 = arith.addf %5, %out : bf16
+      linalg.yield %6 : bf16
+    } -> tensor<32x128xbf16>
+    %1 = linalg.generic {indexing_maps = [#row, #id], iterator_types = ["parallel", "parallel"]} ins(%bias : tensor<128xbf16>) outs(%0 : tensor<32x128xbf16>) {
+    ^bb0(%in: bf16, %out: bf16):
+      %5 = arith.addf %in, %out : bf16
+      linalg.yield %5 : bf16
+    } -> tensor<32x128xbf16>
+    %cst = arith.constant 0.000000e+00 : bf16
+    %2 = linalg.generic {indexing_maps = [#id], iterator_types = ["parallel", "parallel"]} outs(%1 : tensor<32x128xbf16>) {
+    ^bb0(%out: bf16):
+      %5 = arith.maximumf %out, %cst : bf16
+      linalg.yield %5 : bf16
+    } -> tensor<32x128xbf16>
+    return %2 : tensor<32x128xbf16>
+  }
+}
+"""
+
+
+def test_named_matmul_accumulates_into_argument():
+    fn = parse_payload_module(NAMED).lookup("mm")
+    assert fn.entry == "matmul" and fn.arg_order == [2, 0, 1]
+    assert fn.attrs.flags == _lib.GEMM_ACCUMULATE_C
+    assert [a.shape for a in fn.args] == [(8, 24), (24, 16), (8, 16)]
+    assert [a.writable for a in fn.args] == [False, False, True]
+    assert fn.flops == 2 * 8 * 16 * 24
+
+
+def test_zero_fill_means_no_accumulation():
+    fn = parse_payload_module(NAMED_ZERO_INIT).lookup("mm")
+    assert fn.attrs.flags == 0 and fn.arg_order == [2, 0, 1]
+
+
+def test_generic_chain_with_bias_and_relu():
+    fn = parse_payload_module(GENERIC, ["layer"]).lookup("layer")
+    assert fn.arg_order == [3, 0, 1, 2]
+    assert fn.attrs.flags == _lib.GEMM_HAS_BIAS | _lib.GEMM_HAS_RELU | _lib.GEMM_ACCUMULATE_C
+    assert fn.attrs.ab_dtype == _lib.BF16 and fn.attrs.out_dtype == _lib.BF16
+
+
+def test_transposed_contraction_maps():
+    text = GENERIC.replace("#kn = affine_map<(d0, d1, d2) -> (d2, d1)>", "#kn = affine_map<(d0, d1, d2) -> (d1, d2)>")
+    text = text.replace("tensor<64x128xbf16>", "tensor<128x64xbf16>")
+    fn = parse_payload_module(text).lookup("layer")
+    assert fn.attrs.flags & _lib.GEMM_TRANSPOSE_B and not fn.attrs.flags & _lib.GEMM_TRANSPOSE_A
+
+
+@pytest.mark.parametrize("text,match", [
+    (NAMED.replace("linalg.matmul", "linalg.batch_matmul"), "unsupported operation"),
+    (NAMED.replace("tensor<24x16xf32>", "tensor<25x16xf32>"), "inconsistent matmul shapes"),
+    (NAMED.replace("@mm", "@other"), "no function named"),
+    (NAMED.replace("tensor<8x24xf32>", "tensor<?x24xf32>"), "unsupported argument type"),
+])
+def test_rejected_modules(text, match):
+    with pytest.raises(ValueError, match=match):
+        parse_payload_module(text, ["mm"])
+
+
+def test_stage_application(tmp_path):
+    text = GENERIC.replace("32x", "256x").replace("x128", "x384").replace("<128x", "<384x")
+    module = parse_payload_module(text)
+    notes = []
+    apply_stage(module, "canonicalize", notes)                 # an MLIR pass: skipped
+    assert "skipped" in notes[0]
+    yaml_path = tmp_path / "bf16.yaml"
+    yaml_path.write_text('Pipeline:\n  - kernel: "matmul{tile_m=256 tile_n=128}"\n  - pass: cse\n')
+    apply_stage(module, str(yaml_path), notes)
+    assert module.lookup("layer").attrs.flags & 0x700 == _lib.GEMM_TILES[(256, 128)]
+    yaml_path.write_text('Pipeline:\n  - kernel: "matmul{tile_m=256 tile_n=256}"\n')
+    apply_stage(module, str(yaml_path), notes)                 # 384 % 256 != 0: left to the library
+    assert module.lookup("layer").attrs.flags & 0x700 == _lib.GEMM_TILES[(256, 128)]
+    assert "does not apply" in notes[-1]
+
+
+def test_cli_error_codes(tmp_path, capsys):
+    missing = main([str(tmp_path / "nope.mlir"), "--entry-point", "mm", "--input-shape", "8x24xf32x1", "--stage", "cse"])
+    assert missing == 1 and "Error:" in capsys.readouterr().err
+    f = tmp_path / "m.mlir"
+    f.write_text(NAMED)
+    bad_stage = main([str(f), "--entry-point", "mm", "--input-shape", "8x24xf32x1,24x16xf32x1,8x16xf32x0",
+                      "--stage", str(tmp_path / "absent.yaml")])
+    assert bad_stage == 1
+    bad_entry = main([str(f), "--entry-point", "zz", "--input-shape", "8x24xf32x1", "--stage", "cse"])
+    assert bad_entry == 1
