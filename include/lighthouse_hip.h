@@ -214,6 +214,25 @@ typedef struct lh_matmul_attrs {
 /* args: out[M,N], A, B[, bias[N]] */
 int lh_hip_payload_matmul(void** args, int32_t nargs, const lh_matmul_attrs* attrs);
 
+/* Multi-layer perceptron, generate_gpu_mlp_payload
+ * (lighthouse/ingress/mlir_gen/gpu_mlp_payload.py:10-107): layer i computes
+ * epilogue(act_i . W_i) with the matmul payload's epilogue; hidden activations have the A/B type
+ * and get the ReLU, the last layer has out_dtype and gets the ReLU only when
+ * relu_on_final_layer is set; TRANSPOSE_A applies to the first layer's input only,
+ * ACCUMULATE_C to the last layer's output only (the reference accumulates hidden layers into
+ * uninitialised tensors, i.e. leaves them undefined).  Hidden activations live in a
+ * library-owned device buffer that grows on demand. */
+typedef struct lh_mlp_attrs {
+  int32_t ab_dtype;
+  int32_t out_dtype;  /* result type of the last layer: F32 or the A/B type */
+  int32_t bias_dtype; /* type of every bias vector: F32 or the A/B type */
+  uint32_t flags;     /* LH_GEMM_HAS_BIAS | HAS_RELU | ACCUMULATE_C | TRANSPOSE_A | TRANSPOSE_B */
+  int32_t nlayers;
+  int32_t relu_on_final_layer;
+} lh_mlp_attrs;
+/* args: out[M,N_last], in, W_0 .. W_{n-1}[, bias_0 .. bias_{n-1}] */
+int lh_hip_payload_mlp(void** args, int32_t nargs, const lh_mlp_attrs* attrs);
+
 typedef struct lh_matmul_fp8_attrs {
   int32_t out_dtype;
   float scale_a;

@@ -61,6 +61,11 @@ class MatmulAttrs(ctypes.Structure):
     _fields_ = [("ab_dtype", ctypes.c_int32), ("out_dtype", ctypes.c_int32), ("flags", ctypes.c_uint32)]
 
 
+class MlpAttrs(ctypes.Structure):
+    _fields_ = [("ab_dtype", ctypes.c_int32), ("out_dtype", ctypes.c_int32), ("bias_dtype", ctypes.c_int32),
+                ("flags", ctypes.c_uint32), ("nlayers", ctypes.c_int32), ("relu_on_final_layer", ctypes.c_int32)]
+
+
 class MatmulFp8Attrs(ctypes.Structure):
     _fields_ = [("out_dtype", ctypes.c_int32), ("scale_a", ctypes.c_float), ("scale_b", ctypes.c_float)]
 
@@ -113,6 +118,7 @@ PROTOTYPES = {
                                     _vp, _sz, _vp]),
     "lh_hip_payload_matmul": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(MatmulAttrs)]),
     "lh_hip_payload_matmul_fp8": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(MatmulFp8Attrs)]),
+    "lh_hip_payload_mlp": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(MlpAttrs)]),
     "lh_hip_payload_attention": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(AttentionAttrs)]),
     "lh_hip_payload_layer_norm": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(LayerNormAttrs)]),
     "lh_hip_payload_elementwise": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(ElementwiseAttrs)]),

@@ -202,6 +202,85 @@ int lh_hip_payload_matmul(void** args, int32_t nargs, const lh_matmul_attrs* at)
   return sync_default();
 }
 
+// Hidden activations of lh_hip_payload_mlp: two halves used alternately.
+static char* g_mlp_scratch = nullptr;
+static size_t g_mlp_scratch_bytes = 0;
+
+int lh_hip_payload_mlp(void** args, int32_t nargs, const lh_mlp_attrs* at) {
+  LH_REQUIRE(args && at, "lh_hip_payload_mlp: null argument");
+  const int n = at->nlayers;
+  LH_REQUIRE(n >= 1 && n <= 64, "lh_hip_payload_mlp: nlayers %d out of range", n);
+  const bool has_bias = at->flags & LH_GEMM_HAS_BIAS;
+  LH_REQUIRE(nargs == 2 + n * (has_bias ? 2 : 1), "lh_hip_payload_mlp: expected %d arguments, got %d",
+             2 + n * (has_bias ? 2 : 1), nargs);
+  LH_REQUIRE((at->flags & ~(LH_GEMM_HAS_BIAS | LH_GEMM_HAS_RELU | LH_GEMM_ACCUMULATE_C | LH_GEMM_TRANSPOSE_A |
+                            LH_GEMM_TRANSPOSE_B)) == 0,
+             "lh_hip_payload_mlp: unsupported flag bits 0x%x", at->flags);
+  LH_REQUIRE(at->ab_dtype == LH_F32 || at->ab_dtype == LH_BF16 || at->ab_dtype == LH_F16,
+             "lh_hip_payload_mlp: unsupported A/B dtype %d", at->ab_dtype);
+  LH_REQUIRE(at->out_dtype == LH_F32 || at->out_dtype == at->ab_dtype,
+             "lh_hip_payload_mlp: result type must be f32 or the A/B type");
+  LH_REQUIRE(!has_bias || at->bias_dtype == LH_F32 || at->bias_dtype == at->ab_dtype,
+             "lh_hip_payload_mlp: bias type must be f32 or the A/B type");
+  const bool ta = at->flags & LH_GEMM_TRANSPOSE_A, tb = at->flags & LH_GEMM_TRANSPOSE_B;
+  const size_t eab = dtype_size(at->ab_dtype), eout = dtype_size(at->out_dtype);
+  Memref o, in;
+  LH_REQUIRE(get_memref(args, 0, 2, &o) && get_memref(args, 1, 2, &in), "lh_hip_payload_mlp: bad memref descriptor");
+  LH_REQUIRE(o.strides[1] == 1 && in.strides[1] == 1, "lh_hip_payload_mlp: innermost stride must be 1");
+  const int64_t M = ta ? in.sizes[1] : in.sizes[0];
+  LH_REQUIRE(o.sizes[0] == M, "lh_hip_payload_mlp: output rows %lld != batch %lld", (long long)o.sizes[0], (long long)M);
+  int64_t width = ta ? in.sizes[0] : in.sizes[1];
+  int64_t max_hidden = 0;
+  Memref w[64], bias[64];
+  for (int i = 0; i < n; ++i) {
+    LH_REQUIRE(get_memref(args, 2 + i, 2, &w[i]) && w[i].strides[1] == 1, "lh_hip_payload_mlp: bad weight %d", i);
+    const int64_t k = tb ? w[i].sizes[1] : w[i].sizes[0], nn = tb ? w[i].sizes[0] : w[i].sizes[1];
+    LH_REQUIRE(k == width, "lh_hip_payload_mlp: weight %d has %lld input features, expected %lld", i, (long long)k,
+               (long long)width);
+    if (has_bias) {
+      LH_REQUIRE(get_memref(args, 2 + n + i, 1, &bias[i]) && bias[i].sizes[0] == nn && bias[i].strides[0] == 1,
+                 "lh_hip_payload_mlp: bias %d must be contiguous [%lld]", i, (long long)nn);
+    }
+    width = nn;
+    if (i + 1 < n && nn > max_hidden) max_hidden = nn;
+  }
+  LH_REQUIRE(o.sizes[1] == width, "lh_hip_payload_mlp: output has %lld columns, last layer %lld", (long long)o.sizes[1],
+             (long long)width);
+  const size_t half = ((size_t)M * max_hidden * eab + 255) & ~(size_t)255;
+  if (2 * half > g_mlp_scratch_bytes) {
+    if (g_mlp_scratch) LH_HIP_CHECK(hipFree(g_mlp_scratch));
+    g_mlp_scratch = nullptr;
+    g_mlp_scratch_bytes = 0;
+    LH_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&g_mlp_scratch), 2 * half));
+    g_mlp_scratch_bytes = 2 * half;
+  }
+  const void* act = in.data(eab);
+  int64_t lda = in.strides[0];
+  int64_t K = ta ? in.sizes[0] : in.sizes[1];
+  for (int i = 0; i < n; ++i) {
+    const bool last = i + 1 == n;
+    const int64_t N = tb ? w[i].sizes[0] : w[i].sizes[1];
+    uint32_t flags = (at->flags & LH_GEMM_TRANSPOSE_B) | (has_bias ? LH_GEMM_HAS_BIAS : 0);
+    if (i == 0 && ta) flags |= LH_GEMM_TRANSPOSE_A;
+    if ((at->flags & LH_GEMM_HAS_RELU) && (!last || at->relu_on_final_layer)) flags |= LH_GEMM_HAS_RELU;
+    if (last && (at->flags & LH_GEMM_ACCUMULATE_C)) flags |= LH_GEMM_ACCUMULATE_C;
+    void* dst = last ? o.data(eout) : static_cast<void*>(g_mlp_scratch + (i & 1) * half);
+    const int out_dt = last ? at->out_dtype : at->ab_dtype;
+    const void* bias_p = has_bias ? bias[i].data(dtype_size(at->bias_dtype)) : nullptr;
+    const int64_t ldc = last ? o.strides[0] : N;
+    int rc = gemm_common_checks("lh_hip_payload_mlp", dst, act, w[i].data(eab), bias_p, M, N, K, lda, w[i].strides[0],
+                                ldc, flags);
+    if (rc) return rc;
+    rc = gemm_run(dst, dst, act, w[i].data(eab), bias_p, M, N, K, lda, w[i].strides[0], ldc, at->ab_dtype, out_dt,
+                  at->bias_dtype, flags, nullptr);
+    if (rc) return rc;
+    act = dst;
+    lda = N;
+    K = N;
+  }
+  return sync_default();
+}
+
 int lh_hip_payload_matmul_fp8(void** args, int32_t nargs, const lh_matmul_fp8_attrs* at) {
   LH_REQUIRE(args && at, "lh_hip_payload_matmul_fp8: null argument");
   LH_REQUIRE(nargs == 3, "lh_hip_payload_matmul_fp8: expected 3 arguments, got %d", nargs);
@@ -342,6 +421,7 @@ int lh_hip_payload_benchmark(const char* payload, void** args, int32_t nargs, co
   else if (!std::strcmp(payload, "layer_norm")) kind = 3;
   else if (!std::strcmp(payload, "elementwise")) kind = 4;
   else if (!std::strcmp(payload, "nanogpt_block")) kind = 5;
+  else if (!std::strcmp(payload, "mlp")) kind = 6;
   else return fail(LH_ERR_INVALID, "lh_hip_payload_benchmark: unknown payload '%s'", payload);
   auto call = [&]() -> int {
     switch (kind) {
@@ -350,7 +430,8 @@ int lh_hip_payload_benchmark(const char* payload, void** args, int32_t nargs, co
       case 2: return lh_hip_payload_attention(args, nargs, reinterpret_cast<const lh_attention_attrs*>(attrs));
       case 3: return lh_hip_payload_layer_norm(args, nargs, reinterpret_cast<const lh_layer_norm_attrs*>(attrs));
       case 4: return lh_hip_payload_elementwise(args, nargs, reinterpret_cast<const lh_elementwise_attrs*>(attrs));
-      default: return lh_hip_payload_nanogpt_block(args, nargs, reinterpret_cast<const lh_nanogpt_block_attrs*>(attrs));
+      case 5: return lh_hip_payload_nanogpt_block(args, nargs, reinterpret_cast<const lh_nanogpt_block_attrs*>(attrs));
+      default: return lh_hip_payload_mlp(args, nargs, reinterpret_cast<const lh_mlp_attrs*>(attrs));
     }
   };
   for (int64_t i = 0; i < nwarmup; ++i) {

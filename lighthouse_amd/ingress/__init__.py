@@ -3,6 +3,7 @@ from .payloads import (
     PayloadModule,
     generate_gpu_matmul_payload,
     generate_gpu_matmul_fp8_payload,
+    generate_gpu_mlp_payload,
     generate_gpu_attention_payload,
     generate_gpu_layer_norm_payload,
     generate_gpu_softmax_payload,
@@ -11,7 +12,7 @@ from .payloads import (
 )
 
 __all__ = [
-    "PayloadFunction", "PayloadModule", "generate_gpu_matmul_payload", "generate_gpu_matmul_fp8_payload",
+    "PayloadFunction", "PayloadModule", "generate_gpu_matmul_payload", "generate_gpu_matmul_fp8_payload", "generate_gpu_mlp_payload",
     "generate_gpu_attention_payload", "generate_gpu_layer_norm_payload", "generate_gpu_softmax_payload",
     "generate_gpu_elementwise_payload", "generate_nanogpt_block_payload",
 ]

@@ -127,6 +127,52 @@ def generate_gpu_matmul_payload(
     return _single(PayloadFunction(func_name, "matmul", attrs, args, flops, nbytes))
 
 
+def generate_gpu_mlp_payload(
+    func_name: str,
+    batch_size: int,
+    input_size: int,
+    output_size: int,
+    hidden_layer_sizes: list[int],
+    ab_type: str,
+    acc_type: str,
+    bias_type: str,
+    result_type: str,
+    transpose_a: bool = False,
+    transpose_b: bool = False,
+    has_bias: bool = False,
+    has_relu: bool = False,
+    accumulate_c: bool = False,
+    relu_on_final_layer: bool = False,
+) -> PayloadModule:
+    """``payload(out, in, W_0 .. W_n[, bias_0 .. bias_n])``;
+    lighthouse/ingress/mlir_gen/gpu_mlp_payload.py:10-107.  Hidden activations have ``ab_type`` and
+    get the ReLU; the last layer has ``result_type`` and gets it only with ``relu_on_final_layer``;
+    ``transpose_a`` applies to the first layer's input, ``accumulate_c`` to the last layer."""
+    ab, acc, bt, res = (elem_name(t) for t in (ab_type, acc_type, bias_type, result_type))
+    if acc != "f32":
+        raise ValueError("Only f32 accumulation is supported on the HIP target")
+    if ab not in ("f32", "bf16", "f16"):
+        raise ValueError(f"Unsupported A/B element type {ab}")
+    if res not in ("f32", ab) or (has_bias and bt not in ("f32", ab)):
+        raise ValueError(f"result type {res} and bias type {bt} must be f32 or the A/B type {ab}")
+    sizes = [input_size, *hidden_layer_sizes, output_size]
+    features = list(zip(sizes[:-1], sizes[1:]))
+    args = [ArgSpec((batch_size, output_size), res, writable=True),
+            ArgSpec((input_size, batch_size) if transpose_a else (batch_size, input_size), ab)]
+    args += [ArgSpec((o, i) if transpose_b else (i, o), ab) for i, o in features]
+    if has_bias:
+        args += [ArgSpec((o,), bt) for _, o in features]
+    flags = ((_lib.GEMM_HAS_BIAS if has_bias else 0) | (_lib.GEMM_HAS_RELU if has_relu else 0)
+             | (_lib.GEMM_ACCUMULATE_C if accumulate_c else 0) | (_lib.GEMM_TRANSPOSE_A if transpose_a else 0)
+             | (_lib.GEMM_TRANSPOSE_B if transpose_b else 0))
+    attrs = _lib.MlpAttrs(lh_dtype(ab), lh_dtype(res), lh_dtype(bt if has_bias else res), flags, len(features),
+                          1 if relu_on_final_layer else 0)
+    # examples/xegpu/mlp.py sums the per-layer matmul complexity.
+    flops = sum(2 * batch_size * i * o + (batch_size * o if has_bias else 0) for i, o in features)
+    nbytes = sum((batch_size * i + i * o) * _size(ab) for i, o in features) + batch_size * output_size * _size(res)
+    return _single(PayloadFunction(func_name, "mlp", attrs, args, flops, nbytes))
+
+
 def generate_gpu_matmul_fp8_payload(
     func_name: str, M: int, N: int, K: int, scale_a: float, scale_b: float, result_type: str = "bf16"
 ) -> PayloadModule:

@@ -228,6 +228,27 @@ def matmul(
     return out
 
 
+def mlp(x, weights, biases=None, *, has_relu=False, relu_on_final_layer=False, transpose_a=False, transpose_b=False,
+        accumulate_c=None, ab_type: str = "f32", result_type: str = "f32") -> np.ndarray:
+    """``payload(out, in, W_0.., [b_0..])`` of ``generate_gpu_mlp_payload``
+    lighthouse/ingress/mlir_gen/gpu_mlp_payload.py:66-105: every layer is the matmul payload's
+    ``emit_mlp_layer``; hidden layers produce ``ab_type`` and get the ReLU, the last layer produces
+    ``result_type`` (ReLU only with ``relu_on_final_layer``), ``transpose_a`` is applied to the
+    first layer only, and only the last layer accumulates into the passed output
+    (``accumulate_c`` = that initial output).  The example's checker
+    examples/xegpu/mlp.py:47-88 chains the same steps in float32."""
+    act = np.asarray(x, dtype=np.float32)
+    n = len(weights)
+    for i, w in enumerate(weights):
+        last = i == n - 1
+        act = matmul(
+            act, w, c=accumulate_c if last else None, bias=None if biases is None else biases[i],
+            relu=has_relu and (not last or relu_on_final_layer), accumulate_c=last and accumulate_c is not None,
+            transpose_a=transpose_a and i == 0, transpose_b=transpose_b,
+            result_type=result_type if last else ab_type)
+    return act
+
+
 def matmul_check_reference(c, a, b, bias, *, accumulate_c, has_bias, has_relu, truncate_to=None):
     """The example's own float32 checker, restated.
 

@@ -170,3 +170,38 @@ module {
     np.testing.assert_allclose(first_values, np.array(golden["row_values"], dtype=np.float32), rtol=2e-6)
     assert main(common + ["--benchmark"]) == 0
     assert re.match(r"100 runs: [0-9.e-]+ seconds", capsys.readouterr().out)
+
+
+@pytest.mark.parametrize("ab,res,bias_t", [("f32", "f32", "f32"), ("bf16", "bf16", "bf16"), ("bf16", "f32", "f32")])
+@pytest.mark.parametrize("variant", ["plain", "bias_relu", "bias_relu_final_tb", "acc"])
+def test_runner_mlp_payload(ab, res, bias_t, variant):
+    """generate_gpu_mlp_payload: three layers 192 -> 256 -> 128 -> 64 on a batch of 96 (the argument
+    list of gpu_mlp_payload.py:44-48: output, input, weights, biases)."""
+    from lighthouse_amd.execution import Runner
+    from lighthouse_amd.ingress import generate_gpu_mlp_payload
+    from lighthouse_amd.utils.numpy import astype as to_host_array, to_float32
+
+    rng = np.random.default_rng(31)
+    sizes = [192, 256, 128, 64]
+    batch = 96
+    has_bias = variant != "plain" and variant != "acc"
+    has_relu = has_bias
+    tb = variant.endswith("tb")
+    final = "final" in variant
+    acc = variant == "acc"
+    x = orc.round_to(rng.standard_normal((batch, sizes[0])).astype(np.float32), ab)
+    ws = [orc.round_to((rng.standard_normal((i, o)) / np.sqrt(i)).astype(np.float32), ab)
+          for i, o in zip(sizes[:-1], sizes[1:])]
+    bs = [orc.round_to(rng.standard_normal(o).astype(np.float32), bias_t) for o in sizes[1:]] if has_bias else None
+    c0 = orc.round_to(rng.standard_normal((batch, sizes[-1])).astype(np.float32), res)
+    module = generate_gpu_mlp_payload("payload", batch, sizes[0], sizes[-1], sizes[1:-1], ab, "f32", bias_t, res,
+                                      transpose_b=tb, has_bias=has_bias, has_relu=has_relu, accumulate_c=acc,
+                                      relu_on_final_layer=final)
+    out = to_host_array((c0 if acc else np.zeros_like(c0)).copy(), res)
+    bufs = [out, to_host_array(x, ab)] + [to_host_array(w.T.copy() if tb else w, ab) for w in ws]
+    if has_bias:
+        bufs += [to_host_array(b, bias_t) for b in bs]
+    Runner(module).execute("payload", bufs)
+    ref = orc.mlp(x, ws, bs, has_relu=has_relu, relu_on_final_layer=final, accumulate_c=c0 if acc else None,
+                  ab_type=ab, result_type=res)
+    assert_close(to_float32(out), ref, 1e-4 if ab == "f32" else 2e-2, f"mlp {ab}->{res} {variant}")

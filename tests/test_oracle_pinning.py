@@ -367,3 +367,32 @@ def test_complexity_formulas():
     assert orc.matmul_complexity(1024, 1024, 1024, True, True, False, 4, 4)[0] == 2 * 1024**3 + 2 * 1024**2
     assert orc.fused_attention_complexity(4, 16, 2048, 64, 2) == (68719476736, 50331648, 16777216)
     assert orc.layer_norm_complexity(8192, 768, 4) == (8 * 8192 * 768, (8192 * 768 + 2 * 768) * 4, 8192 * 768 * 4)
+
+
+def test_mlp_matches_torch_sequential():
+    """orc.mlp against a library model: torch Linear / ReLU stack in float64 (weights stored
+    [out, in] there, so transpose_b on the oracle side), ReLU on hidden layers only."""
+    import torch
+
+    rng = np.random.default_rng(17)
+    sizes = [12, 20, 9, 5]
+    x = rng.standard_normal((7, sizes[0])).astype(np.float32)
+    layers, ws, bs = [], [], []
+    for i, o in zip(sizes[:-1], sizes[1:]):
+        lin = torch.nn.Linear(i, o, dtype=torch.float64)
+        with torch.no_grad():
+            lin.weight.copy_(torch.from_numpy(rng.standard_normal((o, i))).float().double())
+            lin.bias.copy_(torch.from_numpy(rng.standard_normal(o)).float().double())
+        ws.append(lin.weight.detach().numpy().astype(np.float32))
+        bs.append(lin.bias.detach().numpy().astype(np.float32))
+        layers += [lin, torch.nn.ReLU()]
+    model = torch.nn.Sequential(*layers[:-1])
+    ref = model(torch.from_numpy(x).double()).detach().numpy()
+    got = orc.mlp(x, ws, bs, has_relu=True, transpose_b=True)
+    np.testing.assert_allclose(got, ref, rtol=2e-6, atol=2e-6)
+    with_final = orc.mlp(x, ws, bs, has_relu=True, relu_on_final_layer=True, transpose_b=True)
+    np.testing.assert_allclose(with_final, np.maximum(ref, 0), rtol=2e-6, atol=2e-6)
+    # only the last layer accumulates into the passed output
+    c = rng.standard_normal(ref.shape).astype(np.float32)
+    np.testing.assert_allclose(orc.mlp(x, ws, bs, has_relu=True, transpose_b=True, accumulate_c=c), ref + c,
+                               rtol=2e-6, atol=2e-6)
