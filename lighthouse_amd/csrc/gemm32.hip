@@ -3,63 +3,155 @@
 // (emit_mlp_layer, lighthouse/ingress/mlir_gen/gpu_mlp_payload.py:110-156; the f32
 // generic-form fixture test/opt/pipeline-check.mlir:27-46).
 //
-// Fast kernel: workgroup tile BM x BN x 32, 4 waves (2 x 2), A panel [m][k] and B panel
-// [k][n] double-buffered in LDS in their global orientation.  The MFMA takes one f32 per
-// lane and operand; a lane reads 4 consecutive k of its A row with one 16-byte LDS read and
-// issues 4 MFMAs, and reads the 4 matching B rows with 4-byte reads that are contiguous
-// across the lanes of a half wave.  As in the 16-bit kernel the B panel is the first MFMA
-// operand, so a lane's accumulator holds 4 consecutive columns of one row.
+// Fast kernel: A panel [m][k] and B panel [k][n] in LDS in their global orientation.  The MFMA
+// takes one f32 per lane and operand; a lane reads 4 consecutive k of its A row with one 16-byte
+// LDS read and issues 4 MFMAs, and reads the 4 matching B rows with 4-byte reads that are
+// contiguous across the lanes of a half wave.  As in the 16-bit kernel the B panel is the first
+// MFMA operand, so a lane's accumulator holds 4 consecutive columns of one row.
 #include "gemm_common.h"
 
 namespace lh {
 
 constexpr int kBK32 = 32;
-constexpr int kAStride32 = kBK32 + 4;  // floats; 144-byte rows: 16-byte reads of 16 rows are conflict free
 
-template <int BM, int BN>
-__global__ void __launch_bounds__(256) gemm32_fast(GemmArgs g) {
-  constexpr int NT = 256;
-  constexpr int BSTR = BN + 8;  // rows 4 apart land 32 banks apart
-  constexpr int WTM = BM / 2, WTN = BN / 2, TM = WTM / 32, TN = WTN / 32;
-  constexpr int A_CH = BM * (kBK32 / 4) / NT;
-  constexpr int B_CH = kBK32 * (BN / 4) / NT;
-  extern __shared__ __attribute__((aligned(16))) float smem32[];
-  float(*As)[BM * kAStride32] = reinterpret_cast<float(*)[BM * kAStride32]>(smem32);
-  float(*Bs)[kBK32 * BSTR] = reinterpret_cast<float(*)[kBK32 * BSTR]>(smem32 + 2 * BM * kAStride32);
+// ---- direct-to-LDS kernel ---------------------------------------------------------------
+// Workgroup tile (64 TM) x (64 TN) x 32, 4 waves (2 x 2).  Both panels go global -> LDS with
+// global_load_lds_dwordx4 in their global orientation through a ring of NS stages, NS - 1 of
+// them in flight: at f32 rates a k-step lasts about as long as a global load takes, so a
+// register-staged double buffer stalls on every step.  A wave-wide load writes 1 KiB
+// contiguously, so rows cannot be padded; which 16-byte chunk of a row a lane fetches is
+// XOR-swizzled instead (A rows of 128 bytes: chunk ^ ((row / 2) % 8); B rows: chunk ^ 8 for the
+// k rows with (k / 4) odd, which are the rows the upper half wave reads).
+typedef __attribute__((address_space(3))) void lds32_void_t;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm0 = (wave >> 1) * WTM, wn0 = (wave & 1) * WTN;
+__device__ __forceinline__ void async_copy16_f32(const float* gsrc, uint8_t* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(gsrc, (lds32_void_t*)lds_wave_base, 16, 0, 0);
+}
+
+template <int TM, int TN>
+struct Direct32Ctx {
+  static constexpr int NW = 4;                 // waves
+  static constexpr int LA = 8 * TM / NW;       // A loads per lane and stage
+  static constexpr int LB = 8 * TN / NW;       // B loads per lane and stage
+  const float* a_src[LA];
+  const float* b_src[LB];
+  int64_t ldb;
+  int wave, h;
+  int a_off[TM], a_swz[TM];  // byte offset of the lane's A row, its swizzle
+  int b_off[TN];             // byte offset of the lane's B column inside a k row (swizzle applied)
+};
+
+template <int TM, int TN>
+__device__ __forceinline__ void direct32_issue(const Direct32Ctx<TM, TN>& c, int kt, uint8_t* __restrict__ stage) {
+  using C = Direct32Ctx<TM, TN>;
+  constexpr int a_bytes = 64 * TM * 128;
+#pragma unroll
+  for (int i = 0; i < C::LA; ++i) async_copy16_f32(c.a_src[i] + kt * 32, stage + (C::NW * i + c.wave) * 1024);
+#pragma unroll
+  for (int i = 0; i < C::LB; ++i)
+    async_copy16_f32(c.b_src[i] + (int64_t)(kt * 32) * c.ldb, stage + a_bytes + (C::NW * i + c.wave) * 1024);
+}
+
+// One k-step: refill `wr` (if `prefetch`) and multiply the stage in `rd`.
+// Separate restrict pointers keep the compiler from making the LDS reads wait for the
+// asynchronous writes.
+template <int TM, int TN>
+__device__ __forceinline__ void direct32_step(const Direct32Ctx<TM, TN>& c, f32x16 (&acc)[TN][TM],
+                                              const uint8_t* __restrict__ rd, uint8_t* __restrict__ wr, int next_kt,
+                                              bool prefetch) {
+  constexpr int a_bytes = 64 * TM * 128, b_row = 64 * TN * 4;
+  constexpr int NKK = 4;  // groups of 8 k per stage
+  if (prefetch) direct32_issue(c, next_kt, wr);
+  const uint8_t* as = rd;
+  const uint8_t* bs = rd + a_bytes;
+  // Fragments of k-group kk (k = 8 kk + 4 h + t, t = 0..3) are read while the MFMAs of group
+  // kk - 1 run.
+  f32x4 fa[2][TM];
+  float fb[2][TN][4];
+  auto read = [&](int kk, int buf) {
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+      fa[buf][j] = *reinterpret_cast<const f32x4*>(as + c.a_off[j] + (((2 * kk + c.h) ^ c.a_swz[j]) << 4));
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        fb[buf][i][t] = *reinterpret_cast<const float*>(bs + (8 * kk + 4 * c.h + t) * b_row + c.b_off[i]);
+  };
+  read(0, 0);
+#pragma unroll
+  for (int q = 0; q < NKK; ++q) {
+    const int cur = q & 1;
+    if (q + 1 < NKK) read(q + 1, cur ^ 1);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int j = 0; j < TM; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[cur][i][t], fa[cur][j][t], acc[i][j], 0, 0, 0);
+    if (q + 1 < NKK) {
+      // keep the reads of the next group ahead of this group's MFMAs in the issue order
+      __builtin_amdgcn_sched_group_barrier(0x100, TM + 4 * TN, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 4 * TM * TN, 0);
+    }
+  }
+}
+
+template <int N>
+__device__ __forceinline__ void direct32_wait_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+template <int TM, int TN, int NS>
+__global__ void __launch_bounds__(256) gemm32_direct(GemmArgs g) {
+  using C = Direct32Ctx<TM, TN>;
+  constexpr int BM = 64 * TM, BN = 64 * TN;
+  constexpr int a_bytes = BM * 128, b_row = BN * 4, stage_bytes = a_bytes + 32 * b_row;
+  constexpr int L = C::LA + C::LB;  // loads a lane has in flight per stage
+  static_assert(C::LA >= 1 && C::LB >= 1 && NS >= 3 && NS <= 6 && L * (NS - 2) < 64, "ring shape");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem32d[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave >> 1) * 32 * TM, wn0 = (wave & 1) * 32 * TN;
   const int tiles_n = g.N / BN;
   const int id = xcd_remap(blockIdx.x, gridDim.x);
   const int m0 = (id / tiles_n) * BM, n0 = (id % tiles_n) * BN;
   const float* A = reinterpret_cast<const float*>(g.a);
   const float* B = reinterpret_cast<const float*>(g.b);
+  const int r32 = lane & 31, h = lane >> 5;
 
-  f32x4 ra[A_CH], rb[B_CH];
-  auto load_global = [&](int k0) {
+  C c;
+  c.ldb = g.ldb;
+  c.wave = wave;
+  c.h = h;
+  // A: load i of wave w fills rows (NW i + w) 8 .. +8; lane -> row += lane / 8, LDS chunk lane % 8.
 #pragma unroll
-    for (int i = 0; i < A_CH; ++i) {
-      int c = tid + i * NT, row = c >> 3, kc = c & 7;
-      ra[i] = *reinterpret_cast<const f32x4*>(A + (int64_t)(m0 + row) * g.lda + k0 + kc * 4);
-    }
+  for (int i = 0; i < C::LA; ++i) {
+    const int row = (C::NW * i + wave) * 8 + (lane >> 3);
+    const int gc = (lane & 7) ^ ((row >> 1) & 7);
+    c.a_src[i] = A + (int64_t)(m0 + row) * g.lda + gc * 4;
+  }
+  // B: a k row is 16 TN chunks; load i of wave w fills k rows (NW i + w) (4 / TN) .. ; lane ->
+  // row += lane / (16 TN), LDS chunk lane % (16 TN).
 #pragma unroll
-    for (int i = 0; i < B_CH; ++i) {
-      int c = tid + i * NT, row = c / (BN / 4), nc = c % (BN / 4);
-      rb[i] = *reinterpret_cast<const f32x4*>(B + (int64_t)(k0 + row) * g.ldb + n0 + nc * 4);
-    }
-  };
-  auto store_lds = [&](int buf) {
+  for (int i = 0; i < C::LB; ++i) {
+    constexpr int chunks = 16 * TN;
+    const int k = (C::NW * i + wave) * (64 / chunks) + lane / chunks;
+    const int gc = (lane % chunks) ^ (8 * ((k >> 2) & 1));
+    c.b_src[i] = B + (int64_t)k * g.ldb + n0 + gc * 4;
+  }
 #pragma unroll
-    for (int i = 0; i < A_CH; ++i) {
-      int c = tid + i * NT, row = c >> 3, kc = c & 7;
-      *reinterpret_cast<f32x4*>(&As[buf][row * kAStride32 + kc * 4]) = ra[i];
-    }
+  for (int j = 0; j < TM; ++j) {
+    const int row = wm0 + 32 * j + r32;
+    c.a_off[j] = row * 128;
+    c.a_swz[j] = (row >> 1) & 7;
+  }
 #pragma unroll
-    for (int i = 0; i < B_CH; ++i) {
-      int c = tid + i * NT, row = c / (BN / 4), nc = c % (BN / 4);
-      *reinterpret_cast<f32x4*>(&Bs[buf][row * BSTR + nc * 4]) = rb[i];
-    }
-  };
+  for (int i = 0; i < TN; ++i) {
+    const int n = wn0 + 32 * i + r32;
+    c.b_off[i] = (((n >> 2) ^ (8 * h)) << 4) + (n & 3) * 4;  // rows 8 kk + 4 h + t have (k / 4) % 2 == h
+  }
 
   f32x16 acc[TN][TM];
 #pragma unroll
@@ -69,36 +161,21 @@ __global__ void __launch_bounds__(256) gemm32_fast(GemmArgs g) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-  const int nk = g.K / kBK32;
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
-  const int r32 = lane & 31, h = lane >> 5;
+  const int nk = g.K / 32;
+#pragma unroll
+  for (int st = 0; st < NS - 1; ++st)
+    if (st < nk) direct32_issue(c, st, smem32d + st * stage_bytes);
   for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < nk) load_global((kt + 1) * kBK32);
-#pragma unroll
-    for (int kk = 0; kk < kBK32 / 8; ++kk) {
-      // The lane's k indices for the next 4 MFMAs are kk*8 + 4h + t, t = 0..3.
-      f32x4 fa[TM];
-      float fb[TN][4];
-#pragma unroll
-      for (int j = 0; j < TM; ++j)
-        fa[j] = *reinterpret_cast<const f32x4*>(&As[buf][(wm0 + 32 * j + r32) * kAStride32 + kk * 8 + 4 * h]);
-#pragma unroll
-      for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int t = 0; t < 4; ++t) fb[i][t] = Bs[buf][(kk * 8 + 4 * h + t) * BSTR + wn0 + 32 * i + r32];
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int i = 0; i < TN; ++i)
-#pragma unroll
-          for (int j = 0; j < TM; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[i][t], fa[j][t], acc[i][j], 0, 0, 0);
-    }
-    if (kt + 1 < nk) store_lds(buf ^ 1);
-    __syncthreads();
+    // Stages kt + 1 .. kt + NS - 2 may stay in flight; one asm block per case because a
+    // __syncthreads() would add a fence that waits for every outstanding load.
+    const int younger = min(nk - 1 - kt, NS - 2);
+    if (younger >= 4) direct32_wait_barrier<L * 4>();
+    else if (younger == 3) direct32_wait_barrier<L * 3>();
+    else if (younger == 2) direct32_wait_barrier<L * 2>();
+    else if (younger == 1) direct32_wait_barrier<L>();
+    else direct32_wait_barrier<0>();
+    const int nxt = kt + NS - 1;
+    direct32_step(c, acc, smem32d + (kt % NS) * stage_bytes, smem32d + (nxt % NS) * stage_bytes, nxt, nxt < nk);
   }
 
   const int m_base = m0 + wm0 + r32;
@@ -111,6 +188,20 @@ __global__ void __launch_bounds__(256) gemm32_fast(GemmArgs g) {
       for (int q = 0; q < 4; ++q)
         epilogue4<LH_F32>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
                           acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+}
+
+template <int TM, int TN, int NS>
+static int launch_direct32(const GemmArgs& g, hipStream_t s) {
+  auto kern = gemm32_direct<TM, TN, NS>;
+  constexpr size_t lds = (size_t)NS * (64 * TM * 128 + 32 * 64 * TN * 4);
+  static bool configured = false;
+  if (!configured) {
+    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)lds));
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((g.M / (64 * TM)) * (g.N / (64 * TN))), dim3(256), lds, s, g);
+  return check_launch("gemm32_direct");
 }
 
 // Any shape / stride / transpose; 64 x 64 x 16 tiles, bounds-checked scalar loads.
@@ -164,30 +255,18 @@ __global__ void __launch_bounds__(256) gemm32_generic(GemmArgs g) {
   }
 }
 
-template <int BM, int BN>
-static int launch_fast32(const GemmArgs& g, hipStream_t s) {
-  auto kern = gemm32_fast<BM, BN>;
-  constexpr size_t lds = (size_t)2 * (BM * kAStride32 + kBK32 * (BN + 8)) * sizeof(float);
-  static bool configured = false;
-  if (!configured) {
-    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                     (int)lds));
-    configured = true;
-  }
-  hipLaunchKernelGGL(kern, dim3((g.M / BM) * (g.N / BN)), dim3(256), lds, s, g);
-  return check_launch("gemm32_fast");
-}
-
 int gemm32(const GemmArgs& g, hipStream_t s) {
   const bool trans = g.flags & (LH_GEMM_TRANSPOSE_A | LH_GEMM_TRANSPOSE_B);
   const bool vec_ok = !trans && g.K % kBK32 == 0 && g.lda % 4 == 0 && g.ldb % 4 == 0 && g.ldc % 4 == 0 &&
                       aligned16(g.a) && aligned16(g.b) && aligned16(g.out) &&
                       (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias));
-  if (vec_ok && g.M % 128 == 0 && g.N % 128 == 0 && (int64_t)(g.M / 128) * (g.N / 128) >= 512) {
-    return launch_fast32<128, 128>(g, s);
+  if (vec_ok && g.M % 128 == 0 && g.N % 128 == 0 && (int64_t)(g.M / 128) * (g.N / 128) >= 256) {
+    return launch_direct32<2, 2, 4>(g, s);
   }
   if (vec_ok && g.M % 64 == 0 && g.N % 64 == 0) {
-    return launch_fast32<64, 64>(g, s);
+    // Up to two workgroups per CU: a deep ring; more: a shallow ring so that three share a CU.
+    if ((int64_t)(g.M / 64) * (g.N / 64) <= 512) return launch_direct32<1, 1, 6>(g, s);
+    return launch_direct32<1, 1, 3>(g, s);
   }
   dim3 grid((g.N + 63) / 64, (g.M + 63) / 64);
   hipLaunchKernelGGL(gemm32_generic, grid, dim3(256), 0, s, g);
