@@ -359,17 +359,16 @@ __device__ __forceinline__ void direct_step_pair(const DirectCtx<TM, TN>& c, f32
   direct_interleave_hint<TM, TN>();
 }
 
+// One output tile; `id` is the tile's position in the XCD-grouped order.
 template <int DT, int TM, int TN>
-__global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
+__device__ __forceinline__ void direct_tile(const GemmArgs& g, int id, uint8_t* smem_d) {
   using Cfg = DirectCfg<TM, TN>;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, WN = 4, WTM = Cfg::WTM, WTN = Cfg::WTN;
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_d[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
 
   const int tiles_m = g.M / BM, tiles_n = g.N / BN;
-  int id = xcd_remap(blockIdx.x, gridDim.x);
   constexpr int GROUP_M = 4;
   const int group_size = GROUP_M * tiles_n;
   const int first_m = (id / group_size) * GROUP_M;
@@ -504,6 +503,21 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
                       acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
 }
 
+// Persistent workgroups: one (two for the 128 x 128 tile, whose rings are 64 KiB) per CU, each
+// walking the tile list with the grid as stride.  Tile ids congruent modulo 8 stay on one XCD,
+// which is what xcd_remap assumes.  Launching one workgroup per tile instead costs a
+// workgroup launch plus a cold prologue per tile, about a third of a K = 768 tile's time.
+template <int DT, int TM, int TN>
+__global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
+  using Cfg = DirectCfg<TM, TN>;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_d[];
+  const int ntiles = (g.M / Cfg::BM) * (g.N / Cfg::BN);
+  for (int t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    if (t != (int)blockIdx.x) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS is reused
+    direct_tile<DT, TM, TN>(g, xcd_remap(t, ntiles), smem_d);
+  }
+}
+
 template <int DT, int TM, int TN>
 static int launch_direct(const GemmArgs& g, hipStream_t s) {
   using Cfg = DirectCfg<TM, TN>;
@@ -515,7 +529,9 @@ static int launch_direct(const GemmArgs& g, hipStream_t s) {
                                      (int)lds));
     configured = true;
   }
-  hipLaunchKernelGGL(kern, dim3((g.M / Cfg::BM) * (g.N / Cfg::BN)), dim3(512), lds, s, g);
+  const int ntiles = (g.M / Cfg::BM) * (g.N / Cfg::BN);
+  const int resident = 256 * (2 * lds <= 160 * 1024 ? 2 : 1);
+  hipLaunchKernelGGL(kern, dim3(ntiles < resident ? ntiles : resident), dim3(512), lds, s, g);
   return check_launch("gemm16_direct");
 }
 
