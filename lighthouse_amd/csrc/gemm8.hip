@@ -448,74 +448,124 @@ __global__ void __launch_bounds__(64) gemm8_generic(GemmArgs g) {
 }
 
 // ---- skinny (decode) path ---------------------------------------------------------------
-// Workgroup: 256 threads, tile 16 (padded M) x 128 n x 128 k per step, over a K chunk.
-// partial[split][16][N] f32.  Wave w owns columns 32 w .. 32 w + 31 (two 16-wide MFMA tiles).
-constexpr int kSkinnyBN = 128;
+// M <= 16: the job is streaming B once from HBM.  Grid (N / 256, splits); a workgroup of 4 waves
+// owns 256 columns and a K chunk, wave w the columns 64 w .. 64 w + 63 (four 16-wide MFMA tiles,
+// v_mfma_scale_f32_16x16x128_f8f6f4 with M padded to 16).  B goes global -> LDS with
+// global_load_lds_dwordx4 in its global orientation (k rows of 256 contiguous bytes) through a
+// ring of 4 stages of 128 k, three of them in flight (96 KiB per CU, what the HBM
+// latency-bandwidth product needs); fragments come from ds_read_b64_tr_b8.  The A chunk (16 rows)
+// is staged once, as one 16 x 128-byte block per k-step.  Rows cannot be padded (a wave-wide load
+// writes 1 KiB contiguously): the 16-byte chunk a lane fetches is XOR-swizzled, B chunk ^
+// (k % 8 + 8 ((k / 32) % 2)), A chunk ^ ((m / 2) % 8).
+// Partial sums go to partial[split][16][N] (f32); gemm8_skinny_reduce adds them and runs the
+// epilogue.
+constexpr int kSkinnyBN = 256;
+constexpr int kSkinnyStages = 4;
+constexpr int kSkinnyStageBytes = kBK8 * kSkinnyBN;  // 32 KiB
+constexpr int kSkinnyMaxChunk = 1024;                // K chunk whose A block fits the 16 KiB A area
+constexpr int kSkinnyLdsBytes = kSkinnyStages * kSkinnyStageBytes + 16 * kSkinnyMaxChunk;
+
+__device__ __forceinline__ void skinny_issue_b(const uint8_t* const (&b_src)[8], int64_t ldb, int kt, int wave,
+                                               uint8_t* __restrict__ stage) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    async8_copy16(b_src[i] + (int64_t)(kt * kBK8) * ldb, stage + (4 * i + wave) * 1024);
+}
+
+// One k-step: refill `wr` (if `prefetch`) and multiply the stage in `bs`.  The LDS reads and the
+// asynchronous LDS writes go through separate restrict pointers of one function, otherwise the
+// compiler makes every LDS read wait for all outstanding loads.
+__device__ __forceinline__ void skinny_step(f32x4 (&acc)[4], const uint8_t* __restrict__ bs,
+                                            const uint8_t* __restrict__ as, uint8_t* __restrict__ wr,
+                                            const uint8_t* const (&b_src)[8], int64_t ldb, int next_kt, bool prefetch,
+                                            int wave, int a_off, int a_swz, int qd, int b_off, int b_chunk, int b_swz) {
+  if (prefetch) skinny_issue_b(b_src, ldb, next_kt, wave, wr);
+  const int c0 = 2 * qd;
+  i32x4 alo = *reinterpret_cast<const i32x4*>(as + a_off + ((c0 ^ a_swz) << 4));
+  i32x4 ahi = *reinterpret_cast<const i32x4*>(as + a_off + (((c0 + 1) ^ a_swz) << 4));
+  i32x8 fa = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint8_t* p0 = bs + b_off + (((b_chunk + i) ^ b_swz) << 4);
+    i32x2 r[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      r[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(p0 + q * 8 * kSkinnyBN));
+    i32x8 fb = {r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]};
+    // First operand = B panel: the accumulator of lane (m = r16, quarter qd) holds columns
+    // n = 4 qd + v of row m.
+    acc[i] = mfma_f8_16(fb, fa, acc[i]);
+  }
+}
+
+template <int N>
+__device__ __forceinline__ void skinny_wait_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
+}
 
 __global__ void __launch_bounds__(256) gemm8_skinny(GemmArgs g, float* partial, int k_chunk) {
-  __shared__ __attribute__((aligned(16))) uint8_t As[2][16 * kStride8];
-  __shared__ __attribute__((aligned(16))) uint8_t Bs[2][kSkinnyBN * kStride8];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_sk[];
+  uint8_t* const ring = smem_sk;
+  uint8_t* const a_lds = smem_sk + kSkinnyStages * kSkinnyStageBytes;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n0 = blockIdx.x * kSkinnyBN;
   const int kbeg = blockIdx.y * k_chunk;
+  const int nk = k_chunk / kBK8;
   const uint8_t* A = reinterpret_cast<const uint8_t*>(g.a);
   const uint8_t* B = reinterpret_cast<const uint8_t*>(g.b);
+  const int r16 = lane & 15, qd = lane >> 4;
 
-  // Loader: B tile 128 k x 128 n = 256 units of 16k x 4n (one per thread); A tile 16 x 128 =
-  // 128 chunks of 16 bytes (threads 0..127; rows >= M read as zero).
-  const int ngrp = tid % (kSkinnyBN / 4), kgrp = tid / (kSkinnyBN / 4);
-  const int a_row = tid >> 3, a_kc = tid & 7;
-  uint32_t rb[16];
-  u32x4 ra = {0, 0, 0, 0};
-  auto load_global = [&](int k0) {
-    const uint8_t* p = B + (int64_t)(k0 + kgrp * 16) * g.ldb + n0 + ngrp * 4;
+  // A: k-step t is a 16 x 128-byte block (2 KiB = 2 wave-wide loads); wave w loads the halves
+  // u = w, w + 4, ... of the 2 nk halves.  Rows >= M repeat row M - 1 (their results are unused).
+  for (int u = wave; u < 2 * nk; u += 4) {
+    const int m = 8 * (u & 1) + (lane >> 3);
+    const int gc = (lane & 7) ^ ((m >> 1) & 7);
+    const int row = m < g.M ? m : g.M - 1;
+    async8_copy16(A + (int64_t)row * g.lda + kbeg + (u >> 1) * kBK8 + gc * 16, a_lds + u * 1024);
+  }
+  // B: load i of wave w fills k rows (4 i + w) 4 .. +4 of a stage; lane -> row += lane / 16, LDS
+  // chunk lane % 16.
+  const uint8_t* b_src[8];
 #pragma unroll
-    for (int kk = 0; kk < 16; ++kk) rb[kk] = *reinterpret_cast<const uint32_t*>(p + (int64_t)kk * g.ldb);
-    if (tid < 128 && a_row < g.M) ra = *reinterpret_cast<const u32x4*>(A + (int64_t)a_row * g.lda + k0 + a_kc * 16);
-  };
-  auto store_lds = [&](int buf) {
+  for (int i = 0; i < 8; ++i) {
+    const int k = (4 * i + wave) * 4 + (lane >> 4);
+    const int gc = (lane & 15) ^ ((k & 7) | (((k >> 5) & 1) << 3));
+    b_src[i] = B + (int64_t)(kbeg + k) * g.ldb + n0 + gc * 16;
+  }
 #pragma unroll
-    for (int q = 0; q < 4; ++q) transpose4x4_bytes(rb[4 * q], rb[4 * q + 1], rb[4 * q + 2], rb[4 * q + 3]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      u32x4 w = {rb[j], rb[4 + j], rb[8 + j], rb[12 + j]};
-      *reinterpret_cast<u32x4*>(&Bs[buf][(ngrp * 4 + j) * kStride8 + kgrp * 16]) = w;
-    }
-    if (tid < 128) *reinterpret_cast<u32x4*>(&As[buf][a_row * kStride8 + a_kc * 16]) = ra;
-  };
+  for (int st = 0; st < kSkinnyStages - 1; ++st)
+    if (st < nk) skinny_issue_b(b_src, g.ldb, st, wave, ring + st * kSkinnyStageBytes);
 
-  f32x4 acc[2];
+  // Fragment addressing.  A: row r16 of the step's block, logical chunks 2 qd, 2 qd + 1.  B
+  // through the transposing read: lane (j = lane % 16, quarter qd) addresses k row
+  // 32 qd + 8 q + j / 2, bytes 16 (4 w + i) + 8 (j % 2) .. +8 of it.
+  const int a_off = r16 * 128, a_swz = (r16 >> 1) & 7;
+  const int b_off = (32 * qd + (r16 >> 1)) * kSkinnyBN + 8 * (r16 & 1);
+  const int b_chunk = 4 * wave;
+  const int b_swz = (r16 >> 1) | ((qd & 1) << 3);
+
+  f32x4 acc[4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int v = 0; v < 4; ++v) acc[i][v] = 0.0f;
-  const int nk = k_chunk / kBK8;
-  load_global(kbeg);
-  store_lds(0);
-  __syncthreads();
-  const int r16 = lane & 15, qd = lane >> 4;  // row/col within the MFMA tile, k quarter
+
   for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < nk) load_global(kbeg + (kt + 1) * kBK8);
-    i32x4 alo = *reinterpret_cast<const i32x4*>(&As[buf][r16 * kStride8 + 32 * qd]);
-    i32x4 ahi = *reinterpret_cast<const i32x4*>(&As[buf][r16 * kStride8 + 32 * qd + 16]);
-    i32x8 fa = {alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const uint8_t* bp = &Bs[buf][(wave * 32 + 16 * i + r16) * kStride8 + 32 * qd];
-      i32x4 blo = *reinterpret_cast<const i32x4*>(bp);
-      i32x4 bhi = *reinterpret_cast<const i32x4*>(bp + 16);
-      i32x8 fb = {blo[0], blo[1], blo[2], blo[3], bhi[0], bhi[1], bhi[2], bhi[3]};
-      // First operand = B panel: the accumulator of lane (m = r16, quarter qd) holds
-      // columns n = 4 qd + v of row m.
-      acc[i] = mfma_f8_16(fb, fa, acc[i]);
-    }
-    if (kt + 1 < nk) store_lds(buf ^ 1);
-    __syncthreads();
+    // Stages kt + 1, kt + 2 may stay in flight (8 loads per lane each); the A loads were issued
+    // first and are older than every B stage.
+    const int younger = min(nk - 1 - kt, kSkinnyStages - 2);
+    if (younger >= 2) skinny_wait_barrier<16>();
+    else if (younger == 1) skinny_wait_barrier<8>();
+    else skinny_wait_barrier<0>();
+    const int nxt = kt + kSkinnyStages - 1;
+    skinny_step(acc, ring + (kt % kSkinnyStages) * kSkinnyStageBytes, a_lds + kt * 2048,
+                ring + (nxt % kSkinnyStages) * kSkinnyStageBytes, b_src, g.ldb, nxt, nxt < nk, wave, a_off, a_swz, qd,
+                b_off, b_chunk, b_swz);
   }
-  float* dst = partial + ((int64_t)blockIdx.y * 16 + r16) * g.N + n0 + wave * 32 + 4 * qd;
+  float* dst = partial + ((int64_t)blockIdx.y * 16 + r16) * g.N + n0 + wave * 64 + 4 * qd;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) *reinterpret_cast<f32x4*>(dst + 16 * i) = acc[i];
+  for (int i = 0; i < 4; ++i) *reinterpret_cast<f32x4*>(dst + 16 * i) = acc[i];
 }
 
 __global__ void __launch_bounds__(256) gemm8_skinny_reduce(GemmArgs g, const float* partial, int splits) {
@@ -547,26 +597,35 @@ static int launch_fast8(const GemmArgs& g, hipStream_t s) {
 int gemm8(const GemmArgs& g, hipStream_t s) {
   const bool vec_ok = g.K % kBK8 == 0 && g.lda % 16 == 0 && g.ldb % 4 == 0 && g.ldc % 4 == 0 && aligned16(g.a) &&
                       aligned16(g.b) && aligned16(g.out);
-  if (vec_ok && g.M <= 16 && g.N % kSkinnyBN == 0) {
-    // Split K so that about 512 workgroups stream B.
-    int splits = 1;
+  if (vec_ok && g.M <= 16 && g.N % kSkinnyBN == 0 && g.ldb % 16 == 0) {
+    // Split K so that about one workgroup per CU streams B (its ring alone keeps 96 KiB in
+    // flight) and the A chunk fits its LDS area.
     const int nblk = g.N / kSkinnyBN;
-    while (nblk * splits < 512 && (g.K / kBK8) % (splits * 2) == 0 && splits < 64) splits *= 2;
-    const size_t need = (size_t)splits * 16 * g.N * sizeof(float);
-    if (need > g_partial_bytes) {
-      if (g_partial) LH_HIP_CHECK(hipFree(g_partial));
-      g_partial = nullptr;
-      g_partial_bytes = 0;
-      LH_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&g_partial), need));
-      g_partial_bytes = need;
+    int splits = 1;
+    while ((nblk * splits < 256 || g.K / splits > kSkinnyMaxChunk) && (g.K / kBK8) % (splits * 2) == 0) splits *= 2;
+    if (g.K / splits <= kSkinnyMaxChunk) {
+      const size_t need = (size_t)splits * 16 * g.N * sizeof(float);
+      if (need > g_partial_bytes) {
+        if (g_partial) LH_HIP_CHECK(hipFree(g_partial));
+        g_partial = nullptr;
+        g_partial_bytes = 0;
+        LH_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&g_partial), need));
+        g_partial_bytes = need;
+      }
+      static bool configured = false;
+      if (!configured) {
+        LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_skinny),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, kSkinnyLdsBytes));
+        configured = true;
+      }
+      hipLaunchKernelGGL(gemm8_skinny, dim3(nblk, splits), dim3(256), kSkinnyLdsBytes, s, g, g_partial, g.K / splits);
+      int rc = check_launch("gemm8_skinny");
+      if (rc) return rc;
+      const int64_t total = (int64_t)g.M * g.N;
+      hipLaunchKernelGGL(gemm8_skinny_reduce, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, g, g_partial,
+                         splits);
+      return check_launch("gemm8_skinny_reduce");
     }
-    hipLaunchKernelGGL(gemm8_skinny, dim3(nblk, splits), dim3(256), 0, s, g, g_partial, g.K / splits);
-    int rc = check_launch("gemm8_skinny");
-    if (rc) return rc;
-    const int64_t total = (int64_t)g.M * g.N;
-    hipLaunchKernelGGL(gemm8_skinny_reduce, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, g, g_partial,
-                       splits);
-    return check_launch("gemm8_skinny_reduce");
   }
   if (vec_ok && g.M % 256 == 0 && g.N % 256 == 0 && (int64_t)(g.M / 256) * (g.N / 256) >= 128) {
     if (g.ldb % 16 == 0 && g.ldc % 8 == 0) return launch_direct8(g, s);

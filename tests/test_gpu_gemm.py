@@ -11,6 +11,7 @@ pytestmark = pytest.mark.gpu
 
 F32_RTOL = 1e-4   # benchmark definition: f32 within rtol 1e-4
 BF16_RTOL = 2e-2  # bf16 within rtol 2e-2 of the f32 reference
+FP8_RTOL = 5e-2   # fp8 within rtol 5e-2 of the dequantised f32 reference
 
 
 def _dev(x, dtype):
@@ -232,3 +233,26 @@ def test_gemm_fp8_all_codes():
                        torch.from_numpy(b).cuda().view(torch.float8_e4m3fn), 1.0, 1.0, out_dtype=torch.float32)
     ref = np.outer(table[a[:, 0]].astype(np.float64), table[b[0, :]].astype(np.float64))
     np.testing.assert_array_equal(_host(out), ref.astype(np.float32))
+
+
+@pytest.mark.parametrize("shape", [(16, 1024, 8192), (7, 384, 4096), (1, 128, 2048), (16, 2048, 384)])
+def test_gemm_fp8_decode_path(shape):
+    """M <= 16: split-K streaming kernel with the reduction fused into the last workgroup; called
+    three times in a row (the per-column-block counters must return to zero) and with an f32 output."""
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(5 + M + N + K)
+    aq, sa = orc.quantize_per_tensor_e4m3(rng.standard_normal((M, K)).astype(np.float32))
+    bq, sb = orc.quantize_per_tensor_e4m3(rng.standard_normal((K, N)).astype(np.float32))
+    da = torch.from_numpy(aq).to("cuda").view(torch.float8_e4m3fn)
+    db = torch.from_numpy(bq).to("cuda").view(torch.float8_e4m3fn)
+    ref = orc.matmul_fp8(aq, bq, sa, sb, result_type="bf16")
+    first = None
+    for _ in range(3):
+        out = ops.gemm_fp8(da, db, float(sa), float(sb))
+        assert_close(_host(out), ref, FP8_RTOL, f"fp8 decode {shape}")
+        first = out if first is None else first
+        assert torch.equal(out, first)
+    out32 = ops.gemm_fp8(da, db, float(sa), float(sb), out_dtype=torch.float32)
+    assert_close(_host(out32), orc.matmul_fp8(aq, bq, sa, sb, result_type="f32"), FP8_RTOL, f"fp8 decode f32 {shape}")
