@@ -195,6 +195,19 @@ int lh_hip_nanogpt_block(float* y, const float* x, const lh_nanogpt_block_params
                          int64_t C, int64_t n_head, float eps, int32_t dtype, void* workspace,
                          size_t workspace_bytes, void* stream);
 
+/*
+ * n_layer blocks followed by the final LayerNorm and the lm_head projection with bias, the shape
+ * of build_gpt_fused_payload (examples/xegpu/nanoGPT_payload.py:318-407; embeddings stay on the
+ * host side there too): logits[B*T, vocab] (f32) = LN_f(block_n(...block_1(x))) W_lm + b_lm.
+ * Blocks are lh_hip_nanogpt_block's; lm_w [C, vocab] and lm_b [vocab] have `dtype`.  `workspace`
+ * must hold lh_hip_nanogpt_forward_workspace_bytes(...) bytes.
+ */
+size_t lh_hip_nanogpt_forward_workspace_bytes(int64_t B, int64_t T, int64_t C, int32_t dtype);
+int lh_hip_nanogpt_forward(float* logits, const float* x, const lh_nanogpt_block_params* blocks, int64_t n_layer,
+                           const float* lnf_g, const float* lnf_b, const void* lm_w, const void* lm_b, int64_t B,
+                           int64_t T, int64_t C, int64_t n_head, int64_t vocab, float eps, int32_t dtype,
+                           void* workspace, size_t workspace_bytes, void* stream);
+
 /* ------------------------------------------------- packed-argument payloads ---- */
 
 /*

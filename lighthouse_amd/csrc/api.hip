@@ -170,6 +170,42 @@ int lh_hip_nanogpt_block(float* y, const float* x, const lh_nanogpt_block_params
                   LH_GEMM_HAS_BIAS | LH_GEMM_ACCUMULATE_C, s);
 }
 
+size_t lh_hip_nanogpt_forward_workspace_bytes(int64_t B, int64_t T, int64_t C, int32_t dtype) {
+  const size_t rows = (size_t)B * T;
+  return lh_hip_nanogpt_block_workspace_bytes(B, T, C, dtype) + 2 * align256(rows * C * 4); /* residual streams */
+}
+
+int lh_hip_nanogpt_forward(float* logits, const float* x, const lh_nanogpt_block_params* blocks, int64_t n_layer,
+                           const float* lnf_g, const float* lnf_b, const void* lm_w, const void* lm_b, int64_t B,
+                           int64_t T, int64_t C, int64_t n_head, int64_t vocab, float eps, int32_t dtype,
+                           void* workspace, size_t workspace_bytes, void* stream) {
+  LH_REQUIRE(logits && x && lnf_g && lnf_b && lm_w && workspace, "lh_hip_nanogpt_forward: null pointer");
+  LH_REQUIRE(n_layer >= 0 && (n_layer == 0 || blocks), "lh_hip_nanogpt_forward: bad layer list");
+  LH_REQUIRE(dtype == LH_F32 || dtype == LH_BF16, "lh_hip_nanogpt_forward: dtype must be f32 or bf16");
+  LH_REQUIRE(B > 0 && T > 0 && C > 0 && vocab > 0, "lh_hip_nanogpt_forward: bad shape");
+  LH_REQUIRE(workspace_bytes >= lh_hip_nanogpt_forward_workspace_bytes(B, T, C, dtype),
+             "lh_hip_nanogpt_forward: workspace too small (%zu bytes)", workspace_bytes);
+  LH_REQUIRE(aligned16(workspace), "lh_hip_nanogpt_forward: workspace must be 16-byte aligned");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const int64_t rows = B * T;
+  const size_t block_ws = lh_hip_nanogpt_block_workspace_bytes(B, T, C, dtype);
+  char* w = reinterpret_cast<char*>(workspace);
+  float* h[2] = {reinterpret_cast<float*>(w + block_ws),
+                 reinterpret_cast<float*>(w + block_ws + align256((size_t)rows * C * 4))};
+  const float* cur = x;
+  for (int64_t l = 0; l < n_layer; ++l) {
+    float* nxt = h[l & 1];
+    int rc = lh_hip_nanogpt_block(nxt, cur, &blocks[l], B, T, C, n_head, eps, dtype, workspace, block_ws, stream);
+    if (rc) return rc;
+    cur = nxt;
+  }
+  // hf = LN_f(h) rounded to the matmul input type (first area of the block workspace), then lm_head.
+  int rc = lh_hip_layer_norm(workspace, cur, lnf_g, lnf_b, rows, C, eps, LH_F32, dtype, s);
+  if (rc) return rc;
+  return gemm_run(logits, nullptr, workspace, lm_w, lm_b, rows, vocab, C, C, vocab, vocab, dtype, LH_F32, dtype,
+                  lm_b ? LH_GEMM_HAS_BIAS : 0, s);
+}
+
 // ---- packed-argument payloads -------------------------------------------------------------
 
 int lh_hip_payload_matmul(void** args, int32_t nargs, const lh_matmul_attrs* at) {

@@ -183,3 +183,25 @@ def nanogpt_block(x, params: dict, n_head: int, *, eps=1e-5, out=None, workspace
         out.data_ptr(), x.data_ptr(), ctypes.byref(p), B, T, C, n_head, float(eps), lh_dtype(dtype),
         workspace.data_ptr(), workspace.numel(), _stream()), "nanogpt_block")
     return out
+
+
+def nanogpt_forward(x, layers: list, lnf_g, lnf_b, lm_w, lm_b, n_head: int, *, eps=1e-5, out=None, workspace=None):
+    """n blocks + final LayerNorm + lm_head. x: [B,T,C] float32; `layers`: one parameter dict per
+    block (see nanogpt_block); lm_w [C, vocab] and lm_b [vocab] in the blocks' dtype. Returns float32
+    logits [B,T,vocab]."""
+    _need_cuda(x, out, workspace, lnf_g, lnf_b, lm_w, lm_b, *[t for p in layers for t in p.values()])
+    B, T, C = x.shape
+    vocab = lm_w.shape[1]
+    dtype = lm_w.dtype
+    if out is None:
+        out = torch.empty((B, T, vocab), dtype=torch.float32, device=x.device)
+    need = int(_lib.load().lh_hip_nanogpt_forward_workspace_bytes(B, T, C, lh_dtype(dtype)))
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=x.device)
+    blocks = (_lib.NanoGPTBlockParams * max(len(layers), 1))(
+        *[_lib.NanoGPTBlockParams(*[p[n].data_ptr() for n in BLOCK_PARAM_NAMES]) for p in layers])
+    _lib.check(_lib.load().lh_hip_nanogpt_forward(
+        out.data_ptr(), x.data_ptr(), blocks, len(layers), lnf_g.data_ptr(), lnf_b.data_ptr(), lm_w.data_ptr(),
+        lm_b.data_ptr() if lm_b is not None else None, B, T, C, n_head, vocab, float(eps), lh_dtype(dtype),
+        workspace.data_ptr(), workspace.numel(), _stream()), "nanogpt_forward")
+    return out

@@ -468,6 +468,20 @@ def nanogpt_block(x, p: dict, n_head: int, *, mode: str = "f32", eps: float = 1e
     return (a + o).astype(np.float32).reshape(bsz, t, c)
 
 
+def nanogpt_forward(x, layers, lnf_g, lnf_b, lm_w, lm_b, n_head: int, *, mode: str = "f32", eps: float = 1e-5):
+    """n blocks, final LayerNorm, lm_head with bias: the tail of ``build_gpt_fused_payload``
+    examples/xegpu/nanoGPT_payload.py:401-407 (``hf = LN(h)``, cast to the matmul input type,
+    ``logits = hf W + b`` in float32) after ``nanogpt_block`` applied per layer (:399-400)."""
+    elt = "f32" if mode == "f32" else "bf16"
+    h = np.asarray(x, dtype=np.float32)
+    for p in layers:
+        h = nanogpt_block(h, p, n_head, mode=mode, eps=eps)
+    bsz, t, c = h.shape
+    hf = layer_norm(h.reshape(bsz * t, c), lnf_g, lnf_b, eps, elt)
+    logits = matmul(hf, round_to(lm_w, elt), bias=None if lm_b is None else round_to(lm_b, elt), result_type="f32")
+    return logits.reshape(bsz, t, -1)
+
+
 def _attention_rounded_p(q, k, v, *, causal: bool, elt: str):
     """Attention with the probabilities rounded to ``elt`` before P.V and the row sum
     taken over the unrounded probabilities (the fused kernel's rounding points,

@@ -205,3 +205,24 @@ def test_runner_mlp_payload(ab, res, bias_t, variant):
     ref = orc.mlp(x, ws, bs, has_relu=has_relu, relu_on_final_layer=final, accumulate_c=c0 if acc else None,
                   ab_type=ab, result_type=res)
     assert_close(to_float32(out), ref, 1e-4 if ab == "f32" else 2e-2, f"mlp {ab}->{res} {variant}")
+
+
+@pytest.mark.parametrize("mode,dtype,rtol", [("f32", torch.float32, 1e-4), ("bf16", torch.bfloat16, 2e-2)])
+def test_nanogpt_forward_two_layers(mode, dtype, rtol):
+    """Two blocks + ln_f + lm_head (the tail of build_gpt_fused_payload, nanoGPT_payload.py:399-407)."""
+    from lighthouse_amd import ops
+
+    B, T, C, H, V = 2, 128, 256, 4, 384
+    rng = np.random.default_rng(0x6770)
+    layers = [make_block_params(C, rng, bias_std=0.02) for _ in range(2)]
+    lnf_g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    lnf_b = rng.uniform(-0.1, 0.1, C).astype(np.float32)
+    lm_w = (rng.standard_normal((C, V)) * 0.05).astype(np.float32)
+    lm_b = (rng.standard_normal(V) * 0.02).astype(np.float32)
+    x = rng.standard_normal((B, T, C)).astype(np.float32)
+    dev = lambda a, dt=torch.float32: torch.from_numpy(a).cuda().to(dt)  # noqa: E731
+    y = ops.nanogpt_forward(dev(x), [to_device(p, dtype) for p in layers], dev(lnf_g), dev(lnf_b), dev(lm_w, dtype),
+                            dev(lm_b, dtype), H)
+    ref = orc.nanogpt_forward(x, layers, lnf_g, lnf_b, lm_w, lm_b, H, mode=mode)
+    assert y.shape == (B, T, V)
+    assert_close(y.cpu().numpy(), ref, rtol, f"nanoGPT forward {mode}")
