@@ -140,7 +140,7 @@ def main() -> int:
 
     extras = {}
     if not args.no_extras:
-        def rate(fn, work, steps=20, warmup=5):
+        def rate(fn, work, steps=50, warmup=20):
             _, e = time_region(fn, steps, warmup)
             return work * steps / e
 
@@ -160,7 +160,7 @@ def main() -> int:
         a8 = (torch.randn(n8, n8, device="cuda", generator=g)).clamp(-4, 4).to(torch.float8_e4m3fn)
         b8 = (torch.randn(n8, n8, device="cuda", generator=g)).clamp(-4, 4).to(torch.float8_e4m3fn)
         o8 = torch.empty(n8, n8, device="cuda", dtype=torch.bfloat16)
-        extras["gemm_fp8_8192_tflops"] = rate(lambda: ops.gemm_fp8(a8, b8, 0.01, 0.01, out=o8), 2.0 * n8**3, 10, 3) / 1e12
+        extras["gemm_fp8_8192_tflops"] = rate(lambda: ops.gemm_fp8(a8, b8, 0.01, 0.01, out=o8), 2.0 * n8**3, 20, 5) / 1e12
         a8d = a8[:16].contiguous()
         o8d = torch.empty(16, n8, device="cuda", dtype=torch.bfloat16)
         dec_bytes = n8 * n8 + 16 * n8 + 16 * n8 * 2
@@ -189,7 +189,7 @@ def main() -> int:
             yb = torch.empty_like(xb)
             ws = torch.empty(ops.nanogpt_block_workspace_bytes(B, T, C, dt), dtype=torch.uint8, device="cuda")
             bflops = 128849018880.0  # causal-halved attention
-            extras[f"nanogpt_block_{name}_tflops"] = rate(lambda: ops.nanogpt_block(xb, p, H, out=yb, workspace=ws), bflops, 10, 3) / 1e12
+            extras[f"nanogpt_block_{name}_tflops"] = rate(lambda: ops.nanogpt_block(xb, p, H, out=yb, workspace=ws), bflops, 30, 10) / 1e12
         extras = {k: round(float(v), 3) for k, v in extras.items()}
 
     cpu = None

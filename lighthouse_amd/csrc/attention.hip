@@ -31,6 +31,7 @@ struct AttnArgs {
   float scale_log2e;  // scale * log2(e)
   float scale;
   int causal;
+  int cus;  // compute units of the device (causal launch order)
 };
 
 template <int DT>
@@ -205,20 +206,22 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
   const int nqb = (a.T + kQBlock16 - 1) / kQBlock16;
   int qb, bh;
   if (a.causal) {
-    // Causal work grows with the query block index.  The 1-D grid lists the heavier half of the
-    // query blocks first (heaviest first), then the lighter half lightest first, so that
-    // workgroup L and workgroup L + gridDim/2 -- which share a CU when the whole grid is
-    // resident at two workgroups per CU -- always add up to the same number of key tiles.
+    // Causal work grows with the query block index.  Rank r (0 = heaviest) is query block
+    // nqb - 1 - r / bhn of (batch, head) r % bhn.  With more workgroups than 2 per CU, or at most
+    // 1, the 1-D grid simply lists the ranks heaviest first.  In between every workgroup is
+    // resident at once, workgroup L on CU L % cus, so the first n2 = grid - cus CUs run two: they
+    // get the lightest of the first `cus` ranks, lightest first, each joined by the next of the
+    // remaining ranks (sums stay level), and the other CUs get the heaviest ranks alone.
     const int bhn = a.Z * a.H;
-    const int L = blockIdx.x;
-    const int heavy = (nqb / 2) * bhn;  // workgroups in the heavy half
-    if (L < heavy) {
-      qb = nqb - 1 - L / bhn;
-      bh = L % bhn;
-    } else {
-      qb = (L - heavy) / bhn;
-      bh = (L - heavy) % bhn;
+    const int G = gridDim.x, R = a.cus, L = blockIdx.x;
+    int r = L;
+    if (G > R && G <= 2 * R) {
+      const int n2 = G - R;
+      if (L < n2) r = R - 1 - L;
+      else if (L < R) r = L - n2;
     }
+    qb = nqb - 1 - r / bhn;
+    bh = r % bhn;
   } else {
     qb = blockIdx.x;
     bh = blockIdx.y;
@@ -497,5 +500,12 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   a.scale = scale;
   a.scale_log2e = scale * 1.4426950408889634f;
   a.causal = causal ? 1 : 0;
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    LH_HIP_CHECK(hipGetDevice(&dev));
+    LH_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  }
+  a.cus = cus;
   return attention_launch(a, dtype, reinterpret_cast<hipStream_t>(stream));
 }
