@@ -191,6 +191,12 @@ def main() -> int:
             bflops = 128849018880.0  # causal-halved attention
             extras[f"nanogpt_block_{name}_tflops"] = rate(lambda: ops.nanogpt_block(xb, p, H, out=yb, workspace=ws), bflops, 30, 10) / 1e12
         extras = {k: round(float(v), 3) for k, v in extras.items()}
+        # Register-only MFMA loops: what the matrix cores sustain on zero and on random operands.
+        extras["mfma_register_loop_tflops"] = {
+            f"{name}_{kind}": round(ops.probe_mfma_rate(dt, kind == "random", iters), 1)
+            for name, dt, iters in (("bf16", torch.bfloat16, 20000), ("fp8", torch.float8_e4m3fn, 10000),
+                                    ("f32", torch.float32, 20000))
+            for kind in ("zero", "random")}
 
     cpu = None
     if not args.no_cpu_baseline:

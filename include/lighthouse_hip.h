@@ -208,6 +208,14 @@ int lh_hip_nanogpt_forward(float* logits, const float* x, const lh_nanogpt_block
                            int64_t T, int64_t C, int64_t n_head, int64_t vocab, float eps, int32_t dtype,
                            void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * Measurement aid (no counterpart in the reference): TFLOP/s of a register-only MFMA loop of the
+ * given element type (LH_BF16, LH_F8E4M3, LH_F32) on every SIMD, with all-zero (random_operands
+ * = 0) or random operands.  The matrix-core clock depends on operand bit activity, so this is the
+ * rate a GEMM on such data can approach; bench.py reports it beside the published peak.
+ */
+int lh_hip_probe_mfma_rate(int32_t dtype, int32_t random_operands, int64_t iters, double* tflops);
+
 /* ------------------------------------------------- packed-argument payloads ---- */
 
 /*

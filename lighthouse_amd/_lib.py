@@ -119,6 +119,7 @@ PROTOTYPES = {
     "lh_hip_nanogpt_forward_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
     "lh_hip_nanogpt_forward": (_i32, [_vp, _vp, ctypes.POINTER(NanoGPTBlockParams), _i64, _vp, _vp, _vp, _vp, _i64, _i64,
                                       _i64, _i64, _i64, _f32, _i32, _vp, _sz, _vp]),
+    "lh_hip_probe_mfma_rate": (_i32, [_i32, _i32, _i64, ctypes.POINTER(ctypes.c_double)]),
     "lh_hip_payload_matmul": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(MatmulAttrs)]),
     "lh_hip_payload_matmul_fp8": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(MatmulFp8Attrs)]),
     "lh_hip_payload_mlp": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(MlpAttrs)]),

@@ -19,7 +19,7 @@ LIB_DIR = ROOT / "lighthouse_amd" / "lib"
 LIB_PATH = LIB_DIR / "liblighthouse_hip.so"
 ORACLE_LIB = ROOT / "oracle" / "_build" / "libcpu_ref.so"
 
-HIP_SOURCES = ["runtime.hip", "gemm16.hip", "gemm32.hip", "gemm8.hip", "attention.hip", "rowwise.hip", "api.hip"]
+HIP_SOURCES = ["runtime.hip", "gemm16.hip", "gemm32.hip", "gemm8.hip", "attention.hip", "rowwise.hip", "probe.hip", "api.hip"]
 
 HIPCC_FLAGS = [
     "-O3",

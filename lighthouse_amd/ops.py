@@ -205,3 +205,11 @@ def nanogpt_forward(x, layers: list, lnf_g, lnf_b, lm_w, lm_b, n_head: int, *, e
         lm_b.data_ptr() if lm_b is not None else None, B, T, C, n_head, vocab, float(eps), lh_dtype(dtype),
         workspace.data_ptr(), workspace.numel(), _stream()), "nanogpt_forward")
     return out
+
+
+def probe_mfma_rate(dtype, random_operands: bool, iters: int = 20000) -> float:
+    """TFLOP/s of a register-only MFMA loop on every SIMD (see lh_hip_probe_mfma_rate)."""
+    out = ctypes.c_double(0.0)
+    _lib.check(_lib.load().lh_hip_probe_mfma_rate(lh_dtype(dtype), 1 if random_operands else 0, int(iters),
+                                                  ctypes.byref(out)), "probe_mfma_rate")
+    return out.value
