@@ -191,6 +191,24 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
       }
 }
 
+// Launch order of a causal problem.  Causal work grows with the query block index.  Rank r
+// (0 = heaviest) is query block nqb - 1 - r / bhn of (batch, head) r % bhn.  With more workgroups
+// than 2 per CU, or at most 1, the 1-D grid simply lists the ranks heaviest first (workgroups
+// start as slots free up, so the long ones must not come last).  In between every workgroup is
+// resident at once, workgroup L on CU L % cus, so the first n2 = grid - cus CUs run two: they get
+// the lightest of the first `cus` ranks, lightest first, each joined by the next of the remaining
+// ranks (sums stay level), and the other CUs get the heaviest ranks alone.
+__device__ __forceinline__ void causal_block_of(int L, int G, int R, int nqb, int bhn, int& qb, int& bh) {
+  int r = L;
+  if (G > R && G <= 2 * R) {
+    const int n2 = G - R;
+    if (L < n2) r = R - 1 - L;
+    else if (L < R) r = L - n2;
+  }
+  qb = nqb - 1 - r / bhn;
+  bh = r % bhn;
+}
+
 // 16-bit kernel.  A workgroup owns 256 query rows of one (batch, head): 4 waves x 64 rows (two
 // 32-row sub-tiles per wave share every K and V fragment).  K/V tiles of 64 keys go global ->
 // LDS with global_load_lds_dwordx4 through a ring of 4 stages; K fragments are 16-byte LDS
@@ -206,22 +224,7 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
   const int nqb = (a.T + kQBlock16 - 1) / kQBlock16;
   int qb, bh;
   if (a.causal) {
-    // Causal work grows with the query block index.  Rank r (0 = heaviest) is query block
-    // nqb - 1 - r / bhn of (batch, head) r % bhn.  With more workgroups than 2 per CU, or at most
-    // 1, the 1-D grid simply lists the ranks heaviest first.  In between every workgroup is
-    // resident at once, workgroup L on CU L % cus, so the first n2 = grid - cus CUs run two: they
-    // get the lightest of the first `cus` ranks, lightest first, each joined by the next of the
-    // remaining ranks (sums stay level), and the other CUs get the heaviest ranks alone.
-    const int bhn = a.Z * a.H;
-    const int G = gridDim.x, R = a.cus, L = blockIdx.x;
-    int r = L;
-    if (G > R && G <= 2 * R) {
-      const int n2 = G - R;
-      if (L < n2) r = R - 1 - L;
-      else if (L < R) r = L - n2;
-    }
-    qb = nqb - 1 - r / bhn;
-    bh = r % bhn;
+    causal_block_of(blockIdx.x, gridDim.x, a.cus, nqb, a.Z * a.H, qb, bh);
   } else {
     qb = blockIdx.x;
     bh = blockIdx.y;
@@ -327,19 +330,119 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
   }
 }
 
-// f32 variant (all tensors f32, f32 MFMA): same structure; P stays f32, K and V tiles keep
-// their global orientation in LDS because the f32 MFMA takes a single value per lane.
-constexpr int kAttn32KStride = 68;  // floats per K row (64 + 4): 16-byte reads of 16 rows conflict free
-constexpr int kAttn32VStride = 72;  // floats per V row: rows 4 apart land 32 banks apart
+// f32 variant (all tensors f32, v_mfma_f32_32x32x2_f32): same transposed formulation; P stays
+// f32.  A workgroup owns 128 query rows (4 waves x 32).  K and V tiles of 64 keys keep their
+// global orientation in LDS (rows of 256 bytes), loaded with global_load_lds_dwordx4 one tile
+// ahead into the other of two 32 KiB stages.  Unpadded rows again: the 16-byte chunk a lane
+// fetches is XOR-swizzled, K chunk ^ (key % 16) (a lane reads 4 consecutive d of its key row),
+// V chunk ^ 8 ((key / 4) % 2) (the two half waves read rows 4 apart at the same columns).
+constexpr int kAttn32StageBytes = 2 * kKvTile * kHeadDim * 4;  // K tile + V tile
+
+struct Attn32Ctx {
+  const float* k_src[4];
+  const float* v_src[4];
+  int64_t k_step, v_step;
+  int wave, r32, h;
+  int k_off[2], k_swz[2];
+  int v_col[2];  // byte offset of the lane's V column inside a row, per head-dim sub-tile (unswizzled half)
+};
+
+__device__ __forceinline__ void attn32_copy16(const float* gsrc, uint8_t* lds_wave_base) {
+  __builtin_amdgcn_global_load_lds(gsrc, (attn_lds_void_t*)lds_wave_base, 16, 0, 0);
+}
+
+__device__ __forceinline__ void attn32_issue(const Attn32Ctx& c, int jt, uint8_t* __restrict__ stage) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    attn32_copy16(c.k_src[i] + jt * c.k_step, stage + (4 * i + c.wave) * 1024);
+    attn32_copy16(c.v_src[i] + jt * c.v_step, stage + 16384 + (4 * i + c.wave) * 1024);
+  }
+}
+
+// One key tile for the wave's 32 query rows; `wr` receives the next tile meanwhile.
+__device__ __forceinline__ void attn32_tile(const Attn32Ctx& c, const AttnArgs& a, const f32x4 (&qf)[8],
+                                            f32x16 (&acc_o)[2], float& m_run, float& l_run,
+                                            const uint8_t* __restrict__ rd, uint8_t* __restrict__ wr, int next_jt,
+                                            bool prefetch, int j0, int wq0, bool active, bool need_mask) {
+  if (prefetch) attn32_issue(c, next_jt, wr);
+  if (!active) return;
+  const uint8_t* ks = rd;
+  const uint8_t* vs = rd + 16384;
+  f32x16 s_acc[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s_acc[i][v] = 0.0f;
+  // The two key sub-tiles alternate so that consecutive MFMAs never depend on each other.
+#pragma unroll
+  for (int kk = 0; kk < 8; ++kk) {
+    f32x4 kf[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      kf[i] = *reinterpret_cast<const f32x4*>(ks + c.k_off[i] + (((2 * kk + c.h) ^ c.k_swz[i]) << 4));
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        s_acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[i][t], qf[kk][t], s_acc[i], 0, 0, 0);
+  }
+  // s_acc[i][v] = S[q = wq0 + r32][key = j0 + 32 i + 8 (v/4) + 4 h + v%4] (unscaled)
+  if (need_mask) {
+    const int qrow = wq0 + c.r32;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        int key = j0 + 32 * i + 8 * (v >> 2) + 4 * c.h + (v & 3);
+        if (key > qrow) s_acc[i][v] = -INFINITY;
+      }
+  }
+  float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
+#pragma unroll
+  for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[0][v]), s_acc[1][v]);
+  mx = halfwave_max(mx);
+  const float m_new = fmaxf(m_run, mx);
+  const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+  // exp(x) as exp2(x log2 e): v_exp_f32 is accurate to about 1 ulp, the scaled argument (|x| < 100)
+  // to 1e-5 absolute, well inside the f32 tolerance of the payload.
+  const float alpha = exp2_fast((m_run - m_safe) * a.scale_log2e);
+  const float mc = m_safe * a.scale_log2e;
+  float l_tile = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      s_acc[i][v] = exp2_fast(s_acc[i][v] * a.scale_log2e - mc);
+      l_tile += s_acc[i][v];
+    }
+  l_run = l_run * alpha + l_tile;
+  m_run = m_new;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc_o[j][v] *= alpha;
+  // O^T += V^T P^T, one key (pair) per MFMA: lane (d = r32, half h) reads V[key][32 j + r32].
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int key = 32 * i + 8 * (v >> 2) + 4 * c.h + (v & 3);  // (key / 4) % 2 == h
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        float vf = *reinterpret_cast<const float*>(vs + key * 256 + c.v_col[j]);
+        acc_o[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf, s_acc[i][v], acc_o[j], 0, 0, 0);
+      }
+    }
+}
 
 __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
-  __shared__ __attribute__((aligned(16))) float Ks[kKvTile * kAttn32KStride];
-  __shared__ __attribute__((aligned(16))) float Vs[kKvTile * kAttn32VStride];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn32[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, h = lane >> 5;
   const int nqb = a.T / kQBlock;
-  const int qb = a.causal ? (nqb - 1 - (int)blockIdx.x) : (int)blockIdx.x;
-  const int bh = blockIdx.y;
+  int qb = blockIdx.x, bh = blockIdx.y;
+  if (a.causal) causal_block_of(blockIdx.x, gridDim.x, a.cus, nqb, a.Z * a.H, qb, bh);
   const int z = bh / a.H, hd = bh % a.H;
   const int q0 = qb * kQBlock;
   const int wq0 = q0 + wave * 32;
@@ -347,6 +450,31 @@ __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
   const float* K = reinterpret_cast<const float*>(a.k) + (int64_t)z * a.sk.z + (int64_t)hd * a.sk.h;
   const float* V = reinterpret_cast<const float*>(a.v) + (int64_t)z * a.sv.z + (int64_t)hd * a.sv.h;
   float* O = reinterpret_cast<float*>(a.out) + (int64_t)z * a.so.z + (int64_t)hd * a.so.h;
+
+  Attn32Ctx c;
+  c.wave = wave; c.r32 = r32; c.h = h;
+  c.k_step = (int64_t)kKvTile * a.sk.t;
+  c.v_step = (int64_t)kKvTile * a.sv.t;
+  // Loader: load i of wave w fills keys (4 i + w) 4 .. +4; lane -> key += lane / 16, LDS chunk
+  // p = lane % 16 holds global chunk p ^ swizzle(key).
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int key = (4 * i + wave) * 4 + (lane >> 4);
+    const int p = lane & 15;
+    c.k_src[i] = K + (int64_t)key * a.sk.t + ((p ^ (key & 15)) << 2);
+    c.v_src[i] = V + (int64_t)key * a.sv.t + ((p ^ (8 * ((key >> 2) & 1))) << 2);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int key = 32 * i + r32;
+    c.k_off[i] = key * 256;
+    c.k_swz[i] = key & 15;
+  }
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int col = 32 * j + r32;
+    c.v_col[j] = (((col >> 2) ^ (8 * h)) << 4) + (col & 3) * 4;
+  }
 
   // Lane (q = r32, half h) holds Q[q][8 kk + 4 h + t], kk = 0..7, t = 0..3.
   f32x4 qf[8];
@@ -361,79 +489,21 @@ __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
     for (int v = 0; v < 16; ++v) acc_o[j][v] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
   const int kv_end = a.causal ? min(a.T, q0 + kQBlock) : a.T;
+  const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
 
-  for (int j0 = 0; j0 < kv_end; j0 += kKvTile) {
-    __syncthreads();
-    for (int c = tid; c < kKvTile * 16; c += 256) {
-      int row = c >> 4, ch = c & 15;
-      *reinterpret_cast<f32x4*>(&Ks[row * kAttn32KStride + ch * 4]) =
-          *reinterpret_cast<const f32x4*>(K + (int64_t)(j0 + row) * a.sk.t + ch * 4);
-      *reinterpret_cast<f32x4*>(&Vs[row * kAttn32VStride + ch * 4]) =
-          *reinterpret_cast<const f32x4*>(V + (int64_t)(j0 + row) * a.sv.t + ch * 4);
-    }
-    __syncthreads();
+  attn32_issue(c, 0, smem_attn32);
+  for (int jt = 0; jt < ntiles; ++jt) {
+    // Tile jt is the only load in flight: wait for it, and the barrier also says every wave is
+    // done reading the stage the next tile is about to overwrite.
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    const int j0 = jt * kKvTile;
     const bool active = !a.causal || (j0 <= wq0 + 31);
-    if (!active) continue;
-    f32x16 s_acc[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-#pragma unroll
-      for (int v = 0; v < 16; ++v) s_acc[i][v] = 0.0f;
-#pragma unroll
-      for (int kk = 0; kk < 8; ++kk) {
-        f32x4 kf = *reinterpret_cast<const f32x4*>(&Ks[(32 * i + r32) * kAttn32KStride + 8 * kk + 4 * h]);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) s_acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[t], qf[kk][t], s_acc[i], 0, 0, 0);
-      }
-    }
-    if (a.causal && (j0 + kKvTile - 1 > wq0)) {
-      const int qrow = wq0 + r32;
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          int key = j0 + 32 * i + 8 * (v >> 2) + 4 * h + (v & 3);
-          if (key > qrow) s_acc[i][v] = -INFINITY;
-        }
-    }
-    float mx = s_acc[0][0];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s_acc[i][v]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m_run, mx);
-    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-    // f32 path: exact exp (not the exp2 shortcut) to stay within the f32 tolerance.
-    const float alpha = expf((m_run - m_safe) * a.scale);
-    float l_tile = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        s_acc[i][v] = expf((s_acc[i][v] - m_safe) * a.scale);
-        l_tile += s_acc[i][v];
-      }
-    l_run = l_run * alpha + l_tile;
-    m_run = m_new;
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc_o[j][v] *= alpha;
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int key = 32 * i + 8 * (v >> 2) + 4 * h + (v & 3);
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          float vf = Vs[key * kAttn32VStride + 32 * j + r32];
-          acc_o[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf, s_acc[i][v], acc_o[j], 0, 0, 0);
-        }
-      }
+    const bool need_mask = a.causal && (j0 + kKvTile - 1 > wq0);
+    attn32_tile(c, a, qf, acc_o, m_run, l_run, smem_attn32 + (jt & 1) * kAttn32StageBytes,
+                smem_attn32 + ((jt + 1) & 1) * kAttn32StageBytes, jt + 1, jt + 1 < ntiles, j0, wq0, active, need_mask);
   }
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-  const float inv_l = 1.0f / l_tot;
+
+  const float inv_l = 1.0f / halfwave_sum(l_run);
   float* orow = O + (int64_t)(wq0 + r32) * a.so.t;
 #pragma unroll
   for (int j = 0; j < 2; ++j)
@@ -464,7 +534,15 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
 int attention_launch(const AttnArgs& a, int dtype, hipStream_t s) {
   if (dtype == LH_BF16) return attention16_launch<LH_BF16>(a, s);
   if (dtype == LH_F16) return attention16_launch<LH_F16>(a, s);
-  hipLaunchKernelGGL(attention32_kernel, dim3(a.T / kQBlock, a.Z * a.H), dim3(256), 0, s, a);
+  static bool configured32 = false;
+  if (!configured32) {
+    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention32_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kAttn32StageBytes));
+    configured32 = true;
+  }
+  const int nqb32 = a.T / kQBlock;
+  const dim3 grid32 = a.causal ? dim3(nqb32 * a.Z * a.H) : dim3(nqb32, a.Z * a.H);
+  hipLaunchKernelGGL(attention32_kernel, grid32, dim3(256), 2 * kAttn32StageBytes, s, a);
   return check_launch("attention32");
 }
 
