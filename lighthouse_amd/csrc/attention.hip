@@ -97,9 +97,9 @@ __device__ __forceinline__ void attn_issue_loads(const AttnCtx& c, int jt, uint8
 // One key tile (64 keys) for the wave's two 32-row query sub-tiles.  `rd` holds the tile, `wr`
 // is the ring slot that receives a later tile meanwhile (separate restrict pointers so that LDS
 // reads do not wait for the asynchronous writes).
-template <int DT>
-__device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, const u32x4 (&qf)[2][4],
-                                          f32x16 (&acc_o)[2][2], float (&m_run)[2], float (&l_run)[2],
+template <int DT, int NQ>
+__device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, const u32x4 (&qf)[NQ][4],
+                                          f32x16 (&acc_o)[NQ][2], float (&m_run)[NQ], float (&l_run)[NQ],
                                           const uint8_t* __restrict__ rd, uint8_t* __restrict__ wr, int next_jt,
                                           bool prefetch, int j0, int wq0, bool active, bool need_mask) {
   if (prefetch) attn_issue_loads(c, next_jt, wr);
@@ -107,9 +107,9 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
   const uint8_t* ks = rd;
   const uint8_t* vs = rd + 8192;
   // S^T = K Q^T: key sub-tile i (32 keys) x query sub-tile qt (32 rows).
-  f32x16 s_acc[2][2];
+  f32x16 s_acc[NQ][2];
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt)
+  for (int qt = 0; qt < NQ; ++qt)
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -120,12 +120,12 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
     for (int sd = 0; sd < 4; ++sd) {
       u32x4 kf = *reinterpret_cast<const u32x4*>(ks + c.k_off[i] + (((2 * sd + c.h) ^ c.k_swz[i]) << 4));
 #pragma unroll
-      for (int qt = 0; qt < 2; ++qt) s_acc[qt][i] = mfma16<DT>(kf, qf[qt][sd], s_acc[qt][i]);
+      for (int qt = 0; qt < NQ; ++qt) s_acc[qt][i] = mfma16<DT>(kf, qf[qt][sd], s_acc[qt][i]);
     }
   // s_acc[qt][i][v] = S[q = wq0 + 32 qt + r32][key = j0 + 32 i + 8 (v/4) + 4 h + v%4] (unscaled)
-  u32x4 pf[2][2][2];
+  u32x4 pf[NQ][2][2];
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
+  for (int qt = 0; qt < NQ; ++qt) {
     if (need_mask) {
       const int qrow = wq0 + 32 * qt + c.r32;
 #pragma unroll
@@ -187,7 +187,7 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
         u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
         u32x4 vf = {l2[0], l2[1], h2[0], h2[1]};
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt) acc_o[qt][j] = mfma16<DT>(vf, pf[qt][i][u], acc_o[qt][j]);
+        for (int qt = 0; qt < NQ; ++qt) acc_o[qt][j] = mfma16<DT>(vf, pf[qt][i][u], acc_o[qt][j]);
       }
 }
 
@@ -215,13 +215,14 @@ __device__ __forceinline__ void causal_block_of(int L, int G, int R, int nqb, in
 // reads, V^T fragments come from ds_read_b64_tr_b16 on the row-major V tile.  Rows of a tile
 // are 128 bytes and cannot be padded (a wave-wide load writes 1 KiB contiguous), so the
 // 16-byte chunk a lane fetches is XOR-swizzled: K chunk ^ ((key / 2) % 8), V chunk ^ 4 ((key / 2) % 2).
-template <int DT>
+template <int DT, int NQ>
 __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
+  constexpr int kRowsPerWave = 32 * NQ, kRowsPerGroup = 4 * kRowsPerWave;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, h = lane >> 5;
-  const int nqb = (a.T + kQBlock16 - 1) / kQBlock16;
+  const int nqb = (a.T + kRowsPerGroup - 1) / kRowsPerGroup;
   int qb, bh;
   if (a.causal) {
     causal_block_of(blockIdx.x, gridDim.x, a.cus, nqb, a.Z * a.H, qb, bh);
@@ -230,9 +231,9 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
     bh = blockIdx.y;
   }
   const int z = bh / a.H, hd = bh % a.H;
-  const int q0 = qb * kQBlock16;
-  const int wq0 = q0 + wave * 64;
-  // T is a multiple of 64: a wave's 64 rows are all inside the sequence or all outside (last
+  const int q0 = qb * kRowsPerGroup;
+  const int wq0 = q0 + wave * kRowsPerWave;
+  // T is a multiple of 64: a wave's rows are all inside the sequence or all outside (last
   // workgroup only); an outside wave still takes part in the loads and barriers.
   const bool wave_valid = wq0 < a.T;
   const int wq_load = wave_valid ? wq0 : 0;
@@ -276,23 +277,28 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
   }
   // Q fragments: second MFMA operand of S^T = K Q^T; lane (q = r32, half h) holds
   // Q[q][16 sd + 8 h .. +8] for the 4 k-steps over the head dimension, for both sub-tiles.
-  u32x4 qf[2][4];
+  u32x4 qf[NQ][4];
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt)
+  for (int qt = 0; qt < NQ; ++qt)
 #pragma unroll
     for (int sd = 0; sd < 4; ++sd)
       qf[qt][sd] = *reinterpret_cast<const u32x4*>(Q + (int64_t)(wq_load + 32 * qt + r32) * a.sq.t + 16 * sd + 8 * h);
 
-  f32x16 acc_o[2][2];
+  f32x16 acc_o[NQ][2];
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt)
+  for (int qt = 0; qt < NQ; ++qt)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc_o[qt][j][v] = 0.0f;
-  float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.0f, 0.0f};
+  float m_run[NQ], l_run[NQ];
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) {
+    m_run[qt] = -INFINITY;
+    l_run[qt] = 0.0f;
+  }
 
-  const int kv_end = a.causal ? min(a.T, q0 + kQBlock16) : a.T;
+  const int kv_end = a.causal ? min(a.T, q0 + kRowsPerGroup) : a.T;
   const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
 #pragma unroll
   for (int st = 0; st < kAttnStages - 1; ++st)
@@ -306,17 +312,17 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
     else if (younger == 1) asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     const int j0 = jt * kKvTile;
-    const bool active = wave_valid && (!a.causal || (j0 <= wq0 + 63));
+    const bool active = wave_valid && (!a.causal || (j0 <= wq0 + kRowsPerWave - 1));
     const bool need_mask = a.causal && (j0 + kKvTile - 1 > wq0);
     const int nxt = jt + kAttnStages - 1;
-    attn_tile<DT>(c, a, qf, acc_o, m_run, l_run, smem_attn + (jt % kAttnStages) * kAttnStageBytes,
+    attn_tile<DT, NQ>(c, a, qf, acc_o, m_run, l_run, smem_attn + (jt % kAttnStages) * kAttnStageBytes,
                   smem_attn + (nxt % kAttnStages) * kAttnStageBytes, nxt, nxt < ntiles, j0, wq0, active, need_mask);
   }
 
   // acc_o[qt][j][v] = O[q = wq0 + 32 qt + r32][d = 32 j + 8 (v/4) + 4 h + v%4] * l
   if (!wave_valid) return;
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
+  for (int qt = 0; qt < NQ; ++qt) {
     const float inv_l = 1.0f / halfwave_sum(l_run[qt]);
     uint16_t* orow = O + (int64_t)(wq0 + 32 * qt + r32) * a.so.t;
 #pragma unroll
@@ -515,9 +521,9 @@ __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
     }
 }
 
-template <int DT>
-static int attention16_launch(const AttnArgs& a, hipStream_t s) {
-  auto kern = attention16_kernel<DT>;
+template <int DT, int NQ>
+static int attention16_launch_nq(const AttnArgs& a, hipStream_t s) {
+  auto kern = attention16_kernel<DT, NQ>;
   constexpr size_t lds = (size_t)kAttnStages * kAttnStageBytes;
   static bool configured = false;
   if (!configured) {
@@ -525,10 +531,23 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
                                      (int)lds));
     configured = true;
   }
-  const int nqb = (a.T + kQBlock16 - 1) / kQBlock16;
+  const int nqb = (a.T + 128 * NQ - 1) / (128 * NQ);
   const dim3 grid = a.causal ? dim3(nqb * a.Z * a.H) : dim3(nqb, a.Z * a.H);
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, a);
   return check_launch("attention16");
+}
+
+// 64 query rows per wave share every K/V fragment between two sub-tiles; 32 rows per wave give
+// twice the workgroups, each half as long, which is what a problem needs that would otherwise
+// leave CUs with fewer than two workgroups or hang on its heaviest causal block.
+template <int DT>
+static int attention16_launch(const AttnArgs& a, hipStream_t s) {
+  const int64_t groups64 = (int64_t)((a.T + kQBlock16 - 1) / kQBlock16) * a.Z * a.H;
+  // Measured on [4,16,2048]: 32 rows per wave 105 us non-causal (64 rows: 99) but 54 us causal
+  // (64 rows: 58), hence the different limits.
+  const int64_t limit = a.causal ? 2 * (int64_t)a.cus + 1 : 2 * (int64_t)a.cus;
+  if (groups64 < limit) return attention16_launch_nq<DT, 1>(a, s);
+  return attention16_launch_nq<DT, 2>(a, s);
 }
 
 int attention_launch(const AttnArgs& a, int dtype, hipStream_t s) {
