@@ -110,6 +110,22 @@ def test_attention_benchmark_size(causal):
         assert_close(_host(out[z, h]), ref, 2e-2, f"attention bench size z={z} h={h} causal={causal}")
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype,shape,rtol", [(torch.bfloat16, (8, 20, 1024, 64), 2e-2), (torch.float32, (3, 8, 1024, 64), 1e-4)])
+def test_attention_many_groups(dtype, shape, rtol, causal):
+    """More workgroups than two per CU: the 64-rows-per-wave kernel with the heaviest-first causal
+    launch order (16-bit), and the 1-D causal grid of the f32 kernel; sampled (batch, head) pairs."""
+    from lighthouse_amd import ops
+
+    g = torch.Generator(device="cuda").manual_seed(78)
+    q, k, v = (torch.randn(shape, device="cuda", generator=g).to(dtype) for _ in range(3))
+    out = ops.attention(q, k, v, causal=causal)
+    assert torch.isfinite(out.float()).all()
+    for z, h in [(0, 0), (shape[0] - 1, shape[1] - 1), (1, 5)]:
+        ref = orc.attention(_host(q[z, h]), _host(k[z, h]), _host(v[z, h]), causal=causal)
+        assert_close(_host(out[z, h]), ref, rtol, f"attention {shape} z={z} h={h} causal={causal}")
+
+
 def test_attention_errors():
     from lighthouse_amd import ops
 
