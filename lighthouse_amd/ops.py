@@ -52,6 +52,12 @@ def gemm(a, b, bias=None, *, out=None, out_dtype=None, relu=False, gelu=False, a
     flags = ((_lib.GEMM_HAS_BIAS if bias is not None else 0) | (_lib.GEMM_HAS_RELU if relu else 0)
              | (_lib.GEMM_HAS_GELU if gelu else 0) | (_lib.GEMM_ACCUMULATE_C if accumulate_c else 0)
              | (_lib.GEMM_TRANSPOSE_A if transpose_a else 0) | (_lib.GEMM_TRANSPOSE_B if transpose_b else 0))
+    if tile is None and a.dtype in (torch.bfloat16, torch.float16) and not (transpose_a or transpose_b):
+        from .tuning.tile_db import active_db  # a tuned tile for this shape, if a database is in use
+
+        db = active_db()
+        if db is not None:
+            tile = db.lookup("bf16" if a.dtype == torch.bfloat16 else "f16", M, N, K)
     if tile is not None:
         if tuple(tile) not in _lib.GEMM_TILES:
             raise ValueError(f"unsupported tile {tile}; choose from {sorted(_lib.GEMM_TILES)}")

@@ -1,0 +1,6 @@
+from .csv_logger import CSVLogger
+from .tile_db import TileDB, active_db, use_db
+from .tune_gemm import candidate_tiles, estimate_cost, prefilter, run_with_timeout, tune_shape
+
+__all__ = ["CSVLogger", "TileDB", "active_db", "use_db", "candidate_tiles", "estimate_cost", "prefilter",
+           "run_with_timeout", "tune_shape"]

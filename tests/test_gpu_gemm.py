@@ -256,3 +256,27 @@ def test_gemm_fp8_decode_path(shape):
         assert torch.equal(out, first)
     out32 = ops.gemm_fp8(da, db, float(sa), float(sb), out_dtype=torch.float32)
     assert_close(_host(out32), orc.matmul_fp8(aq, bq, sa, sb, result_type="f32"), FP8_RTOL, f"fp8 decode f32 {shape}")
+
+
+def test_tile_search_and_database(tmp_path):
+    """The tuner times every fitting tile for a shape, logs the trials, records the winner, and
+    ops.gemm picks the recorded tile up when the database is in use (same results either way)."""
+    from lighthouse_amd import ops
+    from lighthouse_amd.tuning import CSVLogger, TileDB, tune_shape, use_db
+
+    M, N, K = 1024, 768, 256
+    db = TileDB(str(tmp_path / "tiles.json"))
+    logger = CSVLogger(str(tmp_path / "trials.csv"), echo_stdout=False)
+    best = tune_shape(M, N, K, "bf16", db, logger, nruns=5, nwarmup=2, exhaustive=True, isolate=False)
+    rows = (tmp_path / "trials.csv").read_text().strip().splitlines()
+    assert len(rows) == 1 + 4 and best is not None and best["error"] == "" and best["tflops"] > 0
+    assert db.lookup("bf16", M, N, K) == (best["tile_m"], best["tile_n"])
+    a = torch.randn(M, K, device="cuda").to(torch.bfloat16)
+    b = torch.randn(K, N, device="cuda").to(torch.bfloat16)
+    plain = ops.gemm(a, b)
+    try:
+        use_db(db)
+        tuned = ops.gemm(a, b)
+    finally:
+        use_db(None)
+    assert torch.equal(plain, tuned)  # every tile accumulates k in the same order

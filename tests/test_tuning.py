@@ -1,0 +1,72 @@
+"""Tile search harness: candidates, cost-model pre-filter, isolated trials, CSV log, database."""
+
+import csv
+import time
+
+import pytest
+
+from lighthouse_amd.tuning import CSVLogger, TileDB, active_db, candidate_tiles, estimate_cost, prefilter, \
+    run_with_timeout, use_db
+
+
+def test_candidates_and_prefilter():
+    assert candidate_tiles(8192, 768, 768) == [(256, 256), (256, 128), (128, 256), (128, 128)]
+    assert candidate_tiles(384, 128, 64) == [(128, 128)]
+    assert candidate_tiles(256, 256, 96) == []          # K must be a multiple of 64
+    # 4096^3: 256 tiles of 256 x 256 are exactly one round, every smaller tile costs more
+    assert prefilter(4096, 4096, 4096)[0] == (256, 256)
+    # N = 768: 96 big tiles leave CUs idle; halves and quarters are estimated cheaper
+    assert prefilter(8192, 768, 768)[0] in ((256, 128), (128, 256))
+    assert estimate_cost(8192, 768, 768, (256, 256)) > estimate_cost(8192, 768, 768, (256, 128))
+    assert all(t in candidate_tiles(8192, 2304, 768) for t in prefilter(8192, 2304, 768))
+
+
+def _ok(res, x):
+    res["time"] = 0.5
+    res["throughput"] = float(x)
+
+
+def _boom(res):
+    raise RuntimeError("tile does not fit\\nsecond line")
+
+
+def _hang(res):
+    time.sleep(30)
+
+
+def test_run_with_timeout_isolates_failures():
+    assert run_with_timeout(_ok, 3, timeout=20) == {"time": 0.5, "throughput": 3.0, "error": ""}
+    assert "tile does not fit" in run_with_timeout(_boom, timeout=20)["error"]
+    assert run_with_timeout(_hang, timeout=0.5)["error"] == "TIMEOUT"
+
+
+def test_csv_logger(tmp_path, capsys):
+    path = tmp_path / "log.csv"
+    path.write_text("taken\\n")
+    logger = CSVLogger(str(path))
+    assert logger.filename.endswith("log_1.csv")        # never overwrites an existing log
+    logger.log({"M": 1, "tile": "a", "tflops": 2.5})
+    logger.log({"M": 2, "tile": "b", "tflops": 3.5})
+    with pytest.raises(ValueError):
+        logger.log({"M": 3})
+    rows = list(csv.DictReader(open(logger.filename)))
+    assert rows == [{"M": "1", "tile": "a", "tflops": "2.5"}, {"M": "2", "tile": "b", "tflops": "3.5"}]
+    assert capsys.readouterr().out.splitlines()[0] == "M,tile,tflops"
+
+
+def test_tile_db_round_trip(tmp_path):
+    db = TileDB(str(tmp_path / "tiles.json"))
+    assert db.lookup("bf16", 8192, 768, 768) is None
+    db.record("bf16", 8192, 768, 768, (256, 128), 19.7, 491.0)
+    db.save()
+    again = TileDB(str(tmp_path / "tiles.json"))
+    assert again.lookup("bf16", 8192, 768, 768) == (256, 128)
+    assert again.lookup("f16", 8192, 768, 768) is None
+    (tmp_path / "bad.json").write_text('{"bf16:1x1x1": {"time_us": 1}}')
+    with pytest.raises(ValueError):
+        TileDB(str(tmp_path / "bad.json"))
+    try:
+        assert use_db(again) is again and active_db() is again
+    finally:
+        use_db(None)
+    assert active_db() is None
