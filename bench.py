@@ -190,6 +190,10 @@ def main() -> int:
             ws = torch.empty(ops.nanogpt_block_workspace_bytes(B, T, C, dt), dtype=torch.uint8, device="cuda")
             bflops = 128849018880.0  # causal-halved attention
             extras[f"nanogpt_block_{name}_tflops"] = rate(lambda: ops.nanogpt_block(xb, p, H, out=yb, workspace=ws), bflops, 30, 10) / 1e12
+        # Vendor library kernels through torch on the same tensors, for orientation only.
+        extras["torch_matmul_bf16_4096_tflops"] = rate(lambda: torch.matmul(a, b, out=out), flops) / 1e12
+        extras["torch_sdpa_bf16_noncausal_tflops"] = rate(
+            lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v), aflops) / 1e12
         extras = {k: round(float(v), 3) for k, v in extras.items()}
         # Register-only MFMA loops: what the matrix cores sustain on zero and on random operands.
         extras["mfma_register_loop_tflops"] = {
