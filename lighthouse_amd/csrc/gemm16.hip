@@ -359,8 +359,11 @@ __device__ __forceinline__ void direct_step_pair(const DirectCtx<TM, TN>& c, f32
   direct_interleave_hint<TM, TN>();
 }
 
-// One output tile; `id` is the tile's position in the XCD-grouped order.
-template <int DT, int TM, int TN>
+// One output tile; `id` is the tile's position in the XCD-grouped order.  EDGE: M and N need not
+// be multiples of the tile (N still a multiple of 8, K of 64): loads of rows / column chunks past
+// the end are redirected to the last valid row / chunk (their products land in accumulators that
+// are never stored) and the epilogue skips what lies outside the matrix.
+template <int DT, int TM, int TN, bool EDGE>
 __device__ __forceinline__ void direct_tile(const GemmArgs& g, int id, uint8_t* smem_d) {
   using Cfg = DirectCfg<TM, TN>;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, WN = 4, WTM = Cfg::WTM, WTN = Cfg::WTN;
@@ -368,7 +371,7 @@ __device__ __forceinline__ void direct_tile(const GemmArgs& g, int id, uint8_t* 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
 
-  const int tiles_m = g.M / BM, tiles_n = g.N / BN;
+  const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
   constexpr int GROUP_M = 4;
   const int group_size = GROUP_M * tiles_n;
   const int first_m = (id / group_size) * GROUP_M;
@@ -390,7 +393,8 @@ __device__ __forceinline__ void direct_tile(const GemmArgs& g, int id, uint8_t* 
   for (int i = 0; i < TM; ++i) {
     const int ar = (8 * i + wave) * 8 + (lane >> 3);
     const int ac = (lane & 7) ^ ((ar >> 1) & 7);
-    c.a_src[i] = A + (int64_t)(m0 + ar) * g.lda + ac * 8;
+    const int arow = EDGE ? min(m0 + ar, g.M - 1) : m0 + ar;
+    c.a_src[i] = A + (int64_t)arow * g.lda + ac * 8;
   }
   // B: load i of wave w fills k rows (8 i + w) R .. +R with R = 1024 / row bytes; lane ->
   // row += lane / chunks-per-row, LDS chunk p holds global chunk p ^ 4 (k % 4).
@@ -398,7 +402,8 @@ __device__ __forceinline__ void direct_tile(const GemmArgs& g, int id, uint8_t* 
   for (int i = 0; i < TN; ++i) {
     const int bk = (8 * i + wave) * Cfg::kBRowsPerLoad + lane / Cfg::kBChunks;
     const int bc = (lane % Cfg::kBChunks) ^ (4 * (bk & 3));
-    c.b_src[i] = B + (int64_t)bk * g.ldb + n0 + bc * 8;
+    const int bcol = EDGE ? min(n0 + bc * 8, g.N - 8) : n0 + bc * 8;
+    c.b_src[i] = B + (int64_t)bk * g.ldb + bcol;
   }
   // A fragment (second MFMA operand): row wm0 + 32 j + r32, logical chunk 2 kc + h.
 #pragma unroll
@@ -480,8 +485,10 @@ __device__ __forceinline__ void direct_tile(const GemmArgs& g, int id, uint8_t* 
       for (int j = 0; j < TM; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          u32x2 w = epilogue4_pack<DT>(g, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
-                                       acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+          u32x2 w = {0u, 0u};
+          if (!EDGE || n_base + 32 * i + 8 * q < g.N)  // the bias row ends at N
+            w = epilogue4_pack<DT>(g, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                                   acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
           *reinterpret_cast<u32x2*>(cw + (32 * j + r32) * cstride + (32 * i + 8 * q + 4 * h) * 2) = w;
         }
     uint16_t* outp = reinterpret_cast<uint16_t*>(g.out);
@@ -489,7 +496,8 @@ __device__ __forceinline__ void direct_tile(const GemmArgs& g, int id, uint8_t* 
     for (int t = 0; t < WTM / rows_per_pass; ++t) {
       const int row = rows_per_pass * t + lane / chunks, ch = lane % chunks;
       u32x4 w = *reinterpret_cast<const u32x4*>(cw + row * cstride + ch * 16);
-      *reinterpret_cast<u32x4*>(outp + (int64_t)(m0 + wm0 + row) * g.ldc + n0 + wn0 + ch * 8) = w;
+      if (!EDGE || (m0 + wm0 + row < g.M && n0 + wn0 + ch * 8 < g.N))
+        *reinterpret_cast<u32x4*>(outp + (int64_t)(m0 + wm0 + row) * g.ldc + n0 + wn0 + ch * 8) = w;
     }
     return;
   }
@@ -499,29 +507,30 @@ __device__ __forceinline__ void direct_tile(const GemmArgs& g, int id, uint8_t* 
     for (int j = 0; j < TM; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q)
-        epilogue4<DT>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
-                      acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+        if (!EDGE || (m_base + 32 * j < g.M && n_base + 32 * i + 8 * q < g.N))
+          epilogue4<DT>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                        acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
 }
 
 // Persistent workgroups: one (two for the 128 x 128 tile, whose rings are 64 KiB) per CU, each
 // walking the tile list with the grid as stride.  Tile ids congruent modulo 8 stay on one XCD,
 // which is what xcd_remap assumes.  Launching one workgroup per tile instead costs a
 // workgroup launch plus a cold prologue per tile, about a third of a K = 768 tile's time.
-template <int DT, int TM, int TN>
+template <int DT, int TM, int TN, bool EDGE>
 __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
   using Cfg = DirectCfg<TM, TN>;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_d[];
-  const int ntiles = (g.M / Cfg::BM) * (g.N / Cfg::BN);
+  const int ntiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
   for (int t = blockIdx.x; t < ntiles; t += gridDim.x) {
     if (t != (int)blockIdx.x) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS is reused
-    direct_tile<DT, TM, TN>(g, xcd_remap(t, ntiles), smem_d);
+    direct_tile<DT, TM, TN, EDGE>(g, xcd_remap(t, ntiles), smem_d);
   }
 }
 
-template <int DT, int TM, int TN>
-static int launch_direct(const GemmArgs& g, hipStream_t s) {
+template <int DT, int TM, int TN, bool EDGE>
+static int launch_direct_edge(const GemmArgs& g, hipStream_t s) {
   using Cfg = DirectCfg<TM, TN>;
-  auto kern = gemm16_direct<DT, TM, TN>;
+  auto kern = gemm16_direct<DT, TM, TN, EDGE>;
   constexpr size_t lds = Cfg::kLdsBytes;
   static bool configured = false;
   if (!configured) {
@@ -529,10 +538,17 @@ static int launch_direct(const GemmArgs& g, hipStream_t s) {
                                      (int)lds));
     configured = true;
   }
-  const int ntiles = (g.M / Cfg::BM) * (g.N / Cfg::BN);
+  const int ntiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
   const int resident = 256 * (2 * lds <= 160 * 1024 ? 2 : 1);
   hipLaunchKernelGGL(kern, dim3(ntiles < resident ? ntiles : resident), dim3(512), lds, s, g);
   return check_launch("gemm16_direct");
+}
+
+template <int DT, int TM, int TN>
+static int launch_direct(const GemmArgs& g, hipStream_t s) {
+  using Cfg = DirectCfg<TM, TN>;
+  if (g.M % Cfg::BM == 0 && g.N % Cfg::BN == 0) return launch_direct_edge<DT, TM, TN, false>(g, s);
+  return launch_direct_edge<DT, TM, TN, true>(g, s);
 }
 
 // Any shape / stride / transpose; 64 x 64 x 32 tiles, 256 threads, bounds-checked.
@@ -602,17 +618,16 @@ static int launch_fast(const GemmArgs& g, hipStream_t s) {
   return check_launch("gemm16_fast");
 }
 
-// Tile choice for the direct kernels: 0 = 256 x 256, 1 = 256 x 128, 2 = 128 x 256, 3 = 128 x 128,
-// -1 = none fits.  Cost model: rounds of 256 workgroups (one per CU) times the tile area, with a
-// penalty for the smaller tiles' extra operand traffic per flop.
+// Tile choice for the direct kernels: 0 = 256 x 256, 1 = 256 x 128, 2 = 128 x 256, 3 = 128 x 128.
+// Cost model: rounds of 256 workgroups (one per CU) times the tile area (edge tiles count in
+// full), with a penalty for the smaller tiles' extra operand traffic per flop.
 static int direct_variant(int M, int N) {
   static const int bm[4] = {256, 256, 128, 128}, bn[4] = {256, 128, 256, 128};
   static const double penalty[4] = {1.0, 1.1, 1.1, 1.25};
   int best = -1;
   double best_cost = 0.0;
   for (int v = 0; v < 4; ++v) {
-    if (M % bm[v] || N % bn[v]) continue;
-    const int64_t tiles = (int64_t)(M / bm[v]) * (N / bn[v]);
+    const int64_t tiles = (int64_t)((M + bm[v] - 1) / bm[v]) * ((N + bn[v] - 1) / bn[v]);
     const double cost = (double)((tiles + 255) / 256) * bm[v] * bn[v] * penalty[v];
     if (best < 0 || cost < best_cost) {
       best = v;
@@ -638,7 +653,7 @@ static int gemm16_dispatch(const GemmArgs& g, hipStream_t s) {
                bm[v], bn[v], bm[v], bn[v], g.M, g.N, g.K);
   }
   if (vec_ok) {
-    if (!tb && g.ldc % 8 == 0) {
+    if (!tb && g.ldc % 8 == 0 && g.N % 8 == 0) {
       const int v = tile != LH_GEMM_TILE_AUTO ? (int)(tile >> 8) - 1 : direct_variant(g.M, g.N);
       if (v == 0) return launch_direct<DT, 4, 2>(g, s);
       if (v == 1) return launch_direct<DT, 4, 1>(g, s);

@@ -103,6 +103,42 @@ def test_gemm_16bit_requested_tile(tile, K, epi):
     assert_close(_host(out), ref, rtol, f"bf16 gemm tile {tile} K={K} {epi}")
 
 
+@pytest.mark.parametrize("shape", [(1000, 520, 192), (130, 264, 64), (257, 8, 128), (1, 1000, 256), (3000, 776, 320)])
+@pytest.mark.parametrize("epi", ["none", "bias_relu", "f32out_acc_bias"])
+def test_gemm_16bit_ragged_shapes(shape, epi):
+    """M and N that no tile divides (N a multiple of 8, K of 64): the direct kernel's edge
+    instantiation; rows and columns past the end must be neither read as bias nor written."""
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(3 * M + 5 * N + K)
+    a = orc.round_to(rng.standard_normal((M, K)).astype(np.float32), "bf16")
+    b = orc.round_to(rng.standard_normal((K, N)).astype(np.float32), "bf16")
+    bias = orc.round_to(rng.standard_normal((N,)).astype(np.float32), "bf16")
+    da, db = _dev(a, torch.bfloat16), _dev(b, torch.bfloat16)
+    # output embedded in a larger canvas: everything around it must stay untouched
+    pad = 8
+    if epi == "f32out_acc_bias":
+        c = rng.standard_normal((M, N)).astype(np.float32)
+        canvas = torch.full((M + 2, N + 2 * pad), 7.0, device="cuda")
+        view = canvas[1:M + 1, pad:pad + N]
+        view.copy_(_dev(c, torch.float32))
+        ops.gemm(da, db, _dev(bias.astype(np.float32), torch.float32), out=view, accumulate_c=True)
+        ref = orc.matmul(a, b, c=c, bias=bias, accumulate_c=True, result_type="f32")
+        rtol = F32_RTOL
+    else:
+        canvas = torch.full((M + 2, N + 2 * pad), 7.0, device="cuda", dtype=torch.bfloat16)
+        view = canvas[1:M + 1, pad:pad + N]
+        has = epi == "bias_relu"
+        ops.gemm(da, db, _dev(bias, torch.bfloat16) if has else None, relu=has, out=view)
+        ref = orc.matmul(a, b, bias=bias if has else None, relu=has, result_type="bf16")
+        rtol = BF16_RTOL
+    assert_close(_host(view), ref, rtol, f"ragged bf16 gemm {shape} {epi}")
+    border = canvas.float().clone()
+    border[1:M + 1, pad:pad + N] = 7.0
+    assert (border == 7.0).all(), "the kernel wrote outside the output matrix"
+
+
 def test_gemm_tile_request_errors():
     from lighthouse_amd import ops
 
