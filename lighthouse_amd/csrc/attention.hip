@@ -597,12 +597,6 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   a.scale = scale;
   a.scale_log2e = scale * 1.4426950408889634f;
   a.causal = causal ? 1 : 0;
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0;
-    LH_HIP_CHECK(hipGetDevice(&dev));
-    LH_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  }
-  a.cus = cus;
+  a.cus = num_cus();
   return attention_launch(a, dtype, reinterpret_cast<hipStream_t>(stream));
 }

@@ -146,5 +146,7 @@ __device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
 }
 
 hipStream_t default_stream();
+// Compute units of the current device (cached; 256 if the query fails).
+int num_cus();
 
 }  // namespace lh

@@ -539,7 +539,7 @@ static int launch_direct_edge(const GemmArgs& g, hipStream_t s) {
     configured = true;
   }
   const int ntiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
-  const int resident = 256 * (2 * lds <= 160 * 1024 ? 2 : 1);
+  const int resident = num_cus() * (2 * lds <= 160 * 1024 ? 2 : 1);
   hipLaunchKernelGGL(kern, dim3(ntiles < resident ? ntiles : resident), dim3(512), lds, s, g);
   return check_launch("gemm16_direct");
 }
@@ -619,16 +619,17 @@ static int launch_fast(const GemmArgs& g, hipStream_t s) {
 }
 
 // Tile choice for the direct kernels: 0 = 256 x 256, 1 = 256 x 128, 2 = 128 x 256, 3 = 128 x 128.
-// Cost model: rounds of 256 workgroups (one per CU) times the tile area (edge tiles count in
+// Cost model: rounds of one workgroup per CU times the tile area (edge tiles count in
 // full), with a penalty for the smaller tiles' extra operand traffic per flop.
 static int direct_variant(int M, int N) {
   static const int bm[4] = {256, 256, 128, 128}, bn[4] = {256, 128, 256, 128};
   static const double penalty[4] = {1.0, 1.1, 1.1, 1.25};
   int best = -1;
   double best_cost = 0.0;
+  const int cus = num_cus();
   for (int v = 0; v < 4; ++v) {
     const int64_t tiles = (int64_t)((M + bm[v] - 1) / bm[v]) * ((N + bn[v] - 1) / bn[v]);
-    const double cost = (double)((tiles + 255) / 256) * bm[v] * bn[v] * penalty[v];
+    const double cost = (double)((tiles + cus - 1) / cus) * bm[v] * bn[v] * penalty[v];
     if (best < 0 || cost < best_cost) {
       best = v;
       best_cost = cost;
@@ -660,7 +661,7 @@ static int gemm16_dispatch(const GemmArgs& g, hipStream_t s) {
       if (v == 2) return launch_direct<DT, 2, 2>(g, s);
       if (v == 3) return launch_direct<DT, 2, 1>(g, s);
     }
-    const int cus = 256;
+    const int cus = num_cus();
     const bool big = g.M % 256 == 0 && g.N % 256 == 0 && (int64_t)(g.M / 256) * (g.N / 256) >= cus;
     if (big) {
       return tb ? launch_fast<DT, 256, 256, 2, 4, true>(g, s) : launch_fast<DT, 256, 256, 2, 4, false>(g, s);

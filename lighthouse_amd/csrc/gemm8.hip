@@ -602,7 +602,7 @@ int gemm8(const GemmArgs& g, hipStream_t s) {
     // flight) and the A chunk fits its LDS area.
     const int nblk = g.N / kSkinnyBN;
     int splits = 1;
-    while ((nblk * splits < 256 || g.K / splits > kSkinnyMaxChunk) && (g.K / kBK8) % (splits * 2) == 0) splits *= 2;
+    while ((nblk * splits < num_cus() || g.K / splits > kSkinnyMaxChunk) && (g.K / kBK8) % (splits * 2) == 0) splits *= 2;
     if (g.K / splits <= kSkinnyMaxChunk) {
       const size_t need = (size_t)splits * 16 * g.N * sizeof(float);
       if (need > g_partial_bytes) {

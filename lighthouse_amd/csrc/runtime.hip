@@ -24,6 +24,19 @@ int fail(int code, const char* fmt, ...) {
 
 hipStream_t default_stream() { return nullptr; }
 
+int num_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      cus = n;
+    else
+      cus = 256;
+  }
+  return cus;
+}
+
 }  // namespace lh
 
 using namespace lh;
