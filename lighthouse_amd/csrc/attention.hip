@@ -550,6 +550,76 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
   return attention16_launch_nq<DT, 2>(a, s);
 }
 
+// Any sequence length and head dimension up to 256: one wave per query row, keys in chunks of 64
+// (one per lane), the same online-softmax recurrence and rounding points as the fast kernels
+// (f32 statistics, P rounded to the element type before P V, output rounded once).  Throughput is
+// not a goal here; the MFMA kernels take every shape they can.
+constexpr int kGenericMaxD = 256;
+
+template <int DT>
+__global__ void __launch_bounds__(64) attention_generic_kernel(AttnArgs a, int d) {
+  __shared__ float qs[kGenericMaxD];
+  __shared__ float ps[64];
+  const int lane = threadIdx.x;
+  const int i = blockIdx.x, bh = blockIdx.y;
+  const int z = bh / a.H, hd = bh % a.H;
+  const int64_t qoff = (int64_t)z * a.sq.z + (int64_t)hd * a.sq.h + (int64_t)i * a.sq.t;
+  const int64_t koff = (int64_t)z * a.sk.z + (int64_t)hd * a.sk.h;
+  const int64_t voff = (int64_t)z * a.sv.z + (int64_t)hd * a.sv.h;
+  const int64_t ooff = (int64_t)z * a.so.z + (int64_t)hd * a.so.h + (int64_t)i * a.so.t;
+  for (int c = lane; c < d; c += 64) qs[c] = load_as_f32<DT>(a.q, qoff + c);
+  __syncthreads();
+  float acc[kGenericMaxD / 64];
+#pragma unroll
+  for (int r = 0; r < kGenericMaxD / 64; ++r) acc[r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+  const int kv_end = a.causal ? i + 1 : a.T;
+  for (int j0 = 0; j0 < kv_end; j0 += 64) {
+    const int j = j0 + lane;
+    float sc = -INFINITY;
+    if (j < kv_end) {
+      float dot = 0.0f;
+      for (int c = 0; c < d; ++c) dot += qs[c] * load_as_f32<DT>(a.k, koff + (int64_t)j * a.sk.t + c);
+      sc = dot * a.scale;
+    }
+    float mx = sc;
+    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+    const float m_new = fmaxf(m_run, mx);  // finite: key j0 is always valid
+    const float alpha = expf(m_run - m_new);
+    const float pexp = (j < kv_end) ? expf(sc - m_new) : 0.0f;
+    float lsum = pexp;
+    for (int off = 32; off > 0; off >>= 1) lsum += __shfl_xor(lsum, off, 64);
+    l_run = l_run * alpha + lsum;
+    m_run = m_new;
+    __syncthreads();  // previous chunk's ps fully consumed
+    ps[lane] = round_through<DT>(pexp);
+    __syncthreads();
+    const int nvalid = min(64, kv_end - j0);
+#pragma unroll
+    for (int r = 0; r < kGenericMaxD / 64; ++r) {
+      const int c = lane + 64 * r;
+      if (c < d) {
+        float s2 = 0.0f;
+        for (int jj = 0; jj < nvalid; ++jj) s2 += ps[jj] * load_as_f32<DT>(a.v, voff + (int64_t)(j0 + jj) * a.sv.t + c);
+        acc[r] = acc[r] * alpha + s2;
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < kGenericMaxD / 64; ++r) {
+    const int c = lane + 64 * r;
+    if (c < d) store_from_f32<DT>(a.out, ooff + c, acc[r] / l_run);
+  }
+}
+
+int attention_generic_launch(const AttnArgs& a, int d, int dtype, hipStream_t s) {
+  const dim3 grid(a.T, a.Z * a.H);
+  if (dtype == LH_BF16) hipLaunchKernelGGL(attention_generic_kernel<LH_BF16>, grid, dim3(64), 0, s, a, d);
+  else if (dtype == LH_F16) hipLaunchKernelGGL(attention_generic_kernel<LH_F16>, grid, dim3(64), 0, s, a, d);
+  else hipLaunchKernelGGL(attention_generic_kernel<LH_F32>, grid, dim3(64), 0, s, a, d);
+  return check_launch("attention_generic");
+}
+
 int attention_launch(const AttnArgs& a, int dtype, hipStream_t s) {
   if (dtype == LH_BF16) return attention16_launch<LH_BF16>(a, s);
   if (dtype == LH_F16) return attention16_launch<LH_F16>(a, s);
@@ -576,19 +646,19 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   LH_REQUIRE(dtype == LH_BF16 || dtype == LH_F16 || dtype == LH_F32, "lh_hip_attention: unsupported dtype %d", dtype);
   LH_REQUIRE(Z > 0 && H > 0 && T > 0, "lh_hip_attention: empty problem Z=%lld H=%lld T=%lld", (long long)Z,
              (long long)H, (long long)T);
-  if (d != kHeadDim) return fail(LH_ERR_UNSUPPORTED, "lh_hip_attention: head_dim %lld not supported (only 64)", (long long)d);
-  const int qblock = (dtype == LH_F32) ? kQBlock : kKvTile;
-  if (T % qblock != 0)
-    return fail(LH_ERR_UNSUPPORTED, "lh_hip_attention: seq_len %lld must be a multiple of %d", (long long)T, qblock);
+  if (d < 1 || d > kGenericMaxD)
+    return fail(LH_ERR_UNSUPPORTED, "lh_hip_attention: head_dim %lld not supported (1 .. %d)", (long long)d, kGenericMaxD);
   LH_REQUIRE(Z * H <= 65535 && T < (1 << 30), "lh_hip_attention: problem too large");
-  const int vec = (dtype == LH_F32) ? 4 : 8;  // elements per 16-byte access
   const lh_strides3* ss[4] = {&so, &sq, &sk, &sv};
   const void* ps[4] = {out, q, k, v};
-  for (int i = 0; i < 4; ++i) {
-    LH_REQUIRE(ss[i]->t >= d && ss[i]->t % vec == 0 && ss[i]->h % vec == 0 && ss[i]->z % vec == 0,
-               "lh_hip_attention: strides of tensor %d must be multiples of %d elements", i, vec);
-    LH_REQUIRE(aligned16(ps[i]), "lh_hip_attention: tensor %d is not 16-byte aligned", i);
-  }
+  for (int i = 0; i < 4; ++i) LH_REQUIRE(ss[i]->t >= d, "lh_hip_attention: row stride of tensor %d is below head_dim", i);
+  // The MFMA kernels need head_dim 64, whole query blocks and 16-byte aligned rows; every other
+  // problem runs on the generic kernel.
+  const int qblock = (dtype == LH_F32) ? kQBlock : kKvTile;
+  const int vec = (dtype == LH_F32) ? 4 : 8;  // elements per 16-byte access
+  bool fast = d == kHeadDim && T % qblock == 0;
+  for (int i = 0; i < 4 && fast; ++i)
+    fast = ss[i]->t % vec == 0 && ss[i]->h % vec == 0 && ss[i]->z % vec == 0 && aligned16(ps[i]);
   if (scale <= 0.0f) scale = 1.0f / sqrtf((float)d);
   AttnArgs a;
   a.out = out; a.q = q; a.k = k; a.v = v;
@@ -598,5 +668,6 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   a.scale_log2e = scale * 1.4426950408889634f;
   a.causal = causal ? 1 : 0;
   a.cus = num_cus();
+  if (!fast) return attention_generic_launch(a, (int)d, dtype, reinterpret_cast<hipStream_t>(stream));
   return attention_launch(a, dtype, reinterpret_cast<hipStream_t>(stream));
 }

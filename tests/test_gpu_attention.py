@@ -126,12 +126,31 @@ def test_attention_many_groups(dtype, shape, rtol, causal):
         assert_close(_host(out[z, h]), ref, rtol, f"attention {shape} z={z} h={h} causal={causal}")
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype,elt,rtol", [(torch.bfloat16, "bf16", 2e-2), (torch.float32, "f32", 1e-4)])
+@pytest.mark.parametrize("shape", [(1, 2, 100, 32), (2, 1, 77, 64), (1, 1, 130, 128), (1, 3, 64, 64), (1, 1, 1, 8),
+                                   (1, 1, 200, 256)])
+def test_attention_any_shape(shape, dtype, elt, rtol, causal):
+    """Sequence lengths and head dimensions the MFMA kernels do not take (and f32 with T % 128 != 0)
+    run on the generic kernel with the same rounding points."""
+    from lighthouse_amd import ops
+
+    rng = np.random.default_rng(sum(shape) + causal)
+    q, k, v = (orc.round_to(rng.standard_normal(shape).astype(np.float32), elt) for _ in range(3))
+    out = ops.attention(_dev(q, dtype), _dev(k, dtype), _dev(v, dtype), causal=causal)
+    ref = orc.attention(q, k, v, causal=causal, result_type=elt)
+    assert_close(_host(out), ref, rtol, f"generic attention {shape} {elt} causal={causal}")
+
+
 def test_attention_errors():
     from lighthouse_amd import ops
 
-    x = torch.zeros(1, 1, 128, 32, device="cuda", dtype=torch.bfloat16)
+    x = torch.zeros(1, 1, 128, 320, device="cuda", dtype=torch.bfloat16)
     with pytest.raises(ValueError):
-        ops.attention(x, x, x)
-    y = torch.zeros(1, 1, 100, 64, device="cuda", dtype=torch.bfloat16)
+        ops.attention(x, x, x)          # head_dim above 256
+    y = torch.zeros(1, 1, 64, 64, dtype=torch.bfloat16)
     with pytest.raises(ValueError):
-        ops.attention(y, y, y)
+        ops.attention(y, y, y)          # not on the GPU
+    z = torch.zeros(1, 1, 64, 64, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        ops.attention(z, z[:, :, :32], z)
