@@ -50,6 +50,7 @@ constexpr int kQBlock = 128;        // query rows per workgroup of the f32 kerne
 constexpr int kQBlock16 = 256;      // query rows per workgroup of the 16-bit kernel (4 waves x 64)
 constexpr int kAttnStages = 4;      // K/V ring depth
 constexpr int kAttnStageBytes = 2 * kKvTile * kHeadDim * 2;  // K tile + V tile, 16 KiB
+constexpr float kOffsetSlack = 1024.0f;  // largest partial row sum of P the softmax offset tolerates
 
 typedef __attribute__((address_space(3))) void attn_lds_void_t;
 typedef short attn_s16x4 __attribute__((ext_vector_type(4)));
@@ -136,41 +137,51 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
           if (key > qrow) s_acc[qt][i][v] = -INFINITY;
         }
     }
-    float mx = fmaxf(s_acc[qt][0][0], s_acc[qt][1][0]);
+    // Lazy offset: P = exp(S - offset) is first computed with the offset already in use.  Softmax
+    // does not depend on the offset and 16-bit P is as accurate at 2^10 as below 1, so the offset
+    // only has to move when P would grow without bound: the lane's partial row sum (needed anyway)
+    // is the test.  It bounds every P of the lane, cannot exceed 32 while no score has passed the
+    // offset, and is inf or NaN on the first tile (offset -inf).  Only then is the row maximum
+    // computed, the offset raised, l and acc rescaled and P recomputed, for the whole wave.
+    float mc = m_run[qt];
+    float p[2][16];
+    float l_tile = 0.0f;
 #pragma unroll
-    for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[qt][0][v]), s_acc[qt][1][v]);
-    mx = halfwave_max(mx);
-    // Deferred rescaling: m_run is the offset in use, not necessarily the running maximum.  It
-    // is raised (and l, acc rescaled by alpha) only when some row of the wave has grown past it
-    // by more than 2^8 after scaling; until then P = exp(S - m_run) stays below 256, exactly as
-    // accurate in 16 bit as values below 1, and softmax does not depend on the offset.
-    const bool grow = (mx - m_run[qt]) * a.scale_log2e > 8.0f;
-    if (__builtin_amdgcn_ballot_w64(grow) != 0) {
-      const float m_new = fmaxf(m_run[qt], mx);
-      const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-      const float alpha = exp2_fast((m_run[qt] - m_safe) * a.scale_log2e);
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        p[i][v] = exp2_fast(s_acc[qt][i][v] * a.scale_log2e - mc);
+        l_tile += p[i][v];
+      }
+    if (__builtin_amdgcn_ballot_w64(!(l_tile <= kOffsetSlack)) != 0) {
+      float mx = fmaxf(s_acc[qt][0][0], s_acc[qt][1][0]);
+#pragma unroll
+      for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[qt][0][v]), s_acc[qt][1][v]);
+      mx = halfwave_max(mx);
+      const float m_new = fmaxf(mc, mx * a.scale_log2e);
+      const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // row without a visible key so far
+      const float alpha = exp2_fast(mc - m_safe);
       l_run[qt] *= alpha;
       m_run[qt] = m_new;
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc_o[qt][j][v] *= alpha;
+      l_tile = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          p[i][v] = exp2_fast(s_acc[qt][i][v] * a.scale_log2e - m_safe);
+          l_tile += p[i][v];
+        }
     }
-    const float mc = ((m_run[qt] == -INFINITY) ? 0.0f : m_run[qt]) * a.scale_log2e;
-    float l_tile = 0.0f;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      float p[16];
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        p[v] = exp2_fast(s_acc[qt][i][v] * a.scale_log2e - mc);
-        l_tile += p[v];
-      }
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int d = 0; d < 4; ++d) pf[qt][i][u][d] = pack2<DT>(p[8 * u + 2 * d], p[8 * u + 2 * d + 1]);
-    }
+        for (int d = 0; d < 4; ++d) pf[qt][i][u][d] = pack2<DT>(p[i][8 * u + 2 * d], p[i][8 * u + 2 * d + 1]);
     l_run[qt] += l_tile;
   }
   // O^T += V^T P^T: head-dim sub-tile j (32 of d) x query sub-tile qt, over 4 k-steps of 16 keys.

@@ -127,6 +127,31 @@ def test_attention_many_groups(dtype, shape, rtol, causal):
 
 
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype,elt", [(torch.bfloat16, "bf16"), (torch.float16, "f16")])
+@pytest.mark.parametrize("shape", [(1, 2, 512, 64), (8, 20, 1024, 64)])
+def test_attention_scores_outgrow_the_offset(shape, dtype, elt, causal):
+    """The softmax offset is only raised when a partial row sum of P says so: scores that climb
+    from one key tile to the next (by little, by 2^10 and more, and by more than f32 exp can hold)
+    must still give the one-shot softmax.  Both row-per-wave variants (few / many groups)."""
+    from lighthouse_amd import ops
+
+    Z, H, T, d = shape
+    rng = np.random.default_rng(5 + T)
+    # score(q, key t) = 0.125 * 64 * 0.25 * ramp[t] + noise = 2 ramp[t] + noise (natural-log units)
+    steps = np.array([0, 1, 3, 3.5, 9, 9, 30, 31, 90, 90, 91, 160, 40, 0, 161, 161], dtype=np.float32)
+    ramp = np.repeat(steps[: T // 64], 64) if T // 64 <= 16 else np.repeat(steps, T // 16)
+    q = 0.5 + 0.05 * rng.standard_normal((Z, H, T, d)).astype(np.float32)
+    k = 0.5 * ramp[None, None, :, None] + 0.05 * rng.standard_normal((Z, H, T, d)).astype(np.float32)
+    v = rng.standard_normal((Z, H, T, d)).astype(np.float32)
+    q, k, v = (orc.round_to(t, elt) for t in (q, k, v))
+    out = ops.attention(_dev(q, dtype), _dev(k, dtype), _dev(v, dtype), causal=causal)
+    assert torch.isfinite(out.float()).all()
+    for z, h in [(0, 0), (Z - 1, H - 1)]:
+        ref = orc.attention(q[z, h], k[z, h], v[z, h], causal=causal)
+        assert_close(_host(out[z, h]), ref, 2e-2, f"attention ramp {shape} {elt} z={z} h={h} causal={causal}")
+
+
+@pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype,elt,rtol", [(torch.bfloat16, "bf16", 2e-2), (torch.float32, "f32", 1e-4)])
 @pytest.mark.parametrize("shape", [(1, 2, 100, 32), (2, 1, 77, 64), (1, 1, 130, 128), (1, 3, 64, 64), (1, 1, 1, 8),
                                    (1, 1, 200, 256)])
