@@ -83,6 +83,46 @@ def cpu_baseline_gemm_bf16(n: int, target_seconds: float = 12.0):
     }
 
 
+def compiled_block_step(torch, gen, B, T, C, H):
+    """The nanoGPT block as a torch module (fused QKV Linear, causal SDPA, tanh-GELU MLP; weights
+    N(0, 0.02), biases 0) compiled with this package's torch.compile backend: every operator of
+    the traced graph is lowered to the HIP kernels.  Returns a callable running one forward."""
+    import torch.nn as nn
+    import torch.nn.functional as F
+
+    from lighthouse_amd.ingress.torch import gpu_backend
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.ln_1, self.ln_2 = nn.LayerNorm(C), nn.LayerNorm(C)
+            self.c_attn, self.c_proj = nn.Linear(C, 3 * C), nn.Linear(C, C)
+            self.c_fc, self.mlp_proj = nn.Linear(C, 4 * C), nn.Linear(4 * C, C)
+
+        def forward(self, x):
+            q, k, v = self.c_attn(self.ln_1(x)).split(C, dim=2)
+            q, k, v = (t.view(B, T, H, C // H).transpose(1, 2) for t in (q, k, v))
+            y = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+            x = x + self.c_proj(y.transpose(1, 2).contiguous().view(B, T, C))
+            return x + self.mlp_proj(F.gelu(self.c_fc(self.ln_2(x)), approximate="tanh"))
+
+    model = Block().cuda()
+    with torch.no_grad():
+        for m in model.modules():
+            if isinstance(m, nn.Linear):
+                m.weight.copy_(torch.randn(m.weight.shape, device="cuda", generator=gen) * 0.02)
+                m.bias.zero_()
+    model = model.bfloat16()
+    x = torch.randn(B, T, C, device="cuda", generator=gen).bfloat16()
+    compiled = torch.compile(model, backend=gpu_backend(), dynamic=False)
+
+    def step():
+        with torch.no_grad():
+            compiled(x)
+
+    return step
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -140,7 +180,7 @@ def main() -> int:
 
     extras = {}
     if not args.no_extras:
-        def rate(fn, work, steps=50, warmup=20):
+        def rate(fn, work, steps=200, warmup=100):
             _, e = time_region(fn, steps, warmup)
             return work * steps / e
 
@@ -190,6 +230,8 @@ def main() -> int:
             ws = torch.empty(ops.nanogpt_block_workspace_bytes(B, T, C, dt), dtype=torch.uint8, device="cuda")
             bflops = 128849018880.0  # causal-halved attention
             extras[f"nanogpt_block_{name}_tflops"] = rate(lambda: ops.nanogpt_block(xb, p, H, out=yb, workspace=ws), bflops, 30, 10) / 1e12
+        extras["nanogpt_block_bf16_torch_compile_tflops"] = rate(
+            compiled_block_step(torch, g, 8, 1024, 768, 12), 128849018880.0, 30, 10) / 1e12
         # Vendor library kernels through torch on the same tensors, for orientation only.
         extras["torch_matmul_bf16_4096_tflops"] = rate(lambda: torch.matmul(a, b, out=out), flops) / 1e12
         extras["torch_sdpa_bf16_noncausal_tflops"] = rate(

@@ -219,10 +219,9 @@ struct DirectCfg {
   static constexpr int kBBytes = 32 * kBRow;              // one B stage (32 k)
   static constexpr int kBBase = 2 * kABytes;
   static constexpr int kRingBytes = kBBase + 4 * kBBytes;
-  static constexpr int kCStride = WTN * 2 + 8;            // staged output row: +8 bytes keeps the
-                                                          // 8-byte writes of 32 rows on distinct banks
-  static constexpr int kStageBytes = 8 * WTM * kCStride;
-  static constexpr int kLdsBytes = kRingBytes > kStageBytes ? kRingBytes : kStageBytes;
+  static constexpr int kStageBytes = 8 * 32 * WTN * 2;    // output staging: 32 rows of each wave's sub-tile
+  static constexpr int kStagedStores = 2 * TM * TN;       // 16-byte stores per lane of a staged epilogue
+  static constexpr int kLdsBytes = kRingBytes + kStageBytes;
   static constexpr int kBChunks = kBRow / 16;             // 16-byte chunks per B row
   static constexpr int kBRowsPerLoad = 1024 / kBRow;      // k rows one wave-wide load covers
   // Loads a lane has in flight per stage, hence the s_waitcnt immediates of the main loop.
@@ -359,39 +358,29 @@ __device__ __forceinline__ void direct_step_pair(const DirectCtx<TM, TN>& c, f32
   direct_interleave_hint<TM, TN>();
 }
 
-// One output tile; `id` is the tile's position in the XCD-grouped order.  EDGE: M and N need not
-// be multiples of the tile (N still a multiple of 8, K of 64): loads of rows / column chunks past
-// the end are redirected to the last valid row / chunk (their products land in accumulators that
-// are never stored) and the epilogue skips what lies outside the matrix.
-template <int DT, int TM, int TN, bool EDGE>
-__device__ __forceinline__ void direct_tile(const GemmArgs& g, int id, uint8_t* smem_d) {
+// Source pointers of tile `id` (its position in the XCD-grouped order) and the tile's origin.
+// EDGE: M and N need not be multiples of the tile (N still a multiple of 8, K of 64): loads of
+// rows / column chunks past the end are redirected to the last valid row / chunk (their products
+// land in accumulators that are never stored) and the epilogue skips what lies outside the matrix.
+template <int TM, int TN, bool EDGE>
+__device__ __forceinline__ void direct_place(const GemmArgs& g, int id, int lane, DirectCtx<TM, TN>& c, int& m0,
+                                             int& n0) {
   using Cfg = DirectCfg<TM, TN>;
-  constexpr int BM = Cfg::BM, BN = Cfg::BN, WN = 4, WTM = Cfg::WTM, WTN = Cfg::WTN;
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm0 = (wave / WN) * WTM, wn0 = (wave % WN) * WTN;
-
+  constexpr int BM = Cfg::BM, BN = Cfg::BN;
   const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
   constexpr int GROUP_M = 4;
   const int group_size = GROUP_M * tiles_n;
   const int first_m = (id / group_size) * GROUP_M;
   const int gm = min(tiles_m - first_m, GROUP_M);
-  const int m0 = (first_m + (id % group_size) % gm) * BM;
-  const int n0 = ((id % group_size) / gm) * BN;
-
+  m0 = (first_m + (id % group_size) % gm) * BM;
+  n0 = ((id % group_size) / gm) * BN;
   const uint16_t* A = reinterpret_cast<const uint16_t*>(g.a);
   const uint16_t* B = reinterpret_cast<const uint16_t*>(g.b);
-
-  DirectCtx<TM, TN> c;
-  c.ldb = g.ldb;
-  c.wave = wave;
-  const int r32 = lane & 31, h = lane >> 5;
-  c.h = h;
-  // Loader addressing.  A: load i of wave w fills rows (8 i + w) 8 .. +8 (1024 bytes); lane ->
-  // row += lane / 8, LDS chunk p = lane % 8 holds global chunk p ^ ((row / 2) % 8).
+  // A: load i of wave w fills rows (8 i + w) 8 .. +8 (1024 bytes); lane -> row += lane / 8, LDS
+  // chunk p = lane % 8 holds global chunk p ^ ((row / 2) % 8).
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
-    const int ar = (8 * i + wave) * 8 + (lane >> 3);
+    const int ar = (8 * i + c.wave) * 8 + (lane >> 3);
     const int ac = (lane & 7) ^ ((ar >> 1) & 7);
     const int arow = EDGE ? min(m0 + ar, g.M - 1) : m0 + ar;
     c.a_src[i] = A + (int64_t)arow * g.lda + ac * 8;
@@ -400,11 +389,189 @@ __device__ __forceinline__ void direct_tile(const GemmArgs& g, int id, uint8_t* 
   // row += lane / chunks-per-row, LDS chunk p holds global chunk p ^ 4 (k % 4).
 #pragma unroll
   for (int i = 0; i < TN; ++i) {
-    const int bk = (8 * i + wave) * Cfg::kBRowsPerLoad + lane / Cfg::kBChunks;
+    const int bk = (8 * i + c.wave) * Cfg::kBRowsPerLoad + lane / Cfg::kBChunks;
     const int bc = (lane % Cfg::kBChunks) ^ (4 * (bk & 3));
     const int bcol = EDGE ? min(n0 + bc * 8, g.N - 8) : n0 + bc * 8;
     c.b_src[i] = B + (int64_t)bk * g.ldb + bcol;
   }
+}
+
+// First loads of a tile: A stages 0, 1 and B stages 0 .. 3 (nk = K / 32 >= 2).
+template <int TM, int TN>
+__device__ __forceinline__ void direct_prologue(const DirectCtx<TM, TN>& c, int nk, uint8_t* __restrict__ ring) {
+  using Cfg = DirectCfg<TM, TN>;
+  direct_load_a(c, 0, ring);
+  if (nk > 2) direct_load_a(c, 1, ring + Cfg::kABytes);
+#pragma unroll
+  for (int st = 0; st < 4; ++st)
+    if (st < nk) direct_load_b(c, st, ring + Cfg::kBBase + st * Cfg::kBBytes);
+}
+
+// Main loop of one tile, whose first loads have been issued.
+// The lane's 16-bit bias values for a staged epilogue, columns n_base + 32 i + 8 q .. +4, as packed
+// pairs; all loads are issued back to back.  (An f32 bias is read by the epilogue itself.)
+template <int TN, bool EDGE>
+__device__ __forceinline__ void direct_load_bias(const GemmArgs& g, int n_base, u32x2 (&bias)[TN][4]) {
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) bias[i][q] = u32x2{0u, 0u};
+  if (!(g.flags & LH_GEMM_HAS_BIAS) || g.bias_dt == LH_F32) return;
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int n = n_base + 32 * i + 8 * q;
+      bias[i][q] = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.bias) + (EDGE ? min(n, g.N - 4) : n));
+    }
+}
+
+// `stores_behind`: the previous tile's staged epilogue issued exactly Cfg::kStagedStores stores
+// per lane AFTER this tile's first loads; vector memory operations complete in issue order, so
+// those stores may stay in flight.
+// `staged`: the epilogue will want `bias` (for columns from n_base); it is loaded ahead of the
+// last two steps, whose full wait covers it.
+template <int DT, int TM, int TN, bool EDGE>
+__device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectCtx<TM, TN>& c, f32x16 (&acc)[TN][TM],
+                                                uint8_t* smem_d, int nk, bool stores_behind, bool staged, int n_base,
+                                                u32x2 (&bias)[TN][4]) {
+  using Cfg = DirectCfg<TM, TN>;
+  uint8_t* const abuf = smem_d;
+  uint8_t* const bbuf = smem_d + Cfg::kBBase;
+  if (stores_behind) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(Cfg::kStagedStores) : "memory");
+  else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  DirectFrags<TM, TN> f0;
+  direct_read_frags(c, abuf, bbuf, 0, 0, f0);
+  int kt = 0;
+  for (; kt + 2 < nk; kt += 2) {
+    uint8_t* a_cur = abuf + ((kt >> 1) & 1) * Cfg::kABytes;
+    uint8_t* a_nxt = abuf + (((kt >> 1) + 1) & 1) * Cfg::kABytes;
+    uint8_t* b0 = bbuf + (kt & 3) * Cfg::kBBytes;
+    uint8_t* b1 = bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
+    uint8_t* b2 = bbuf + ((kt + 2) & 3) * Cfg::kBBytes;
+    direct_step_pair<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
+  }
+  {
+    // Last two steps: nothing left to load; stage nk - 1 of B must have landed.
+    const uint8_t* a_cur = abuf + ((kt >> 1) & 1) * Cfg::kABytes;
+    const uint8_t* b0 = bbuf + (kt & 3) * Cfg::kBBytes;
+    const uint8_t* b1 = bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
+    DirectFrags<TM, TN> f1;
+    if (staged) direct_load_bias<TN, EDGE>(g, n_base, bias);
+    direct_read_frags(c, a_cur, b0, 1, 1, f1);
+    direct_mfma<DT>(acc, f0);
+    direct_wait_barrier<0>();
+    direct_read_frags(c, a_cur, b1, 2, 0, f0);
+    direct_mfma<DT>(acc, f1);
+    direct_read_frags(c, a_cur, b1, 3, 1, f1);
+    direct_mfma<DT>(acc, f0);
+    direct_mfma<DT>(acc, f1);
+  }
+}
+
+// End of a tile: once every wave has left the rings, the first loads of the workgroup's NEXT tile
+// are issued into them (their latency and the cold start of the pipeline hide behind this tile's
+// stores), then the accumulators are written out.  16-bit outputs are staged through `stage`, an
+// LDS area of its own (32 rows of the wave's sub-tile at a time, 16-byte chunk ^ ((row / 2) % chunks)
+// against bank conflicts), and leave as full row segments of 16 bytes per lane.  `ring` and
+// `stage` are separate restrict parameters so that the staging traffic does not wait for the
+// asynchronous ring writes.
+template <int DT, int TM, int TN, bool EDGE, bool HAS_NEXT>
+__device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx<TM, TN>& next, int nk,
+                                              uint8_t* __restrict__ ring, uint8_t* __restrict__ stage,
+                                              const f32x16 (&acc)[TN][TM], const u32x2 (&bias)[TN][4], int m0, int n0,
+                                              int wm0, int wn0, int lane) {
+  using Cfg = DirectCfg<TM, TN>;
+  constexpr int WTN = Cfg::WTN;
+  // The lane-dependent addresses below do not change from tile to tile; computed from an opaque
+  // copy of the lane index they are recomputed here instead of being kept in registers (and
+  // spilled) across the main loop.
+  asm volatile("" : "+v"(lane));
+  const int r32 = lane & 31, h = lane >> 5;
+  const int m_base = m0 + wm0 + r32;
+  const int n_base = n0 + wn0 + 4 * h;
+  if (g.out_dt != LH_F32 && !(g.flags & LH_GEMM_ACCUMULATE_C)) {
+    // The bias values (loaded by the main loop, whose last wait covered them) are pinned down here:
+    // a wait for them placed after the ring loads below would wait for those loads as well.
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) asm volatile("" ::"v"(bias[i][q][e]));
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the rings
+    if constexpr (HAS_NEXT) direct_prologue(next, nk, ring);
+    constexpr int RB = WTN * 2;                // bytes of a staged row
+    constexpr int chunks = RB / 16;            // 16-byte chunks per staged row
+    constexpr int rows_per_pass = 64 / chunks;
+    // With a next tile loading into the rings, 32 rows at a time go through the wave's slice of
+    // `stage`; the last tile of a workgroup stages its whole sub-tile in the idle rings at once.
+    constexpr int JB = HAS_NEXT ? 1 : TM;
+    uint8_t* cw = HAS_NEXT ? stage + next.wave * (32 * RB) : ring + next.wave * (TM * 32 * RB);
+    uint16_t* outp = reinterpret_cast<uint16_t*>(g.out);
+#pragma unroll
+    for (int j0 = 0; j0 < TM; j0 += JB) {
+#pragma unroll
+      for (int jj = 0; jj < JB; ++jj)
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int j = j0 + jj;
+            const int n = n_base + 32 * i + 8 * q;
+            const f32x4 b4 = (g.bias_dt == LH_F32)
+                                 ? bias4<DT>(g, EDGE ? min(n, g.N - 4) : n)  // the bias row ends at N
+                                 : f32x4{unpack_lo<DT>(bias[i][q][0]), unpack_hi<DT>(bias[i][q][0]),
+                                         unpack_lo<DT>(bias[i][q][1]), unpack_hi<DT>(bias[i][q][1])};
+            const u32x2 w = epilogue4_pack_bias<DT>(g, b4, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                                                    acc[i][j][4 * q + 3]);
+            *reinterpret_cast<u32x2*>(cw + (32 * jj + r32) * RB + (((4 * i + q) ^ ((r32 >> 1) & (chunks - 1))) << 4) +
+                                      8 * h) = w;
+          }
+      // Cfg::kStagedStores stores per lane in all; the main loop's first wait counts on it.
+#pragma unroll
+      for (int t = 0; t < JB * 32 / rows_per_pass; ++t) {
+        const int row = rows_per_pass * t + lane / chunks, ch = lane % chunks;
+        u32x4 w = *reinterpret_cast<const u32x4*>(cw + row * RB + ((ch ^ ((row >> 1) & (chunks - 1))) << 4));
+        const int m = m0 + wm0 + 32 * j0 + row;
+        if (!EDGE || (m < g.M && n0 + wn0 + ch * 8 < g.N))
+          *reinterpret_cast<u32x4*>(outp + (int64_t)m * g.ldc + n0 + wn0 + ch * 8) = w;
+      }
+    }
+    return;
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  if constexpr (HAS_NEXT) direct_prologue(next, nk, ring);
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (!EDGE || (m_base + 32 * j < g.M && n_base + 32 * i + 8 * q < g.N))
+          epilogue4<DT>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                        acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+}
+
+// Persistent workgroups: one (two for the 128 x 128 tile, whose LDS is 80 KiB) per CU, each
+// walking the tile list with the grid as stride.  Tile ids congruent modulo 8 stay on one XCD,
+// which is what xcd_remap assumes.  Launching one workgroup per tile instead costs a
+// workgroup launch plus a cold prologue per tile, about a third of a K = 768 tile's time.
+template <int DT, int TM, int TN, bool EDGE>
+__global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
+  using Cfg = DirectCfg<TM, TN>;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_d[];
+  const int ntiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int WN = 4;
+  const int wm0 = (wave / WN) * Cfg::WTM, wn0 = (wave % WN) * Cfg::WTN;
+  const int r32 = lane & 31, h = lane >> 5;
+
+  DirectCtx<TM, TN> c;
+  c.ldb = g.ldb;
+  c.wave = wave;
+  c.h = h;
   // A fragment (second MFMA operand): row wm0 + 32 j + r32, logical chunk 2 kc + h.
 #pragma unroll
   for (int j = 0; j < TM; ++j) {
@@ -424,106 +591,42 @@ __device__ __forceinline__ void direct_tile(const GemmArgs& g, int id, uint8_t* 
     c.b_off = krow * Cfg::kBRow + 8 * ((col >> 2) & 1);
   }
 
-  f32x16 acc[TN][TM];
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
   const int nk = g.K / 32;  // even: K is a multiple of 64
-  uint8_t* const abuf = smem_d;
-  uint8_t* const bbuf = smem_d + Cfg::kBBase;
-  // Prologue: A stages 0, 1 and B stages 0 .. 3.
-  direct_load_a(c, 0, abuf);
-  if (nk > 2) direct_load_a(c, 1, abuf + Cfg::kABytes);
-#pragma unroll
-  for (int st = 0; st < 4; ++st)
-    if (st < nk) direct_load_b(c, st, bbuf + st * Cfg::kBBytes);
-  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-  DirectFrags<TM, TN> f0;
-  direct_read_frags(c, abuf, bbuf, 0, 0, f0);
-  int kt = 0;
-  for (; kt + 2 < nk; kt += 2) {
-    uint8_t* a_cur = abuf + ((kt >> 1) & 1) * Cfg::kABytes;
-    uint8_t* a_nxt = abuf + (((kt >> 1) + 1) & 1) * Cfg::kABytes;
-    uint8_t* b0 = bbuf + (kt & 3) * Cfg::kBBytes;
-    uint8_t* b1 = bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
-    uint8_t* b2 = bbuf + ((kt + 2) & 3) * Cfg::kBBytes;
-    direct_step_pair<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
-  }
-  {
-    // Last two steps: nothing left to load; stage nk - 1 of B must have landed.
-    const uint8_t* a_cur = abuf + ((kt >> 1) & 1) * Cfg::kABytes;
-    const uint8_t* b0 = bbuf + (kt & 3) * Cfg::kBBytes;
-    const uint8_t* b1 = bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
-    DirectFrags<TM, TN> f1;
-    direct_read_frags(c, a_cur, b0, 1, 1, f1);
-    direct_mfma<DT>(acc, f0);
-    direct_wait_barrier<0>();
-    direct_read_frags(c, a_cur, b1, 2, 0, f0);
-    direct_mfma<DT>(acc, f1);
-    direct_read_frags(c, a_cur, b1, 3, 1, f1);
-    direct_mfma<DT>(acc, f0);
-    direct_mfma<DT>(acc, f1);
-  }
-
-  const int m_base = m0 + wm0 + r32;
-  const int n_base = n0 + wn0 + 4 * h;
-  if (g.out_dt != LH_F32 && !(g.flags & LH_GEMM_ACCUMULATE_C)) {
-    // 16-bit output: stage the wave's sub-tile in LDS and store full row segments of the
-    // sub-tile (128 or 64 bytes) with 16 bytes per lane.
-    constexpr int cstride = Cfg::kCStride;
-    constexpr int chunks = WTN * 2 / 16;       // 16-byte chunks per staged row
-    constexpr int rows_per_pass = 64 / chunks;
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the rings
-    uint8_t* cw = smem_d + wave * (WTM * cstride);
+  int t = blockIdx.x;       // < ntiles: the grid is never larger than the tile list
+  int m0, n0;
+  direct_place<TM, TN, EDGE>(g, xcd_remap(t, ntiles), lane, c, m0, n0);
+  direct_prologue(c, nk, smem_d);
+  // Without EDGE every lane issues all stores of a staged epilogue.
+  const bool staged = g.out_dt != LH_F32 && !(g.flags & LH_GEMM_ACCUMULATE_C);
+  const bool counted_stores = !EDGE && staged;
+  bool first = true;
+  for (;;) {
+    f32x16 acc[TN][TM];
 #pragma unroll
     for (int i = 0; i < TN; ++i)
 #pragma unroll
       for (int j = 0; j < TM; ++j)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          u32x2 w = {0u, 0u};
-          if (!EDGE || n_base + 32 * i + 8 * q < g.N)  // the bias row ends at N
-            w = epilogue4_pack<DT>(g, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
-                                   acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-          *reinterpret_cast<u32x2*>(cw + (32 * j + r32) * cstride + (32 * i + 8 * q + 4 * h) * 2) = w;
-        }
-    uint16_t* outp = reinterpret_cast<uint16_t*>(g.out);
-#pragma unroll
-    for (int t = 0; t < WTM / rows_per_pass; ++t) {
-      const int row = rows_per_pass * t + lane / chunks, ch = lane % chunks;
-      u32x4 w = *reinterpret_cast<const u32x4*>(cw + row * cstride + ch * 16);
-      if (!EDGE || (m0 + wm0 + row < g.M && n0 + wn0 + ch * 8 < g.N))
-        *reinterpret_cast<u32x4*>(outp + (int64_t)(m0 + wm0 + row) * g.ldc + n0 + wn0 + ch * 8) = w;
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+    u32x2 bias[TN][4];
+    direct_mainloop<DT, TM, TN, EDGE>(g, c, acc, smem_d, nk, counted_stores && !first, staged, n0 + wn0 + 4 * h, bias);
+    first = false;
+    const int tn = t + (int)gridDim.x;
+    const bool more = tn < ntiles;
+    DirectCtx<TM, TN> cn = c;
+    int m1 = 0, n1 = 0;
+    uint8_t* const stage = smem_d + Cfg::kRingBytes;
+    if (more) {
+      direct_place<TM, TN, EDGE>(g, xcd_remap(tn, ntiles), lane, cn, m1, n1);
+      direct_finish<DT, TM, TN, EDGE, true>(g, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0, lane);
+    } else {
+      direct_finish<DT, TM, TN, EDGE, false>(g, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0, lane);
     }
-    return;
-  }
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        if (!EDGE || (m_base + 32 * j < g.M && n_base + 32 * i + 8 * q < g.N))
-          epilogue4<DT>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
-                        acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-}
-
-// Persistent workgroups: one (two for the 128 x 128 tile, whose rings are 64 KiB) per CU, each
-// walking the tile list with the grid as stride.  Tile ids congruent modulo 8 stay on one XCD,
-// which is what xcd_remap assumes.  Launching one workgroup per tile instead costs a
-// workgroup launch plus a cold prologue per tile, about a third of a K = 768 tile's time.
-template <int DT, int TM, int TN, bool EDGE>
-__global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
-  using Cfg = DirectCfg<TM, TN>;
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_d[];
-  const int ntiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
-  for (int t = blockIdx.x; t < ntiles; t += gridDim.x) {
-    if (t != (int)blockIdx.x) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS is reused
-    direct_tile<DT, TM, TN, EDGE>(g, xcd_remap(t, ntiles), smem_d);
+    if (!more) break;
+    c = cn;
+    m0 = m1;
+    n0 = n1;
+    t = tn;
   }
 }
 

@@ -68,20 +68,31 @@ __device__ __forceinline__ void epilogue4(const GemmArgs& g, int m, int n, float
   }
 }
 
-// Bias / activation / conversion for 4 consecutive columns of a 16-bit output, returned as two
-// packed dwords (no accumulator input); same order of operations as epilogue4.
+// Bias of 4 consecutive columns as f32 (zeros without a bias).
 template <int DT>
-__device__ __forceinline__ u32x2 epilogue4_pack(const GemmArgs& g, int n, float v0, float v1, float v2, float v3) {
-  float v[4] = {v0 * g.alpha, v1 * g.alpha, v2 * g.alpha, v3 * g.alpha};
+__device__ __forceinline__ f32x4 bias4(const GemmArgs& g, int n) {
+  f32x4 r = {0.0f, 0.0f, 0.0f, 0.0f};
   if (g.flags & LH_GEMM_HAS_BIAS) {
     if (g.bias_dt == LH_F32) {
-      f32x4 bb = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.bias) + n);
-      v[0] += bb[0]; v[1] += bb[1]; v[2] += bb[2]; v[3] += bb[3];
+      r = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.bias) + n);
     } else {
       u32x2 bb = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.bias) + n);
-      v[0] += unpack_lo<DT>(bb[0]); v[1] += unpack_hi<DT>(bb[0]);
-      v[2] += unpack_lo<DT>(bb[1]); v[3] += unpack_hi<DT>(bb[1]);
+      r = f32x4{unpack_lo<DT>(bb[0]), unpack_hi<DT>(bb[0]), unpack_lo<DT>(bb[1]), unpack_hi<DT>(bb[1])};
     }
+  }
+  return r;
+}
+
+// Bias / activation / conversion for 4 consecutive columns of a 16-bit output, returned as two
+// packed dwords (no accumulator input); same order of operations as epilogue4.  `bias` comes from
+// bias4 (loaded ahead of time by kernels that have other loads in flight).
+template <int DT>
+__device__ __forceinline__ u32x2 epilogue4_pack_bias(const GemmArgs& g, f32x4 bias, float v0, float v1, float v2,
+                                                     float v3) {
+  float v[4] = {v0 * g.alpha, v1 * g.alpha, v2 * g.alpha, v3 * g.alpha};
+  if (g.flags & LH_GEMM_HAS_BIAS) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] += bias[e];
   }
   if (g.flags & LH_GEMM_HAS_GELU) {
 #pragma unroll
@@ -92,6 +103,10 @@ __device__ __forceinline__ u32x2 epilogue4_pack(const GemmArgs& g, int n, float 
     for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
   }
   return u32x2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+}
+template <int DT>
+__device__ __forceinline__ u32x2 epilogue4_pack(const GemmArgs& g, int n, float v0, float v1, float v2, float v3) {
+  return epilogue4_pack_bias<DT>(g, bias4<DT>(g, n), v0, v1, v2, v3);
 }
 
 // One output element, any alignment (edge tiles and the generic kernels).
