@@ -164,7 +164,7 @@ constexpr int kD8ABytes = 256 * 128;   // one A stage (128 k): 32 KiB
 constexpr int kD8BBytes = 64 * 256;    // one B stage (64 k): 16 KiB
 constexpr int kD8BBase = 2 * kD8ABytes;
 constexpr int kD8RingBytes = kD8BBase + 4 * kD8BBytes;  // 128 KiB
-constexpr int kD8LdsBytes = 8 * 128 * 136;              // bf16 output staging (139264) >= rings
+constexpr int kD8LdsBytes = kD8RingBytes + 8 * 32 * 128;  // + bf16 output staging, 32 rows per wave at a time
 
 typedef __attribute__((address_space(3))) void lds8_void_t;
 typedef int i32x2 __attribute__((ext_vector_type(2)));
@@ -174,9 +174,14 @@ __device__ __forceinline__ void async8_copy16(const void* gsrc, uint8_t* lds_wav
 }
 
 struct D8Ctx {
-  const uint8_t* a_src[4];
-  const uint8_t* b_src[2];
-  int a_off[4], a_swz[4];
+  // Sources of the lane's loads at k = 0: a wave-uniform base (the tile's first A row / B column)
+  // plus a 32-bit byte offset per load (at most 255 lda, 63 ldb + 255).
+  const uint8_t* a_base;
+  const uint8_t* b_base;
+  uint32_t a_voff[4];
+  uint32_t b_voff[2];
+  int a_off, a_swz;  // byte offset and swizzle of the lane's A row of m-subtile 0; subtile j is 32 rows
+                     // (4096 bytes) further on with the same swizzle
   int64_t ldb;
   int wave, h, b_off, b_chunk, b_swz;
 };
@@ -188,11 +193,11 @@ struct D8Frags {
 
 __device__ __forceinline__ void d8_load_a(const D8Ctx& c, int sa, uint8_t* __restrict__ abuf) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) async8_copy16(c.a_src[i] + sa * 128, abuf + (8 * i + c.wave) * 1024);
+  for (int i = 0; i < 4; ++i) async8_copy16(c.a_base + (c.a_voff[i] + (uint32_t)(sa * 128)), abuf + (8 * i + c.wave) * 1024);
 }
 __device__ __forceinline__ void d8_load_b(const D8Ctx& c, int sb, uint8_t* __restrict__ bbuf) {
 #pragma unroll
-  for (int i = 0; i < 2; ++i) async8_copy16(c.b_src[i] + (int64_t)(sb * 64) * c.ldb, bbuf + (8 * i + c.wave) * 1024);
+  for (int i = 0; i < 2; ++i) async8_copy16(c.b_base + (int64_t)(sb * 64) * c.ldb + c.b_voff[i], bbuf + (8 * i + c.wave) * 1024);
 }
 
 // Fragments of one 64-k step: A bytes 64 kb .. +64 of the stage's rows (kb = 0 / 1), B stage bs.
@@ -201,8 +206,8 @@ __device__ __forceinline__ void d8_read_frags(const D8Ctx& c, const uint8_t* __r
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int c0 = 4 * kb + 2 * c.h;
-    i32x4 lo = *reinterpret_cast<const i32x4*>(as + c.a_off[j] + ((c0 ^ c.a_swz[j]) << 4));
-    i32x4 hi = *reinterpret_cast<const i32x4*>(as + c.a_off[j] + (((c0 + 1) ^ c.a_swz[j]) << 4));
+    i32x4 lo = *reinterpret_cast<const i32x4*>(as + c.a_off + ((c0 ^ c.a_swz) << 4) + 4096 * j);
+    i32x4 hi = *reinterpret_cast<const i32x4*>(as + c.a_off + (((c0 + 1) ^ c.a_swz) << 4) + 4096 * j);
     f.a[j] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   }
 #pragma unroll
@@ -268,73 +273,46 @@ __device__ __forceinline__ void d8_step_pair(const D8Ctx& c, f32x16 (&acc)[2][4]
   d8_interleave_hint();
 }
 
-__global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
-  constexpr int BM = 256, BN = 256, TM = 4, TN = 2, WN = 4, WTN = 64;
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_8[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm0 = (wave / WN) * 128, wn0 = (wave % WN) * WTN;
+// Source pointers of tile `id` (its position in the XCD-grouped order) and the tile's origin.
+__device__ __forceinline__ void d8_place(const GemmArgs& g, int id, int lane, D8Ctx& c, int& m0, int& n0) {
+  constexpr int BM = 256, BN = 256;
+  asm volatile("" : "+v"(lane));  // recompute the lane's offsets per tile rather than keep them in registers
   const int tiles_m = g.M / BM, tiles_n = g.N / BN;
-  int id = xcd_remap(blockIdx.x, gridDim.x);
   constexpr int GROUP_M = 4;
   const int group_size = GROUP_M * tiles_n;
   const int first_m = (id / group_size) * GROUP_M;
   const int gm = min(tiles_m - first_m, GROUP_M);
-  const int m0 = (first_m + (id % group_size) % gm) * BM;
-  const int n0 = ((id % group_size) / gm) * BN;
-  const uint8_t* A = reinterpret_cast<const uint8_t*>(g.a);
-  const uint8_t* B = reinterpret_cast<const uint8_t*>(g.b);
-
-  D8Ctx c;
-  c.ldb = g.ldb;
-  c.wave = wave;
-  const int r32 = lane & 31, h = lane >> 5;
-  c.h = h;
+  m0 = (first_m + (id % group_size) % gm) * BM;
+  n0 = ((id % group_size) / gm) * BN;
+  c.a_base = reinterpret_cast<const uint8_t*>(g.a) + (int64_t)m0 * g.lda;
+  c.b_base = reinterpret_cast<const uint8_t*>(g.b) + n0;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int ar = (8 * i + wave) * 8 + (lane >> 3);
+    const int ar = (8 * i + c.wave) * 8 + (lane >> 3);
     const int ac = (lane & 7) ^ ((ar >> 1) & 7);
-    c.a_src[i] = A + (int64_t)(m0 + ar) * g.lda + ac * 16;
+    c.a_voff[i] = (uint32_t)ar * (uint32_t)g.lda + ac * 16;
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    const int bk = (8 * i + wave) * 4 + (lane >> 4);
+    const int bk = (8 * i + c.wave) * 4 + (lane >> 4);
     const int bc = (lane & 15) ^ (2 * (bk & 7));
-    c.b_src[i] = B + (int64_t)bk * g.ldb + n0 + bc * 16;
+    c.b_voff[i] = (uint32_t)bk * (uint32_t)g.ldb + bc * 16;
   }
-#pragma unroll
-  for (int j = 0; j < TM; ++j) {
-    const int r = wm0 + 32 * j + r32;
-    c.a_off[j] = r * 128;
-    c.a_swz[j] = (r >> 1) & 7;
-  }
-  {
-    // Lane (grp = lane / 16, j = lane % 16) addresses k row 32 h + 8 q + j / 2 (q = 0..3), columns
-    // wn0 + 32 i + 16 (grp % 2) + 8 (j % 2) .. +8.
-    const int j16 = lane & 15, grp = lane >> 4;
-    const int krow = 32 * h + (j16 >> 1);
-    const int col = wn0 + 16 * (grp & 1) + 8 * (j16 & 1);
-    c.b_chunk = col >> 4;
-    c.b_swz = 2 * (krow & 7);
-    c.b_off = krow * 256 + (col & 8);
-  }
+}
 
-  f32x16 acc[TN][TM];
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-  const int nk = g.K / 64;  // even: K is a multiple of 128
-  uint8_t* const abuf = smem_8;
-  uint8_t* const bbuf = smem_8 + kD8BBase;
-  d8_load_a(c, 0, abuf);
-  if (nk > 2) d8_load_a(c, 1, abuf + kD8ABytes);
+// First loads of a tile: A stages 0, 1 and B stages 0 .. 3 (nk = K / 64 >= 2).
+__device__ __forceinline__ void d8_prologue(const D8Ctx& c, int nk, uint8_t* __restrict__ ring) {
+  d8_load_a(c, 0, ring);
+  if (nk > 2) d8_load_a(c, 1, ring + kD8ABytes);
 #pragma unroll
   for (int st = 0; st < 4; ++st)
-    if (st < nk) d8_load_b(c, st, bbuf + st * kD8BBytes);
+    if (st < nk) d8_load_b(c, st, ring + kD8BBase + st * kD8BBytes);
+}
+
+// Main loop of one tile, whose first loads have been issued.
+__device__ __forceinline__ void d8_mainloop(const D8Ctx& c, f32x16 (&acc)[2][4], uint8_t* smem_8, int nk) {
+  uint8_t* const abuf = smem_8;
+  uint8_t* const bbuf = smem_8 + kD8BBase;
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
   D8Frags f;
   d8_read_frags(c, abuf, bbuf, 0, f);
@@ -356,29 +334,49 @@ __global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
     d8_mfma(acc, f);
     d8_mfma(acc, gfr);
   }
+}
 
+// End of a tile: once every wave has left the rings, the first loads of the workgroup's next tile
+// are issued into them, then the accumulators are written out.  bf16 outputs are staged through
+// `stage`, an LDS area of its own (32 rows of the wave's 128 x 64 sub-tile at a time, 16-byte
+// chunk ^ ((row / 2) % 8) against bank conflicts); the last tile of a workgroup stages its whole
+// sub-tile in the idle rings at once.  `ring` and `stage` are separate restrict parameters so
+// that the staging traffic does not wait for the asynchronous ring writes.
+template <bool HAS_NEXT>
+__device__ __forceinline__ void d8_finish(const GemmArgs& g, const D8Ctx& next, int nk, uint8_t* __restrict__ ring,
+                                          uint8_t* __restrict__ stage, const f32x16 (&acc)[2][4], int m0, int n0, int wm0,
+                                          int wn0, int lane) {
+  constexpr int TM = 4, TN = 2, RB = 128, chunks = 8, rows_per_pass = 8;
+  asm volatile("" : "+v"(lane));  // keeps the addresses below out of registers during the main loop
+  const int r32 = lane & 31, h = lane >> 5;
   const int m_base = m0 + wm0 + r32;
   const int n_base = n0 + wn0 + 4 * h;
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the rings
+  if constexpr (HAS_NEXT) d8_prologue(next, nk, ring);
   if (g.out_dt != LH_F32) {
-    constexpr int cstride = WTN * 2 + 8;
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    uint8_t* cw = smem_8 + wave * (128 * cstride);
-#pragma unroll
-    for (int i = 0; i < TN; ++i)
-#pragma unroll
-      for (int j = 0; j < TM; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          u32x2 w = epilogue4_pack<LH_BF16>(g, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
-                                            acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-          *reinterpret_cast<u32x2*>(cw + (32 * j + r32) * cstride + (32 * i + 8 * q + 4 * h) * 2) = w;
-        }
+    constexpr int JB = HAS_NEXT ? 1 : TM;
+    uint8_t* cw = HAS_NEXT ? stage + next.wave * (32 * RB) : ring + next.wave * (TM * 32 * RB);
     uint16_t* outp = reinterpret_cast<uint16_t*>(g.out);
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-      const int row = 8 * t + (lane >> 3), ch = lane & 7;
-      u32x4 w = *reinterpret_cast<const u32x4*>(cw + row * cstride + ch * 16);
-      *reinterpret_cast<u32x4*>(outp + (int64_t)(m0 + wm0 + row) * g.ldc + n0 + wn0 + ch * 8) = w;
+    for (int j0 = 0; j0 < TM; j0 += JB) {
+#pragma unroll
+      for (int jj = 0; jj < JB; ++jj)
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int j = j0 + jj;
+            const u32x2 w = epilogue4_pack<LH_BF16>(g, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                                                    acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+            *reinterpret_cast<u32x2*>(cw + (32 * jj + r32) * RB + (((4 * i + q) ^ ((r32 >> 1) & (chunks - 1))) << 4) +
+                                      8 * h) = w;
+          }
+#pragma unroll
+      for (int t = 0; t < JB * 32 / rows_per_pass; ++t) {
+        const int row = rows_per_pass * t + lane / chunks, ch = lane % chunks;
+        u32x4 w = *reinterpret_cast<const u32x4*>(cw + row * RB + ((ch ^ ((row >> 1) & (chunks - 1))) << 4));
+        *reinterpret_cast<u32x4*>(outp + (int64_t)(m0 + wm0 + 32 * j0 + row) * g.ldc + n0 + wn0 + ch * 8) = w;
+      }
     }
     return;
   }
@@ -392,15 +390,76 @@ __global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
                            acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
 }
 
+// Persistent workgroups, one per CU, each walking the tile list with the grid as stride (tile
+// ids congruent modulo 8 stay on one XCD, which is what xcd_remap assumes).
+__global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
+  constexpr int TM = 4, TN = 2, WN = 4, WTN = 64;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_8[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave / WN) * 128, wn0 = (wave % WN) * WTN;
+  const int ntiles = (g.M / 256) * (g.N / 256);
+
+  D8Ctx c;
+  c.ldb = g.ldb;
+  c.wave = wave;
+  const int r32 = lane & 31, h = lane >> 5;
+  c.h = h;
+  c.a_off = (wm0 + r32) * 128;
+  c.a_swz = (r32 >> 1) & 7;  // wm0 and 32 j are multiples of 16
+  {
+    // Lane (grp = lane / 16, j = lane % 16) addresses k row 32 h + 8 q + j / 2 (q = 0..3), columns
+    // wn0 + 32 i + 16 (grp % 2) + 8 (j % 2) .. +8.
+    const int j16 = lane & 15, grp = lane >> 4;
+    const int krow = 32 * h + (j16 >> 1);
+    const int col = wn0 + 16 * (grp & 1) + 8 * (j16 & 1);
+    c.b_chunk = col >> 4;
+    c.b_swz = 2 * (krow & 7);
+    c.b_off = krow * 256 + (col & 8);
+  }
+
+  const int nk = g.K / 64;  // even: K is a multiple of 128
+  int t = blockIdx.x;       // < ntiles: the grid is never larger than the tile list
+  int m0, n0;
+  d8_place(g, xcd_remap(t, ntiles), lane, c, m0, n0);
+  d8_prologue(c, nk, smem_8);
+  for (;;) {
+    f32x16 acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+    d8_mainloop(c, acc, smem_8, nk);
+    const int tn = t + (int)gridDim.x;
+    const bool more = tn < ntiles;
+    D8Ctx cn = c;
+    int m1 = 0, n1 = 0;
+    uint8_t* const stage = smem_8 + kD8RingBytes;
+    if (more) {
+      d8_place(g, xcd_remap(tn, ntiles), lane, cn, m1, n1);
+      d8_finish<true>(g, cn, nk, smem_8, stage, acc, m0, n0, wm0, wn0, lane);
+    } else {
+      d8_finish<false>(g, cn, nk, smem_8, stage, acc, m0, n0, wm0, wn0, lane);
+    }
+    if (!more) break;
+    c = cn;
+    m0 = m1;
+    n0 = n1;
+    t = tn;
+  }
+}
+
 static int launch_direct8(const GemmArgs& g, hipStream_t s) {
-  static_assert(kD8LdsBytes >= kD8RingBytes, "rings must fit");
   static bool configured = false;
   if (!configured) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_direct),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kD8LdsBytes));
     configured = true;
   }
-  hipLaunchKernelGGL(gemm8_direct, dim3((g.M / 256) * (g.N / 256)), dim3(512), kD8LdsBytes, s, g);
+  const int ntiles = (g.M / 256) * (g.N / 256), cus = num_cus();
+  hipLaunchKernelGGL(gemm8_direct, dim3(ntiles < cus ? ntiles : cus), dim3(512), kD8LdsBytes, s, g);
   return check_launch("gemm8_direct");
 }
 
@@ -628,7 +687,8 @@ int gemm8(const GemmArgs& g, hipStream_t s) {
     }
   }
   if (vec_ok && g.M % 256 == 0 && g.N % 256 == 0 && (int64_t)(g.M / 256) * (g.N / 256) >= 128) {
-    if (g.ldb % 16 == 0 && g.ldc % 8 == 0) return launch_direct8(g, s);
+    // the direct kernel addresses a tile's rows with 32-bit byte offsets from the tile's origin
+    if (g.ldb % 16 == 0 && g.ldc % 8 == 0 && g.lda < (1 << 24) && g.ldb < (1 << 24)) return launch_direct8(g, s);
     return launch_fast8<256, 256, 2, 4>(g, s);
   }
   if (vec_ok && g.M % 128 == 0 && g.N % 128 == 0) return launch_fast8<128, 128, 2, 2>(g, s);
