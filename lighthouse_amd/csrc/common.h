@@ -128,11 +128,12 @@ __device__ __forceinline__ float relu_nan(float v) { return (v != v) ? v : fmaxf
 
 // tanh-GELU, 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))), via one exp:
 // 0.5 (1 + tanh(u)) = 1 / (1 + exp(-2u)).
+// exp(-2u) = exp2(x (c + 0.044715 c x^2)) with c = -2 sqrt(2/pi) log2(e); the quotient uses the
+// hardware reciprocal (1 ulp).  7 instructions per element.
 __device__ __forceinline__ float gelu_tanh(float x) {
-  const float k = 0.7978845608028654f;
-  float u = k * (x + 0.044715f * x * x * x);
-  float e = __expf(-2.0f * u);
-  return x / (1.0f + e);
+  const float c = -2.0f * 0.7978845608028654f * 1.4426950408889634f;
+  const float e = __builtin_amdgcn_exp2f(x * __builtin_fmaf(x * x, 0.044715f * c, c));
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 // Workgroup id -> tile id so that the workgroups resident on one XCD (ids congruent

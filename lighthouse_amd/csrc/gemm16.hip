@@ -723,10 +723,13 @@ static int launch_fast(const GemmArgs& g, hipStream_t s) {
 
 // Tile choice for the direct kernels: 0 = 256 x 256, 1 = 256 x 128, 2 = 128 x 256, 3 = 128 x 128.
 // Cost model: rounds of one workgroup per CU times the tile area (edge tiles count in
-// full), with a penalty for the smaller tiles' extra operand traffic per flop.
-static int direct_variant(int M, int N) {
+// full), with a penalty for the smaller tiles' extra operand traffic per flop.  For short K a
+// tile's prologue and epilogue weigh as much as its main loop, and the 128 x 128 tile, of which
+// two share a CU and cover each other's, costs little more per flop than the large ones
+// (measured at M = 8192, K = 768: N = 768 24 vs 28 us, N = 2304 38 vs 46, N = 3072 50 vs 51).
+static int direct_variant(int M, int N, int K) {
   static const int bm[4] = {256, 256, 128, 128}, bn[4] = {256, 128, 256, 128};
-  static const double penalty[4] = {1.0, 1.1, 1.1, 1.25};
+  const double penalty[4] = {1.0, 1.1, 1.1, K <= 1536 ? 1.08 : 1.25};
   int best = -1;
   double best_cost = 0.0;
   const int cus = num_cus();
@@ -758,7 +761,7 @@ static int gemm16_dispatch(const GemmArgs& g, hipStream_t s) {
   }
   if (vec_ok) {
     if (!tb && g.ldc % 8 == 0 && g.N % 8 == 0) {
-      const int v = tile != LH_GEMM_TILE_AUTO ? (int)(tile >> 8) - 1 : direct_variant(g.M, g.N);
+      const int v = tile != LH_GEMM_TILE_AUTO ? (int)(tile >> 8) - 1 : direct_variant(g.M, g.N, g.K);
       if (v == 0) return launch_direct<DT, 4, 2>(g, s);
       if (v == 1) return launch_direct<DT, 4, 1>(g, s);
       if (v == 2) return launch_direct<DT, 2, 2>(g, s);

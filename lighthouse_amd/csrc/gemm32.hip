@@ -15,7 +15,8 @@ namespace lh {
 constexpr int kBK32 = 32;
 
 // ---- direct-to-LDS kernel ---------------------------------------------------------------
-// Workgroup tile (64 TM) x (64 TN) x 32, 4 waves (2 x 2).  Both panels go global -> LDS with
+// Workgroup tile (64 TM) x (64 TN) x 32 with NW = 4 waves (2 x 2) or 8 waves (4 x 2, two per
+// SIMD: one wave's waits and barriers are covered by the other's MFMAs).  Both panels go global -> LDS with
 // global_load_lds_dwordx4 in their global orientation through a ring of NS stages, NS - 1 of
 // them in flight: at f32 rates a k-step lasts about as long as a global load takes, so a
 // register-staged double buffer stalls on every step.  A wave-wide load writes 1 KiB
@@ -28,22 +29,24 @@ __device__ __forceinline__ void async_copy16_f32(const float* gsrc, uint8_t* lds
   __builtin_amdgcn_global_load_lds(gsrc, (lds32_void_t*)lds_wave_base, 16, 0, 0);
 }
 
-template <int TM, int TN>
+template <int TM, int TN, int NW_>
 struct Direct32Ctx {
-  static constexpr int NW = 4;                 // waves
+  static constexpr int NW = NW_;               // waves, as (NW / 2) x 2
+  static constexpr int WTM = 4 * TM / NW;      // 32-row sub-tiles per wave (a wave spans 32 TN columns)
   static constexpr int LA = 8 * TM / NW;       // A loads per lane and stage
   static constexpr int LB = 8 * TN / NW;       // B loads per lane and stage
+  static_assert(WTM >= 1 && LA >= 1 && LB >= 1, "tile too small for the wave count");
   const float* a_src[LA];
   const float* b_src[LB];
   int64_t ldb;
   int wave, h;
-  int a_off[TM], a_swz[TM];  // byte offset of the lane's A row, its swizzle
-  int b_off[TN];             // byte offset of the lane's B column inside a k row (swizzle applied)
+  int a_off[WTM], a_swz[WTM];  // byte offset of the lane's A row, its swizzle
+  int b_off[TN];               // byte offset of the lane's B column inside a k row (swizzle applied)
 };
 
-template <int TM, int TN>
-__device__ __forceinline__ void direct32_issue(const Direct32Ctx<TM, TN>& c, int kt, uint8_t* __restrict__ stage) {
-  using C = Direct32Ctx<TM, TN>;
+template <int TM, int TN, int NW>
+__device__ __forceinline__ void direct32_issue(const Direct32Ctx<TM, TN, NW>& c, int kt, uint8_t* __restrict__ stage) {
+  using C = Direct32Ctx<TM, TN, NW>;
   constexpr int a_bytes = 64 * TM * 128;
 #pragma unroll
   for (int i = 0; i < C::LA; ++i) async_copy16_f32(c.a_src[i] + kt * 32, stage + (C::NW * i + c.wave) * 1024);
@@ -55,22 +58,23 @@ __device__ __forceinline__ void direct32_issue(const Direct32Ctx<TM, TN>& c, int
 // One k-step: refill `wr` (if `prefetch`) and multiply the stage in `rd`.
 // Separate restrict pointers keep the compiler from making the LDS reads wait for the
 // asynchronous writes.
-template <int TM, int TN>
-__device__ __forceinline__ void direct32_step(const Direct32Ctx<TM, TN>& c, f32x16 (&acc)[TN][TM],
+template <int TM, int TN, int NW>
+__device__ __forceinline__ void direct32_step(const Direct32Ctx<TM, TN, NW>& c,
+                                              f32x16 (&acc)[TN][Direct32Ctx<TM, TN, NW>::WTM],
                                               const uint8_t* __restrict__ rd, uint8_t* __restrict__ wr, int next_kt,
                                               bool prefetch) {
-  constexpr int a_bytes = 64 * TM * 128, b_row = 64 * TN * 4;
+  constexpr int a_bytes = 64 * TM * 128, b_row = 64 * TN * 4, WTM = Direct32Ctx<TM, TN, NW>::WTM;
   constexpr int NKK = 4;  // groups of 8 k per stage
   if (prefetch) direct32_issue(c, next_kt, wr);
   const uint8_t* as = rd;
   const uint8_t* bs = rd + a_bytes;
   // Fragments of k-group kk (k = 8 kk + 4 h + t, t = 0..3) are read while the MFMAs of group
   // kk - 1 run.
-  f32x4 fa[2][TM];
+  f32x4 fa[2][WTM];
   float fb[2][TN][4];
   auto read = [&](int kk, int buf) {
 #pragma unroll
-    for (int j = 0; j < TM; ++j)
+    for (int j = 0; j < WTM; ++j)
       fa[buf][j] = *reinterpret_cast<const f32x4*>(as + c.a_off[j] + (((2 * kk + c.h) ^ c.a_swz[j]) << 4));
 #pragma unroll
     for (int i = 0; i < TN; ++i)
@@ -88,12 +92,12 @@ __device__ __forceinline__ void direct32_step(const Direct32Ctx<TM, TN>& c, f32x
 #pragma unroll
       for (int i = 0; i < TN; ++i)
 #pragma unroll
-        for (int j = 0; j < TM; ++j)
+        for (int j = 0; j < WTM; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[cur][i][t], fa[cur][j][t], acc[i][j], 0, 0, 0);
     if (q + 1 < NKK) {
       // keep the reads of the next group ahead of this group's MFMAs in the issue order
-      __builtin_amdgcn_sched_group_barrier(0x100, TM + 4 * TN, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, 4 * TM * TN, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, WTM + 4 * TN, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, 4 * WTM * TN, 0);
     }
   }
 }
@@ -103,32 +107,22 @@ __device__ __forceinline__ void direct32_wait_barrier() {
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-template <int TM, int TN, int NS>
-__global__ void __launch_bounds__(256) gemm32_direct(GemmArgs g) {
-  using C = Direct32Ctx<TM, TN>;
+// Source pointers of tile `id` (row-major over the tile grid) and the tile's origin.
+template <int TM, int TN, int NW>
+__device__ __forceinline__ void direct32_place(const GemmArgs& g, int id, int lane, Direct32Ctx<TM, TN, NW>& c, int& m0,
+                                               int& n0) {
+  using C = Direct32Ctx<TM, TN, NW>;
   constexpr int BM = 64 * TM, BN = 64 * TN;
-  constexpr int a_bytes = BM * 128, b_row = BN * 4, stage_bytes = a_bytes + 32 * b_row;
-  constexpr int L = C::LA + C::LB;  // loads a lane has in flight per stage
-  static_assert(C::LA >= 1 && C::LB >= 1 && NS >= 3 && NS <= 6 && L * (NS - 2) < 64, "ring shape");
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem32d[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm0 = (wave >> 1) * 32 * TM, wn0 = (wave & 1) * 32 * TN;
+  asm volatile("" : "+v"(lane));  // recompute the lane's offsets per tile rather than keep them in registers
   const int tiles_n = g.N / BN;
-  const int id = xcd_remap(blockIdx.x, gridDim.x);
-  const int m0 = (id / tiles_n) * BM, n0 = (id % tiles_n) * BN;
+  m0 = (id / tiles_n) * BM;
+  n0 = (id % tiles_n) * BN;
   const float* A = reinterpret_cast<const float*>(g.a);
   const float* B = reinterpret_cast<const float*>(g.b);
-  const int r32 = lane & 31, h = lane >> 5;
-
-  C c;
-  c.ldb = g.ldb;
-  c.wave = wave;
-  c.h = h;
   // A: load i of wave w fills rows (NW i + w) 8 .. +8; lane -> row += lane / 8, LDS chunk lane % 8.
 #pragma unroll
   for (int i = 0; i < C::LA; ++i) {
-    const int row = (C::NW * i + wave) * 8 + (lane >> 3);
+    const int row = (C::NW * i + c.wave) * 8 + (lane >> 3);
     const int gc = (lane & 7) ^ ((row >> 1) & 7);
     c.a_src[i] = A + (int64_t)(m0 + row) * g.lda + gc * 4;
   }
@@ -137,12 +131,37 @@ __global__ void __launch_bounds__(256) gemm32_direct(GemmArgs g) {
 #pragma unroll
   for (int i = 0; i < C::LB; ++i) {
     constexpr int chunks = 16 * TN;
-    const int k = (C::NW * i + wave) * (64 / chunks) + lane / chunks;
+    const int k = (C::NW * i + c.wave) * (64 / chunks) + lane / chunks;
     const int gc = (lane % chunks) ^ (8 * ((k >> 2) & 1));
     c.b_src[i] = B + (int64_t)k * g.ldb + n0 + gc * 4;
   }
+}
+
+// Persistent workgroups, each walking the tile list with the grid as stride (tile ids congruent
+// modulo 8 stay on one XCD, which is what xcd_remap assumes).  At the end of a tile, once every
+// wave has left the ring, the first NS - 1 stages of the workgroup's next tile are issued before
+// the epilogue, so their latency and the cold start of the pipeline hide behind its stores.
+template <int TM, int TN, int NS, int NW>
+__global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
+  using C = Direct32Ctx<TM, TN, NW>;
+  constexpr int WTM = C::WTM;
+  constexpr int BM = 64 * TM, BN = 64 * TN;
+  constexpr int a_bytes = BM * 128, b_row = BN * 4, stage_bytes = a_bytes + 32 * b_row;
+  constexpr int L = C::LA + C::LB;  // loads a lane has in flight per stage
+  static_assert(NS >= 3 && NS <= 6 && L * (NS - 2) < 64, "ring shape");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem32d[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm0 = (wave >> 1) * 32 * WTM, wn0 = (wave & 1) * 32 * TN;
+  const int ntiles = (g.M / BM) * (g.N / BN);
+  const int r32 = lane & 31, h = lane >> 5;
+
+  C c;
+  c.ldb = g.ldb;
+  c.wave = wave;
+  c.h = h;
 #pragma unroll
-  for (int j = 0; j < TM; ++j) {
+  for (int j = 0; j < WTM; ++j) {
     const int row = wm0 + 32 * j + r32;
     c.a_off[j] = row * 128;
     c.a_swz[j] = (row >> 1) & 7;
@@ -153,46 +172,65 @@ __global__ void __launch_bounds__(256) gemm32_direct(GemmArgs g) {
     c.b_off[i] = (((n >> 2) ^ (8 * h)) << 4) + (n & 3) * 4;  // rows 8 kk + 4 h + t have (k / 4) % 2 == h
   }
 
-  f32x16 acc[TN][TM];
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
   const int nk = g.K / 32;
+  int t = blockIdx.x;  // < ntiles: the grid is never larger than the tile list
+  int m0, n0;
+  direct32_place(g, xcd_remap(t, ntiles), lane, c, m0, n0);
 #pragma unroll
   for (int st = 0; st < NS - 1; ++st)
     if (st < nk) direct32_issue(c, st, smem32d + st * stage_bytes);
-  for (int kt = 0; kt < nk; ++kt) {
-    // Stages kt + 1 .. kt + NS - 2 may stay in flight; one asm block per case because a
-    // __syncthreads() would add a fence that waits for every outstanding load.
-    const int younger = min(nk - 1 - kt, NS - 2);
-    if (younger >= 4) direct32_wait_barrier<L * 4>();
-    else if (younger == 3) direct32_wait_barrier<L * 3>();
-    else if (younger == 2) direct32_wait_barrier<L * 2>();
-    else if (younger == 1) direct32_wait_barrier<L>();
-    else direct32_wait_barrier<0>();
-    const int nxt = kt + NS - 1;
-    direct32_step(c, acc, smem32d + (kt % NS) * stage_bytes, smem32d + (nxt % NS) * stage_bytes, nxt, nxt < nk);
+  for (;;) {
+    f32x16 acc[TN][WTM];
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < WTM; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+    for (int kt = 0; kt < nk; ++kt) {
+      // Stages kt + 1 .. kt + NS - 2 may stay in flight (anything issued after them, such as the
+      // previous tile's stores, only makes the wait longer); one asm block per case because a
+      // __syncthreads() would add a fence that waits for every outstanding load.
+      const int younger = min(nk - 1 - kt, NS - 2);
+      if (younger >= 4) direct32_wait_barrier<L * 4>();
+      else if (younger == 3) direct32_wait_barrier<L * 3>();
+      else if (younger == 2) direct32_wait_barrier<L * 2>();
+      else if (younger == 1) direct32_wait_barrier<L>();
+      else direct32_wait_barrier<0>();
+      const int nxt = kt + NS - 1;
+      direct32_step(c, acc, smem32d + (kt % NS) * stage_bytes, smem32d + (nxt % NS) * stage_bytes, nxt, nxt < nk);
+    }
+    const int tn = t + (int)gridDim.x;
+    const bool more = tn < ntiles;
+    const int em0 = m0, en0 = n0;
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the ring
+    if (more) {
+      direct32_place(g, xcd_remap(tn, ntiles), lane, c, m0, n0);
+#pragma unroll
+      for (int st = 0; st < NS - 1; ++st)
+        if (st < nk) direct32_issue(c, st, smem32d + st * stage_bytes);
+    }
+    int elane = lane;
+    asm volatile("" : "+v"(elane));  // as in direct32_place
+    const int m_base = em0 + wm0 + (elane & 31);
+    const int n_base = en0 + wn0 + 4 * (elane >> 5);
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int j = 0; j < WTM; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          epilogue4<LH_F32>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                            acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+    if (!more) break;
+    t = tn;
   }
-
-  const int m_base = m0 + wm0 + r32;
-  const int n_base = n0 + wn0 + 4 * h;
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        epilogue4<LH_F32>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
-                          acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
 }
 
-template <int TM, int TN, int NS>
+// `per_cu`: workgroups of this shape that fit a CU's LDS together.
+template <int TM, int TN, int NS, int NW = 4>
 static int launch_direct32(const GemmArgs& g, hipStream_t s) {
-  auto kern = gemm32_direct<TM, TN, NS>;
+  auto kern = gemm32_direct<TM, TN, NS, NW>;
   constexpr size_t lds = (size_t)NS * (64 * TM * 128 + 32 * 64 * TN * 4);
   static bool configured = false;
   if (!configured) {
@@ -200,7 +238,9 @@ static int launch_direct32(const GemmArgs& g, hipStream_t s) {
                                      (int)lds));
     configured = true;
   }
-  hipLaunchKernelGGL(kern, dim3((g.M / (64 * TM)) * (g.N / (64 * TN))), dim3(256), lds, s, g);
+  const int ntiles = (g.M / (64 * TM)) * (g.N / (64 * TN));
+  const int resident = num_cus() * (int)((160 * 1024) / lds);
+  hipLaunchKernelGGL(kern, dim3(ntiles < resident ? ntiles : resident), dim3(NW * 64), lds, s, g);
   return check_launch("gemm32_direct");
 }
 
@@ -261,7 +301,13 @@ int gemm32(const GemmArgs& g, hipStream_t s) {
                       aligned16(g.a) && aligned16(g.b) && aligned16(g.out) &&
                       (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias));
   if (vec_ok && g.M % 128 == 0 && g.N % 128 == 0 && (int64_t)(g.M / 128) * (g.N / 128) >= 256) {
-    return launch_direct32<2, 2, 4>(g, s);
+    // 128 x 128 or 128 x 64 tiles, one workgroup per CU: whichever needs less time in whole
+    // rounds of tiles (the narrow tile pays about 8 % more operand traffic per flop).
+    const int cus = num_cus();
+    const int64_t t128 = (int64_t)(g.M / 128) * (g.N / 128);
+    const double wide = (double)((t128 + cus - 1) / cus), narrow = (double)((2 * t128 + cus - 1) / cus) * 0.54;
+    if (narrow < wide) return launch_direct32<2, 1, 4, 8>(g, s);
+    return launch_direct32<2, 2, 4, 8>(g, s);
   }
   if (vec_ok && g.M % 64 == 0 && g.N % 64 == 0) {
     // Up to two workgroups per CU: a deep ring; more: a shallow ring so that three share a CU.
