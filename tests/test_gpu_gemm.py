@@ -23,7 +23,9 @@ def _host(t):
 
 
 @pytest.mark.parametrize("shape", [(64, 64, 32), (128, 128, 64), (256, 192, 96), (1024, 1024, 1024), (100, 70, 50),
-                                   (1, 1, 1), (33, 65, 17)])
+                                   (1, 1, 1), (33, 65, 17),
+                                   # 128 x 128 tiles, two per workgroup; 128 x 64 tiles, three per workgroup; one
+                                   (4096, 2048, 64), (4096, 1536, 96), (2048, 2048, 512)])
 @pytest.mark.parametrize("epi", ["none", "bias_relu"])
 def test_gemm_f32(shape, epi):
     from lighthouse_amd import ops
@@ -234,7 +236,8 @@ def test_gemm_errors():
 
 
 @pytest.mark.parametrize("shape", [(128, 128, 128), (256, 256, 512), (96, 80, 200), (16, 256, 1024), (5, 128, 256),
-                                   (2048, 4096, 128), (4096, 2048, 384)])  # the last two: direct-to-LDS kernel
+                                   # direct-to-LDS kernel: one tile per workgroup (twice), two tiles per workgroup
+                                   (2048, 4096, 128), (4096, 2048, 384), (8192, 4096, 128)])
 def test_gemm_fp8(shape):
     from lighthouse_amd import ops
 
