@@ -105,6 +105,34 @@ def test_gemm_16bit_requested_tile(tile, K, epi):
     assert_close(_host(out), ref, rtol, f"bf16 gemm tile {tile} K={K} {epi}")
 
 
+@pytest.mark.parametrize("epi", ["bias_relu", "f32out_acc"])
+@pytest.mark.parametrize("tile,M,N", [((256, 256), 4608, 4608), ((256, 128), 4608, 2304), ((128, 256), 2304, 4608),
+                                      ((128, 128), 3072, 3072), (None, 4600, 4600)])
+def test_gemm_16bit_several_tiles_per_workgroup(tile, M, N, epi):
+    """More tiles than resident workgroups: a workgroup issues its next tile's first loads before
+    the epilogue of the current one (some workgroups get two tiles, others one).  The last case
+    is the edge instantiation (M, N not multiples of the tile)."""
+    from lighthouse_amd import ops
+
+    K = 128
+    rng = np.random.default_rng(M + N)
+    a = orc.round_to(rng.standard_normal((M, K)).astype(np.float32), "bf16")
+    b = orc.round_to(rng.standard_normal((K, N)).astype(np.float32), "bf16")
+    da, db = _dev(a, torch.bfloat16), _dev(b, torch.bfloat16)
+    if epi == "bias_relu":
+        bias = orc.round_to(rng.standard_normal((N,)).astype(np.float32), "bf16")
+        out = ops.gemm(da, db, _dev(bias, torch.bfloat16), relu=True, tile=tile)
+        ref = orc.matmul(a, b, bias=bias, relu=True, result_type="bf16")
+        rtol = BF16_RTOL
+    else:
+        c = rng.standard_normal((M, N)).astype(np.float32)
+        out = _dev(c, torch.float32)
+        ops.gemm(da, db, out=out, accumulate_c=True, tile=tile)
+        ref = orc.matmul(a, b, c=c, accumulate_c=True, result_type="f32")
+        rtol = F32_RTOL
+    assert_close(_host(out), ref, rtol, f"bf16 gemm {M}x{N} tile {tile} {epi}")
+
+
 @pytest.mark.parametrize("shape", [(1000, 520, 192), (130, 264, 64), (257, 8, 128), (1, 1000, 256), (3000, 776, 320)])
 @pytest.mark.parametrize("epi", ["none", "bias_relu", "f32out_acc_bias"])
 def test_gemm_16bit_ragged_shapes(shape, epi):
