@@ -136,6 +136,16 @@ __device__ __forceinline__ float gelu_tanh(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
+// The lane's index in its wave, recomputed from the execution mask at the point of the call (the
+// opaque zero keeps the compiler from computing it once and holding it in a register).  Persistent
+// kernels use it for per-tile address setup so that lane-dependent offsets do not stay live, or
+// get spilled, across a register-bound main loop.  Requires all 64 lanes active.
+__device__ __forceinline__ int lane_now() {
+  int zero = 0;
+  asm volatile("" : "+v"(zero));
+  return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, zero));
+}
+
 // Workgroup id -> tile id so that the workgroups resident on one XCD (ids congruent
 // modulo 8 are dispatched to the same XCD) cover a compact patch of tiles and share
 // their operand panels through that XCD's L2.

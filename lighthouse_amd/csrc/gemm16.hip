@@ -363,10 +363,10 @@ __device__ __forceinline__ void direct_step_pair(const DirectCtx<TM, TN>& c, f32
 // rows / column chunks past the end are redirected to the last valid row / chunk (their products
 // land in accumulators that are never stored) and the epilogue skips what lies outside the matrix.
 template <int TM, int TN, bool EDGE>
-__device__ __forceinline__ void direct_place(const GemmArgs& g, int id, int lane, DirectCtx<TM, TN>& c, int& m0,
-                                             int& n0) {
+__device__ __forceinline__ void direct_place(const GemmArgs& g, int id, DirectCtx<TM, TN>& c, int& m0, int& n0) {
   using Cfg = DirectCfg<TM, TN>;
   constexpr int BM = Cfg::BM, BN = Cfg::BN;
+  const int lane = lane_now();
   const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
   constexpr int GROUP_M = 4;
   const int group_size = GROUP_M * tiles_n;
@@ -480,13 +480,12 @@ template <int DT, int TM, int TN, bool EDGE, bool HAS_NEXT>
 __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx<TM, TN>& next, int nk,
                                               uint8_t* __restrict__ ring, uint8_t* __restrict__ stage,
                                               const f32x16 (&acc)[TN][TM], const u32x2 (&bias)[TN][4], int m0, int n0,
-                                              int wm0, int wn0, int lane) {
+                                              int wm0, int wn0) {
   using Cfg = DirectCfg<TM, TN>;
   constexpr int WTN = Cfg::WTN;
-  // The lane-dependent addresses below do not change from tile to tile; computed from an opaque
-  // copy of the lane index they are recomputed here instead of being kept in registers (and
-  // spilled) across the main loop.
-  asm volatile("" : "+v"(lane));
+  // The lane-dependent addresses below do not change from tile to tile; lane_now() has them
+  // recomputed here instead of kept in registers (and spilled) across the main loop.
+  const int lane = lane_now();
   const int r32 = lane & 31, h = lane >> 5;
   const int m_base = m0 + wm0 + r32;
   const int n_base = n0 + wn0 + 4 * h;
@@ -542,6 +541,67 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
   }
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   if constexpr (HAS_NEXT) direct_prologue(next, nk, ring);
+  if (g.out_dt == LH_F32) {
+    // f32 output (with or without an accumulator input): the scaled accumulators of a 32 x 8 QH
+    // block go through the wave's slice of `stage` so that the accumulator input is read and the
+    // result written as whole row segments (16 bytes per lane, 64 or 128 bytes per row) instead
+    // of 16-byte pieces of 64 different rows.  Order of operations as in epilogue4.
+    constexpr int QH = TN == 2 ? 4 : 2;        // accumulator column groups (of 8) per staged block
+    constexpr int RB = QH * 32;                // bytes of a staged row
+    constexpr int chunks = RB / 16;
+    constexpr int rows_per_pass = 64 / chunks;
+    uint8_t* cw = stage + next.wave * (32 * RB);
+    float* outp = reinterpret_cast<float*>(g.out);
+    const float* cin = reinterpret_cast<const float*>(g.c);
+    const bool has_c = (g.flags & LH_GEMM_ACCUMULATE_C) != 0;
+    const bool gelu = (g.flags & LH_GEMM_HAS_GELU) != 0, relu = (g.flags & LH_GEMM_HAS_RELU) != 0;
+    const int ch = lane % chunks, row0 = lane / chunks;
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int qh = 0; qh < 4 / QH; ++qh) {
+        const int n = n0 + wn0 + 32 * i + 8 * QH * qh + 4 * ch;  // the lane's 4 output columns
+        const bool n_ok = !EDGE || n < g.N;
+        const f32x4 b4 = bias4<DT>(g, EDGE ? min(n, g.N - 4) : n);
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+#pragma unroll
+          for (int qq = 0; qq < QH; ++qq) {
+            const int q = QH * qh + qq;
+            const f32x4 w = {acc[i][j][4 * q] * g.alpha, acc[i][j][4 * q + 1] * g.alpha, acc[i][j][4 * q + 2] * g.alpha,
+                             acc[i][j][4 * q + 3] * g.alpha};
+            *reinterpret_cast<f32x4*>(cw + r32 * RB + (((2 * qq + h) ^ ((r32 >> 1) & (chunks - 1))) << 4)) = w;
+          }
+#pragma unroll
+          for (int t = 0; t < 32 / rows_per_pass; ++t) {
+            const int row = rows_per_pass * t + row0;
+            f32x4 v = *reinterpret_cast<const f32x4*>(cw + row * RB + ((ch ^ ((row >> 1) & (chunks - 1))) << 4));
+            const int m = m0 + wm0 + 32 * j + row;
+            if (EDGE && !(n_ok && m < g.M)) continue;
+            const int64_t off = (int64_t)m * g.ldc + n;
+            if (has_c) {
+              const f32x4 c4 = *reinterpret_cast<const f32x4*>(cin + off);
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] += c4[e];
+            }
+            if (g.flags & LH_GEMM_HAS_BIAS) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] += b4[e];
+            }
+            if (gelu) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
+            }
+            if (relu) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
+            }
+            *reinterpret_cast<f32x4*>(outp + off) = v;
+          }
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TN; ++i)
 #pragma unroll
@@ -594,7 +654,7 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
   const int nk = g.K / 32;  // even: K is a multiple of 64
   int t = blockIdx.x;       // < ntiles: the grid is never larger than the tile list
   int m0, n0;
-  direct_place<TM, TN, EDGE>(g, xcd_remap(t, ntiles), lane, c, m0, n0);
+  direct_place<TM, TN, EDGE>(g, xcd_remap(t, ntiles), c, m0, n0);
   direct_prologue(c, nk, smem_d);
   // Without EDGE every lane issues all stores of a staged epilogue.
   const bool staged = g.out_dt != LH_F32 && !(g.flags & LH_GEMM_ACCUMULATE_C);
@@ -617,10 +677,10 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
     int m1 = 0, n1 = 0;
     uint8_t* const stage = smem_d + Cfg::kRingBytes;
     if (more) {
-      direct_place<TM, TN, EDGE>(g, xcd_remap(tn, ntiles), lane, cn, m1, n1);
-      direct_finish<DT, TM, TN, EDGE, true>(g, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0, lane);
+      direct_place<TM, TN, EDGE>(g, xcd_remap(tn, ntiles), cn, m1, n1);
+      direct_finish<DT, TM, TN, EDGE, true>(g, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0);
     } else {
-      direct_finish<DT, TM, TN, EDGE, false>(g, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0, lane);
+      direct_finish<DT, TM, TN, EDGE, false>(g, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0);
     }
     if (!more) break;
     c = cn;

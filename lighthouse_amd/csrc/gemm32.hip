@@ -109,11 +109,10 @@ __device__ __forceinline__ void direct32_wait_barrier() {
 
 // Source pointers of tile `id` (row-major over the tile grid) and the tile's origin.
 template <int TM, int TN, int NW>
-__device__ __forceinline__ void direct32_place(const GemmArgs& g, int id, int lane, Direct32Ctx<TM, TN, NW>& c, int& m0,
-                                               int& n0) {
+__device__ __forceinline__ void direct32_place(const GemmArgs& g, int id, Direct32Ctx<TM, TN, NW>& c, int& m0, int& n0) {
   using C = Direct32Ctx<TM, TN, NW>;
   constexpr int BM = 64 * TM, BN = 64 * TN;
-  asm volatile("" : "+v"(lane));  // recompute the lane's offsets per tile rather than keep them in registers
+  const int lane = lane_now();  // the lane's offsets are recomputed per tile rather than kept in registers
   const int tiles_n = g.N / BN;
   m0 = (id / tiles_n) * BM;
   n0 = (id % tiles_n) * BN;
@@ -175,7 +174,7 @@ __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
   const int nk = g.K / 32;
   int t = blockIdx.x;  // < ntiles: the grid is never larger than the tile list
   int m0, n0;
-  direct32_place(g, xcd_remap(t, ntiles), lane, c, m0, n0);
+  direct32_place(g, xcd_remap(t, ntiles), c, m0, n0);
 #pragma unroll
   for (int st = 0; st < NS - 1; ++st)
     if (st < nk) direct32_issue(c, st, smem32d + st * stage_bytes);
@@ -205,13 +204,12 @@ __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
     const int em0 = m0, en0 = n0;
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the ring
     if (more) {
-      direct32_place(g, xcd_remap(tn, ntiles), lane, c, m0, n0);
+      direct32_place(g, xcd_remap(tn, ntiles), c, m0, n0);
 #pragma unroll
       for (int st = 0; st < NS - 1; ++st)
         if (st < nk) direct32_issue(c, st, smem32d + st * stage_bytes);
     }
-    int elane = lane;
-    asm volatile("" : "+v"(elane));  // as in direct32_place
+    const int elane = lane_now();  // as in direct32_place
     const int m_base = em0 + wm0 + (elane & 31);
     const int n_base = en0 + wn0 + 4 * (elane >> 5);
 #pragma unroll

@@ -274,9 +274,9 @@ __device__ __forceinline__ void d8_step_pair(const D8Ctx& c, f32x16 (&acc)[2][4]
 }
 
 // Source pointers of tile `id` (its position in the XCD-grouped order) and the tile's origin.
-__device__ __forceinline__ void d8_place(const GemmArgs& g, int id, int lane, D8Ctx& c, int& m0, int& n0) {
+__device__ __forceinline__ void d8_place(const GemmArgs& g, int id, D8Ctx& c, int& m0, int& n0) {
   constexpr int BM = 256, BN = 256;
-  asm volatile("" : "+v"(lane));  // recompute the lane's offsets per tile rather than keep them in registers
+  const int lane = lane_now();  // the lane's offsets are recomputed per tile rather than kept in registers
   const int tiles_m = g.M / BM, tiles_n = g.N / BN;
   constexpr int GROUP_M = 4;
   const int group_size = GROUP_M * tiles_n;
@@ -345,9 +345,9 @@ __device__ __forceinline__ void d8_mainloop(const D8Ctx& c, f32x16 (&acc)[2][4],
 template <bool HAS_NEXT>
 __device__ __forceinline__ void d8_finish(const GemmArgs& g, const D8Ctx& next, int nk, uint8_t* __restrict__ ring,
                                           uint8_t* __restrict__ stage, const f32x16 (&acc)[2][4], int m0, int n0, int wm0,
-                                          int wn0, int lane) {
+                                          int wn0) {
   constexpr int TM = 4, TN = 2, RB = 128, chunks = 8, rows_per_pass = 8;
-  asm volatile("" : "+v"(lane));  // keeps the addresses below out of registers during the main loop
+  const int lane = lane_now();  // keeps the addresses below out of registers during the main loop
   const int r32 = lane & 31, h = lane >> 5;
   const int m_base = m0 + wm0 + r32;
   const int n_base = n0 + wn0 + 4 * h;
@@ -421,7 +421,7 @@ __global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
   const int nk = g.K / 64;  // even: K is a multiple of 128
   int t = blockIdx.x;       // < ntiles: the grid is never larger than the tile list
   int m0, n0;
-  d8_place(g, xcd_remap(t, ntiles), lane, c, m0, n0);
+  d8_place(g, xcd_remap(t, ntiles), c, m0, n0);
   d8_prologue(c, nk, smem_8);
   for (;;) {
     f32x16 acc[TN][TM];
@@ -438,10 +438,10 @@ __global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
     int m1 = 0, n1 = 0;
     uint8_t* const stage = smem_8 + kD8RingBytes;
     if (more) {
-      d8_place(g, xcd_remap(tn, ntiles), lane, cn, m1, n1);
-      d8_finish<true>(g, cn, nk, smem_8, stage, acc, m0, n0, wm0, wn0, lane);
+      d8_place(g, xcd_remap(tn, ntiles), cn, m1, n1);
+      d8_finish<true>(g, cn, nk, smem_8, stage, acc, m0, n0, wm0, wn0);
     } else {
-      d8_finish<false>(g, cn, nk, smem_8, stage, acc, m0, n0, wm0, wn0, lane);
+      d8_finish<false>(g, cn, nk, smem_8, stage, acc, m0, n0, wm0, wn0);
     }
     if (!more) break;
     c = cn;
