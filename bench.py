@@ -26,7 +26,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM bytes one launch of the headline kernel moves, from two rocprofv3 --pmc runs of
 # `bench.py --only gemm_bf16` (FETCH_SIZE 98560.8 KiB x 2.0, the factor a plain copy of known size
 # gives for that counter, plus WRITE_SIZE 32768 KiB x 1.0); algorithmic minimum 100.7 MB.
-GEMM_BF16_4096_TRAFFIC_BYTES = 235.4e6
+GEMM_BF16_4096_TRAFFIC_BYTES = 235.3e6
 
 
 def time_region(fn, steps, warmup):
