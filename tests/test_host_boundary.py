@@ -212,8 +212,9 @@ def test_c_abi_argument_validation_without_gpu():
     assert lib.lh_hip_gemm(p, p, p, None, 4, 4, 4, 4, 4, 4, _lib.F64, _lib.F64, 0, None) == _lib.LH_ERR_UNSUPPORTED
     assert lib.lh_hip_gemm(p, p, p, None, 4, 4, 4, 4, 4, 4, _lib.BF16, _lib.F16, 0, None) == _lib.LH_ERR_UNSUPPORTED
     assert lib.lh_hip_gemm(p, p, p, None, 4, 4, 4, 4, 4, 4, _lib.F32, _lib.F32, 1 << 9, None) == _lib.LH_ERR_INVALID
-    assert lib.lh_hip_attention(p, p, p, p, 1, 1, 128, 32, z, z, z, z, 1.0, 0, _lib.BF16, None) == _lib.LH_ERR_UNSUPPORTED
-    assert lib.lh_hip_attention(p, p, p, p, 1, 1, 100, 64, z, z, z, z, 1.0, 0, _lib.BF16, None) == _lib.LH_ERR_UNSUPPORTED
+    assert lib.lh_hip_attention(p, p, p, p, 1, 1, 128, 512, z, z, z, z, 1.0, 0, _lib.BF16, None) == _lib.LH_ERR_UNSUPPORTED
+    assert lib.lh_hip_attention(p, p, p, p, 1, 1, 100, 64, z, z, z, z, 1.0, 0, _lib.BF16, None) == _lib.LH_ERR_INVALID  # row stride 0
+    assert lib.lh_hip_attention(p, p, p, p, 0, 1, 100, 64, z, z, z, z, 1.0, 0, _lib.BF16, None) == _lib.LH_ERR_INVALID
     assert lib.lh_hip_layer_norm(p, p, p, p, 0, 8, 1e-5, _lib.F32, _lib.F32, None) == _lib.LH_ERR_INVALID
     assert lib.lh_hip_nanogpt_block(p, p, None, 1, 1, 8, 2, 1e-5, _lib.F32, p, 0, None) == _lib.LH_ERR_INVALID
     with pytest.raises(ValueError):
