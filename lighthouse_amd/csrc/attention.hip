@@ -48,7 +48,6 @@ constexpr int kHeadDim = 64;
 constexpr int kKvTile = 64;
 constexpr int kQBlock = 128;        // query rows per workgroup of the f32 kernel
 constexpr int kQBlock16 = 256;      // query rows per workgroup of the 16-bit kernel (4 waves x 64)
-constexpr int kAttnStages = 4;      // K/V ring depth
 constexpr int kAttnStageBytes = 2 * kKvTile * kHeadDim * 2;  // K tile + V tile, 16 KiB
 constexpr float kOffsetSlack = 1024.0f;  // largest partial row sum of P the softmax offset tolerates
 
@@ -222,11 +221,11 @@ __device__ __forceinline__ void causal_block_of(int L, int G, int R, int nqb, in
 
 // 16-bit kernel.  A workgroup owns 256 query rows of one (batch, head): 4 waves x 64 rows (two
 // 32-row sub-tiles per wave share every K and V fragment).  K/V tiles of 64 keys go global ->
-// LDS with global_load_lds_dwordx4 through a ring of 4 stages; K fragments are 16-byte LDS
+// LDS with global_load_lds_dwordx4 through a ring of NS stages; K fragments are 16-byte LDS
 // reads, V^T fragments come from ds_read_b64_tr_b16 on the row-major V tile.  Rows of a tile
 // are 128 bytes and cannot be padded (a wave-wide load writes 1 KiB contiguous), so the
 // 16-byte chunk a lane fetches is XOR-swizzled: K chunk ^ ((key / 2) % 8), V chunk ^ 4 ((key / 2) % 2).
-template <int DT, int NQ>
+template <int DT, int NQ, int NS>
 __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
   constexpr int kRowsPerWave = 32 * NQ, kRowsPerGroup = 4 * kRowsPerWave;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn[];
@@ -311,12 +310,13 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
 
   const int kv_end = a.causal ? min(a.T, q0 + kRowsPerGroup) : a.T;
   const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
+  constexpr int kAttnStages = NS;  // K/V ring depth, 3 or 4
 #pragma unroll
   for (int st = 0; st < kAttnStages - 1; ++st)
     if (st < ntiles) attn_issue_loads(c, st, smem_attn + st * kAttnStageBytes);
 
   for (int jt = 0; jt < ntiles; ++jt) {
-    // 4 loads per lane and stage; the 2 younger stages may stay in flight.  One asm block: a
+    // 4 loads per lane and stage; the NS - 2 younger stages may stay in flight.  One asm block: a
     // __syncthreads() would add a fence that waits for ALL outstanding loads.
     const int younger = min(ntiles - 1 - jt, kAttnStages - 2);
     if (younger >= 2) asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
@@ -532,10 +532,10 @@ __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
     }
 }
 
-template <int DT, int NQ>
+template <int DT, int NQ, int NS>
 static int attention16_launch_nq(const AttnArgs& a, hipStream_t s) {
-  auto kern = attention16_kernel<DT, NQ>;
-  constexpr size_t lds = (size_t)kAttnStages * kAttnStageBytes;
+  auto kern = attention16_kernel<DT, NQ, NS>;
+  constexpr size_t lds = (size_t)NS * kAttnStageBytes;
   static bool configured = false;
   if (!configured) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -557,8 +557,15 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
   // Measured on [4,16,2048]: 32 rows per wave 105 us non-causal (64 rows: 99) but 54 us causal
   // (64 rows: 58), hence the different limits.
   const int64_t limit = a.causal ? 2 * (int64_t)a.cus + 1 : 2 * (int64_t)a.cus;
-  if (groups64 < limit) return attention16_launch_nq<DT, 1>(a, s);
-  return attention16_launch_nq<DT, 2>(a, s);
+  if (groups64 < limit) {
+    // With more than one 128-row workgroup per CU a ring of 3 stages (48 KiB) lets three of them
+    // share a CU instead of two ([8,12,1024] causal 26.7 -> 25.3 us, [16,16,512] causal 24.2 ->
+    // 22.3); a problem that does not fill the CUs is better off with the deeper ring.
+    const int64_t groups32 = (int64_t)((a.T + 127) / 128) * a.Z * a.H;
+    if (groups32 > a.cus) return attention16_launch_nq<DT, 1, 3>(a, s);
+    return attention16_launch_nq<DT, 1, 4>(a, s);
+  }
+  return attention16_launch_nq<DT, 2, 4>(a, s);
 }
 
 // Any sequence length and head dimension up to 256: one wave per query row, keys in chunks of 64
