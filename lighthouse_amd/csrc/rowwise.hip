@@ -41,40 +41,54 @@ __device__ __forceinline__ void store4(void* p, int64_t i, f32x4 v) {
 // emit_layer_norm_generics (lighthouse/ingress/mlir_gen/gpu_layer_norm_payload.py:15-87)
 // evaluated on the register-resident row: sum -> mean = sum * (1/N); sum of squared centred
 // values -> var = that * (1/N); (x - mean) * rsqrt(var + eps) * gamma + beta.
-template <int XDT, int ODT, int VPL>
+// A wave takes RPW rows (r, r + rows/RPW ...): all of them, gamma and beta are requested up
+// front, so that the loads of a later row and the stores of an earlier one overlap.
+template <int XDT, int ODT, int VPL, int RPW>
 __global__ void __launch_bounds__(256) layer_norm_vec(void* out, const void* x, const float* gamma, const float* beta,
                                                       int M, int N, float eps, float inv_n) {
   const int lane = threadIdx.x & 63;
-  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= M) return;
-  const int64_t base = (int64_t)row * N;
-  f32x4 v[VPL];
-  float s = 0.0f;
+  const int slots = (M + RPW - 1) / RPW;  // waves in the grid that have work
+  const int slot = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (slot >= slots) return;
+  f32x4 v[RPW][VPL];
 #pragma unroll
-  for (int i = 0; i < VPL; ++i) {
-    v[i] = load4<XDT>(x, base + (i * 64 + lane) * 4);
-    s += (v[i][0] + v[i][1]) + (v[i][2] + v[i][3]);
+  for (int r = 0; r < RPW; ++r) {
+    const int row = min(slot + r * slots, M - 1);  // a row past the end repeats the last one and is not stored
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) v[r][i] = load4<XDT>(x, (int64_t)row * N + (i * 64 + lane) * 4);
   }
-  const float mean = wave_sum(s) * inv_n;
-  float q = 0.0f;
+  f32x4 g[VPL], b[VPL];
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
+    g[i] = *reinterpret_cast<const f32x4*>(gamma + (i * 64 + lane) * 4);
+    b[i] = *reinterpret_cast<const f32x4*>(beta + (i * 64 + lane) * 4);
+  }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      float c = v[i][e] - mean;
-      q += c * c;
+  for (int r = 0; r < RPW; ++r) {
+    const int row = slot + r * slots;
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) s += (v[r][i][0] + v[r][i][1]) + (v[r][i][2] + v[r][i][3]);
+    const float mean = wave_sum(s) * inv_n;
+    float q = 0.0f;
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float c = v[r][i][e] - mean;
+        q += c * c;
+      }
     }
-  }
-  const float inv_std = rsqrtf(wave_sum(q) * inv_n + eps);
+    const float inv_std = rsqrtf(wave_sum(q) * inv_n + eps);
+    if (row < M) {
 #pragma unroll
-  for (int i = 0; i < VPL; ++i) {
-    const int col = (i * 64 + lane) * 4;
-    f32x4 g = *reinterpret_cast<const f32x4*>(gamma + col);
-    f32x4 b = *reinterpret_cast<const f32x4*>(beta + col);
-    f32x4 o;
+      for (int i = 0; i < VPL; ++i) {
+        f32x4 o;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = (v[i][e] - mean) * inv_std * g[e] + b[e];
-    store4<ODT>(out, base + col, o);
+        for (int e = 0; e < 4; ++e) o[e] = (v[r][i][e] - mean) * inv_std * g[i][e] + b[i][e];
+        store4<ODT>(out, (int64_t)row * N + (i * 64 + lane) * 4, o);
+      }
+    }
   }
 }
 
@@ -189,9 +203,17 @@ static int layer_norm_launch(void* out, const void* x, const float* gamma, const
   const float inv_n = (float)(1.0 / (double)N);
   dim3 grid((M + 3) / 4), block(256);
   const bool vec = N % 256 == 0 && aligned16(out) && aligned16(x) && aligned16(gamma) && aligned16(beta);
-#define LH_LN_CASE(V)                                                                                          \
-  case V:                                                                                                      \
-    hipLaunchKernelGGL((layer_norm_vec<XDT, ODT, V>), grid, block, 0, s, out, x, gamma, beta, M, N, eps, inv_n); \
+  // Two rows per wave once every CU would otherwise hold 16 waves or more (and rows of at most
+  // 1024 elements, to stay within 64 registers of row data).
+  const bool two = (int64_t)M >= 16ll * 2 * num_cus() && N <= 1024;
+  const dim3 grid2((((M + 1) / 2) + 3) / 4);
+#define LH_LN_CASE(V)                                                                                                 \
+  case V:                                                                                                             \
+    if (two && V <= 4)                                                                                                \
+      hipLaunchKernelGGL((layer_norm_vec<XDT, ODT, V, V <= 4 ? 2 : 1>), grid2, block, 0, s, out, x, gamma, beta, M, N, eps, \
+                         inv_n);                                                                                      \
+    else                                                                                                              \
+      hipLaunchKernelGGL((layer_norm_vec<XDT, ODT, V, 1>), grid, block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);  \
     return check_launch("layer_norm_vec");
   if (vec) {
     switch (N / 256) {
