@@ -57,17 +57,41 @@ class _Ref:
     name: str
 
 
-def _arg(env: dict, a):
-    """Resolve an FX argument (nodes nested in tuples / lists / dicts / slices) against the environment."""
+def _has_node(a) -> bool:
     if isinstance(a, (torch.fx.Node, _Ref)):
-        return env[a.name]
+        return True
     if isinstance(a, dict):
-        return {k: _arg(env, v) for k, v in a.items()}
+        return any(_has_node(v) for v in a.values())
     if isinstance(a, (tuple, list)):
-        return type(a)(_arg(env, x) for x in a)
+        return any(_has_node(x) for x in a)
     if isinstance(a, slice):
-        return slice(_arg(env, a.start), _arg(env, a.stop), _arg(env, a.step))
-    return a
+        return any(_has_node(x) for x in (a.start, a.stop, a.step))
+    return False
+
+
+def _resolver(a) -> Callable[[dict], object]:
+    """A function env -> value for one FX argument (nodes nested in tuples / lists / dicts / slices
+    are looked up in the environment), built at lowering time so that a call of the compiled
+    function does no type dispatch over its arguments: constants are returned as they are, a node
+    is one dictionary lookup."""
+    if not _has_node(a):
+        return lambda env: a
+    if isinstance(a, (torch.fx.Node, _Ref)):
+        name = a.name
+        return lambda env: env[name]
+    if isinstance(a, dict):
+        items = [(k, _resolver(v)) for k, v in a.items()]
+        return lambda env: {k: f(env) for k, f in items}
+    if isinstance(a, (tuple, list)):
+        parts, ctor = [_resolver(x) for x in a], type(a)
+        return lambda env: ctor(f(env) for f in parts)
+    start, stop, step = _resolver(a.start), _resolver(a.stop), _resolver(a.step)  # a slice
+    return lambda env: slice(start(env), stop(env), step(env))
+
+
+def _call_resolver(args, kwargs) -> Callable[[dict], tuple]:
+    """Resolvers of a call's positional and keyword arguments."""
+    return _resolver(tuple(args)), (_resolver(dict(kwargs)) if kwargs else None)
 
 
 class _WeightCache:
@@ -147,9 +171,10 @@ class _Lowering:
             self.fused[act_node.name] = node.name
         cache = self.cache
 
-        def run(env, x_arg=x_arg, w_arg=w_arg, b_arg=b_arg, act=act):
-            x, w = _arg(env, x_arg), _arg(env, w_arg)
-            b = _arg(env, b_arg) if b_arg is not None else None
+        x_f, w_f, b_f = _resolver(x_arg), _resolver(w_arg), _resolver(b_arg)
+
+        def run(env, act=act):
+            x, w, b = x_f(env), w_f(env), b_f(env)
             wt = cache.get(w, "linear_weight", lambda t: t.t().contiguous())
             x2 = _as_2d(x)
             out = ops.gemm(x2, wt, b.detach() if b is not None else None, relu=act == "relu", gelu=act == "gelu")
@@ -162,10 +187,12 @@ class _Lowering:
             raise ValueError(f"{node.name}: LayerNorm over {tuple(shape)}: only the last dimension is supported")
         cache = self.cache
 
+        x_f, w_f, b_f = _resolver(x_arg), _resolver(w_arg), _resolver(b_arg)
+
         def run(env):
-            x = _arg(env, x_arg)
+            x = x_f(env)
             n = x.shape[-1]
-            w, b = _arg(env, w_arg), _arg(env, b_arg)
+            w, b = w_f(env), b_f(env)
             gamma = cache.get(w, "ln", lambda t: t.float().contiguous()) if w is not None else \
                 cache.get(x.new_empty(0), f"ones{n}", lambda t: torch.ones(n, device=x.device))
             beta = cache.get(b, "ln", lambda t: t.float().contiguous()) if b is not None else \
@@ -183,8 +210,10 @@ class _Lowering:
         causal = bool(self._kwarg(node, "is_causal", 5, False))
         scale = self._kwarg(node, "scale", 6)
 
+        q_f, k_f, v_f = _resolver(q_arg), _resolver(k_arg), _resolver(v_arg)
+
         def run(env):
-            q, k, v = _arg(env, q_arg), _arg(env, k_arg), _arg(env, v_arg)
+            q, k, v = q_f(env), k_f(env), v_f(env)
             if q.dim() != 4:
                 raise ValueError("scaled_dot_product_attention expects [batch, heads, seq, head_dim] tensors")
             z, h, t, d = q.shape
@@ -204,8 +233,10 @@ class _Lowering:
         if self._kwarg(node, "alpha", 2, 1) != 1:
             raise ValueError(f"{node.name}: add with alpha is not supported")
 
+        a_f, b_f = _resolver(a_arg), _resolver(b_arg)
+
         def run(env):
-            a, b = _arg(env, a_arg), _arg(env, b_arg)
+            a, b = a_f(env), b_f(env)
             if not (isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor)):
                 return a + b  # Python scalars / sizes
             if a.shape != b.shape or a.dtype != b.dtype:
@@ -223,8 +254,10 @@ class _Lowering:
             self._emit(node.name, "fused", lambda env, src=src: env[src], into=src)
             return
 
+        x_f = _resolver(x_arg)
+
         def run(env):
-            x = _arg(env, x_arg)
+            x = x_f(env)
             x = x if x.is_contiguous() else x.contiguous()
             if kind == "gelu":
                 return ops.gelu_tanh(x)
@@ -240,15 +273,27 @@ class _Lowering:
             raise ValueError(f"no HIP kernel for graph node '{node.name}' ({what}); "
                              "pass allow_torch_fallback=True to run it with torch on the device")
         if node.op == "call_function":
-            fn = node.target
-            run = lambda env: fn(*_arg(env, node.args), **_arg(env, dict(node.kwargs)))  # noqa: E731
+            run = self._call(node.target, node.args, node.kwargs)
         elif node.op == "call_method":
-            run = lambda env: getattr(_arg(env, node.args[0]), node.target)(  # noqa: E731
-                *_arg(env, node.args[1:]), **_arg(env, dict(node.kwargs)))
+            run = self._method_call(node)
         else:
-            mod = self.gm.get_submodule(node.target)
-            run = lambda env: mod(*_arg(env, node.args), **_arg(env, dict(node.kwargs)))  # noqa: E731
+            run = self._call(self.gm.get_submodule(node.target), node.args, node.kwargs)
         self._emit(node.name, f"torch.{what}", run)
+
+    @staticmethod
+    def _call(fn, args, kwargs):
+        args_f, kwargs_f = _call_resolver(args, kwargs)
+        if kwargs_f is None:
+            return lambda env: fn(*args_f(env))
+        return lambda env: fn(*args_f(env), **kwargs_f(env))
+
+    @staticmethod
+    def _method_call(node):
+        self_f, method = _resolver(node.args[0]), node.target
+        args_f, kwargs_f = _call_resolver(node.args[1:], node.kwargs)
+        if kwargs_f is None:
+            return lambda env: getattr(self_f(env), method)(*args_f(env))
+        return lambda env: getattr(self_f(env), method)(*args_f(env), **kwargs_f(env))
 
     # -- dispatch ------------------------------------------------------------------------
     def lower(self) -> tuple[list[str], list[PlanStep], object]:
@@ -276,12 +321,10 @@ class _Lowering:
 
     def _meta(self, node):
         if node.op == "call_function":
-            fn = node.target
-            run = lambda env: fn(*_arg(env, node.args), **_arg(env, dict(node.kwargs)))  # noqa: E731
-            label = getattr(fn, "__name__", str(fn))
+            run = self._call(node.target, node.args, node.kwargs)
+            label = getattr(node.target, "__name__", str(node.target))
         else:
-            run = lambda env: getattr(_arg(env, node.args[0]), node.target)(  # noqa: E731
-                *_arg(env, node.args[1:]), **_arg(env, dict(node.kwargs)))
+            run = self._method_call(node)
             label = node.target
         self._emit(node.name, f"meta.{label}", run)
 
@@ -308,7 +351,7 @@ class _Lowering:
                 return self._fallback(node, f"softmax(dim={dim})")
             return self._unary(node, "softmax", node.args[0])
         if t is F.dropout and (self._kwarg(node, "p", 1, 0.5) == 0.0 or not self._kwarg(node, "training", 2, True)):
-            return self._emit(node.name, "meta.identity", lambda env: _arg(env, node.args[0]))
+            return self._emit(node.name, "meta.identity", _resolver(node.args[0]))
         if t in _METADATA_FUNCTIONS:
             return self._meta(node)
         return self._fallback(node, getattr(t, "__name__", str(t)))
@@ -339,9 +382,9 @@ class _Lowering:
         if isinstance(mod, torch.nn.GELU) and mod.approximate == "tanh":
             return self._unary(node, "gelu", x)
         if isinstance(mod, torch.nn.Dropout) and (mod.p == 0.0 or not mod.training):
-            return self._emit(node.name, "meta.identity", lambda env: _arg(env, x))
+            return self._emit(node.name, "meta.identity", _resolver(x))
         if isinstance(mod, torch.nn.Identity):
-            return self._emit(node.name, "meta.identity", lambda env: _arg(env, x))
+            return self._emit(node.name, "meta.identity", _resolver(x))
         return self._fallback(node, type(mod).__name__)
 
 
@@ -353,6 +396,7 @@ class JITFunction:
         self.placeholders = placeholders
         self.plan = plan
         self.output_spec = output_spec
+        self._output = _resolver(output_spec)
         self.device = device
         self.entry_func = entry_func
 
@@ -371,7 +415,7 @@ class JITFunction:
         with torch.no_grad():
             for step in self.plan:
                 env[step.name] = step.run(env)
-        out = _arg(env, self.output_spec)
+        out = self._output(env)
         return list(out) if isinstance(out, (tuple, list)) else [out]
 
     def benchmark(self, *args: torch.Tensor, nruns: int = 500, nwarmup: int = 500) -> np.ndarray:

@@ -15,7 +15,9 @@ from .utils.numpy import lh_dtype
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """Raw handle of torch's current stream on the current device (the accessor torch's own
+    extensions use: no Stream object is built per launch)."""
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
 
 
 def _need_cuda(*tensors) -> None:

@@ -77,8 +77,23 @@ def mlir_to_numpy_dtype(mlir_type: str) -> np.dtype:
     return _NAME_TO_NUMPY[mlir_type]
 
 
+_TORCH_LH_CACHE: dict = {}  # torch.dtype -> lh_dtype value (the per-launch path of the torch front end)
+
+
 def lh_dtype(dtype) -> int:
     """lh_dtype enum value for a numpy dtype / torch dtype / name."""
+    hit = _TORCH_LH_CACHE.get(dtype) if type(dtype).__module__ == "torch" else None
+    if hit is not None:
+        return hit
+    value = _lh_dtype_uncached(dtype)
+    # numpy dtypes are not cached: the narrow-float dtypes above compare (and hash) equal to the
+    # plain uint16 / uint8 they are built on.
+    if type(dtype).__module__ == "torch":
+        _TORCH_LH_CACHE[dtype] = value
+    return value
+
+
+def _lh_dtype_uncached(dtype) -> int:
     name = elem_name(dtype)
     if name not in _NAME_TO_LH:
         raise ValueError(f"Unsupported element type for the HIP target: {name}")
