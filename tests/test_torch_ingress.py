@@ -96,3 +96,17 @@ def test_fn_compile_hook_and_device_check():
     assert "hip.gemm" in seen
     with pytest.raises(AssertionError):
         gpu_backend(device="cpu")
+
+
+def test_argument_resolvers_follow_nested_structures():
+    """Arguments are resolved by functions built at lowering time: nodes inside tuples, lists,
+    dicts and slices are looked up in the environment, anything else is passed through as it is."""
+    from lighthouse_amd.ingress.torch.compile import _Ref, _resolver
+
+    env = {"a": 3, "b": 5}
+    a, b = _Ref("a"), _Ref("b")
+    assert _resolver(a)(env) == 3
+    assert _resolver((a, [b, 7], {"k": a}, slice(a, None, b)))(env) == (3, [5, 7], {"k": 3}, slice(3, None, 5))
+    const = (1, [2, 3], {"k": None}, slice(0, 4))
+    assert _resolver(const)(env) is const  # no node inside: returned without a walk
+    assert _resolver(None)(env) is None
