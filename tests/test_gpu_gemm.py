@@ -183,6 +183,45 @@ def test_gemm_tile_request_errors():
     ops.gemm(a, b, tile=(256, 128))
 
 
+@pytest.mark.parametrize("kind", ["bf16_bias_relu", "bf16_f32_acc", "f32", "fp8"])
+def test_gemm_row_strided_views(kind):
+    """Operands and output that are column ranges of wider buffers (lda, ldb, ldc larger than the
+    logical widths): results match the contiguous call and nothing outside the output view changes."""
+    from lighthouse_amd import ops
+
+    M, N, K = (2048, 4096, 128) if kind == "fp8" else (512, 768, 256)
+    pad = 64
+    g = torch.Generator(device="cuda").manual_seed(31)
+    if kind == "fp8":
+        dt, odt = torch.float8_e4m3fn, torch.bfloat16
+    elif kind == "f32":
+        dt, odt = torch.float32, torch.float32
+    else:
+        dt, odt = torch.bfloat16, torch.float32 if kind == "bf16_f32_acc" else torch.bfloat16
+    wide_a = torch.randn(M, K + 2 * pad, device="cuda", generator=g).clamp(-4, 4).to(dt)
+    wide_b = torch.randn(K, N + 2 * pad, device="cuda", generator=g).clamp(-4, 4).to(dt)
+    a, b = wide_a[:, pad:pad + K], wide_b[:, pad:pad + N]
+    wide_o = torch.full((M, N + 2 * pad), 7.0, device="cuda").to(odt)
+    out = wide_o[:, pad:pad + N]
+    assert not a.is_contiguous() and not out.is_contiguous()
+    if kind == "fp8":
+        ops.gemm_fp8(a, b, 0.5, 0.25, out=out)
+        ref = ops.gemm_fp8(a.contiguous(), b.contiguous(), 0.5, 0.25)
+    elif kind == "bf16_f32_acc":
+        bias = torch.randn(N, device="cuda", generator=g)
+        c = torch.randn(M, N, device="cuda", generator=g)
+        out.copy_(c)
+        ops.gemm(a, b, bias, out=out, accumulate_c=True)
+        ref = c.clone()
+        ops.gemm(a.contiguous(), b.contiguous(), bias, out=ref, accumulate_c=True)
+    else:
+        bias = torch.randn(N, device="cuda", generator=g).to(odt)
+        ops.gemm(a, b, bias, relu=True, out=out)
+        ref = ops.gemm(a.contiguous(), b.contiguous(), bias, relu=True)
+    assert torch.equal(out.contiguous(), ref)
+    assert torch.all(wide_o[:, :pad].float() == 7.0) and torch.all(wide_o[:, pad + N:].float() == 7.0)
+
+
 @pytest.mark.parametrize("ta,tb", [(True, False), (False, True), (True, True)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_gemm_transposed(dtype, ta, tb):
