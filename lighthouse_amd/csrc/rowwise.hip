@@ -129,14 +129,6 @@ __global__ void __launch_bounds__(256) softmax_rows(void* out, const void* x, in
   for (int j = lane; j < N; j += 64) store_from_f32<DT>(out, base + j, expf(load_as_f32<DT>(x, base + j) - mx) / s);
 }
 
-// tanh-GELU as x / (1 + exp(-2u)), u = sqrt(2/pi) (x + 0.044715 x^3): identical to
-// 0.5 x (1 + tanh u) but without the cancellation of 1 + tanh(u) in the negative tail.
-__device__ __forceinline__ float gelu_tanh_ref(float x) {
-  const float k = 0.7978845608028654f;
-  float u = k * (x + 0.044715f * x * x * x);
-  return x / (1.0f + expf(-2.0f * u));
-}
-
 enum { EW_GELU = 0, EW_ADD = 1, EW_BIAS = 2, EW_BIAS_RELU = 3 };
 
 // n4 groups of 4 elements; `N` is the row length for the bias kinds.
@@ -148,7 +140,7 @@ __global__ void __launch_bounds__(256) elementwise4(void* out, const void* a, co
     f32x4 o;
     if constexpr (KIND == EW_GELU) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = gelu_tanh_ref(x[e]);
+      for (int e = 0; e < 4; ++e) o[e] = gelu_tanh(x[e]);
     } else if constexpr (KIND == EW_ADD) {
       f32x4 y = load4<DT>(b, i * 4);
 #pragma unroll
@@ -170,7 +162,7 @@ __global__ void __launch_bounds__(256) elementwise1(void* out, const void* a, co
   const int64_t stride = (int64_t)gridDim.x * 256;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
     float x = load_as_f32<DT>(a, i), o;
-    if constexpr (KIND == EW_GELU) o = gelu_tanh_ref(x);
+    if constexpr (KIND == EW_GELU) o = gelu_tanh(x);
     else if constexpr (KIND == EW_ADD) o = x + load_as_f32<DT>(b, i);
     else {
       o = x + load_as_f32<DT>(b, i % N);
