@@ -113,6 +113,40 @@ __global__ void __launch_bounds__(256) layer_norm_generic(void* out, const void*
     store_from_f32<ODT>(out, base + j, (load_as_f32<XDT>(x, base + j) - mean) * inv_std * gamma[j] + beta[j]);
 }
 
+// Row softmax with the row resident in registers (N = 256 VPL): one read and one write per
+// element, one exp per element.
+template <int DT, int VPL>
+__global__ void __launch_bounds__(256) softmax_rows_vec(void* out, const void* x, int M, int N) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= M) return;
+  const int64_t base = (int64_t)row * N;
+  f32x4 v[VPL];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    v[i] = load4<DT>(x, base + (i * 64 + lane) * 4);
+    mx = fmaxf(fmaxf(mx, fmaxf(v[i][0], v[i][1])), fmaxf(v[i][2], v[i][3]));
+  }
+  mx = wave_max(mx);
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < VPL; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[i][e] = expf(v[i][e] - mx);
+      s += v[i][e];
+    }
+  s = wave_sum(s);
+#pragma unroll
+  for (int i = 0; i < VPL; ++i) {
+    f32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = v[i][e] / s;
+    store4<DT>(out, base + (i * 64 + lane) * 4, o);
+  }
+}
+
 // Row softmax (lighthouse/ingress/mlir_gen/gpu_softmax_payload.py:46-55), one wave per row.
 template <int DT>
 __global__ void __launch_bounds__(256) softmax_rows(void* out, const void* x, int M, int N) {
@@ -265,6 +299,23 @@ int lh_hip_softmax(void* out, const void* x, int64_t M, int64_t N, int32_t dtype
   LH_REQUIRE(M > 0 && N > 0 && M < (1ll << 31) && N < (1ll << 31), "lh_hip_softmax: bad shape");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   dim3 grid((unsigned)((M + 3) / 4)), block(256);
+  if (N % 256 == 0 && N <= 4096 && aligned16(out) && aligned16(x)) {
+#define LH_SM_CASE(DT, V)                                                                            \
+  case V:                                                                                            \
+    hipLaunchKernelGGL((softmax_rows_vec<DT, V>), grid, block, 0, s, out, x, (int)M, (int)N);        \
+    return check_launch("softmax_rows_vec");
+#define LH_SM_DTYPE(DT)                                                                              \
+  switch (N / 256) {                                                                                 \
+    LH_SM_CASE(DT, 1) LH_SM_CASE(DT, 2) LH_SM_CASE(DT, 3) LH_SM_CASE(DT, 4) LH_SM_CASE(DT, 6)        \
+    LH_SM_CASE(DT, 8) LH_SM_CASE(DT, 12) LH_SM_CASE(DT, 16)                                          \
+    default: break;                                                                                  \
+  }
+    if (dtype == LH_F32) { LH_SM_DTYPE(LH_F32) }
+    else if (dtype == LH_BF16) { LH_SM_DTYPE(LH_BF16) }
+    else if (dtype == LH_F16) { LH_SM_DTYPE(LH_F16) }
+#undef LH_SM_DTYPE
+#undef LH_SM_CASE
+  }
   switch (dtype) {
     case LH_F32: hipLaunchKernelGGL(softmax_rows<LH_F32>, grid, block, 0, s, out, x, (int)M, (int)N); break;
     case LH_BF16: hipLaunchKernelGGL(softmax_rows<LH_BF16>, grid, block, 0, s, out, x, (int)M, (int)N); break;

@@ -61,7 +61,7 @@ def test_layer_norm_special_cases():
     assert (y.var(1, unbiased=False) - 1).abs().max() < 1e-3
 
 
-@pytest.mark.parametrize("shape", [(64, 1024), (5, 77), (128, 4096)])
+@pytest.mark.parametrize("shape", [(64, 1024), (5, 77), (128, 4096), (33, 768), (16, 8192), (7, 260)])
 def test_softmax(shape):
     from lighthouse_amd import ops
 
