@@ -341,10 +341,32 @@ def test_gemm_fp8_all_codes():
     np.testing.assert_array_equal(_host(out), ref.astype(np.float32))
 
 
-@pytest.mark.parametrize("shape", [(16, 1024, 8192), (7, 384, 4096), (1, 128, 2048), (16, 2048, 384)])
+def test_gemm_fp8_8192_properties():
+    """The benchmark's 8192^3 problem (four tiles per persistent workgroup): sampled rows against
+    the oracle, and with B the identity the output is exactly the scaled, bf16-rounded A."""
+    from lighthouse_amd import ops
+
+    n = 8192
+    g = torch.Generator(device="cuda").manual_seed(13)
+    a = torch.randn(n, n, device="cuda", generator=g).clamp(-4, 4).to(torch.float8_e4m3fn)
+    b = torch.randn(n, n, device="cuda", generator=g).clamp(-4, 4).to(torch.float8_e4m3fn)
+    out = ops.gemm_fp8(a, b, 0.5, 0.25)
+    rows = [0, 1, 255, 256, 4095, 4096, 8190, 8191]
+    a_codes = a.view(torch.uint8)[rows].cpu().numpy()
+    b_codes = b.view(torch.uint8).cpu().numpy()
+    ref = orc.matmul_fp8(a_codes, b_codes, 0.5, 0.25)
+    assert_close(_host(out[rows]), ref, FP8_RTOL, "fp8 8192^3 sampled rows")
+    eye = torch.eye(n, device="cuda").to(torch.float8_e4m3fn)
+    out_id = ops.gemm_fp8(a, eye, 0.5, 0.25)
+    expect = (a.float() * 0.125).to(torch.bfloat16)
+    assert torch.equal(out_id, expect)
+
+
+@pytest.mark.parametrize("shape", [(16, 1024, 8192), (7, 384, 4096), (1, 128, 2048), (16, 2048, 384),
+                                   (16, 8192, 8192)])  # the last: the benchmark's decode configuration
 def test_gemm_fp8_decode_path(shape):
-    """M <= 16: split-K streaming kernel with the reduction fused into the last workgroup; called
-    three times in a row (the per-column-block counters must return to zero) and with an f32 output."""
+    """M <= 16: split-K streaming kernel plus the reduction kernel; called three times in a row
+    (the library's partial-sum buffer is reused) and with an f32 output."""
     from lighthouse_amd import ops
 
     M, N, K = shape
