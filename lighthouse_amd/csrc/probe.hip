@@ -65,7 +65,7 @@ extern "C" int lh_hip_probe_mfma_rate(int32_t dtype, int32_t random_operands, in
   const size_t nfrag = 8 * 512;
   std::vector<uint32_t> host(nfrag * 4, 0u);
   if (random_operands) {
-    // Values of magnitude around 1 with random signs and mantissas (what N(0,1) inputs look like
+    // Values of magnitude close to 1 with random signs and mantissas (what N(0,1) inputs look like
     // to the multiplier arrays), from a fixed linear congruential sequence.
     uint64_t state = 0x9E3779B97F4A7C15ull;
     auto next = [&]() {
