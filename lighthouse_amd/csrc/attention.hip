@@ -79,30 +79,41 @@ struct AttnCtx {
   const uint16_t* k_src[2];  // lane's source of K load i at key 0
   const uint16_t* v_src[2];
   int64_t k_step, v_step;    // elements per key tile
+  int64_t k_row, v_row;      // elements per key (row strides), for the clamped loads of a partial tile
+  int key_local[2];          // the key of the tile that load i of this lane fetches
   int wave, r32, h;
   int k_off[2], k_swz[2];    // K fragment: byte offset of the lane's row, its swizzle, per key sub-tile
   int v_off, v_swz;          // V fragment through the transposing read
 };
 
-__device__ __forceinline__ void attn_issue_loads(const AttnCtx& c, int jt, uint8_t* __restrict__ stage) {
+// RAGGED (sequence length T no multiple of the key tile): keys of the last, partial tile that lie
+// past the end are fetched from the last key instead (and masked by the consumer).  Branch-free,
+// and a template parameter, so that the loads of the common case stay one addition each.
+template <bool RAGGED>
+__device__ __forceinline__ void attn_issue_loads(const AttnCtx& c, int jt, int T, uint8_t* __restrict__ stage) {
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    __builtin_amdgcn_global_load_lds(c.k_src[i] + jt * c.k_step, (attn_lds_void_t*)(stage + (4 * i + c.wave) * 1024),
-                                     16, 0, 0);
-    __builtin_amdgcn_global_load_lds(c.v_src[i] + jt * c.v_step,
-                                     (attn_lds_void_t*)(stage + 8192 + (4 * i + c.wave) * 1024), 16, 0, 0);
+    int64_t k_off = jt * c.k_step, v_off = jt * c.v_step;
+    if constexpr (RAGGED) {
+      const int back = max(jt * kKvTile + c.key_local[i] - (T - 1), 0);  // keys past the last one
+      k_off -= back * c.k_row;
+      v_off -= back * c.v_row;
+    }
+    __builtin_amdgcn_global_load_lds(c.k_src[i] + k_off, (attn_lds_void_t*)(stage + (4 * i + c.wave) * 1024), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds(c.v_src[i] + v_off, (attn_lds_void_t*)(stage + 8192 + (4 * i + c.wave) * 1024), 16,
+                                     0, 0);
   }
 }
 
 // One key tile (64 keys) for the wave's two 32-row query sub-tiles.  `rd` holds the tile, `wr`
 // is the ring slot that receives a later tile meanwhile (separate restrict pointers so that LDS
 // reads do not wait for the asynchronous writes).
-template <int DT, int NQ>
+template <int DT, int NQ, bool RAGGED>
 __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, const u32x4 (&qf)[NQ][4],
                                           f32x16 (&acc_o)[NQ][2], float (&m_run)[NQ], float (&l_run)[NQ],
                                           const uint8_t* __restrict__ rd, uint8_t* __restrict__ wr, int next_jt,
                                           bool prefetch, int j0, int wq0, bool active, bool need_mask) {
-  if (prefetch) attn_issue_loads(c, next_jt, wr);
+  if (prefetch) attn_issue_loads<RAGGED>(c, next_jt, a.T, wr);
   if (!active) return;
   const uint8_t* ks = rd;
   const uint8_t* vs = rd + 8192;
@@ -127,13 +138,14 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt) {
     if (need_mask) {
-      const int qrow = wq0 + 32 * qt + c.r32;
+      // last visible key of the row: its own index under the causal mask, and never past the end
+      const int last = a.causal ? min(wq0 + 32 * qt + c.r32, a.T - 1) : a.T - 1;
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           int key = j0 + 32 * i + 8 * (v >> 2) + 4 * c.h + (v & 3);
-          if (key > qrow) s_acc[qt][i][v] = -INFINITY;
+          if (key > last) s_acc[qt][i][v] = -INFINITY;
         }
     }
     // Lazy offset: P = exp(S - offset) is first computed with the offset already in use.  Softmax
@@ -225,7 +237,7 @@ __device__ __forceinline__ void causal_block_of(int L, int G, int R, int nqb, in
 // reads, V^T fragments come from ds_read_b64_tr_b16 on the row-major V tile.  Rows of a tile
 // are 128 bytes and cannot be padded (a wave-wide load writes 1 KiB contiguous), so the
 // 16-byte chunk a lane fetches is XOR-swizzled: K chunk ^ ((key / 2) % 8), V chunk ^ 4 ((key / 2) % 2).
-template <int DT, int NQ, int NS>
+template <int DT, int NQ, int NS, bool RAGGED>
 __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
   constexpr int kRowsPerWave = 32 * NQ, kRowsPerGroup = 4 * kRowsPerWave;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn[];
@@ -243,8 +255,8 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
   const int z = bh / a.H, hd = bh % a.H;
   const int q0 = qb * kRowsPerGroup;
   const int wq0 = q0 + wave * kRowsPerWave;
-  // T is a multiple of 64: a wave's rows are all inside the sequence or all outside (last
-  // workgroup only); an outside wave still takes part in the loads and barriers.
+  // A wave whose rows all lie past the end (last workgroup only) still takes part in the loads
+  // and barriers; rows past the end inside a valid wave compute on the last row and are not stored.
   const bool wave_valid = wq0 < a.T;
   const int wq_load = wave_valid ? wq0 : 0;
 
@@ -257,12 +269,15 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
   c.wave = wave; c.r32 = r32; c.h = h;
   c.k_step = (int64_t)kKvTile * a.sk.t;
   c.v_step = (int64_t)kKvTile * a.sv.t;
+  c.k_row = a.sk.t;
+  c.v_row = a.sv.t;
   // Loader: load i of wave w fills keys (4 i + w) 8 .. +8 of the tile; lane -> key += lane / 8,
   // LDS chunk p = lane % 8 holds global chunk p ^ swizzle(key).
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int key = (4 * i + wave) * 8 + (lane >> 3);
     const int p = lane & 7;
+    c.key_local[i] = key;
     c.k_src[i] = K + (int64_t)key * a.sk.t + ((p ^ ((key >> 1) & 7)) << 3);
     c.v_src[i] = V + (int64_t)key * a.sv.t + ((p ^ (4 * ((key >> 1) & 1))) << 3);
   }
@@ -291,8 +306,10 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt)
 #pragma unroll
-    for (int sd = 0; sd < 4; ++sd)
-      qf[qt][sd] = *reinterpret_cast<const u32x4*>(Q + (int64_t)(wq_load + 32 * qt + r32) * a.sq.t + 16 * sd + 8 * h);
+    for (int sd = 0; sd < 4; ++sd) {
+      const int row = RAGGED ? min(wq_load + 32 * qt + r32, a.T - 1) : wq_load + 32 * qt + r32;
+      qf[qt][sd] = *reinterpret_cast<const u32x4*>(Q + (int64_t)row * a.sq.t + 16 * sd + 8 * h);
+    }
 
   f32x16 acc_o[NQ][2];
 #pragma unroll
@@ -313,7 +330,7 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
   constexpr int kAttnStages = NS;  // K/V ring depth, 3 or 4
 #pragma unroll
   for (int st = 0; st < kAttnStages - 1; ++st)
-    if (st < ntiles) attn_issue_loads(c, st, smem_attn + st * kAttnStageBytes);
+    if (st < ntiles) attn_issue_loads<RAGGED>(c, st, a.T, smem_attn + st * kAttnStageBytes);
 
   for (int jt = 0; jt < ntiles; ++jt) {
     // 4 loads per lane and stage; the NS - 2 younger stages may stay in flight.  One asm block: a
@@ -324,9 +341,9 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
     else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     const int j0 = jt * kKvTile;
     const bool active = wave_valid && (!a.causal || (j0 <= wq0 + kRowsPerWave - 1));
-    const bool need_mask = a.causal && (j0 + kKvTile - 1 > wq0);
+    const bool need_mask = (a.causal && (j0 + kKvTile - 1 > wq0)) || (RAGGED && j0 + kKvTile > a.T);
     const int nxt = jt + kAttnStages - 1;
-    attn_tile<DT, NQ>(c, a, qf, acc_o, m_run, l_run, smem_attn + (jt % kAttnStages) * kAttnStageBytes,
+    attn_tile<DT, NQ, RAGGED>(c, a, qf, acc_o, m_run, l_run, smem_attn + (jt % kAttnStages) * kAttnStageBytes,
                   smem_attn + (nxt % kAttnStages) * kAttnStageBytes, nxt, nxt < ntiles, j0, wq0, active, need_mask);
   }
 
@@ -335,6 +352,7 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt) {
     const float inv_l = 1.0f / halfwave_sum(l_run[qt]);
+    if (RAGGED && wq0 + 32 * qt + r32 >= a.T) continue;  // (after the cross-lane sum, which needs every lane)
     uint16_t* orow = O + (int64_t)(wq0 + 32 * qt + r32) * a.so.t;
 #pragma unroll
     for (int j = 0; j < 2; ++j)
@@ -532,9 +550,9 @@ __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
     }
 }
 
-template <int DT, int NQ, int NS>
-static int attention16_launch_nq(const AttnArgs& a, hipStream_t s) {
-  auto kern = attention16_kernel<DT, NQ, NS>;
+template <int DT, int NQ, int NS, bool RAGGED>
+static int attention16_launch_ragged(const AttnArgs& a, hipStream_t s) {
+  auto kern = attention16_kernel<DT, NQ, NS, RAGGED>;
   constexpr size_t lds = (size_t)NS * kAttnStageBytes;
   static bool configured = false;
   if (!configured) {
@@ -546,6 +564,14 @@ static int attention16_launch_nq(const AttnArgs& a, hipStream_t s) {
   const dim3 grid = a.causal ? dim3(nqb * a.Z * a.H) : dim3(nqb, a.Z * a.H);
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, a);
   return check_launch("attention16");
+}
+
+// Sequence lengths that are no multiple of the key tile take the instantiation that clamps the
+// last tile's loads, masks it and skips rows past the end.
+template <int DT, int NQ, int NS>
+static int attention16_launch_nq(const AttnArgs& a, hipStream_t s) {
+  if (a.T % kKvTile != 0) return attention16_launch_ragged<DT, NQ, NS, true>(a, s);
+  return attention16_launch_ragged<DT, NQ, NS, false>(a, s);
 }
 
 // 64 query rows per wave share every K/V fragment between two sub-tiles; 32 rows per wave give
@@ -670,11 +696,12 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   const lh_strides3* ss[4] = {&so, &sq, &sk, &sv};
   const void* ps[4] = {out, q, k, v};
   for (int i = 0; i < 4; ++i) LH_REQUIRE(ss[i]->t >= d, "lh_hip_attention: row stride of tensor %d is below head_dim", i);
-  // The MFMA kernels need head_dim 64, whole query blocks and 16-byte aligned rows; every other
-  // problem runs on the generic kernel.
+  // The MFMA kernels need head_dim 64 and 16-byte aligned rows (the f32 one also whole query
+  // blocks); every other problem runs on the generic kernel.
   const int qblock = (dtype == LH_F32) ? kQBlock : kKvTile;
   const int vec = (dtype == LH_F32) ? 4 : 8;  // elements per 16-byte access
-  bool fast = d == kHeadDim && T % qblock == 0;
+  // (the 16-bit kernels mask a partial last key tile and skip rows past the end themselves)
+  bool fast = d == kHeadDim && (dtype != LH_F32 || T % qblock == 0);
   for (int i = 0; i < 4 && fast; ++i)
     fast = ss[i]->t % vec == 0 && ss[i]->h % vec == 0 && ss[i]->z % vec == 0 && aligned16(ps[i]);
   if (scale <= 0.0f) scale = 1.0f / sqrtf((float)d);

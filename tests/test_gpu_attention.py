@@ -156,8 +156,8 @@ def test_attention_scores_outgrow_the_offset(shape, dtype, elt, causal):
 @pytest.mark.parametrize("shape", [(1, 2, 100, 32), (2, 1, 77, 64), (1, 1, 130, 128), (1, 3, 64, 64), (1, 1, 1, 8),
                                    (1, 1, 200, 256)])
 def test_attention_any_shape(shape, dtype, elt, rtol, causal):
-    """Sequence lengths and head dimensions the MFMA kernels do not take (and f32 with T % 128 != 0)
-    run on the generic kernel with the same rounding points."""
+    """Head dimensions the MFMA kernels do not take (and f32 with T % 128 != 0) run on the generic
+    kernel with the same rounding points."""
     from lighthouse_amd import ops
 
     rng = np.random.default_rng(sum(shape) + causal)
@@ -165,6 +165,29 @@ def test_attention_any_shape(shape, dtype, elt, rtol, causal):
     out = ops.attention(_dev(q, dtype), _dev(k, dtype), _dev(v, dtype), causal=causal)
     ref = orc.attention(q, k, v, causal=causal, result_type=elt)
     assert_close(_host(out), ref, rtol, f"generic attention {shape} {elt} causal={causal}")
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype,elt", [(torch.bfloat16, "bf16"), (torch.float16, "f16")])
+@pytest.mark.parametrize("shape", [(1, 2, 65, 64), (2, 3, 1000, 64), (1, 1, 300, 64), (1, 2, 63, 64), (1, 1, 1, 64),
+                                   (12, 20, 449, 64)])
+def test_attention_ragged_sequence_16bit(shape, dtype, elt, causal):
+    """head_dim 64 with a sequence length that is no multiple of the key tile: the MFMA kernels mask
+    the partial last key tile and skip rows past the end (the last shape has more than two 256-row
+    groups per CU, i.e. the 64-rows-per-wave instantiation); nothing past the end is written."""
+    from lighthouse_amd import ops
+
+    Z, H, T, d = shape
+    rng = np.random.default_rng(sum(shape) + 3 * causal)
+    q, k, v = (orc.round_to(rng.standard_normal(shape).astype(np.float32), elt) for _ in range(3))
+    # outputs live in a longer buffer whose tail must stay untouched
+    buf = torch.full((Z, H, T + 70, d), 5.0, device="cuda").to(dtype)
+    out = buf[:, :, :T]
+    ops.attention(_dev(q, dtype), _dev(k, dtype), _dev(v, dtype), causal=causal, out=out)
+    assert torch.all(buf[:, :, T:].float() == 5.0)
+    for z, h in {(0, 0), (Z - 1, H - 1)}:
+        ref = orc.attention(q[z, h], k[z, h], v[z, h], causal=causal, result_type=elt)
+        assert_close(_host(out[z, h]), ref, 2e-2, f"ragged attention {shape} {elt} z={z} h={h} causal={causal}")
 
 
 def test_attention_errors():
