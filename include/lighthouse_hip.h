@@ -138,7 +138,7 @@ int lh_hip_gemm_fp8(void* out, const void* a_q, const void* b_q, float scale_a, 
  * (sz, sh, st) per tensor and unit stride along d, so (T, H*d) projection buffers can be
  * passed as strided views without a copy (examples/xegpu/nanoGPT_payload.py:198-217).
  * dtype in {BF16, F16, F32}; d <= 256.  The matrix-core kernels take d = 64 with 16-byte aligned
- * rows (16-bit: any T; f32: T a multiple of 128); every other problem runs on a generic kernel.
+ * rows at any T; every other problem runs on a generic kernel.
  */
 typedef struct lh_strides3 {
   int64_t z, h, t;

@@ -377,6 +377,8 @@ struct Attn32Ctx {
   const float* k_src[4];
   const float* v_src[4];
   int64_t k_step, v_step;
+  int64_t k_row, v_row;  // elements per key, for the clamped loads of a partial last tile
+  int key_local[4];      // the key of the tile that load i of this lane fetches
   int wave, r32, h;
   int k_off[2], k_swz[2];
   int v_col[2];  // byte offset of the lane's V column inside a row, per head-dim sub-tile (unswizzled half)
@@ -386,20 +388,29 @@ __device__ __forceinline__ void attn32_copy16(const float* gsrc, uint8_t* lds_wa
   __builtin_amdgcn_global_load_lds(gsrc, (attn_lds_void_t*)lds_wave_base, 16, 0, 0);
 }
 
-__device__ __forceinline__ void attn32_issue(const Attn32Ctx& c, int jt, uint8_t* __restrict__ stage) {
+// RAGGED: as in the 16-bit kernel, keys past the end of the sequence are fetched from the last key.
+template <bool RAGGED>
+__device__ __forceinline__ void attn32_issue(const Attn32Ctx& c, int jt, int T, uint8_t* __restrict__ stage) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    attn32_copy16(c.k_src[i] + jt * c.k_step, stage + (4 * i + c.wave) * 1024);
-    attn32_copy16(c.v_src[i] + jt * c.v_step, stage + 16384 + (4 * i + c.wave) * 1024);
+    int64_t k_off = jt * c.k_step, v_off = jt * c.v_step;
+    if constexpr (RAGGED) {
+      const int back = max(jt * kKvTile + c.key_local[i] - (T - 1), 0);
+      k_off -= back * c.k_row;
+      v_off -= back * c.v_row;
+    }
+    attn32_copy16(c.k_src[i] + k_off, stage + (4 * i + c.wave) * 1024);
+    attn32_copy16(c.v_src[i] + v_off, stage + 16384 + (4 * i + c.wave) * 1024);
   }
 }
 
 // One key tile for the wave's 32 query rows; `wr` receives the next tile meanwhile.
+template <bool RAGGED>
 __device__ __forceinline__ void attn32_tile(const Attn32Ctx& c, const AttnArgs& a, const f32x4 (&qf)[8],
                                             f32x16 (&acc_o)[2], float& m_run, float& l_run,
                                             const uint8_t* __restrict__ rd, uint8_t* __restrict__ wr, int next_jt,
                                             bool prefetch, int j0, int wq0, bool active, bool need_mask) {
-  if (prefetch) attn32_issue(c, next_jt, wr);
+  if (prefetch) attn32_issue<RAGGED>(c, next_jt, a.T, wr);
   if (!active) return;
   const uint8_t* ks = rd;
   const uint8_t* vs = rd + 16384;
@@ -423,13 +434,14 @@ __device__ __forceinline__ void attn32_tile(const Attn32Ctx& c, const AttnArgs& 
   }
   // s_acc[i][v] = S[q = wq0 + r32][key = j0 + 32 i + 8 (v/4) + 4 h + v%4] (unscaled)
   if (need_mask) {
-    const int qrow = wq0 + c.r32;
+    // last visible key of the row: its own index under the causal mask, and never past the end
+    const int last = a.causal ? min(wq0 + c.r32, a.T - 1) : a.T - 1;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         int key = j0 + 32 * i + 8 * (v >> 2) + 4 * c.h + (v & 3);
-        if (key > qrow) s_acc[i][v] = -INFINITY;
+        if (key > last) s_acc[i][v] = -INFINITY;
       }
   }
   float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
@@ -470,17 +482,22 @@ __device__ __forceinline__ void attn32_tile(const Attn32Ctx& c, const AttnArgs& 
     }
 }
 
+// RAGGED: T is no multiple of the 128-row query block; the last key tile may be partial, rows past
+// the end compute on the last row and are not stored, and a wave entirely past the end only takes
+// part in the loads and barriers.
+template <bool RAGGED>
 __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn32[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, h = lane >> 5;
-  const int nqb = a.T / kQBlock;
+  const int nqb = (a.T + kQBlock - 1) / kQBlock;
   int qb = blockIdx.x, bh = blockIdx.y;
   if (a.causal) causal_block_of(blockIdx.x, gridDim.x, a.cus, nqb, a.Z * a.H, qb, bh);
   const int z = bh / a.H, hd = bh % a.H;
   const int q0 = qb * kQBlock;
   const int wq0 = q0 + wave * 32;
+  const bool wave_valid = !RAGGED || wq0 < a.T;
   const float* Q = reinterpret_cast<const float*>(a.q) + (int64_t)z * a.sq.z + (int64_t)hd * a.sq.h;
   const float* K = reinterpret_cast<const float*>(a.k) + (int64_t)z * a.sk.z + (int64_t)hd * a.sk.h;
   const float* V = reinterpret_cast<const float*>(a.v) + (int64_t)z * a.sv.z + (int64_t)hd * a.sv.h;
@@ -490,12 +507,15 @@ __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
   c.wave = wave; c.r32 = r32; c.h = h;
   c.k_step = (int64_t)kKvTile * a.sk.t;
   c.v_step = (int64_t)kKvTile * a.sv.t;
+  c.k_row = a.sk.t;
+  c.v_row = a.sv.t;
   // Loader: load i of wave w fills keys (4 i + w) 4 .. +4; lane -> key += lane / 16, LDS chunk
   // p = lane % 16 holds global chunk p ^ swizzle(key).
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int key = (4 * i + wave) * 4 + (lane >> 4);
     const int p = lane & 15;
+    c.key_local[i] = key;
     c.k_src[i] = K + (int64_t)key * a.sk.t + ((p ^ (key & 15)) << 2);
     c.v_src[i] = V + (int64_t)key * a.sv.t + ((p ^ (8 * ((key >> 2) & 1))) << 2);
   }
@@ -515,7 +535,8 @@ __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
   f32x4 qf[8];
 #pragma unroll
   for (int kk = 0; kk < 8; ++kk)
-    qf[kk] = *reinterpret_cast<const f32x4*>(Q + (int64_t)(wq0 + r32) * a.sq.t + 8 * kk + 4 * h);
+    qf[kk] = *reinterpret_cast<const f32x4*>(Q + (int64_t)(RAGGED ? min(wq0 + r32, a.T - 1) : wq0 + r32) * a.sq.t +
+                                             8 * kk + 4 * h);
 
   f32x16 acc_o[2];
 #pragma unroll
@@ -526,19 +547,21 @@ __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
   const int kv_end = a.causal ? min(a.T, q0 + kQBlock) : a.T;
   const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
 
-  attn32_issue(c, 0, smem_attn32);
+  attn32_issue<RAGGED>(c, 0, a.T, smem_attn32);
   for (int jt = 0; jt < ntiles; ++jt) {
     // Tile jt is the only load in flight: wait for it, and the barrier also says every wave is
     // done reading the stage the next tile is about to overwrite.
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     const int j0 = jt * kKvTile;
-    const bool active = !a.causal || (j0 <= wq0 + 31);
-    const bool need_mask = a.causal && (j0 + kKvTile - 1 > wq0);
-    attn32_tile(c, a, qf, acc_o, m_run, l_run, smem_attn32 + (jt & 1) * kAttn32StageBytes,
+    const bool active = wave_valid && (!a.causal || (j0 <= wq0 + 31));
+    const bool need_mask = (a.causal && (j0 + kKvTile - 1 > wq0)) || (RAGGED && j0 + kKvTile > a.T);
+    attn32_tile<RAGGED>(c, a, qf, acc_o, m_run, l_run, smem_attn32 + (jt & 1) * kAttn32StageBytes,
                 smem_attn32 + ((jt + 1) & 1) * kAttn32StageBytes, jt + 1, jt + 1 < ntiles, j0, wq0, active, need_mask);
   }
 
+  if (!wave_valid) return;
   const float inv_l = 1.0f / halfwave_sum(l_run);
+  if (RAGGED && wq0 + r32 >= a.T) return;  // (after the cross-lane sum, which needs every lane)
   float* orow = O + (int64_t)(wq0 + r32) * a.so.t;
 #pragma unroll
   for (int j = 0; j < 2; ++j)
@@ -667,15 +690,21 @@ int attention_generic_launch(const AttnArgs& a, int d, int dtype, hipStream_t s)
 int attention_launch(const AttnArgs& a, int dtype, hipStream_t s) {
   if (dtype == LH_BF16) return attention16_launch<LH_BF16>(a, s);
   if (dtype == LH_F16) return attention16_launch<LH_F16>(a, s);
-  static bool configured32 = false;
-  if (!configured32) {
-    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention32_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, 2 * kAttn32StageBytes));
-    configured32 = true;
-  }
-  const int nqb32 = a.T / kQBlock;
+  const int nqb32 = (a.T + kQBlock - 1) / kQBlock;
   const dim3 grid32 = a.causal ? dim3(nqb32 * a.Z * a.H) : dim3(nqb32, a.Z * a.H);
-  hipLaunchKernelGGL(attention32_kernel, grid32, dim3(256), 2 * kAttn32StageBytes, s, a);
+  auto launch = [&](auto kern, bool& configured) -> int {
+    if (!configured) {
+      LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       2 * kAttn32StageBytes));
+      configured = true;
+    }
+    hipLaunchKernelGGL(kern, grid32, dim3(256), 2 * kAttn32StageBytes, s, a);
+    return 0;
+  };
+  static bool configured_whole = false, configured_ragged = false;
+  const int rc = a.T % kQBlock == 0 ? launch(attention32_kernel<false>, configured_whole)
+                                    : launch(attention32_kernel<true>, configured_ragged);
+  if (rc) return rc;
   return check_launch("attention32");
 }
 
@@ -696,12 +725,11 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   const lh_strides3* ss[4] = {&so, &sq, &sk, &sv};
   const void* ps[4] = {out, q, k, v};
   for (int i = 0; i < 4; ++i) LH_REQUIRE(ss[i]->t >= d, "lh_hip_attention: row stride of tensor %d is below head_dim", i);
-  // The MFMA kernels need head_dim 64 and 16-byte aligned rows (the f32 one also whole query
-  // blocks); every other problem runs on the generic kernel.
-  const int qblock = (dtype == LH_F32) ? kQBlock : kKvTile;
+  // The MFMA kernels need head_dim 64 and 16-byte aligned rows; every other problem runs on the
+  // generic kernel.
   const int vec = (dtype == LH_F32) ? 4 : 8;  // elements per 16-byte access
-  // (the 16-bit kernels mask a partial last key tile and skip rows past the end themselves)
-  bool fast = d == kHeadDim && (dtype != LH_F32 || T % qblock == 0);
+  // (the kernels mask a partial last key tile and skip rows past the end themselves)
+  bool fast = d == kHeadDim;
   for (int i = 0; i < 4 && fast; ++i)
     fast = ss[i]->t % vec == 0 && ss[i]->h % vec == 0 && ss[i]->z % vec == 0 && aligned16(ps[i]);
   if (scale <= 0.0f) scale = 1.0f / sqrtf((float)d);
