@@ -107,13 +107,16 @@ __device__ __forceinline__ void direct32_wait_barrier() {
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-// Source pointers of tile `id` (row-major over the tile grid) and the tile's origin.
-template <int TM, int TN, int NW>
+// Source pointers of tile `id` (row-major over the tile grid) and the tile's origin.  EDGE: M and
+// N need not be multiples of the tile (N still a multiple of 4): loads of rows / column chunks
+// past the end are redirected to the last valid row / chunk (their products land in accumulators
+// that are never stored) and the epilogue skips what lies outside the matrix.
+template <bool EDGE, int TM, int TN, int NW>
 __device__ __forceinline__ void direct32_place(const GemmArgs& g, int id, Direct32Ctx<TM, TN, NW>& c, int& m0, int& n0) {
   using C = Direct32Ctx<TM, TN, NW>;
   constexpr int BM = 64 * TM, BN = 64 * TN;
   const int lane = lane_now();  // the lane's offsets are recomputed per tile rather than kept in registers
-  const int tiles_n = g.N / BN;
+  const int tiles_n = (g.N + BN - 1) / BN;
   m0 = (id / tiles_n) * BM;
   n0 = (id % tiles_n) * BN;
   const float* A = reinterpret_cast<const float*>(g.a);
@@ -123,7 +126,7 @@ __device__ __forceinline__ void direct32_place(const GemmArgs& g, int id, Direct
   for (int i = 0; i < C::LA; ++i) {
     const int row = (C::NW * i + c.wave) * 8 + (lane >> 3);
     const int gc = (lane & 7) ^ ((row >> 1) & 7);
-    c.a_src[i] = A + (int64_t)(m0 + row) * g.lda + gc * 4;
+    c.a_src[i] = A + (int64_t)(EDGE ? min(m0 + row, g.M - 1) : m0 + row) * g.lda + gc * 4;
   }
   // B: a k row is 16 TN chunks; load i of wave w fills k rows (NW i + w) (4 / TN) .. ; lane ->
   // row += lane / (16 TN), LDS chunk lane % (16 TN).
@@ -132,7 +135,7 @@ __device__ __forceinline__ void direct32_place(const GemmArgs& g, int id, Direct
     constexpr int chunks = 16 * TN;
     const int k = (C::NW * i + c.wave) * (64 / chunks) + lane / chunks;
     const int gc = (lane % chunks) ^ (8 * ((k >> 2) & 1));
-    c.b_src[i] = B + (int64_t)k * g.ldb + n0 + gc * 4;
+    c.b_src[i] = B + (int64_t)k * g.ldb + (EDGE ? min(n0 + gc * 4, g.N - 4) : n0 + gc * 4);
   }
 }
 
@@ -140,7 +143,7 @@ __device__ __forceinline__ void direct32_place(const GemmArgs& g, int id, Direct
 // modulo 8 stay on one XCD, which is what xcd_remap assumes).  At the end of a tile, once every
 // wave has left the ring, the first NS - 1 stages of the workgroup's next tile are issued before
 // the epilogue, so their latency and the cold start of the pipeline hide behind its stores.
-template <int TM, int TN, int NS, int NW>
+template <int TM, int TN, int NS, int NW, bool EDGE>
 __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
   using C = Direct32Ctx<TM, TN, NW>;
   constexpr int WTM = C::WTM;
@@ -152,7 +155,7 @@ __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave >> 1) * 32 * WTM, wn0 = (wave & 1) * 32 * TN;
-  const int ntiles = (g.M / BM) * (g.N / BN);
+  const int ntiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
   const int r32 = lane & 31, h = lane >> 5;
 
   C c;
@@ -174,7 +177,7 @@ __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
   const int nk = g.K / 32;
   int t = blockIdx.x;  // < ntiles: the grid is never larger than the tile list
   int m0, n0;
-  direct32_place(g, xcd_remap(t, ntiles), c, m0, n0);
+  direct32_place<EDGE>(g, xcd_remap(t, ntiles), c, m0, n0);
 #pragma unroll
   for (int st = 0; st < NS - 1; ++st)
     if (st < nk) direct32_issue(c, st, smem32d + st * stage_bytes);
@@ -204,7 +207,7 @@ __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
     const int em0 = m0, en0 = n0;
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the ring
     if (more) {
-      direct32_place(g, xcd_remap(tn, ntiles), c, m0, n0);
+      direct32_place<EDGE>(g, xcd_remap(tn, ntiles), c, m0, n0);
 #pragma unroll
       for (int st = 0; st < NS - 1; ++st)
         if (st < nk) direct32_issue(c, st, smem32d + st * stage_bytes);
@@ -218,17 +221,17 @@ __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
       for (int j = 0; j < WTM; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          epilogue4<LH_F32>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
-                            acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+          if (!EDGE || (m_base + 32 * j < g.M && n_base + 32 * i + 8 * q < g.N))
+            epilogue4<LH_F32>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                              acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
     if (!more) break;
     t = tn;
   }
 }
 
-// `per_cu`: workgroups of this shape that fit a CU's LDS together.
-template <int TM, int TN, int NS, int NW = 4>
-static int launch_direct32(const GemmArgs& g, hipStream_t s) {
-  auto kern = gemm32_direct<TM, TN, NS, NW>;
+template <int TM, int TN, int NS, int NW, bool EDGE>
+static int launch_direct32_edge(const GemmArgs& g, hipStream_t s) {
+  auto kern = gemm32_direct<TM, TN, NS, NW, EDGE>;
   constexpr size_t lds = (size_t)NS * (64 * TM * 128 + 32 * 64 * TN * 4);
   static bool configured = false;
   if (!configured) {
@@ -236,10 +239,16 @@ static int launch_direct32(const GemmArgs& g, hipStream_t s) {
                                      (int)lds));
     configured = true;
   }
-  const int ntiles = (g.M / (64 * TM)) * (g.N / (64 * TN));
-  const int resident = num_cus() * (int)((160 * 1024) / lds);
+  const int ntiles = ((g.M + 64 * TM - 1) / (64 * TM)) * ((g.N + 64 * TN - 1) / (64 * TN));
+  const int resident = num_cus() * (int)((160 * 1024) / lds);  // workgroups that fit the CUs' LDS together
   hipLaunchKernelGGL(kern, dim3(ntiles < resident ? ntiles : resident), dim3(NW * 64), lds, s, g);
   return check_launch("gemm32_direct");
+}
+
+template <int TM, int TN, int NS, int NW = 4>
+static int launch_direct32(const GemmArgs& g, hipStream_t s) {
+  if (g.M % (64 * TM) == 0 && g.N % (64 * TN) == 0) return launch_direct32_edge<TM, TN, NS, NW, false>(g, s);
+  return launch_direct32_edge<TM, TN, NS, NW, true>(g, s);
 }
 
 // Any shape / stride / transpose; 64 x 64 x 16 tiles, bounds-checked scalar loads.
@@ -298,18 +307,20 @@ int gemm32(const GemmArgs& g, hipStream_t s) {
   const bool vec_ok = !trans && g.K % kBK32 == 0 && g.lda % 4 == 0 && g.ldb % 4 == 0 && g.ldc % 4 == 0 &&
                       aligned16(g.a) && aligned16(g.b) && aligned16(g.out) &&
                       (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias));
-  if (vec_ok && g.M % 128 == 0 && g.N % 128 == 0 && (int64_t)(g.M / 128) * (g.N / 128) >= 256) {
-    // 128 x 128 or 128 x 64 tiles, one workgroup per CU: whichever needs less time in whole
-    // rounds of tiles (the narrow tile pays about 8 % more operand traffic per flop).
+  if (vec_ok && g.N % 4 == 0) {
+    // Tiles are counted with edge tiles in full (M, N need not be multiples of a tile).
     const int cus = num_cus();
-    const int64_t t128 = (int64_t)(g.M / 128) * (g.N / 128);
-    const double wide = (double)((t128 + cus - 1) / cus), narrow = (double)((2 * t128 + cus - 1) / cus) * 0.54;
-    if (narrow < wide) return launch_direct32<2, 1, 4, 8>(g, s);
-    return launch_direct32<2, 2, 4, 8>(g, s);
-  }
-  if (vec_ok && g.M % 64 == 0 && g.N % 64 == 0) {
+    const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
+    if (t128 >= 256) {
+      // 128 x 128 or 128 x 64 tiles, one workgroup per CU: whichever needs less time in whole
+      // rounds of tiles (the narrow tile pays about 8 % more operand traffic per flop).
+      const int64_t t64n = (int64_t)((g.M + 127) / 128) * ((g.N + 63) / 64);
+      const double wide = (double)((t128 + cus - 1) / cus), narrow = (double)((t64n + cus - 1) / cus) * 0.54;
+      if (narrow < wide) return launch_direct32<2, 1, 4, 8>(g, s);
+      return launch_direct32<2, 2, 4, 8>(g, s);
+    }
     // Up to two workgroups per CU: a deep ring; more: a shallow ring so that three share a CU.
-    if ((int64_t)(g.M / 64) * (g.N / 64) <= 512) return launch_direct32<1, 1, 6>(g, s);
+    if ((int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64) <= 512) return launch_direct32<1, 1, 6>(g, s);
     return launch_direct32<1, 1, 3>(g, s);
   }
   dim3 grid((g.N + 63) / 64, (g.M + 63) / 64);

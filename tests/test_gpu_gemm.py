@@ -169,6 +169,38 @@ def test_gemm_16bit_ragged_shapes(shape, epi):
     assert (border == 7.0).all(), "the kernel wrote outside the output matrix"
 
 
+@pytest.mark.parametrize("shape", [(1000, 520, 192), (130, 264, 64), (257, 4, 128), (1, 1000, 256), (3000, 772, 320),
+                                   (4100, 2052, 96)])  # the last: 128-wide tiles, several per workgroup
+@pytest.mark.parametrize("epi", ["none", "bias_relu", "acc_bias"])
+def test_gemm_f32_ragged_shapes(shape, epi):
+    """f32 with M and N that no tile divides (N a multiple of 4, K of 32): the direct kernel's edge
+    instantiation; rows and columns past the end must be neither read as bias nor written."""
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(7 * M + 3 * N + K)
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (N,)).astype(np.float32)
+    pad = 4
+    canvas = torch.full((M + 2, N + 2 * pad), 7.0, device="cuda")
+    view = canvas[1:M + 1, pad:pad + N]
+    da, db = _dev(a, torch.float32), _dev(b, torch.float32)
+    if epi == "acc_bias":
+        c = rng.standard_normal((M, N)).astype(np.float32)
+        view.copy_(_dev(c, torch.float32))
+        ops.gemm(da, db, _dev(bias, torch.float32), out=view, accumulate_c=True)
+        ref = orc.matmul(a, b, c=c, bias=bias, accumulate_c=True)
+    else:
+        has = epi == "bias_relu"
+        ops.gemm(da, db, _dev(bias, torch.float32) if has else None, relu=has, out=view)
+        ref = orc.matmul(a, b, bias=bias if has else None, relu=has)
+    assert_close(_host(view), ref, F32_RTOL, f"ragged f32 gemm {shape} {epi}")
+    border = canvas.clone()
+    border[1:M + 1, pad:pad + N] = 7.0
+    assert (border == 7.0).all(), "the kernel wrote outside the output matrix"
+
+
 def test_gemm_tile_request_errors():
     from lighthouse_amd import ops
 
