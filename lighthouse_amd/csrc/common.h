@@ -157,6 +157,13 @@ __device__ __forceinline__ int xcd_remap(int bid, int nblocks) {
 }
 
 hipStream_t default_stream();
+// out[c][r] = in[r][c] for an R x C matrix of 2- or 4-byte elements (row strides in elements).
+int transpose_matrix(void* out, const void* in, int R, int C, int64_t ld_in, int64_t ld_out, int elem_bytes,
+                     hipStream_t s);
+// A library-owned device buffer of at least `bytes` (grown on demand, kept until the process
+// ends); calls that use it on different streams at the same time race.  nullptr on failure
+// (the error message is set).
+void* transpose_scratch(size_t bytes);
 // Compute units of the current device (cached; 256 if the query fails).
 int num_cus();
 

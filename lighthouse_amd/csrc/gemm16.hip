@@ -805,7 +805,13 @@ static int direct_variant(int M, int N, int K) {
 }
 
 template <int DT>
-static int gemm16_dispatch(const GemmArgs& g, hipStream_t s) {
+static int gemm16_dispatch(const GemmArgs& g_in, hipStream_t s) {
+  GemmArgs g = g_in;
+  if ((g.flags & LH_GEMM_TILE_MASK) == LH_GEMM_TILE_AUTO && g.ldc % 8 == 0 && aligned16(g.out) &&
+      (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias))) {
+    const int rc = untranspose_operands<2>(g, kBK, 8, s);
+    if (rc < 0) return rc;
+  }
   const bool ta = g.flags & LH_GEMM_TRANSPOSE_A, tb = g.flags & LH_GEMM_TRANSPOSE_B;
   const bool vec_ok = !ta && g.K % kBK == 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 && g.ldc % 4 == 0 &&
                       aligned16(g.a) && aligned16(g.b) && aligned16(g.out) &&

@@ -302,7 +302,12 @@ __global__ void __launch_bounds__(256) gemm32_generic(GemmArgs g) {
   }
 }
 
-int gemm32(const GemmArgs& g, hipStream_t s) {
+int gemm32(const GemmArgs& g_in, hipStream_t s) {
+  GemmArgs g = g_in;
+  if (g.ldc % 4 == 0 && aligned16(g.out) && (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias))) {
+    const int rc = untranspose_operands<4>(g, kBK32, 4, s);
+    if (rc < 0) return rc;
+  }
   const bool trans = g.flags & (LH_GEMM_TRANSPOSE_A | LH_GEMM_TRANSPOSE_B);
   const bool vec_ok = !trans && g.K % kBK32 == 0 && g.lda % 4 == 0 && g.ldb % 4 == 0 && g.ldc % 4 == 0 &&
                       aligned16(g.a) && aligned16(g.b) && aligned16(g.out) &&

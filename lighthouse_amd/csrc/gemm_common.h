@@ -109,6 +109,32 @@ __device__ __forceinline__ u32x2 epilogue4_pack(const GemmArgs& g, int n, float 
   return epilogue4_pack_bias<DT>(g, bias4<DT>(g, n), v0, v1, v2, v3);
 }
 
+// Transposed operands (A stored [K,M], B stored [N,K]) of a problem the direct kernels would
+// otherwise take are first transposed into a library-owned buffer (one extra pass over that
+// operand, about a tenth of a 4096^3 problem's time) instead of running the slower kernels that
+// read them in place.  Returns 0 and rewrites `g` on success, 1 when the problem does not qualify.
+template <int ELEM_BYTES>
+inline int untranspose_operands(GemmArgs& g, int k_multiple, int n_multiple, hipStream_t s) {
+  const bool ta = g.flags & LH_GEMM_TRANSPOSE_A, tb = g.flags & LH_GEMM_TRANSPOSE_B;
+  if (!(ta || tb) || g.K % k_multiple != 0 || g.N % n_multiple != 0) return 1;
+  const size_t a_bytes = ta ? ((size_t)g.M * g.K * ELEM_BYTES + 255) / 256 * 256 : 0;
+  const size_t b_bytes = tb ? (size_t)g.K * g.N * ELEM_BYTES : 0;
+  char* buf = static_cast<char*>(transpose_scratch(a_bytes + b_bytes));
+  if (!buf) return LH_ERR_RUNTIME;
+  if (ta) {  // stored [K, M] -> [M, K]
+    if (int rc = transpose_matrix(buf, g.a, g.K, g.M, g.lda, g.K, ELEM_BYTES, s)) return rc;
+    g.a = buf;
+    g.lda = g.K;
+  }
+  if (tb) {  // stored [N, K] -> [K, N]
+    if (int rc = transpose_matrix(buf + a_bytes, g.b, g.N, g.K, g.ldb, g.N, ELEM_BYTES, s)) return rc;
+    g.b = buf + a_bytes;
+    g.ldb = g.N;
+  }
+  g.flags &= ~(uint32_t)(LH_GEMM_TRANSPOSE_A | LH_GEMM_TRANSPOSE_B);
+  return 0;
+}
+
 // One output element, any alignment (edge tiles and the generic kernels).
 template <int DT>
 __device__ __forceinline__ void epilogue1(const GemmArgs& g, int m, int n, float x) {

@@ -37,6 +37,85 @@ int num_cus() {
   return cus;
 }
 
+// Transpose through a padded 64 x 64 LDS tile: rows of 64 elements are read and written whole.
+template <typename T>
+__global__ void __launch_bounds__(256) transpose_tiles(T* out, const T* in, int R, int C, int64_t ld_in, int64_t ld_out) {
+  __shared__ T tile[64][65];
+  const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int r = r0 + i, c = c0 + tx;
+    if (r < R && c < C) tile[i][tx] = in[(int64_t)r * ld_in + c];
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int c = c0 + i, r = r0 + tx;
+    if (c < C && r < R) out[(int64_t)c * ld_out + r] = tile[tx][i];
+  }
+}
+
+// 16-bit elements with R, C and both strides multiples of 8 and 16-byte aligned bases: 16-byte
+// global accesses on both sides, the transposition happens in the 2-byte LDS writes.
+__global__ void __launch_bounds__(256) transpose_tiles16(uint16_t* out, const uint16_t* in, int R, int C,
+                                                         int64_t ld_in, int64_t ld_out) {
+  __shared__ __attribute__((aligned(16))) uint16_t tile[64][72];  // [column][row], rows of 144 bytes
+  const int c0 = blockIdx.x * 64, r0 = blockIdx.y * 64;
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int idx = threadIdx.x + 256 * p, r = idx >> 3, cg = idx & 7;
+    if (r0 + r < R && c0 + 8 * cg < C) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(in + (int64_t)(r0 + r) * ld_in + c0 + 8 * cg);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) tile[8 * cg + e][r] = (uint16_t)(v[e >> 1] >> (16 * (e & 1)));
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    const int idx = threadIdx.x + 256 * p, c = idx >> 3, rg = idx & 7;
+    if (c0 + c < C && r0 + 8 * rg < R)
+      *reinterpret_cast<u32x4*>(out + (int64_t)(c0 + c) * ld_out + r0 + 8 * rg) =
+          *reinterpret_cast<const u32x4*>(&tile[c][8 * rg]);
+  }
+}
+
+int transpose_matrix(void* out, const void* in, int R, int C, int64_t ld_in, int64_t ld_out, int elem_bytes,
+                     hipStream_t s) {
+  const dim3 grid((C + 63) / 64, (R + 63) / 64);
+  if (elem_bytes == 2 && R % 8 == 0 && C % 8 == 0 && ld_in % 8 == 0 && ld_out % 8 == 0 && aligned16(out) && aligned16(in))
+    hipLaunchKernelGGL(transpose_tiles16, grid, dim3(256), 0, s, static_cast<uint16_t*>(out),
+                       static_cast<const uint16_t*>(in), R, C, ld_in, ld_out);
+  else if (elem_bytes == 2)
+    hipLaunchKernelGGL(transpose_tiles<uint16_t>, grid, dim3(256), 0, s, static_cast<uint16_t*>(out),
+                       static_cast<const uint16_t*>(in), R, C, ld_in, ld_out);
+  else if (elem_bytes == 4)
+    hipLaunchKernelGGL(transpose_tiles<uint32_t>, grid, dim3(256), 0, s, static_cast<uint32_t*>(out),
+                       static_cast<const uint32_t*>(in), R, C, ld_in, ld_out);
+  else
+    return fail(LH_ERR_UNSUPPORTED, "transpose: element size %d", elem_bytes);
+  return check_launch("transpose_tiles");
+}
+
+static char* g_transpose_scratch = nullptr;
+static size_t g_transpose_scratch_bytes = 0;
+
+void* transpose_scratch(size_t bytes) {
+  if (bytes > g_transpose_scratch_bytes) {
+    if (g_transpose_scratch && hipFree(g_transpose_scratch) != hipSuccess) (void)hipGetLastError();
+    g_transpose_scratch = nullptr;
+    g_transpose_scratch_bytes = 0;
+    const hipError_t e = hipMalloc(reinterpret_cast<void**>(&g_transpose_scratch), bytes);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      set_error("transpose scratch: hipMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+      g_transpose_scratch = nullptr;
+      return nullptr;
+    }
+    g_transpose_scratch_bytes = bytes;
+  }
+  return g_transpose_scratch;
+}
+
 }  // namespace lh
 
 using namespace lh;

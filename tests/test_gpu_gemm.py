@@ -256,17 +256,21 @@ def test_gemm_row_strided_views(kind):
 
 @pytest.mark.parametrize("ta,tb", [(True, False), (False, True), (True, True)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-def test_gemm_transposed(dtype, ta, tb):
+@pytest.mark.parametrize("shape", [(256, 128, 192),   # operands transposed into the library's buffer first
+                                   (1000, 776, 512),  # the same with several tiles and an M no tile divides
+                                   (100, 72, 64),     # M no multiple of 8: the element-wise transpose
+                                   (70, 50, 33)])     # K no multiple of a k-step: the kernels that read in place
+def test_gemm_transposed(dtype, ta, tb, shape):
     from lighthouse_amd import ops
 
-    M, N, K = 256, 128, 192
+    M, N, K = shape
     elt = "bf16" if dtype == torch.bfloat16 else "f32"
     rng = np.random.default_rng(99)
     a = orc.round_to(rng.standard_normal((K, M) if ta else (M, K)).astype(np.float32), elt)
     b = orc.round_to(rng.standard_normal((N, K) if tb else (K, N)).astype(np.float32), elt)
     out = ops.gemm(_dev(a, dtype), _dev(b, dtype), out_dtype=torch.float32, transpose_a=ta, transpose_b=tb)
     ref = orc.matmul(a, b, transpose_a=ta, transpose_b=tb)
-    assert_close(_host(out), ref, F32_RTOL, f"transposed gemm ta={ta} tb={tb} {elt}")
+    assert_close(_host(out), ref, F32_RTOL, f"transposed gemm {shape} ta={ta} tb={tb} {elt}")
 
 
 def test_gemm_integer_inputs_exact():
