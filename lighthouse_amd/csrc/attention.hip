@@ -111,29 +111,27 @@ __device__ __forceinline__ void attn_issue_loads(const AttnCtx& c, int jt, int T
 template <int DT, int NQ, bool RAGGED>
 __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, const u32x4 (&qf)[NQ][4],
                                           f32x16 (&acc_o)[NQ][2], float (&m_run)[NQ], float (&l_run)[NQ],
-                                          const uint8_t* __restrict__ rd, uint8_t* __restrict__ wr, int next_jt,
+                                          f32x16 (&neg_m)[NQ], const uint8_t* __restrict__ rd,
+                                          uint8_t* __restrict__ wr, int next_jt,
                                           bool prefetch, int j0, int wq0, bool active, bool need_mask) {
   if (prefetch) attn_issue_loads<RAGGED>(c, next_jt, a.T, wr);
   if (!active) return;
   const uint8_t* ks = rd;
   const uint8_t* vs = rd + 8192;
-  // S^T = K Q^T: key sub-tile i (32 keys) x query sub-tile qt (32 rows).
+  // S^T = K Q^T: key sub-tile i (32 keys) x query sub-tile qt (32 rows).  Q carries the factor
+  // scale * log2(e) and the first MFMA of a sub-tile starts from neg_m (every element of a lane's
+  // block = minus the softmax offset of the lane's query row), so the accumulators come out as
+  // the exponents themselves: no per-element multiply-subtract before the exp.
   f32x16 s_acc[NQ][2];
-#pragma unroll
-  for (int qt = 0; qt < NQ; ++qt)
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) s_acc[qt][i][v] = 0.0f;
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int sd = 0; sd < 4; ++sd) {
       u32x4 kf = *reinterpret_cast<const u32x4*>(ks + c.k_off[i] + (((2 * sd + c.h) ^ c.k_swz[i]) << 4));
 #pragma unroll
-      for (int qt = 0; qt < NQ; ++qt) s_acc[qt][i] = mfma16<DT>(kf, qf[qt][sd], s_acc[qt][i]);
+      for (int qt = 0; qt < NQ; ++qt) s_acc[qt][i] = mfma16<DT>(kf, qf[qt][sd], sd == 0 ? neg_m[qt] : s_acc[qt][i]);
     }
-  // s_acc[qt][i][v] = S[q = wq0 + 32 qt + r32][key = j0 + 32 i + 8 (v/4) + 4 h + v%4] (unscaled)
+  // s_acc[qt][i][v] = S[q = wq0 + 32 qt + r32][key = j0 + 32 i + 8 (v/4) + 4 h + v%4] scale log2e - offset
   u32x4 pf[NQ][2][2];
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt) {
@@ -151,26 +149,31 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
     // Lazy offset: P = exp(S - offset) is first computed with the offset already in use.  Softmax
     // does not depend on the offset and 16-bit P is as accurate at 2^10 as below 1, so the offset
     // only has to move when P would grow without bound: the lane's partial row sum (needed anyway)
-    // is the test.  It bounds every P of the lane, cannot exceed 32 while no score has passed the
-    // offset, and is inf or NaN on the first tile (offset -inf).  Only then is the row maximum
-    // computed, the offset raised, l and acc rescaled and P recomputed, for the whole wave.
-    float mc = m_run[qt];
+    // is the test.  It bounds every P of the lane and cannot exceed 32 while no score has passed
+    // the offset.  A row that has no offset yet (m = -inf; computed against 0) always takes the
+    // slow path, so that its first visible maximum becomes the offset and l >= 1 from then on.
+    // Only there is the row maximum computed, the offset raised, l and acc rescaled and P
+    // recomputed, for the whole wave.
+    const float mc = m_run[qt];
     float p[2][16];
     float l_tile = 0.0f;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        p[i][v] = exp2_fast(s_acc[qt][i][v] * a.scale_log2e - mc);
+        p[i][v] = exp2_fast(s_acc[qt][i][v]);
         l_tile += p[i][v];
       }
-    if (__builtin_amdgcn_ballot_w64(!(l_tile <= kOffsetSlack)) != 0) {
+    if (__builtin_amdgcn_ballot_w64(!(l_tile <= kOffsetSlack) || mc == -INFINITY) != 0) {
       float mx = fmaxf(s_acc[qt][0][0], s_acc[qt][1][0]);
 #pragma unroll
       for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[qt][0][v]), s_acc[qt][1][v]);
-      mx = halfwave_max(mx);
-      const float m_new = fmaxf(mc, mx * a.scale_log2e);
-      const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // row without a visible key so far
+      mx = halfwave_max(mx);  // relative to the offset in use (0 for a row without one)
+      const float m_old = (mc == -INFINITY) ? 0.0f : mc;
+      // The offset only moves up; a row with no visible key so far (mx = -inf) stays without one.
+      const float m_new = (mc == -INFINITY) ? mx : mc + fmaxf(mx, 0.0f);
+      const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+      const float delta = m_safe - m_old;
       const float alpha = exp2_fast(mc - m_safe);
       l_run[qt] *= alpha;
       m_run[qt] = m_new;
@@ -183,9 +186,12 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          p[i][v] = exp2_fast(s_acc[qt][i][v] * a.scale_log2e - m_safe);
+          p[i][v] = exp2_fast(s_acc[qt][i][v] - delta);
           l_tile += p[i][v];
         }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) neg_m[qt][v] = -m_safe;
+      asm volatile("" : "+v"(neg_m[qt]));  // a register block, not a constant to re-create per tile
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -308,7 +314,10 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
 #pragma unroll
     for (int sd = 0; sd < 4; ++sd) {
       const int row = RAGGED ? min(wq_load + 32 * qt + r32, a.T - 1) : wq_load + 32 * qt + r32;
-      qf[qt][sd] = *reinterpret_cast<const u32x4*>(Q + (int64_t)row * a.sq.t + 16 * sd + 8 * h);
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(Q + (int64_t)row * a.sq.t + 16 * sd + 8 * h);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        qf[qt][sd][e] = pack2<DT>(unpack_lo<DT>(raw[e]) * a.scale_log2e, unpack_hi<DT>(raw[e]) * a.scale_log2e);
     }
 
   f32x16 acc_o[NQ][2];
@@ -319,10 +328,14 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc_o[qt][j][v] = 0.0f;
   float m_run[NQ], l_run[NQ];
+  f32x16 neg_m[NQ];  // minus the softmax offset of the lane's row, 16 times: the C operand of S
 #pragma unroll
   for (int qt = 0; qt < NQ; ++qt) {
     m_run[qt] = -INFINITY;
     l_run[qt] = 0.0f;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) neg_m[qt][v] = 0.0f;
+    asm volatile("" : "+v"(neg_m[qt]));
   }
 
   const int kv_end = a.causal ? min(a.T, q0 + kRowsPerGroup) : a.T;
@@ -343,7 +356,7 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
     const bool active = wave_valid && (!a.causal || (j0 <= wq0 + kRowsPerWave - 1));
     const bool need_mask = (a.causal && (j0 + kKvTile - 1 > wq0)) || (RAGGED && j0 + kKvTile > a.T);
     const int nxt = jt + kAttnStages - 1;
-    attn_tile<DT, NQ, RAGGED>(c, a, qf, acc_o, m_run, l_run, smem_attn + (jt % kAttnStages) * kAttnStageBytes,
+    attn_tile<DT, NQ, RAGGED>(c, a, qf, acc_o, m_run, l_run, neg_m, smem_attn + (jt % kAttnStages) * kAttnStageBytes,
                   smem_attn + (nxt % kAttnStages) * kAttnStageBytes, nxt, nxt < ntiles, j0, wq0, active, need_mask);
   }
 
