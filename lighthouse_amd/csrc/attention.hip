@@ -108,7 +108,7 @@ __device__ __forceinline__ void attn_issue_loads(const AttnCtx& c, int jt, int T
 // One key tile (64 keys) for the wave's two 32-row query sub-tiles.  `rd` holds the tile, `wr`
 // is the ring slot that receives a later tile meanwhile (separate restrict pointers so that LDS
 // reads do not wait for the asynchronous writes).
-template <int DT, int NQ, bool RAGGED>
+template <int DT, int NQ, bool RAGGED, bool AHEAD>
 __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, const u32x4 (&qf)[NQ][4],
                                           f32x16 (&acc_o)[NQ][2], float (&m_run)[NQ], float (&l_run)[NQ],
                                           f32x16 (&neg_m)[NQ], const uint8_t* __restrict__ rd,
@@ -122,15 +122,24 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
   // scale * log2(e) and the first MFMA of a sub-tile starts from neg_m (every element of a lane's
   // block = minus the softmax offset of the lane's query row), so the accumulators come out as
   // the exponents themselves: no per-element multiply-subtract before the exp.
+  // AHEAD: all K fragments are requested before the first MFMA (the registers are free in this
+  // phase); left to the compiler each read is followed by its wait, one exposed LDS latency per
+  // pair of MFMAs.  (Not for the instantiation that runs three waves per SIMD on 168 registers.)
   f32x16 s_acc[NQ][2];
+  u32x4 kf[2][4];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int sd = 0; sd < 4; ++sd) {
-      u32x4 kf = *reinterpret_cast<const u32x4*>(ks + c.k_off[i] + (((2 * sd + c.h) ^ c.k_swz[i]) << 4));
+    for (int sd = 0; sd < 4; ++sd)
+      kf[i][sd] = *reinterpret_cast<const u32x4*>(ks + c.k_off[i] + (((2 * sd + c.h) ^ c.k_swz[i]) << 4));
+  if constexpr (AHEAD) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int qt = 0; qt < NQ; ++qt) s_acc[qt][i] = mfma16<DT>(kf, qf[qt][sd], sd == 0 ? neg_m[qt] : s_acc[qt][i]);
-    }
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int sd = 0; sd < 4; ++sd)
+#pragma unroll
+      for (int qt = 0; qt < NQ; ++qt)
+        s_acc[qt][i] = mfma16<DT>(kf[i][sd], qf[qt][sd], sd == 0 ? neg_m[qt] : s_acc[qt][i]);
   // s_acc[qt][i][v] = S[q = wq0 + 32 qt + r32][key = j0 + 32 i + 8 (v/4) + 4 h + v%4] scale log2e - offset
   u32x4 pf[NQ][2][2];
 #pragma unroll
@@ -202,6 +211,8 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
     l_run[qt] += l_tile;
   }
   // O^T += V^T P^T: head-dim sub-tile j (32 of d) x query sub-tile qt, over 4 k-steps of 16 keys.
+  // The V^T fragments too are all requested first.
+  u32x4 vf[2][2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -213,10 +224,17 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
         attn_s16x4 hi =
             __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) attn_s16x4*)(p0 + 8 * 128));
         u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-        u32x4 vf = {l2[0], l2[1], h2[0], h2[1]};
-#pragma unroll
-        for (int qt = 0; qt < NQ; ++qt) acc_o[qt][j] = mfma16<DT>(vf, pf[qt][i][u], acc_o[qt][j]);
+        vf[i][u][j] = u32x4{l2[0], l2[1], h2[0], h2[1]};
       }
+  if constexpr (AHEAD) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int qt = 0; qt < NQ; ++qt) acc_o[qt][j] = mfma16<DT>(vf[i][u][j], pf[qt][i][u], acc_o[qt][j]);
 }
 
 // Launch order of a causal problem.  Causal work grows with the query block index.  Rank r
@@ -244,7 +262,7 @@ __device__ __forceinline__ void causal_block_of(int L, int G, int R, int nqb, in
 // are 128 bytes and cannot be padded (a wave-wide load writes 1 KiB contiguous), so the
 // 16-byte chunk a lane fetches is XOR-swizzled: K chunk ^ ((key / 2) % 8), V chunk ^ 4 ((key / 2) % 2).
 template <int DT, int NQ, int NS, bool RAGGED>
-__global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
+__global__ void __launch_bounds__(256, (NQ == 1 && NS == 3 ? 3 : 2)) attention16_kernel(AttnArgs a) {
   constexpr int kRowsPerWave = 32 * NQ, kRowsPerGroup = 4 * kRowsPerWave;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -356,7 +374,7 @@ __global__ void __launch_bounds__(256, 2) attention16_kernel(AttnArgs a) {
     const bool active = wave_valid && (!a.causal || (j0 <= wq0 + kRowsPerWave - 1));
     const bool need_mask = (a.causal && (j0 + kKvTile - 1 > wq0)) || (RAGGED && j0 + kKvTile > a.T);
     const int nxt = jt + kAttnStages - 1;
-    attn_tile<DT, NQ, RAGGED>(c, a, qf, acc_o, m_run, l_run, neg_m, smem_attn + (jt % kAttnStages) * kAttnStageBytes,
+    attn_tile<DT, NQ, RAGGED, !(NQ == 1 && NS == 3) && !(NQ == 2 && RAGGED)>(c, a, qf, acc_o, m_run, l_run, neg_m, smem_attn + (jt % kAttnStages) * kAttnStageBytes,
                   smem_attn + (nxt % kAttnStages) * kAttnStageBytes, nxt, nxt < ntiles, j0, wq0, active, need_mask);
   }
 
