@@ -140,6 +140,10 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
 #pragma unroll
       for (int qt = 0; qt < NQ; ++qt)
         s_acc[qt][i] = mfma16<DT>(kf[i][sd], qf[qt][sd], sd == 0 ? neg_m[qt] : s_acc[qt][i]);
+  // A use of neg_m behind its last MFMA: without it the compiler treats that MFMA as the end of the
+  // block's life, accumulates in place and first copies the block (16 moves per tile and sub-tile).
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) asm volatile("" ::"v"(neg_m[qt]));
   // s_acc[qt][i][v] = S[q = wq0 + 32 qt + r32][key = j0 + 32 i + 8 (v/4) + 4 h + v%4] scale log2e - offset
   u32x4 pf[NQ][2][2];
 #pragma unroll
