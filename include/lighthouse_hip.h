@@ -122,6 +122,18 @@ int lh_hip_gemm(void* out, const void* a, const void* b, const void* bias, int64
                 void* stream);
 
 /*
+ * lh_hip_gemm whose accumulation starts from a separate matrix: out = epilogue(c + A.B), with
+ * `c` [M,N] of out_dtype and row stride ldc (ACCUMULATE_C is implied; c may be `out`, which is
+ * lh_hip_gemm with the flag).  The reference's payload accumulates in place only
+ * (gpu_mlp_payload.py:123-131); this form is what a residual connection x + linear(y) needs when
+ * x must survive (the torch ingress lowers that pattern to one call, and the nanoGPT block
+ * kernel sequence uses it internally).
+ */
+int lh_hip_gemm_residual(void* out, const void* c, const void* a, const void* b, const void* bias, int64_t M,
+                         int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype,
+                         int32_t out_dtype, uint32_t flags, void* stream);
+
+/*
  * fp8 GEMM of the benchmark's quantised configuration (no counterpart in the
  * reference): out[M,N] = out_dtype( (Aq.Bq)_f32 * (scale_a*scale_b) ), Aq [M,K] and
  * Bq [K,N] hold OCP e4m3fn codes; out_dtype BF16 or F32.

@@ -104,6 +104,7 @@ PROTOTYPES = {
     "lh_hip_memset": (_i32, [_vp, _i32, _sz]),
     "lh_hip_sync": (_i32, [_vp]),
     "lh_hip_gemm": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp]),
+    "lh_hip_gemm_residual": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp]),
     "lh_hip_gemm_fp8": (_i32, [_vp, _vp, _vp, _f32, _f32, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _vp]),
     "lh_hip_attention": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, Strides3, Strides3, Strides3, Strides3,
                                 _f32, _i32, _i32, _vp]),

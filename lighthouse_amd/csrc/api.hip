@@ -93,6 +93,21 @@ int lh_hip_gemm(void* out, const void* a, const void* b, const void* bias, int64
                   reinterpret_cast<hipStream_t>(stream));
 }
 
+int lh_hip_gemm_residual(void* out, const void* c, const void* a, const void* b, const void* bias, int64_t M, int64_t N,
+                         int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype, int32_t out_dtype,
+                         uint32_t flags, void* stream) {
+  int rc = gemm_common_checks("lh_hip_gemm_residual", out, a, b, bias, M, N, K, lda, ldb, ldc, flags);
+  if (rc) return rc;
+  LH_REQUIRE(c != nullptr, "lh_hip_gemm_residual: null accumulator input");
+  if (!(ab_dtype == LH_F32 || ab_dtype == LH_BF16 || ab_dtype == LH_F16))
+    return fail(LH_ERR_UNSUPPORTED, "lh_hip_gemm_residual: unsupported A/B dtype %d", ab_dtype);
+  if (!(out_dtype == LH_F32 || (out_dtype == ab_dtype)))
+    return fail(LH_ERR_UNSUPPORTED, "lh_hip_gemm_residual: out dtype %d must be f32 or the A/B dtype %d", out_dtype,
+                ab_dtype);
+  return gemm_run(out, c, a, b, bias, M, N, K, lda, ldb, ldc, ab_dtype, out_dtype, out_dtype,
+                  flags | LH_GEMM_ACCUMULATE_C, reinterpret_cast<hipStream_t>(stream));
+}
+
 int lh_hip_gemm_fp8(void* out, const void* a_q, const void* b_q, float scale_a, float scale_b, int64_t M, int64_t N,
                     int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int32_t out_dtype, void* stream) {
   int rc = gemm_common_checks("lh_hip_gemm_fp8", out, a_q, b_q, nullptr, M, N, K, lda, ldb, ldc, 0);

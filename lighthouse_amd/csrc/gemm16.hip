@@ -487,7 +487,6 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
   // recomputed here instead of kept in registers (and spilled) across the main loop.
   const int lane = lane_now();
   const int r32 = lane & 31, h = lane >> 5;
-  const int m_base = m0 + wm0 + r32;
   const int n_base = n0 + wn0 + 4 * h;
   if (g.out_dt != LH_F32 && !(g.flags & LH_GEMM_ACCUMULATE_C)) {
     // The bias values (loaded by the main loop, whose last wait covered them) are pinned down here:
@@ -541,18 +540,18 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
   }
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
   if constexpr (HAS_NEXT) direct_prologue(next, nk, ring);
-  if (g.out_dt == LH_F32) {
-    // f32 output (with or without an accumulator input): the scaled accumulators of a 32 x 8 QH
-    // block go through the wave's slice of `stage` so that the accumulator input is read and the
-    // result written as whole row segments (16 bytes per lane, 64 or 128 bytes per row) instead
-    // of 16-byte pieces of 64 different rows.  Order of operations as in epilogue4.
+  {
+    // f32 output (with or without an accumulator input), or a 16-bit output with an accumulator
+    // input: the scaled f32 accumulators of a 32 x 8 QH block go through the wave's slice of `stage`
+    // so that the accumulator input is read and the result written as whole row segments (4
+    // elements per lane, 32 to 128 bytes per row) instead of pieces of 64 different rows.  Order
+    // of operations as in epilogue4 (one rounding, after the sum).
     constexpr int QH = TN == 2 ? 4 : 2;        // accumulator column groups (of 8) per staged block
     constexpr int RB = QH * 32;                // bytes of a staged row
     constexpr int chunks = RB / 16;
     constexpr int rows_per_pass = 64 / chunks;
     uint8_t* cw = stage + next.wave * (32 * RB);
-    float* outp = reinterpret_cast<float*>(g.out);
-    const float* cin = reinterpret_cast<const float*>(g.c);
+    const bool out32 = g.out_dt == LH_F32;
     const bool has_c = (g.flags & LH_GEMM_ACCUMULATE_C) != 0;
     const bool gelu = (g.flags & LH_GEMM_HAS_GELU) != 0, relu = (g.flags & LH_GEMM_HAS_RELU) != 0;
     const int ch = lane % chunks, row0 = lane / chunks;
@@ -580,7 +579,13 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
             if (EDGE && !(n_ok && m < g.M)) continue;
             const int64_t off = (int64_t)m * g.ldc + n;
             if (has_c) {
-              const f32x4 c4 = *reinterpret_cast<const f32x4*>(cin + off);
+              f32x4 c4;
+              if (out32) {
+                c4 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.c) + off);
+              } else {
+                const u32x2 cc = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.c) + off);
+                c4 = f32x4{unpack_lo<DT>(cc[0]), unpack_hi<DT>(cc[0]), unpack_lo<DT>(cc[1]), unpack_hi<DT>(cc[1])};
+              }
 #pragma unroll
               for (int e = 0; e < 4; ++e) v[e] += c4[e];
             }
@@ -596,21 +601,15 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
 #pragma unroll
               for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
             }
-            *reinterpret_cast<f32x4*>(outp + off) = v;
+            if (out32)
+              *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(g.out) + off) = v;
+            else
+              *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(g.out) + off) =
+                  u32x2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
           }
         }
       }
-    return;
   }
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        if (!EDGE || (m_base + 32 * j < g.M && n_base + 32 * i + 8 * q < g.N))
-          epilogue4<DT>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
-                        acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
 }
 
 // Persistent workgroups: one (two for the 128 x 128 tile, whose LDS is 80 KiB) per CU, each

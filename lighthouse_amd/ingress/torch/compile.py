@@ -123,7 +123,8 @@ class _Lowering:
         self.allow_torch_fallback = allow_torch_fallback
         self.cache = _WeightCache()
         self.steps: list[PlanStep] = []
-        self.fused: dict[str, str] = {}  # activation node name -> name of the linear it is fused into
+        self.fused: dict[str, str] = {}  # activation / residual-add node name -> name of the linear it is fused into
+        self.order = {n: i for i, n in enumerate(gm.graph.nodes)}
 
     # -- helpers -------------------------------------------------------------------------
     @staticmethod
@@ -156,6 +157,22 @@ class _Lowering:
                 return "gelu", u
         return None, None
 
+    def _single_user_residual_add(self, node):
+        """(add node, residual operand) if `node` feeds exactly one `r + node` / `node + r` whose other
+        operand is a tensor computed before `node`: the GEMM then starts its accumulation from r."""
+        users = list(node.users)
+        if len(users) != 1:
+            return None, None
+        u = users[0]
+        is_add = (u.op == "call_function" and u.target in (operator.add, torch.add, operator.iadd)) or \
+                 (u.op == "call_method" and u.target in ("add", "__add__"))
+        if not is_add or len(u.args) < 2 or self._kwarg(u, "alpha", 2, 1) != 1:
+            return None, None
+        other = u.args[1] if u.args[0] is node else u.args[0]
+        if not isinstance(other, torch.fx.Node) or other is node or self.order[other] > self.order[node]:
+            return None, None
+        return u, other
+
     def _emit(self, name, kind, run, **detail):
         self.steps.append(PlanStep(name, kind, run, detail))
 
@@ -167,20 +184,30 @@ class _Lowering:
     # -- compute nodes -------------------------------------------------------------------
     def _linear(self, node, x_arg, w_arg, b_arg):
         act, act_node = self._single_user_activation(node)
+        add_node, res_arg = (None, None) if act_node is not None else self._single_user_residual_add(node)
         if act_node is not None:
             self.fused[act_node.name] = node.name
+        if add_node is not None:
+            self.fused[add_node.name] = node.name
         cache = self.cache
 
-        x_f, w_f, b_f = _resolver(x_arg), _resolver(w_arg), _resolver(b_arg)
+        x_f, w_f, b_f, r_f = _resolver(x_arg), _resolver(w_arg), _resolver(b_arg), _resolver(res_arg)
 
         def run(env, act=act):
-            x, w, b = x_f(env), w_f(env), b_f(env)
+            x, w, b, r = x_f(env), w_f(env), b_f(env), r_f(env)
             wt = cache.get(w, "linear_weight", lambda t: t.t().contiguous())
             x2 = _as_2d(x)
-            out = ops.gemm(x2, wt, b.detach() if b is not None else None, relu=act == "relu", gelu=act == "gelu")
-            return out.view(*x.shape[:-1], wt.shape[1])
+            shape = (*x.shape[:-1], wt.shape[1])
+            if r is not None:
+                # x + linear(y): the accumulation starts from the residual, which is only read.
+                if not isinstance(r, torch.Tensor) or tuple(r.shape) != shape or r.dtype != x.dtype:
+                    raise ValueError(f"{node.name}: broadcasting / mixed-type add is not supported")
+                r = _as_2d(r)
+            out = ops.gemm(x2, wt, b.detach() if b is not None else None, relu=act == "relu", gelu=act == "gelu",
+                           residual=r)
+            return out.view(shape)
 
-        self._emit(node.name, "hip.gemm", run, bias=b_arg is not None, activation=act)
+        self._emit(node.name, "hip.gemm", run, bias=b_arg is not None, activation=act, residual=add_node is not None)
 
     def _layer_norm(self, node, x_arg, shape, w_arg, b_arg, eps):
         if len(tuple(shape)) != 1:
@@ -230,6 +257,10 @@ class _Lowering:
 
     def _binary_add(self, node):
         a_arg, b_arg = node.args[:2]
+        if node.name in self.fused:
+            src = self.fused[node.name]
+            self._emit(node.name, "fused", lambda env, src=src: env[src], into=src)
+            return
         if self._kwarg(node, "alpha", 2, 1) != 1:
             raise ValueError(f"{node.name}: add with alpha is not supported")
 

@@ -38,9 +38,10 @@ def device_info() -> dict:
 
 
 def gemm(a, b, bias=None, *, out=None, out_dtype=None, relu=False, gelu=False, accumulate_c=False,
-         transpose_a=False, transpose_b=False, tile=None):
-    """out = epilogue(A @ B); see lh_hip_gemm.  `tile=(bm, bn)` requests a workgroup tile."""
-    _need_cuda(a, b, bias, out)
+         transpose_a=False, transpose_b=False, tile=None, residual=None):
+    """out = epilogue(A @ B); see lh_hip_gemm.  `tile=(bm, bn)` requests a workgroup tile;
+    `residual` [M, N] is added to A @ B before the epilogue (lh_hip_gemm_residual) and is left intact."""
+    _need_cuda(a, b, bias, out, residual)
     if a.dim() != 2 or b.dim() != 2:
         raise ValueError("gemm expects 2-D tensors")
     if a.stride(1) != 1 or b.stride(1) != 1:
@@ -68,6 +69,17 @@ def gemm(a, b, bias=None, *, out=None, out_dtype=None, relu=False, gelu=False, a
         raise ValueError("bias must have the output dtype")
     if a.dtype != b.dtype:
         raise ValueError("A and B must have the same dtype")
+    if residual is not None:
+        if accumulate_c:
+            raise ValueError("residual and accumulate_c are exclusive")
+        if tuple(residual.shape) != (M, N) or residual.dtype != out.dtype or residual.stride(1) != 1 \
+                or residual.stride(0) != out.stride(0):
+            raise ValueError("residual must be an [M, N] matrix of the output dtype with the output's row stride")
+        _lib.check(_lib.load().lh_hip_gemm_residual(
+            out.data_ptr(), residual.data_ptr(), a.data_ptr(), b.data_ptr(),
+            bias.data_ptr() if bias is not None else None, M, N, K, a.stride(0), b.stride(0), out.stride(0),
+            lh_dtype(a.dtype), lh_dtype(out.dtype), flags, _stream()), "gemm")
+        return out
     _lib.check(_lib.load().lh_hip_gemm(
         out.data_ptr(), a.data_ptr(), b.data_ptr(), bias.data_ptr() if bias is not None else None,
         M, N, K, a.stride(0), b.stride(0), out.stride(0), lh_dtype(a.dtype), lh_dtype(out.dtype), flags, _stream()),

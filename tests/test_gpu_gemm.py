@@ -444,3 +444,27 @@ def test_tile_search_and_database(tmp_path):
     finally:
         use_db(None)
     assert torch.equal(plain, tuned)  # every tile accumulates k in the same order
+
+
+@pytest.mark.parametrize("shape", [(512, 768, 768), (8192, 768, 3072), (130, 264, 64), (96, 50, 40)])
+@pytest.mark.parametrize("elt,out_elt", [("bf16", "bf16"), ("f16", "f16"), ("bf16", "f32"), ("f32", "f32")])
+def test_gemm_residual_input(shape, elt, out_elt):
+    """lh_hip_gemm_residual: the accumulation starts from a separate matrix (the x of x + linear(y)),
+    which is only read; bias is added as in the in-place form.  Shapes cover the staged epilogues
+    of the direct kernels, their edge instantiation and the generic kernel."""
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(M * 7 + N + K)
+    dt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}
+    a = orc.round_to(rng.standard_normal((M, K)).astype(np.float32), elt)
+    b = orc.round_to(rng.standard_normal((K, N)).astype(np.float32) * 0.1, elt)
+    bias = orc.round_to(rng.standard_normal((N,)).astype(np.float32), out_elt)
+    res = orc.round_to(rng.standard_normal((M, N)).astype(np.float32), out_elt)
+    d_res = _dev(res, dt[out_elt])
+    out = ops.gemm(_dev(a, dt[elt]), _dev(b, dt[elt]), _dev(bias, dt[out_elt]), out_dtype=dt[out_elt], residual=d_res)
+    ref = orc.matmul(a, b, c=res, accumulate_c=True, bias=bias, result_type=out_elt)
+    rtol = F32_RTOL if elt == "f32" else BF16_RTOL
+    assert_close(_host(out), ref, rtol, f"{elt}->{out_elt} gemm {shape} + residual")
+    assert np.array_equal(_host(d_res), res), "the residual input was modified"
+    assert out.data_ptr() != d_res.data_ptr()

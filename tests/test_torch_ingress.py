@@ -55,15 +55,37 @@ def test_activation_with_second_user_is_not_fused():
     assert jit.kinds == ["hip.gemm", "hip.relu", "hip.add"]
 
 
+def test_residual_add_is_fused_only_when_the_residual_exists_before_the_linear():
+    class M(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc, self.ln = nn.Linear(8, 8), nn.LayerNorm(8)
+
+        def forward(self, x):
+            early = self.ln(x)
+            a = early + self.fc(x)      # residual computed before the linear: one GEMM
+            h = self.fc(a)
+            late = self.ln(a)           # computed after the linear it is added to: a separate add
+            return h + late
+
+    jit = gpu_backend()(torch.fx.symbolic_trace(M()), [torch.randn(2, 8)])
+    assert jit.kinds == ["hip.layer_norm", "hip.gemm", "hip.gemm", "hip.layer_norm", "hip.add"]
+    assert [s.detail["residual"] for s in jit.plan if s.kind == "hip.gemm"] == [True, False]
+
+
 def test_block_plan_through_dynamo():
     backend = gpu_backend()
     compiled = torch.compile(Block(), backend=backend, dynamic=False)
     with pytest.raises(ValueError, match="compiled for cuda"):  # the plan exists; running needs the GPU
         with torch.no_grad():
             compiled(torch.randn(2, 8, 64))
+    # both residual adds start the accumulation of the projection GEMM in front of them
     assert backend.last_jit_function.kinds == [
-        "hip.layer_norm", "hip.gemm", "hip.attention", "hip.gemm", "hip.add",
-        "hip.layer_norm", "hip.gemm", "hip.gemm", "hip.add"]
+        "hip.layer_norm", "hip.gemm", "hip.attention", "hip.gemm",
+        "hip.layer_norm", "hip.gemm", "hip.gemm"]
+    gemms = [s for s in backend.last_jit_function.plan if s.kind == "hip.gemm"]
+    assert [g.detail["residual"] for g in gemms] == [False, True, False, True]
+    assert [g.detail["activation"] for g in gemms] == [None, None, "gelu", None]
     attn = next(s for s in backend.last_jit_function.plan if s.kind == "hip.attention")
     assert attn.detail["causal"] is True
 
