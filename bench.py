@@ -229,10 +229,10 @@ def main() -> int:
             yb = torch.empty_like(xb)
             ws = torch.empty(ops.nanogpt_block_workspace_bytes(B, T, C, dt), dtype=torch.uint8, device="cuda")
             bflops = 128849018880.0  # causal-halved attention
-            extras[f"nanogpt_block_{name}_tflops"] = rate(lambda: ops.nanogpt_block(xb, p, H, out=yb, workspace=ws), bflops, 30, 10) / 1e12
+            extras[f"nanogpt_block_{name}_tflops"] = rate(lambda: ops.nanogpt_block(xb, p, H, out=yb, workspace=ws), bflops, 200, 50) / 1e12
         try:
             extras["nanogpt_block_bf16_torch_compile_tflops"] = rate(
-                compiled_block_step(torch, g, 8, 1024, 768, 12), 128849018880.0, 30, 10) / 1e12
+                compiled_block_step(torch, g, 8, 1024, 768, 12), 128849018880.0, 200, 50) / 1e12
         except Exception as exc:  # torch.compile's tracer is outside this package: report, do not lose the line
             print(f"bench.py: torch.compile block line skipped: {exc!r}", file=sys.stderr)
         # Vendor library kernels through torch on the same tensors, for orientation only.

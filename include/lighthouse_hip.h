@@ -124,10 +124,11 @@ int lh_hip_gemm(void* out, const void* a, const void* b, const void* bias, int64
 /*
  * lh_hip_gemm whose accumulation starts from a separate matrix: out = epilogue(c + A.B), with
  * `c` [M,N] of out_dtype and row stride ldc (ACCUMULATE_C is implied; c may be `out`, which is
- * lh_hip_gemm with the flag).  The reference's payload accumulates in place only
- * (gpu_mlp_payload.py:123-131); this form is what a residual connection x + linear(y) needs when
- * x must survive (the torch ingress lowers that pattern to one call, and the nanoGPT block
- * kernel sequence uses it internally).
+ * lh_hip_gemm with the flag).  This is emit_mlp_layer's `acc_tensor` argument in its general
+ * form (lighthouse/ingress/mlir_gen/gpu_mlp_payload.py:115,124-127,144); the payload generator
+ * itself only ever passes the output matrix (gpu_mlp_payload.py:83-95).  It is what a residual
+ * connection x + linear(y) needs when x must survive: the torch ingress lowers that pattern to
+ * one call, and the nanoGPT block kernel sequence uses it internally.
  */
 int lh_hip_gemm_residual(void* out, const void* c, const void* a, const void* b, const void* bias, int64_t M,
                          int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype,
