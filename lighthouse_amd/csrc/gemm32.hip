@@ -150,7 +150,7 @@ __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
   constexpr int BM = 64 * TM, BN = 64 * TN;
   constexpr int a_bytes = BM * 128, b_row = BN * 4, stage_bytes = a_bytes + 32 * b_row;
   constexpr int L = C::LA + C::LB;  // loads a lane has in flight per stage
-  static_assert(NS >= 3 && NS <= 6 && L * (NS - 2) < 64, "ring shape");
+  static_assert(NS >= 3 && NS <= 8, "ring shape");
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem32d[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -175,11 +175,18 @@ __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
   }
 
   const int nk = g.K / 32;
+  // G k-steps per barrier.  The 64 x 64 tile runs one wave per SIMD: nobody covers its barrier
+  // wait and the LDS latency of a step's first fragments, so it takes G > 1 steps behind one
+  // barrier (fewer waits, and the next step's first reads are issued under this step's MFMAs).
+  // Loads then run NS - G stages ahead.
+  constexpr int G = (TM == 1 && TN == 1 && NW == 4) ? (NS == 8 ? 4 : NS == 6 ? 2 : 1) : 1;
+  constexpr int kAhead = NS - G;
+  static_assert(NS >= 2 * G && L * (NS - 2 * G) < 64, "ring shape");
   int t = blockIdx.x;  // < ntiles: the grid is never larger than the tile list
   int m0, n0;
   direct32_place<EDGE>(g, xcd_remap(t, ntiles), c, m0, n0);
 #pragma unroll
-  for (int st = 0; st < NS - 1; ++st)
+  for (int st = 0; st < kAhead; ++st)
     if (st < nk) direct32_issue(c, st, smem32d + st * stage_bytes);
   for (;;) {
     f32x16 acc[TN][WTM];
@@ -189,18 +196,27 @@ __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
       for (int j = 0; j < WTM; ++j)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-    for (int kt = 0; kt < nk; ++kt) {
-      // Stages kt + 1 .. kt + NS - 2 may stay in flight (anything issued after them, such as the
-      // previous tile's stores, only makes the wait longer); one asm block per case because a
+    int kt = 0;
+    for (; kt + G <= nk; kt += G) {
+      // Stages kt + G .. kt + NS - G - 1 may stay in flight (anything issued after them, such as
+      // the previous tile's stores, only makes the wait longer); one asm block per case because a
       // __syncthreads() would add a fence that waits for every outstanding load.
-      const int younger = min(nk - 1 - kt, NS - 2);
+      const int younger = min(nk - G - kt, NS - 2 * G);
       if (younger >= 4) direct32_wait_barrier<L * 4>();
       else if (younger == 3) direct32_wait_barrier<L * 3>();
       else if (younger == 2) direct32_wait_barrier<L * 2>();
       else if (younger == 1) direct32_wait_barrier<L>();
       else direct32_wait_barrier<0>();
-      const int nxt = kt + NS - 1;
-      direct32_step(c, acc, smem32d + (kt % NS) * stage_bytes, smem32d + (nxt % NS) * stage_bytes, nxt, nxt < nk);
+#pragma unroll
+      for (int sg = 0; sg < G; ++sg) {
+        const int nxt = kt + kAhead + sg;
+        direct32_step(c, acc, smem32d + ((kt + sg) % NS) * stage_bytes, smem32d + (nxt % NS) * stage_bytes, nxt,
+                      nxt < nk);
+      }
+    }
+    for (; kt < nk; ++kt) {  // G > 1: the steps left over at the end of a tile, every stage issued already
+      direct32_wait_barrier<0>();
+      direct32_step(c, acc, smem32d + (kt % NS) * stage_bytes, smem32d, 0, false);
     }
     const int tn = t + (int)gridDim.x;
     const bool more = tn < ntiles;
@@ -209,7 +225,7 @@ __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
     if (more) {
       direct32_place<EDGE>(g, xcd_remap(tn, ntiles), c, m0, n0);
 #pragma unroll
-      for (int st = 0; st < NS - 1; ++st)
+      for (int st = 0; st < kAhead; ++st)
         if (st < nk) direct32_issue(c, st, smem32d + st * stage_bytes);
     }
     const int elane = lane_now();  // as in direct32_place
@@ -324,8 +340,9 @@ int gemm32(const GemmArgs& g_in, hipStream_t s) {
       if (narrow < wide) return launch_direct32<2, 1, 4, 8>(g, s);
       return launch_direct32<2, 2, 4, 8>(g, s);
     }
-    // Up to two workgroups per CU: a deep ring; more: a shallow ring so that three share a CU.
-    if ((int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64) <= 512) return launch_direct32<1, 1, 6>(g, s);
+    // Up to two rounds of one workgroup per CU: a deep ring, four k-steps per barrier (1024^3: 26.7 ->
+    // 24.3 us); more tiles: a shallow ring so that three workgroups share a CU.
+    if ((int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64) <= 512) return launch_direct32<1, 1, 8>(g, s);
     return launch_direct32<1, 1, 3>(g, s);
   }
   dim3 grid((g.N + 63) / 64, (g.M + 63) / 64);

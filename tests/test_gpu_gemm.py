@@ -24,6 +24,8 @@ def _host(t):
 
 @pytest.mark.parametrize("shape", [(64, 64, 32), (128, 128, 64), (256, 192, 96), (1024, 1024, 1024), (100, 70, 50),
                                    (1, 1, 1), (33, 65, 17),
+                                   # 64 x 64 tiles take four k-steps per barrier: K = 5, 7, 9 and 13 steps
+                                   (128, 128, 160), (192, 64, 224), (64, 128, 288), (256, 256, 416),
                                    # 128 x 128 tiles, two per workgroup; 128 x 64 tiles, three per workgroup; one
                                    (4096, 2048, 64), (4096, 1536, 96), (2048, 2048, 512)])
 @pytest.mark.parametrize("epi", ["none", "bias_relu"])
