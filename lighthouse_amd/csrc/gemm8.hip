@@ -36,7 +36,9 @@ __device__ __forceinline__ void transpose4x4_bytes(uint32_t& r0, uint32_t& r1, u
 constexpr int kBK8 = 128;
 constexpr int kStride8 = kBK8 + 16;  // bytes per LDS row
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+// EDGE_M: M need not be a multiple of the tile: rows past the end are loaded from the last row
+// (their products land in accumulators that are never stored) and the epilogue skips them.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool EDGE_M>
 __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm8_fast(GemmArgs g) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N, TM = WTM / 32, TN = WTN / 32;
@@ -49,7 +51,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm8_fast(GemmArgs g) 
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm0 = (wave / WAVES_N) * WTM, wn0 = (wave % WAVES_N) * WTN;
-  const int tiles_m = g.M / BM, tiles_n = g.N / BN;
+  const int tiles_m = (g.M + BM - 1) / BM, tiles_n = g.N / BN;
   const int id = xcd_remap(blockIdx.x, gridDim.x);
   constexpr int GROUP_M = 4;
   const int group_size = GROUP_M * tiles_n;
@@ -66,7 +68,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm8_fast(GemmArgs g) 
 #pragma unroll
     for (int i = 0; i < A_CH; ++i) {
       int c = tid + i * NT, row = c >> 3, kc = c & 7;
-      ra[i] = *reinterpret_cast<const u32x4*>(A + (int64_t)(m0 + row) * g.lda + k0 + kc * 16);
+      const int arow = EDGE_M ? min(m0 + row, g.M - 1) : m0 + row;
+      ra[i] = *reinterpret_cast<const u32x4*>(A + (int64_t)arow * g.lda + k0 + kc * 16);
     }
 #pragma unroll
     for (int i = 0; i < B_UN; ++i) {
@@ -147,8 +150,9 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm8_fast(GemmArgs g) 
     for (int j = 0; j < TM; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q)
-        epilogue4<LH_BF16>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
-                           acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+        if (!EDGE_M || m_base + 32 * j < g.M)
+          epilogue4<LH_BF16>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                             acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
 }
 
 // ---- direct-to-LDS kernel ---------------------------------------------------------------
@@ -627,21 +631,138 @@ __global__ void __launch_bounds__(256) gemm8_skinny(GemmArgs g, float* partial, 
   for (int i = 0; i < 4; ++i) *reinterpret_cast<f32x4*>(dst + 16 * i) = acc[i];
 }
 
-__global__ void __launch_bounds__(256) gemm8_skinny_reduce(GemmArgs g, const float* partial, int splits) {
+// 16 < M <= 128 (decode batches): the same streaming scheme with MT = 2, 4 or 8 row groups of 16, so
+// that B is still read once.  The A block of a k-step (16 MT rows x 128 bytes; rows >= M repeat the
+// last row) travels through the ring next to the B stage it belongs to, so the K chunk of a
+// workgroup is not limited by an A area and the waits count A and B loads alike.  A stage is
+// 32 + 2 MT KiB; MT <= 4: a ring of 4 stages (the whole 160 KiB of a CU with MT = 4), MT = 8: 3
+// stages of 48 KiB.  Partial sums: partial[split][16 MT][N].
+template <int MT>
+struct SkinnyMt {
+  static constexpr int kStages = MT == 8 ? 3 : 4;
+  static constexpr int kStageBytes = kSkinnyStageBytes + (MT < 4 ? 4 : MT) * 16 * kBK8;
+  static constexpr int kLdsBytes = kStages * kStageBytes;
+};
+
+template <int MT>
+__device__ __forceinline__ void skinny_mt_issue(const uint8_t* const (&b_src)[8], const uint8_t* const (&a_src)[MT / 2],
+                                                int64_t ldb, int kt, int wave, uint8_t* __restrict__ stage) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+    async8_copy16(b_src[i] + (int64_t)(kt * kBK8) * ldb, stage + (4 * i + wave) * 1024);
+#pragma unroll
+  for (int i = 0; i < MT / 2; ++i)
+    async8_copy16(a_src[i] + kt * kBK8, stage + kSkinnyStageBytes + (4 * i + wave) * 1024);
+}
+
+template <int MT>
+__device__ __forceinline__ void skinny_mt_step(f32x4 (&acc)[MT][4], const uint8_t* __restrict__ st,
+                                               uint8_t* __restrict__ wr, const uint8_t* const (&b_src)[8],
+                                               const uint8_t* const (&a_src)[MT / 2], int64_t ldb, int next_kt,
+                                               bool prefetch, int wave, int a_off, int a_swz, int qd, int b_off,
+                                               int b_chunk, int b_swz) {
+  if (prefetch) skinny_mt_issue<MT>(b_src, a_src, ldb, next_kt, wave, wr);
+  const uint8_t* as = st + kSkinnyStageBytes;
+  const int c0 = 2 * qd;
+  i32x8 fa[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    i32x4 alo = *reinterpret_cast<const i32x4*>(as + mt * 2048 + a_off + ((c0 ^ a_swz) << 4));
+    i32x4 ahi = *reinterpret_cast<const i32x4*>(as + mt * 2048 + a_off + (((c0 + 1) ^ a_swz) << 4));
+    fa[mt] = i32x8{alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint8_t* p0 = st + b_off + (((b_chunk + i) ^ b_swz) << 4);
+    i32x2 r[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      r[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(p0 + q * 8 * kSkinnyBN));
+    i32x8 fb = {r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]};
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt][i] = mfma_f8_16(fb, fa[mt], acc[mt][i]);
+  }
+}
+
+template <int MT>
+__global__ void __launch_bounds__(256) gemm8_skinny_mt(GemmArgs g, float* partial, int k_chunk) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_sk[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n0 = blockIdx.x * kSkinnyBN;
+  const int kbeg = blockIdx.y * k_chunk;
+  const int nk = k_chunk / kBK8;
+  const uint8_t* A = reinterpret_cast<const uint8_t*>(g.a);
+  const uint8_t* B = reinterpret_cast<const uint8_t*>(g.b);
+  const int r16 = lane & 15, qd = lane >> 4;
+
+  // A: load i of wave w fills rows (4 i + w) 8 .. +8 of the step's block; lane -> row += lane / 8,
+  // LDS chunk lane % 8 holds global chunk (lane % 8) ^ ((row / 2) % 8).
+  const uint8_t* a_src[MT / 2];
+#pragma unroll
+  for (int i = 0; i < MT / 2; ++i) {
+    const int m = (4 * i + wave) * 8 + (lane >> 3);
+    const int gc = (lane & 7) ^ ((m >> 1) & 7);
+    a_src[i] = A + (int64_t)min(m, g.M - 1) * g.lda + kbeg + gc * 16;
+  }
+  const uint8_t* b_src[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int k = (4 * i + wave) * 4 + (lane >> 4);
+    const int gc = (lane & 15) ^ ((k & 7) | (((k >> 5) & 1) << 3));
+    b_src[i] = B + (int64_t)(kbeg + k) * g.ldb + n0 + gc * 16;
+  }
+#pragma unroll
+  for (int st = 0; st < SkinnyMt<MT>::kStages - 1; ++st)
+    if (st < nk) skinny_mt_issue<MT>(b_src, a_src, g.ldb, st, wave, smem_sk + st * SkinnyMt<MT>::kStageBytes);
+
+  const int a_off = r16 * 128, a_swz = (r16 >> 1) & 7;
+  const int b_off = (32 * qd + (r16 >> 1)) * kSkinnyBN + 8 * (r16 & 1);
+  const int b_chunk = 4 * wave;
+  const int b_swz = (r16 >> 1) | ((qd & 1) << 3);
+
+  f32x4 acc[MT][4];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[mt][i][v] = 0.0f;
+
+  constexpr int L = 8 + MT / 2;  // loads per lane and stage
+  for (int kt = 0; kt < nk; ++kt) {
+    const int younger = min(nk - 1 - kt, SkinnyMt<MT>::kStages - 2);
+    if (younger >= 2) skinny_wait_barrier<2 * L>();
+    else if (younger == 1) skinny_wait_barrier<L>();
+    else skinny_wait_barrier<0>();
+    const int nxt = kt + SkinnyMt<MT>::kStages - 1;
+    skinny_mt_step<MT>(acc, smem_sk + (kt % SkinnyMt<MT>::kStages) * SkinnyMt<MT>::kStageBytes,
+                       smem_sk + (nxt % SkinnyMt<MT>::kStages) * SkinnyMt<MT>::kStageBytes, b_src, a_src, g.ldb, nxt, nxt < nk, wave,
+                       a_off, a_swz, qd, b_off, b_chunk, b_swz);
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    float* dst = partial + ((int64_t)blockIdx.y * (16 * MT) + 16 * mt + r16) * g.N + n0 + wave * 64 + 4 * qd;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<f32x4*>(dst + 16 * i) = acc[mt][i];
+  }
+}
+
+__global__ void __launch_bounds__(256) gemm8_skinny_reduce(GemmArgs g, const float* partial, int splits, int rows) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (int64_t)g.M * g.N) return;
   const int m = (int)(idx / g.N), n = (int)(idx % g.N);
   float s = 0.0f;
-  for (int sp = 0; sp < splits; ++sp) s += partial[((int64_t)sp * 16 + m) * g.N + n];
+  for (int sp = 0; sp < splits; ++sp) s += partial[((int64_t)sp * rows + m) * g.N + n];
   epilogue1<LH_BF16>(g, m, n, s);
 }
 
 static float* g_partial = nullptr;
 static size_t g_partial_bytes = 0;
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool EDGE_M = false>
 static int launch_fast8(const GemmArgs& g, hipStream_t s) {
-  auto kern = gemm8_fast<BM, BN, WAVES_M, WAVES_N>;
+  auto kern = gemm8_fast<BM, BN, WAVES_M, WAVES_N, EDGE_M>;
   constexpr size_t lds = (size_t)2 * (BM + BN) * kStride8;
   static bool configured = false;
   if (!configured) {
@@ -649,8 +770,43 @@ static int launch_fast8(const GemmArgs& g, hipStream_t s) {
                                      (int)lds));
     configured = true;
   }
-  hipLaunchKernelGGL(kern, dim3((g.M / BM) * (g.N / BN)), dim3(WAVES_M * WAVES_N * 64), lds, s, g);
+  hipLaunchKernelGGL(kern, dim3(((g.M + BM - 1) / BM) * (g.N / BN)), dim3(WAVES_M * WAVES_N * 64), lds, s, g);
   return check_launch("gemm8_fast");
+}
+
+static int skinny_partial_buffer(size_t need) {
+  if (need > g_partial_bytes) {
+    if (g_partial) LH_HIP_CHECK(hipFree(g_partial));
+    g_partial = nullptr;
+    g_partial_bytes = 0;
+    LH_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&g_partial), need));
+    g_partial_bytes = need;
+  }
+  return LH_OK;
+}
+
+template <int MT>
+static int launch_skinny_mt(const GemmArgs& g, hipStream_t s) {
+  // Split K until about one workgroup per CU streams B.
+  const int nblk = g.N / kSkinnyBN;
+  int splits = 1;
+  while (nblk * splits < num_cus() && (g.K / kBK8) % (splits * 2) == 0) splits *= 2;
+  int rc = skinny_partial_buffer((size_t)splits * 16 * MT * g.N * sizeof(float));
+  if (rc) return rc;
+  static bool configured = false;
+  if (!configured) {
+    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_skinny_mt<MT>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, SkinnyMt<MT>::kLdsBytes));
+    configured = true;
+  }
+  hipLaunchKernelGGL(gemm8_skinny_mt<MT>, dim3(nblk, splits), dim3(256), SkinnyMt<MT>::kLdsBytes, s, g, g_partial,
+                     g.K / splits);
+  rc = check_launch("gemm8_skinny_mt");
+  if (rc) return rc;
+  const int64_t total = (int64_t)g.M * g.N;
+  hipLaunchKernelGGL(gemm8_skinny_reduce, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, g, g_partial, splits,
+                     16 * MT);
+  return check_launch("gemm8_skinny_reduce");
 }
 
 int gemm8(const GemmArgs& g, hipStream_t s) {
@@ -663,14 +819,8 @@ int gemm8(const GemmArgs& g, hipStream_t s) {
     int splits = 1;
     while ((nblk * splits < num_cus() || g.K / splits > kSkinnyMaxChunk) && (g.K / kBK8) % (splits * 2) == 0) splits *= 2;
     if (g.K / splits <= kSkinnyMaxChunk) {
-      const size_t need = (size_t)splits * 16 * g.N * sizeof(float);
-      if (need > g_partial_bytes) {
-        if (g_partial) LH_HIP_CHECK(hipFree(g_partial));
-        g_partial = nullptr;
-        g_partial_bytes = 0;
-        LH_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&g_partial), need));
-        g_partial_bytes = need;
-      }
+      int prc = skinny_partial_buffer((size_t)splits * 16 * g.N * sizeof(float));
+      if (prc) return prc;
       static bool configured = false;
       if (!configured) {
         LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_skinny),
@@ -682,9 +832,14 @@ int gemm8(const GemmArgs& g, hipStream_t s) {
       if (rc) return rc;
       const int64_t total = (int64_t)g.M * g.N;
       hipLaunchKernelGGL(gemm8_skinny_reduce, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, g, g_partial,
-                         splits);
+                         splits, 16);
       return check_launch("gemm8_skinny_reduce");
     }
+  }
+  if (vec_ok && g.M > 16 && g.M <= 128 && g.N % kSkinnyBN == 0 && g.ldb % 16 == 0) {
+    if (g.M <= 32) return launch_skinny_mt<2>(g, s);
+    if (g.M <= 64) return launch_skinny_mt<4>(g, s);
+    return launch_skinny_mt<8>(g, s);
   }
   if (vec_ok && g.M % 256 == 0 && g.N % 256 == 0 && (int64_t)(g.M / 256) * (g.N / 256) >= 128) {
     // the direct kernel addresses a tile's rows with 32-bit byte offsets from the tile's origin
@@ -692,6 +847,7 @@ int gemm8(const GemmArgs& g, hipStream_t s) {
     return launch_fast8<256, 256, 2, 4>(g, s);
   }
   if (vec_ok && g.M % 128 == 0 && g.N % 128 == 0) return launch_fast8<128, 128, 2, 2>(g, s);
+  if (vec_ok && g.N % 128 == 0) return launch_fast8<128, 128, 2, 2, true>(g, s);  // any M
   dim3 grid((g.N + 31) / 32, (g.M + 31) / 32);
   hipLaunchKernelGGL(gemm8_generic, grid, dim3(64), 0, s, g);
   return check_launch("gemm8_generic");

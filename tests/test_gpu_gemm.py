@@ -424,6 +424,33 @@ def test_gemm_fp8_decode_path(shape):
     assert_close(_host(out32), orc.matmul_fp8(aq, bq, sa, sb, result_type="f32"), FP8_RTOL, f"fp8 decode f32 {shape}")
 
 
+@pytest.mark.parametrize("shape", [(17, 256, 1024), (32, 1024, 4096), (33, 512, 2048), (48, 256, 384),
+                                   (64, 2048, 8192), (64, 8192, 8192), (65, 512, 1024), (100, 1024, 2048),
+                                   (128, 8192, 8192),
+                                   # M that no tile divides, N a multiple of 128: the fast kernel's M-edge form
+                                   (100, 384, 512), (129, 256, 256), (1000, 1024, 1024)])
+def test_gemm_fp8_decode_batches_and_ragged_m(shape):
+    """16 < M <= 128: the streaming kernel with 2, 4 or 8 row groups (B still read once; rows past M
+    repeat the last row and are not stored); other M: tile kernel with clamped rows.  Run twice
+    (the partial-sum buffer is reused) with a guard row behind the output."""
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(11 + M + N + K)
+    aq, sa = orc.quantize_per_tensor_e4m3(rng.standard_normal((M, K)).astype(np.float32))
+    bq, sb = orc.quantize_per_tensor_e4m3(rng.standard_normal((K, N)).astype(np.float32))
+    da = torch.from_numpy(aq).to("cuda").view(torch.float8_e4m3fn)
+    db = torch.from_numpy(bq).to("cuda").view(torch.float8_e4m3fn)
+    ref = orc.matmul_fp8(aq, bq, sa, sb, result_type="bf16")
+    buf = torch.full((M + 1, N), 7.0, device="cuda", dtype=torch.bfloat16)
+    for _ in range(2):
+        ops.gemm_fp8(da, db, float(sa), float(sb), out=buf[:M])
+        assert_close(_host(buf[:M]), ref, FP8_RTOL, f"fp8 gemm {shape}")
+        assert bool((buf[M] == 7.0).all()), "a row past M was written"
+    out32 = ops.gemm_fp8(da, db, float(sa), float(sb), out_dtype=torch.float32)
+    assert_close(_host(out32), orc.matmul_fp8(aq, bq, sa, sb, result_type="f32"), FP8_RTOL, f"fp8 f32 {shape}")
+
+
 def test_tile_search_and_database(tmp_path):
     """The tuner times every fitting tile for a shape, logs the trials, records the winner, and
     ops.gemm picks the recorded tile up when the database is in use (same results either way)."""
