@@ -164,6 +164,10 @@ int transpose_matrix(void* out, const void* in, int R, int C, int64_t ld_in, int
 // ends); calls that use it on different streams at the same time race.  nullptr on failure
 // (the error message is set).
 void* transpose_scratch(size_t bytes);
+// dst (rows_dst x cols_dst) = src (rows_src x cols_src) padded with zeros or cut; any alignment.
+int pad_copy_matrix(void* dst, int64_t ld_dst, int rows_dst, int cols_dst, const void* src, int64_t ld_src, int rows_src,
+                    int cols_src, int elem_bytes, hipStream_t s);
+void* pad_scratch(size_t bytes);
 // Compute units of the current device (cached; 256 if the query fails).
 int num_cus();
 

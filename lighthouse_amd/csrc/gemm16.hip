@@ -816,6 +816,12 @@ static int gemm16_dispatch(const GemmArgs& g_in, hipStream_t s) {
                       aligned16(g.a) && aligned16(g.b) && aligned16(g.out) &&
                       (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias));
   const uint32_t tile = g.flags & LH_GEMM_TILE_MASK;
+  if (tile == LH_GEMM_TILE_AUTO && !(vec_ok && !tb && g.ldc % 8 == 0 && g.N % 8 == 0) &&
+      (int64_t)g.M * g.N * g.K >= (1 << 22)) {
+    // not a shape for the direct kernels as it stands: run it on padded copies of the operands
+    const int rc = gemm_padded<2>(g, kBK, 8, s, [&](const GemmArgs& p) { return gemm16_dispatch<DT>(p, s); });
+    if (rc <= 0) return rc;
+  }
   if (tile != LH_GEMM_TILE_AUTO) {
     static const int bm[4] = {256, 256, 128, 128}, bn[4] = {256, 128, 256, 128};
     const int v = (int)(tile >> 8) - 1;

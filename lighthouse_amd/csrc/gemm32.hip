@@ -328,6 +328,11 @@ int gemm32(const GemmArgs& g_in, hipStream_t s) {
   const bool vec_ok = !trans && g.K % kBK32 == 0 && g.lda % 4 == 0 && g.ldb % 4 == 0 && g.ldc % 4 == 0 &&
                       aligned16(g.a) && aligned16(g.b) && aligned16(g.out) &&
                       (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias));
+  if (!(vec_ok && g.N % 4 == 0) && (int64_t)g.M * g.N * g.K >= (1 << 22)) {
+    // not a shape for the direct kernels as it stands: run it on padded copies of the operands
+    const int rc = gemm_padded<4>(g, kBK32, 4, s, [&](const GemmArgs& p) { return gemm32(p, s); });
+    if (rc <= 0) return rc;
+  }
   if (vec_ok && g.N % 4 == 0) {
     // Tiles are counted with edge tiles in full (M, N need not be multiples of a tile).
     const int cus = num_cus();

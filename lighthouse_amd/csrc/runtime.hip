@@ -96,25 +96,67 @@ int transpose_matrix(void* out, const void* in, int R, int C, int64_t ld_in, int
   return check_launch("transpose_tiles");
 }
 
+// dst[r][c] = src[r][c] inside the source matrix, 0 outside: the copies of a GEMM whose K or N the
+// fast kernels cannot take (and the copy of its padded result back).  Any alignment on either side;
+// a thread handles 8 consecutive elements of a row.
+template <typename T>
+__global__ void __launch_bounds__(256) pad_copy_kernel(T* dst, int64_t ld_dst, int rows_dst, int cols_dst, const T* src,
+                                                       int64_t ld_src, int rows_src, int cols_src) {
+  const int r = blockIdx.y;
+  const int c0 = (blockIdx.x * 256 + threadIdx.x) * 8;
+  if (c0 >= cols_dst) return;
+  T* d = dst + (int64_t)r * ld_dst + c0;
+  const T* sp = src + (int64_t)r * ld_src + c0;
+  const bool row_in = r < rows_src;
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    if (c0 + e < cols_dst) d[e] = (row_in && c0 + e < cols_src) ? sp[e] : (T)0;
+}
+
+int pad_copy_matrix(void* dst, int64_t ld_dst, int rows_dst, int cols_dst, const void* src, int64_t ld_src, int rows_src,
+                    int cols_src, int elem_bytes, hipStream_t s) {
+  if (rows_dst <= 0 || cols_dst <= 0) return LH_OK;
+  const dim3 grid((cols_dst + 2047) / 2048, rows_dst);
+  if (elem_bytes == 2)
+    hipLaunchKernelGGL(pad_copy_kernel<uint16_t>, grid, dim3(256), 0, s, static_cast<uint16_t*>(dst), ld_dst, rows_dst,
+                       cols_dst, static_cast<const uint16_t*>(src), ld_src, rows_src, cols_src);
+  else if (elem_bytes == 4)
+    hipLaunchKernelGGL(pad_copy_kernel<uint32_t>, grid, dim3(256), 0, s, static_cast<uint32_t*>(dst), ld_dst, rows_dst,
+                       cols_dst, static_cast<const uint32_t*>(src), ld_src, rows_src, cols_src);
+  else
+    return fail(LH_ERR_UNSUPPORTED, "pad copy: element size %d", elem_bytes);
+  return check_launch("pad_copy");
+}
+
 static char* g_transpose_scratch = nullptr;
 static size_t g_transpose_scratch_bytes = 0;
 
-void* transpose_scratch(size_t bytes) {
-  if (bytes > g_transpose_scratch_bytes) {
-    if (g_transpose_scratch && hipFree(g_transpose_scratch) != hipSuccess) (void)hipGetLastError();
-    g_transpose_scratch = nullptr;
-    g_transpose_scratch_bytes = 0;
-    const hipError_t e = hipMalloc(reinterpret_cast<void**>(&g_transpose_scratch), bytes);
+// Library-owned buffers that only grow (hipFree waits for the work that may still use the old one).
+static void* grow_buffer(char*& buf, size_t& have, size_t bytes, const char* what) {
+  if (bytes > have) {
+    if (buf && hipFree(buf) != hipSuccess) (void)hipGetLastError();
+    buf = nullptr;
+    have = 0;
+    const hipError_t e = hipMalloc(reinterpret_cast<void**>(&buf), bytes);
     if (e != hipSuccess) {
       (void)hipGetLastError();
-      set_error("transpose scratch: hipMalloc of %zu bytes failed: %s", bytes, hipGetErrorString(e));
-      g_transpose_scratch = nullptr;
+      set_error("%s: hipMalloc of %zu bytes failed: %s", what, bytes, hipGetErrorString(e));
+      buf = nullptr;
       return nullptr;
     }
-    g_transpose_scratch_bytes = bytes;
+    have = bytes;
   }
-  return g_transpose_scratch;
+  return buf;
 }
+
+void* transpose_scratch(size_t bytes) {
+  return grow_buffer(g_transpose_scratch, g_transpose_scratch_bytes, bytes, "transpose scratch");
+}
+
+static char* g_pad_scratch = nullptr;
+static size_t g_pad_scratch_bytes = 0;
+
+void* pad_scratch(size_t bytes) { return grow_buffer(g_pad_scratch, g_pad_scratch_bytes, bytes, "padding scratch"); }
 
 }  // namespace lh
 

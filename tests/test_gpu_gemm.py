@@ -451,6 +451,46 @@ def test_gemm_fp8_decode_batches_and_ragged_m(shape):
     assert_close(_host(out32), orc.matmul_fp8(aq, bq, sa, sb, result_type="f32"), FP8_RTOL, f"fp8 f32 {shape}")
 
 
+@pytest.mark.parametrize("elt", ["bf16", "f16", "f32"])
+@pytest.mark.parametrize("shape", [(512, 521, 200), (300, 1000, 1000), (257, 136, 4100), (1024, 4097, 96)])
+@pytest.mark.parametrize("epi", ["none", "bias_relu", "acc", "residual"])
+def test_gemm_shapes_run_on_padded_copies(shape, elt, epi):
+    """K that is no multiple of the k-step, N that is no multiple of the vector width (rows of B
+    and of the output not 16-byte aligned): operands are copied into zero-padded library buffers,
+    the direct kernels run, the result is copied back.  The output is a view with two guard
+    columns, which must stay as they were."""
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(M + 3 * N + 7 * K)
+    dt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[elt]
+    a = orc.round_to(rng.standard_normal((M, K)).astype(np.float32), elt)
+    b = orc.round_to(rng.standard_normal((K, N)).astype(np.float32) * 0.1, elt)
+    bias = orc.round_to(rng.standard_normal((N,)).astype(np.float32), elt)
+    c = orc.round_to(rng.standard_normal((M, N)).astype(np.float32), elt)
+    da, db = _dev(a, dt), _dev(b, dt)
+    buf = torch.full((M, N + 2), 5.0, device="cuda", dtype=dt)
+    out = buf[:, :N]
+    if epi == "none":
+        ops.gemm(da, db, out=out)
+        ref = orc.matmul(a, b, result_type=elt)
+    elif epi == "bias_relu":
+        ops.gemm(da, db, _dev(bias, dt), relu=True, out=out)
+        ref = orc.matmul(a, b, bias=bias, relu=True, result_type=elt)
+    elif epi == "acc":
+        out.copy_(_dev(c, dt))
+        ops.gemm(da, db, out=out, accumulate_c=True)
+        ref = orc.matmul(a, b, c=c, accumulate_c=True, result_type=elt)
+    else:
+        res = torch.full((M, N + 2), 0.0, device="cuda", dtype=dt)
+        res[:, :N] = _dev(c, dt)
+        ops.gemm(da, db, _dev(bias, dt), out=out, residual=res[:, :N])
+        ref = orc.matmul(a, b, c=c, accumulate_c=True, bias=bias, result_type=elt)
+    rtol = F32_RTOL if elt == "f32" else BF16_RTOL
+    assert_close(_host(out), ref, rtol, f"{elt} gemm {shape} {epi} (padded)")
+    assert bool((buf[:, N:] == 5.0).all()), "columns behind the output were written"
+
+
 def test_tile_search_and_database(tmp_path):
     """The tuner times every fitting tile for a shape, logs the trials, records the winner, and
     ops.gemm picks the recorded tile up when the database is in use (same results either way)."""
