@@ -652,6 +652,190 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
   return attention16_launch_nq<DT, 2, 4>(a, s);
 }
 
+// 16-bit tensors, head dimension D = 32 DB other than 64 (32, 96, 128, 192, 256): the same
+// transposed formulation on the matrix cores (S^T = K Q^T, O^T = V^T P^T, a lane owns a query row)
+// without the streaming machinery of the head-dimension-64 kernel.  A workgroup owns 128 query
+// rows (4 waves x 32); a tile of 64 keys is copied through registers into LDS, K row-major with
+// rows padded by 16 bytes, V transposed (rows = head-dim columns, 64 keys + 16 bytes), two
+// barriers per tile.  Row statistics follow the plain online-softmax recurrence (maximum per
+// tile).  Any sequence length: keys past the end are loaded from the last key and masked, rows
+// past the end are computed on the last row and not stored.
+template <int DT, int DB>
+__global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kernel(AttnArgs a) {
+  constexpr int D = 32 * DB;
+  constexpr int KROW = D + 8, VROW = kKvTile + 8;  // elements per LDS row
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem_anyd[];
+  uint16_t* Ks = reinterpret_cast<uint16_t*>(smem_anyd);  // [64][KROW]
+  uint16_t* Vt = Ks + kKvTile * KROW;                     // [D][VROW]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r32 = lane & 31, h = lane >> 5;
+  const int nqb = (a.T + 127) / 128;
+  const int qb = a.causal ? nqb - 1 - (int)blockIdx.x : (int)blockIdx.x;  // causal: heavy blocks first
+  const int bh = blockIdx.y;
+  const int z = bh / a.H, hd = bh % a.H;
+  const int q0 = qb * 128, wq0 = q0 + 32 * wave;
+  const bool wave_valid = wq0 < a.T;
+
+  const uint16_t* Q = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)z * a.sq.z + (int64_t)hd * a.sq.h;
+  const uint16_t* K = reinterpret_cast<const uint16_t*>(a.k) + (int64_t)z * a.sk.z + (int64_t)hd * a.sk.h;
+  const uint16_t* V = reinterpret_cast<const uint16_t*>(a.v) + (int64_t)z * a.sv.z + (int64_t)hd * a.sv.h;
+  uint16_t* O = reinterpret_cast<uint16_t*>(a.out) + (int64_t)z * a.so.z + (int64_t)hd * a.so.h;
+
+  // Q fragments (second MFMA operand of S^T), times scale * log2(e): lane (row r32, half h) holds
+  // Q[row][16 sd + 8 h .. +8].  They live in registers, or for the largest head dimension (whose
+  // output accumulators alone take 128 registers) in the wave's own 16 KiB of LDS, in fragment order.
+  constexpr bool Q_LDS = DB >= 8;
+  u32x4 qf[Q_LDS ? 1 : D / 16];
+  u32x4* q_lds = reinterpret_cast<u32x4*>(Vt + D * VROW) + wave * (D / 16) * 64 + lane;
+  {
+    const int row = min(wq0 + r32, a.T - 1);
+#pragma unroll
+    for (int sd = 0; sd < D / 16; ++sd) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(Q + (int64_t)row * a.sq.t + 16 * sd + 8 * h);
+      u32x4 scaled;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        scaled[e] = pack2<DT>(unpack_lo<DT>(raw[e]) * a.scale_log2e, unpack_hi<DT>(raw[e]) * a.scale_log2e);
+      if constexpr (Q_LDS) q_lds[sd * 64] = scaled;
+      else qf[sd] = scaled;
+    }
+  }
+  f32x16 acc_o[DB];
+#pragma unroll
+  for (int j = 0; j < DB; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc_o[j][v] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  const int kv_end = a.causal ? min(a.T, q0 + 128) : a.T;
+  const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
+  for (int jt = 0; jt < ntiles; ++jt) {
+    const int j0 = jt * kKvTile;
+    __syncthreads();  // the previous tile has been consumed
+    // 8 D 16-byte chunks per tile and tensor, DB per thread: chunk c = key c / (D / 8), columns 8 (c % (D / 8)) .. +8.
+#pragma unroll
+    for (int i = 0; i < DB; ++i) {
+      const int c = tid + 256 * i, key = c / (D / 8), ch = c % (D / 8);
+      const int kg = min(j0 + key, a.T - 1);
+      const u32x4 kv = *reinterpret_cast<const u32x4*>(K + (int64_t)kg * a.sk.t + 8 * ch);
+      const u32x4 vv = *reinterpret_cast<const u32x4*>(V + (int64_t)kg * a.sv.t + 8 * ch);
+      *reinterpret_cast<u32x4*>(Ks + key * KROW + 8 * ch) = kv;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) Vt[(8 * ch + e) * VROW + key] = (uint16_t)(vv[e >> 1] >> (16 * (e & 1)));
+    }
+    __syncthreads();
+    if (!wave_valid || (a.causal && j0 > wq0 + 31)) continue;
+    // S^T = K Q^T - nothing: the accumulators are the scores times scale * log2(e).
+    f32x16 s_acc[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s_acc[i][v] = 0.0f;
+#pragma unroll
+      for (int sd = 0; sd < D / 16; ++sd) {
+        const u32x4 kf = *reinterpret_cast<const u32x4*>(Ks + (32 * i + r32) * KROW + 16 * sd + 8 * h);
+        if constexpr (Q_LDS) s_acc[i] = mfma16<DT>(kf, q_lds[sd * 64], s_acc[i]);
+        else s_acc[i] = mfma16<DT>(kf, qf[sd], s_acc[i]);
+      }
+    }
+    // s_acc[i][v] = score of (query wq0 + r32, key j0 + 32 i + 8 (v / 4) + 4 h + v % 4)
+    if ((a.causal && j0 + kKvTile - 1 > wq0) || j0 + kKvTile > a.T) {
+      const int last = a.causal ? min(wq0 + r32, a.T - 1) : a.T - 1;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          if (j0 + 32 * i + 8 * (v >> 2) + 4 * h + (v & 3) > last) s_acc[i][v] = -INFINITY;
+    }
+    float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
+#pragma unroll
+    for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[0][v]), s_acc[1][v]);
+    mx = halfwave_max(mx);
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // a row without a visible key so far
+    const float alpha = exp2_fast(m_run - m_safe);
+    m_run = m_new;
+    float p[2][16];
+    float l_tile = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        p[i][v] = exp2_fast(s_acc[i][v] - m_safe);
+        l_tile += p[i][v];
+      }
+    l_run = l_run * alpha + l_tile;
+#pragma unroll
+    for (int j = 0; j < DB; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc_o[j][v] *= alpha;
+    // O^T += V^T P^T.  The packed P registers of lane half h hold keys 4 h .. 4 h + 3 and
+    // 8 + 4 h .. 8 + 4 h + 3 of a 16-key step, so the V^T fragment is read in that order.
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        u32x4 pf;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) pf[d] = pack2<DT>(p[i][8 * u + 2 * d], p[i][8 * u + 2 * d + 1]);
+#pragma unroll
+        for (int j = 0; j < DB; ++j) {
+          const uint16_t* vrow = Vt + (32 * j + r32) * VROW + 32 * i + 16 * u + 4 * h;
+          const u32x2 lo = *reinterpret_cast<const u32x2*>(vrow), hi = *reinterpret_cast<const u32x2*>(vrow + 8);
+          acc_o[j] = mfma16<DT>(u32x4{lo[0], lo[1], hi[0], hi[1]}, pf, acc_o[j]);
+        }
+      }
+  }
+  // acc_o[j][v] = O[q = wq0 + r32][d = 32 j + 8 (v / 4) + 4 h + v % 4] * l
+  if (!wave_valid) return;
+  const float inv_l = 1.0f / halfwave_sum(l_run);
+  if (wq0 + r32 >= a.T) return;
+  uint16_t* orow = O + (int64_t)(wq0 + r32) * a.so.t;
+#pragma unroll
+  for (int j = 0; j < DB; ++j)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      u32x2 w = {pack2<DT>(acc_o[j][4 * g] * inv_l, acc_o[j][4 * g + 1] * inv_l),
+                 pack2<DT>(acc_o[j][4 * g + 2] * inv_l, acc_o[j][4 * g + 3] * inv_l)};
+      *reinterpret_cast<u32x2*>(orow + 32 * j + 8 * g + 4 * h) = w;
+    }
+}
+
+template <int DT, int DB>
+static int attention16_anyd_launch(const AttnArgs& a, hipStream_t s) {
+  constexpr int D = 32 * DB;
+  constexpr size_t lds = (size_t)(kKvTile * (D + 8) + D * (kKvTile + 8)) * 2 + (DB >= 8 ? 4 * 32 * D * 2 : 0);
+  auto kern = attention16_anyd_kernel<DT, DB>;
+  static bool configured = false;
+  if (!configured) {
+    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)lds));
+    configured = true;
+  }
+  hipLaunchKernelGGL(kern, dim3((a.T + 127) / 128, a.Z * a.H), dim3(256), lds, s, a);
+  return check_launch("attention16_anyd");
+}
+
+// Returns 1 when no instantiation takes the head dimension.
+template <int DT>
+static int attention16_anyd_dispatch(const AttnArgs& a, int d, hipStream_t s) {
+  switch (d) {
+    case 32: return attention16_anyd_launch<DT, 1>(a, s);
+    case 96: return attention16_anyd_launch<DT, 3>(a, s);
+    case 128: return attention16_anyd_launch<DT, 4>(a, s);
+    case 192: return attention16_anyd_launch<DT, 6>(a, s);
+    case 256: return attention16_anyd_launch<DT, 8>(a, s);
+    default: return 1;
+  }
+}
+
+int attention16_anyd(const AttnArgs& a, int d, int dtype, hipStream_t s) {
+  if (dtype == LH_BF16) return attention16_anyd_dispatch<LH_BF16>(a, d, s);
+  if (dtype == LH_F16) return attention16_anyd_dispatch<LH_F16>(a, d, s);
+  return 1;
+}
+
 // Any sequence length and head dimension up to 256: one wave per query row, keys in chunks of 64
 // (one per lane), the same online-softmax recurrence and rounding points as the fast kernels
 // (f32 statistics, P rounded to the element type before P V, output rounded once).  Throughput is
@@ -764,9 +948,10 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   // generic kernel.
   const int vec = (dtype == LH_F32) ? 4 : 8;  // elements per 16-byte access
   // (the kernels mask a partial last key tile and skip rows past the end themselves)
-  bool fast = d == kHeadDim;
-  for (int i = 0; i < 4 && fast; ++i)
-    fast = ss[i]->t % vec == 0 && ss[i]->h % vec == 0 && ss[i]->z % vec == 0 && aligned16(ps[i]);
+  bool vec_ok = true;
+  for (int i = 0; i < 4 && vec_ok; ++i)
+    vec_ok = ss[i]->t % vec == 0 && ss[i]->h % vec == 0 && ss[i]->z % vec == 0 && aligned16(ps[i]);
+  const bool fast = vec_ok && d == kHeadDim;
   if (scale <= 0.0f) scale = 1.0f / sqrtf((float)d);
   AttnArgs a;
   a.out = out; a.q = q; a.k = k; a.v = v;
@@ -776,6 +961,12 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   a.scale_log2e = scale * 1.4426950408889634f;
   a.causal = causal ? 1 : 0;
   a.cus = num_cus();
-  if (!fast) return attention_generic_launch(a, (int)d, dtype, reinterpret_cast<hipStream_t>(stream));
+  if (!fast) {
+    if (vec_ok) {  // 16-bit tensors with another head dimension the matrix-core kernel takes
+      const int rc = attention16_anyd(a, (int)d, dtype, reinterpret_cast<hipStream_t>(stream));
+      if (rc <= 0) return rc;
+    }
+    return attention_generic_launch(a, (int)d, dtype, reinterpret_cast<hipStream_t>(stream));
+  }
   return attention_launch(a, dtype, reinterpret_cast<hipStream_t>(stream));
 }

@@ -152,12 +152,37 @@ def test_attention_scores_outgrow_the_offset(shape, dtype, elt, causal):
 
 
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype,elt", [(torch.bfloat16, "bf16"), (torch.float16, "f16")])
+@pytest.mark.parametrize("shape", [(2, 3, 256, 128), (1, 2, 333, 128), (1, 2, 512, 32), (1, 2, 200, 96), (1, 1, 384, 192),
+                                   (1, 2, 257, 256), (1, 1, 1, 128), (2, 2, 64, 32)])
+def test_attention_other_head_dims_on_the_matrix_cores(shape, dtype, elt, causal):
+    """16-bit tensors with head_dim 32, 96, 128, 192 or 256: the matrix-core kernel for head
+    dimensions other than 64 (key tiles copied through registers, V transposed in LDS), at sequence
+    lengths that are and are not multiples of its 64-key tile and 128-row query block; also on
+    head-innermost views ([batch, seq, heads, d] seen as [batch, heads, seq, d])."""
+    from lighthouse_amd import ops
+
+    Z, H, T, D = shape
+    rng = np.random.default_rng(sum(shape) + 2 * causal)
+    q, k, v = (orc.round_to(rng.standard_normal(shape).astype(np.float32), elt) for _ in range(3))
+    ref = orc.attention(q, k, v, causal=causal, result_type=elt)
+    out = ops.attention(_dev(q, dtype), _dev(k, dtype), _dev(v, dtype), causal=causal)
+    assert_close(_host(out), ref, 2e-2, f"attention {shape} {elt} causal={causal}")
+    # the same problem on strided views
+    qs, ks, vs = (_dev(x, dtype).transpose(1, 2).contiguous().transpose(1, 2) for x in (q, k, v))
+    outs = torch.empty((Z, T, H, D), dtype=dtype, device="cuda").transpose(1, 2)
+    ops.attention(qs, ks, vs, causal=causal, out=outs)
+    assert torch.equal(outs, out)
+
+
+@pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype,elt,rtol", [(torch.bfloat16, "bf16", 2e-2), (torch.float32, "f32", 1e-4)])
-@pytest.mark.parametrize("shape", [(1, 2, 100, 32), (2, 1, 77, 64), (1, 1, 130, 128), (1, 3, 64, 64), (1, 1, 1, 8),
+@pytest.mark.parametrize("shape", [(1, 2, 100, 40), (2, 1, 77, 64), (1, 1, 130, 128), (1, 3, 64, 64), (1, 1, 1, 8),
                                    (1, 1, 200, 256)])
 def test_attention_any_shape(shape, dtype, elt, rtol, causal):
-    """Head dimensions the MFMA kernels do not take run on the generic kernel with the same
-    rounding points (head_dim 64 takes the MFMA kernels at any sequence length)."""
+    """Head dimensions (and element types) the MFMA kernels do not take run on the generic kernel
+    with the same rounding points (16-bit head_dim 32 / 64 / 96 / 128 / 192 / 256 and f32 head_dim 64
+    take the MFMA kernels at any sequence length)."""
     from lighthouse_amd import ops
 
     rng = np.random.default_rng(sum(shape) + causal)
