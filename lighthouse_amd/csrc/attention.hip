@@ -655,18 +655,17 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
 // 16-bit tensors, head dimension D = 32 DB other than 64 (32, 96, 128, 192, 256): the same
 // transposed formulation on the matrix cores (S^T = K Q^T, O^T = V^T P^T, a lane owns a query row)
 // without the streaming machinery of the head-dimension-64 kernel.  A workgroup owns 128 query
-// rows (4 waves x 32); a tile of 64 keys is copied through registers into LDS, K row-major with
-// rows padded by 16 bytes, V transposed (rows = head-dim columns, 64 keys + 16 bytes), two
-// barriers per tile.  Row statistics follow the plain online-softmax recurrence (maximum per
+// rows (4 waves x 32); a tile of 64 keys is copied through registers into LDS, K and V row-major
+// with rows padded by 16 bytes (V^T fragments through ds_read_b64_tr_b16), two barriers per tile.  Row statistics follow the plain online-softmax recurrence (maximum per
 // tile).  Any sequence length: keys past the end are loaded from the last key and masked, rows
 // past the end are computed on the last row and not stored.
 template <int DT, int DB>
 __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kernel(AttnArgs a) {
   constexpr int D = 32 * DB;
-  constexpr int KROW = D + 8, VROW = kKvTile + 8;  // elements per LDS row
+  constexpr int KROW = D + 8;  // elements per LDS row
   extern __shared__ __attribute__((aligned(16))) uint8_t smem_anyd[];
   uint16_t* Ks = reinterpret_cast<uint16_t*>(smem_anyd);  // [64][KROW]
-  uint16_t* Vt = Ks + kKvTile * KROW;                     // [D][VROW]
+  uint16_t* Vs = Ks + kKvTile * KROW;                     // [64][KROW]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, h = lane >> 5;
@@ -687,7 +686,7 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
   // output accumulators alone take 128 registers) in the wave's own 16 KiB of LDS, in fragment order.
   constexpr bool Q_LDS = DB >= 8;
   u32x4 qf[Q_LDS ? 1 : D / 16];
-  u32x4* q_lds = reinterpret_cast<u32x4*>(Vt + D * VROW) + wave * (D / 16) * 64 + lane;
+  u32x4* q_lds = reinterpret_cast<u32x4*>(Vs + kKvTile * KROW) + wave * (D / 16) * 64 + lane;
   {
     const int row = min(wq0 + r32, a.T - 1);
 #pragma unroll
@@ -721,8 +720,7 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
       const u32x4 kv = *reinterpret_cast<const u32x4*>(K + (int64_t)kg * a.sk.t + 8 * ch);
       const u32x4 vv = *reinterpret_cast<const u32x4*>(V + (int64_t)kg * a.sv.t + 8 * ch);
       *reinterpret_cast<u32x4*>(Ks + key * KROW + 8 * ch) = kv;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) Vt[(8 * ch + e) * VROW + key] = (uint16_t)(vv[e >> 1] >> (16 * (e & 1)));
+      *reinterpret_cast<u32x4*>(Vs + key * KROW + 8 * ch) = vv;
     }
     __syncthreads();
     if (!wave_valid || (a.causal && j0 > wq0 + 31)) continue;
@@ -770,8 +768,11 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
     for (int j = 0; j < DB; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc_o[j][v] *= alpha;
-    // O^T += V^T P^T.  The packed P registers of lane half h hold keys 4 h .. 4 h + 3 and
-    // 8 + 4 h .. 8 + 4 h + 3 of a 16-key step, so the V^T fragment is read in that order.
+    // O^T += V^T P^T.  V^T fragments come from the row-major tile through the transposing read:
+    // lane (g4 = lane / 16, j16 = lane % 16) addresses key row 4 h + j16 / 4 of the 16-key step
+    // (+8 for the second read), columns 32 j + 16 (g4 % 2) + 4 (j16 % 4) .. +4, and receives 8 keys
+    // of one column in exactly the key order of the packed P registers.
+    const int tr_row = 4 * h + ((lane & 15) >> 2), tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -781,9 +782,13 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
         for (int d = 0; d < 4; ++d) pf[d] = pack2<DT>(p[i][8 * u + 2 * d], p[i][8 * u + 2 * d + 1]);
 #pragma unroll
         for (int j = 0; j < DB; ++j) {
-          const uint16_t* vrow = Vt + (32 * j + r32) * VROW + 32 * i + 16 * u + 4 * h;
-          const u32x2 lo = *reinterpret_cast<const u32x2*>(vrow), hi = *reinterpret_cast<const u32x2*>(vrow + 8);
-          acc_o[j] = mfma16<DT>(u32x4{lo[0], lo[1], hi[0], hi[1]}, pf, acc_o[j]);
+          const uint16_t* p0 = Vs + (32 * i + 16 * u + tr_row) * KROW + 32 * j + tr_col;
+          const attn_s16x4 lo =
+              __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) attn_s16x4*)p0);
+          const attn_s16x4 hi =
+              __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) attn_s16x4*)(p0 + 8 * KROW));
+          const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+          acc_o[j] = mfma16<DT>(u32x4{l2[0], l2[1], h2[0], h2[1]}, pf, acc_o[j]);
         }
       }
   }
@@ -805,7 +810,7 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
 template <int DT, int DB>
 static int attention16_anyd_launch(const AttnArgs& a, hipStream_t s) {
   constexpr int D = 32 * DB;
-  constexpr size_t lds = (size_t)(kKvTile * (D + 8) + D * (kKvTile + 8)) * 2 + (DB >= 8 ? 4 * 32 * D * 2 : 0);
+  constexpr size_t lds = (size_t)2 * kKvTile * (D + 8) * 2 + (DB >= 8 ? 4 * 32 * D * 2 : 0);
   auto kern = attention16_anyd_kernel<DT, DB>;
   static bool configured = false;
   if (!configured) {
