@@ -163,6 +163,179 @@ __global__ void __launch_bounds__(256) softmax_rows(void* out, const void* x, in
   for (int j = lane; j < N; j += 64) store_from_f32<DT>(out, base + j, expf(load_as_f32<DT>(x, base + j) - mx) / s);
 }
 
+// Long rows (N >= 1024 outside the register-resident cases): one workgroup of 256 threads per row,
+// the same three passes with block-wide reductions; the row comes from HBM once and from the cache
+// twice.  VEC: rows start 16-byte aligned and N % 4 == 0, 4 elements per access.  One wave per row
+// leaves a 50000-column row to 64 lanes and a short matrix to a handful of waves.
+__device__ __forceinline__ float block_reduce(float v, bool is_max, float* red) {
+  v = is_max ? wave_max(v) : wave_sum(v);
+  __syncthreads();  // `red` may still be read from the previous reduction
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  const float a = red[0], b = red[1], c = red[2], d = red[3];
+  return is_max ? fmaxf(fmaxf(a, b), fmaxf(c, d)) : (a + b) + (c + d);
+}
+
+template <int XDT, int ODT, bool VEC>
+__global__ void __launch_bounds__(256) layer_norm_block(void* out, const void* x, const float* gamma, const float* beta,
+                                                        int M, int N, float eps, float inv_n) {
+  __shared__ float red[4];
+  const int64_t base = (int64_t)blockIdx.x * N;
+  const int tid = threadIdx.x;
+  float s = 0.0f;
+  if constexpr (VEC) {
+    for (int j = 4 * tid; j < N; j += 1024) {
+      const f32x4 v = load4<XDT>(x, base + j);
+      s += (v[0] + v[1]) + (v[2] + v[3]);
+    }
+  } else {
+    for (int j = tid; j < N; j += 256) s += load_as_f32<XDT>(x, base + j);
+  }
+  const float mean = block_reduce(s, false, red) * inv_n;
+  float q = 0.0f;
+  if constexpr (VEC) {
+    for (int j = 4 * tid; j < N; j += 1024) {
+      const f32x4 v = load4<XDT>(x, base + j);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) q += (v[e] - mean) * (v[e] - mean);
+    }
+  } else {
+    for (int j = tid; j < N; j += 256) {
+      const float c = load_as_f32<XDT>(x, base + j) - mean;
+      q += c * c;
+    }
+  }
+  const float inv_std = rsqrtf(block_reduce(q, false, red) * inv_n + eps);
+  if constexpr (VEC) {
+    for (int j = 4 * tid; j < N; j += 1024) {
+      const f32x4 v = load4<XDT>(x, base + j);
+      const f32x4 g = *reinterpret_cast<const f32x4*>(gamma + j), b = *reinterpret_cast<const f32x4*>(beta + j);
+      f32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (v[e] - mean) * inv_std * g[e] + b[e];
+      store4<ODT>(out, base + j, o);
+    }
+  } else {
+    for (int j = tid; j < N; j += 256)
+      store_from_f32<ODT>(out, base + j, (load_as_f32<XDT>(x, base + j) - mean) * inv_std * gamma[j] + beta[j]);
+  }
+}
+
+// Rows of up to 16384 elements (N % 4 == 0, aligned) stay in the workgroup's registers between
+// the passes: 16 groups of 4 elements per thread at most, one read and one write per element.
+constexpr int kBlockRegGroups = 16;
+
+template <int XDT, int ODT>
+__global__ void __launch_bounds__(256) layer_norm_block_reg(void* out, const void* x, const float* gamma,
+                                                            const float* beta, int M, int N, float eps, float inv_n) {
+  __shared__ float red[4];
+  const int64_t base = (int64_t)blockIdx.x * N;
+  const int j0 = 4 * threadIdx.x;
+  f32x4 v[kBlockRegGroups];
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kBlockRegGroups; ++i) {
+    v[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (j0 + 1024 * i < N) {
+      v[i] = load4<XDT>(x, base + j0 + 1024 * i);
+      s += (v[i][0] + v[i][1]) + (v[i][2] + v[i][3]);
+    }
+  }
+  const float mean = block_reduce(s, false, red) * inv_n;
+  float q = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kBlockRegGroups; ++i)
+    if (j0 + 1024 * i < N) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) q += (v[i][e] - mean) * (v[i][e] - mean);
+    }
+  const float inv_std = rsqrtf(block_reduce(q, false, red) * inv_n + eps);
+#pragma unroll
+  for (int i = 0; i < kBlockRegGroups; ++i)
+    if (j0 + 1024 * i < N) {
+      const int j = j0 + 1024 * i;
+      const f32x4 g = *reinterpret_cast<const f32x4*>(gamma + j), b = *reinterpret_cast<const f32x4*>(beta + j);
+      f32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (v[i][e] - mean) * inv_std * g[e] + b[e];
+      store4<ODT>(out, base + j, o);
+    }
+}
+
+template <int DT>
+__global__ void __launch_bounds__(256) softmax_block_reg(void* out, const void* x, int M, int N) {
+  __shared__ float red[4];
+  const int64_t base = (int64_t)blockIdx.x * N;
+  const int j0 = 4 * threadIdx.x;
+  f32x4 v[kBlockRegGroups];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < kBlockRegGroups; ++i)
+    if (j0 + 1024 * i < N) {
+      v[i] = load4<DT>(x, base + j0 + 1024 * i);
+      mx = fmaxf(fmaxf(mx, fmaxf(v[i][0], v[i][1])), fmaxf(v[i][2], v[i][3]));
+    }
+  mx = block_reduce(mx, true, red);
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kBlockRegGroups; ++i)
+    if (j0 + 1024 * i < N) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[i][e] = expf(v[i][e] - mx);
+        s += v[i][e];
+      }
+    }
+  s = block_reduce(s, false, red);
+#pragma unroll
+  for (int i = 0; i < kBlockRegGroups; ++i)
+    if (j0 + 1024 * i < N) {
+      f32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = v[i][e] / s;
+      store4<DT>(out, base + j0 + 1024 * i, o);
+    }
+}
+
+template <int DT, bool VEC>
+__global__ void __launch_bounds__(256) softmax_block(void* out, const void* x, int M, int N) {
+  __shared__ float red[4];
+  const int64_t base = (int64_t)blockIdx.x * N;
+  const int tid = threadIdx.x;
+  float mx = -INFINITY;
+  if constexpr (VEC) {
+    for (int j = 4 * tid; j < N; j += 1024) {
+      const f32x4 v = load4<DT>(x, base + j);
+      mx = fmaxf(fmaxf(mx, fmaxf(v[0], v[1])), fmaxf(v[2], v[3]));
+    }
+  } else {
+    for (int j = tid; j < N; j += 256) mx = fmaxf(mx, load_as_f32<DT>(x, base + j));
+  }
+  mx = block_reduce(mx, true, red);
+  float s = 0.0f;
+  if constexpr (VEC) {
+    for (int j = 4 * tid; j < N; j += 1024) {
+      const f32x4 v = load4<DT>(x, base + j);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s += expf(v[e] - mx);
+    }
+  } else {
+    for (int j = tid; j < N; j += 256) s += expf(load_as_f32<DT>(x, base + j) - mx);
+  }
+  s = block_reduce(s, false, red);
+  if constexpr (VEC) {
+    for (int j = 4 * tid; j < N; j += 1024) {
+      const f32x4 v = load4<DT>(x, base + j);
+      f32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = expf(v[e] - mx) / s;
+      store4<DT>(out, base + j, o);
+    }
+  } else {
+    for (int j = tid; j < N; j += 256) store_from_f32<DT>(out, base + j, expf(load_as_f32<DT>(x, base + j) - mx) / s);
+  }
+}
+
 enum { EW_GELU = 0, EW_ADD = 1, EW_BIAS = 2, EW_BIAS_RELU = 3 };
 
 // n4 groups of 4 elements; `N` is the row length for the bias kinds.
@@ -248,6 +421,17 @@ static int layer_norm_launch(void* out, const void* x, const float* gamma, const
     }
   }
 #undef LH_LN_CASE
+  const bool vec4 = N % 4 == 0 && aligned16(out) && aligned16(x) && aligned16(gamma) && aligned16(beta);
+  if (N >= 1024 || (vec4 && N >= 512)) {
+    if (vec4 && N <= 1024 * kBlockRegGroups)
+      hipLaunchKernelGGL((layer_norm_block_reg<XDT, ODT>), dim3(M), block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);
+    else if (vec4)
+      hipLaunchKernelGGL((layer_norm_block<XDT, ODT, true>), dim3(M), block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);
+    else
+      hipLaunchKernelGGL((layer_norm_block<XDT, ODT, false>), dim3(M), block, 0, s, out, x, gamma, beta, M, N, eps,
+                         inv_n);
+    return check_launch("layer_norm_block");
+  }
   hipLaunchKernelGGL((layer_norm_generic<XDT, ODT>), grid, block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);
   return check_launch("layer_norm_generic");
 }
@@ -315,6 +499,22 @@ int lh_hip_softmax(void* out, const void* x, int64_t M, int64_t N, int32_t dtype
     else if (dtype == LH_F16) { LH_SM_DTYPE(LH_F16) }
 #undef LH_SM_DTYPE
 #undef LH_SM_CASE
+  }
+  const bool vec = N % 4 == 0 && aligned16(out) && aligned16(x);
+  if (N >= 1024 || (vec && N >= 512)) {
+    const dim3 rows((unsigned)M);
+#define LH_SMB_CASE(DT)                                                                                    \
+  case DT:                                                                                                 \
+    if (vec && N <= 1024 * kBlockRegGroups)                                                                \
+      hipLaunchKernelGGL((softmax_block_reg<DT>), rows, block, 0, s, out, x, (int)M, (int)N);              \
+    else if (vec) hipLaunchKernelGGL((softmax_block<DT, true>), rows, block, 0, s, out, x, (int)M, (int)N); \
+    else hipLaunchKernelGGL((softmax_block<DT, false>), rows, block, 0, s, out, x, (int)M, (int)N);        \
+    return check_launch("softmax_block");
+    switch (dtype) {
+      LH_SMB_CASE(LH_F32) LH_SMB_CASE(LH_BF16) LH_SMB_CASE(LH_F16)
+      default: return fail(LH_ERR_UNSUPPORTED, "lh_hip_softmax: unsupported dtype %d", dtype);
+    }
+#undef LH_SMB_CASE
   }
   switch (dtype) {
     case LH_F32: hipLaunchKernelGGL(softmax_rows<LH_F32>, grid, block, 0, s, out, x, (int)M, (int)N); break;

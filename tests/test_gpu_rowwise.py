@@ -31,6 +31,30 @@ def test_layer_norm_f32(shape):
     assert_close(_host(out), orc.layer_norm(x, g, b, 1e-5), 1e-4, f"layer_norm {shape}")
 
 
+@pytest.mark.parametrize("shape", [(100, 50000), (64, 8192), (33, 5001), (7, 1026), (3, 50257), (300, 1280)])
+@pytest.mark.parametrize("elt", ["f32", "bf16"])
+def test_long_rows_one_workgroup_per_row(shape, elt):
+    """Rows that do not stay in a wave's registers: LayerNorm and softmax with one workgroup per row,
+    vector accesses when the row length and alignment allow (N % 4 == 0), scalar otherwise."""
+    from lighthouse_amd import ops
+
+    rng = np.random.default_rng(shape[0] + shape[1])
+    dt = torch.float32 if elt == "f32" else torch.bfloat16
+    x = orc.round_to(rng.standard_normal(shape).astype(np.float32) * 2 + 0.5, elt)
+    g = rng.uniform(0.5, 1.5, shape[1:]).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, shape[1:]).astype(np.float32)
+    out = ops.layer_norm(_dev(x, dt), _dev(g), _dev(b), 1e-5)
+    rtol = 1e-4 if elt == "f32" else 2e-2
+    assert_close(_host(out), orc.layer_norm(x, g, b, 1e-5, result_type=elt), rtol, f"layer_norm {shape} {elt}")
+    sm = _host(ops.softmax(_dev(x, dt)))
+    ref = orc.softmax(x, result_type=elt)
+    if elt == "f32":
+        assert np.allclose(sm.sum(1), 1.0, rtol=1e-5, atol=1e-6)
+        assert np.allclose(sm, ref, rtol=1e-4, atol=1e-6)
+    else:
+        assert_close(sm, ref, 2e-2, f"softmax {shape} bf16")
+
+
 def test_layer_norm_bf16_out_and_in():
     from lighthouse_amd import ops
 
