@@ -168,6 +168,7 @@ void* transpose_scratch(size_t bytes);
 int pad_copy_matrix(void* dst, int64_t ld_dst, int rows_dst, int cols_dst, const void* src, int64_t ld_src, int rows_src,
                     int cols_src, int elem_bytes, hipStream_t s);
 void* pad_scratch(size_t bytes);
+void* splitk_scratch(size_t bytes);  // f32 partial results of split-K GEMM launches
 // Compute units of the current device (cached; 256 if the query fails).
 int num_cus();
 

@@ -616,11 +616,27 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
 // walking the tile list with the grid as stride.  Tile ids congruent modulo 8 stay on one XCD,
 // which is what xcd_remap assumes.  Launching one workgroup per tile instead costs a
 // workgroup launch plus a cold prologue per tile, about a third of a K = 768 tile's time.
-template <int DT, int TM, int TN, bool EDGE>
+// SPLITK: the tile list is g.splits copies of the problem's tiles, copy sp working on its own K
+// columns of A / rows of B and its own block of the (f32) output; a second kernel adds the blocks.
+// For problems with few tiles and a long K (decode shapes), where the tile count cannot fill the CUs.
+template <int DT, int TM, int TN, bool EDGE, bool SPLITK = false>
 __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
   using Cfg = DirectCfg<TM, TN>;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_d[];
-  const int ntiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
+  const int tiles1 = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
+  const int ntiles = SPLITK ? tiles1 * g.splits : tiles1;
+  GemmArgs g_cur = g, g_nxt = g;  // (SPLITK) the problem copy that the current / next tile belongs to
+  auto select = [&](int t, GemmArgs& ga) -> int {  // -> the tile's id within its copy
+    if constexpr (SPLITK) {
+      const int sp = t / tiles1;
+      ga.a = reinterpret_cast<const uint16_t*>(g.a) + (int64_t)sp * g.K;
+      ga.b = reinterpret_cast<const uint16_t*>(g.b) + (int64_t)sp * g.K * g.ldb;
+      ga.out = reinterpret_cast<float*>(g.out) + (int64_t)sp * g.M * g.ldc;
+      ga.c = ga.out;
+      return t - sp * tiles1;
+    }
+    return t;
+  };
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr int WN = 4;
@@ -653,7 +669,10 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
   const int nk = g.K / 32;  // even: K is a multiple of 64
   int t = blockIdx.x;       // < ntiles: the grid is never larger than the tile list
   int m0, n0;
-  direct_place<TM, TN, EDGE>(g, xcd_remap(t, ntiles), c, m0, n0);
+  {
+    const int id = select(t, g_cur);
+    direct_place<TM, TN, EDGE>(SPLITK ? g_cur : g, xcd_remap(id, tiles1), c, m0, n0);
+  }
   direct_prologue(c, nk, smem_d);
   // Without EDGE every lane issues all stores of a staged epilogue.
   const bool staged = g.out_dt != LH_F32 && !(g.flags & LH_GEMM_ACCUMULATE_C);
@@ -668,7 +687,8 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
     u32x2 bias[TN][4];
-    direct_mainloop<DT, TM, TN, EDGE>(g, c, acc, smem_d, nk, counted_stores && !first, staged, n0 + wn0 + 4 * h, bias);
+    const GemmArgs& ga = SPLITK ? g_cur : g;
+    direct_mainloop<DT, TM, TN, EDGE>(ga, c, acc, smem_d, nk, counted_stores && !first, staged, n0 + wn0 + 4 * h, bias);
     first = false;
     const int tn = t + (int)gridDim.x;
     const bool more = tn < ntiles;
@@ -676,12 +696,14 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
     int m1 = 0, n1 = 0;
     uint8_t* const stage = smem_d + Cfg::kRingBytes;
     if (more) {
-      direct_place<TM, TN, EDGE>(g, xcd_remap(tn, ntiles), cn, m1, n1);
-      direct_finish<DT, TM, TN, EDGE, true>(g, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0);
+      const int idn = select(tn, g_nxt);
+      direct_place<TM, TN, EDGE>(SPLITK ? g_nxt : g, xcd_remap(idn, tiles1), cn, m1, n1);
+      direct_finish<DT, TM, TN, EDGE, true>(ga, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0);
     } else {
-      direct_finish<DT, TM, TN, EDGE, false>(g, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0);
+      direct_finish<DT, TM, TN, EDGE, false>(ga, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0);
     }
     if (!more) break;
+    if constexpr (SPLITK) g_cur = g_nxt;
     c = cn;
     m0 = m1;
     n0 = n1;
@@ -803,6 +825,63 @@ static int direct_variant(int M, int N, int K) {
   return best;
 }
 
+// Sum of the split-K blocks (f32, [splits][M][N]) and the problem's own epilogue, 4 columns per thread.
+template <int DT>
+__global__ void __launch_bounds__(256) gemm16_splitk_reduce(GemmArgs g, const float* partial, int splits) {
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (idx >= (int64_t)g.M * g.N) return;
+  const int m = (int)(idx / g.N), n = (int)(idx % g.N);
+  f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int sp = 0; sp < splits; ++sp) {
+    const f32x4 p = *reinterpret_cast<const f32x4*>(partial + ((int64_t)sp * g.M + m) * g.N + n);
+    v[0] += p[0]; v[1] += p[1]; v[2] += p[2]; v[3] += p[3];
+  }
+  epilogue4<DT>(g, m, n, v[0], v[1], v[2], v[3]);
+}
+
+// Decode shapes: so few 128 x 128 tiles that most CUs would idle, and a K long enough to cut.
+// Returns 1 when the problem does not qualify.
+template <int DT>
+static int gemm16_splitk(const GemmArgs& g, hipStream_t s) {
+  using Cfg = DirectCfg<2, 1>;
+  const int cus = num_cus();
+  const int64_t tiles = (int64_t)((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
+  if (tiles * 2 > cus || g.K < 2048) return 1;
+  int splits = 1;
+  while (splits < 8 && tiles * splits * 2 <= 2 * cus && (g.K / (splits * 2)) % kBK == 0 && g.K / (splits * 2) >= 512)
+    splits *= 2;
+  if (splits == 1) return 1;
+  float* partial = static_cast<float*>(splitk_scratch((size_t)splits * g.M * g.N * sizeof(float)));
+  if (!partial) return LH_ERR_RUNTIME;
+  GemmArgs p = g;
+  p.K = g.K / splits;
+  p.splits = splits;
+  p.out = partial;
+  p.c = partial;
+  p.ldc = g.N;
+  p.out_dt = LH_F32;
+  p.bias = nullptr;
+  p.flags = 0;
+  const bool edge = g.M % Cfg::BM != 0 || g.N % Cfg::BN != 0;
+  auto launch = [&](auto kern, bool& configured) -> int {
+    if (!configured) {
+      LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)Cfg::kLdsBytes));
+      configured = true;
+    }
+    const int64_t total = tiles * splits, resident = 2 * (int64_t)cus;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(total < resident ? total : resident)), dim3(512), Cfg::kLdsBytes, s, p);
+    return check_launch("gemm16_direct (split K)");
+  };
+  static bool configured_edge = false, configured_whole = false;
+  const int rc = edge ? launch(gemm16_direct<DT, 2, 1, true, true>, configured_edge)
+                      : launch(gemm16_direct<DT, 2, 1, false, true>, configured_whole);
+  if (rc) return rc;
+  const int64_t groups = (int64_t)g.M * g.N / 4;
+  hipLaunchKernelGGL(gemm16_splitk_reduce<DT>, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s, g, partial, splits);
+  return check_launch("gemm16_splitk_reduce");
+}
+
 template <int DT>
 static int gemm16_dispatch(const GemmArgs& g_in, hipStream_t s) {
   GemmArgs g = g_in;
@@ -832,6 +911,10 @@ static int gemm16_dispatch(const GemmArgs& g_in, hipStream_t s) {
   }
   if (vec_ok) {
     if (!tb && g.ldc % 8 == 0 && g.N % 8 == 0) {
+      if (tile == LH_GEMM_TILE_AUTO) {
+        const int rc = gemm16_splitk<DT>(g, s);
+        if (rc <= 0) return rc;
+      }
       const int v = tile != LH_GEMM_TILE_AUTO ? (int)(tile >> 8) - 1 : direct_variant(g.M, g.N, g.K);
       if (v == 0) return launch_direct<DT, 4, 2>(g, s);
       if (v == 1) return launch_direct<DT, 4, 1>(g, s);

@@ -17,6 +17,9 @@ struct GemmArgs {
   int out_dt;
   int bias_dt;  // element type of bias
   float alpha;  // accumulator scale applied first (1 for the unquantised payloads)
+  // Split-K launches of the 16-bit direct kernel: `splits` problems of K columns each, problem sp reads
+  // A from column sp K, B from row sp K and writes its own M x ldc block of `out`.
+  int splits = 1;
 };
 
 // Epilogue for 4 consecutive columns of one row.

@@ -158,6 +158,13 @@ static size_t g_pad_scratch_bytes = 0;
 
 void* pad_scratch(size_t bytes) { return grow_buffer(g_pad_scratch, g_pad_scratch_bytes, bytes, "padding scratch"); }
 
+static char* g_splitk_scratch = nullptr;
+static size_t g_splitk_scratch_bytes = 0;
+
+void* splitk_scratch(size_t bytes) {
+  return grow_buffer(g_splitk_scratch, g_splitk_scratch_bytes, bytes, "split-K scratch");
+}
+
 }  // namespace lh
 
 using namespace lh;

@@ -491,6 +491,41 @@ def test_gemm_shapes_run_on_padded_copies(shape, elt, epi):
     assert bool((buf[:, N:] == 5.0).all()), "columns behind the output were written"
 
 
+@pytest.mark.parametrize("elt", ["bf16", "f16"])
+@pytest.mark.parametrize("shape", [(16, 1024, 4096), (1, 520, 2048), (64, 512, 8192), (130, 256, 4096), (256, 1024, 2048)])
+@pytest.mark.parametrize("epi", ["none", "bias_gelu", "f32_acc", "residual"])
+def test_gemm_16bit_split_k(shape, elt, epi):
+    """Few tiles and a long K (decode shapes): the tile list is cut along K, each part writes an
+    f32 block, a second kernel adds them and runs the epilogue.  Called twice (the library's
+    partial-result buffer is reused)."""
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(M + 5 * N + 11 * K)
+    dt = {"bf16": torch.bfloat16, "f16": torch.float16}[elt]
+    a = orc.round_to(rng.standard_normal((M, K)).astype(np.float32), elt)
+    b = orc.round_to(rng.standard_normal((K, N)).astype(np.float32) * 0.05, elt)
+    bias = orc.round_to(rng.standard_normal((N,)).astype(np.float32), elt)
+    c = rng.standard_normal((M, N)).astype(np.float32)
+    da, db = _dev(a, dt), _dev(b, dt)
+    for _ in range(2):
+        if epi == "none":
+            out = ops.gemm(da, db)
+            ref, rtol = orc.matmul(a, b, result_type=elt), BF16_RTOL
+        elif epi == "bias_gelu":
+            out = ops.gemm(da, db, _dev(bias, dt), gelu=True)
+            ref, rtol = orc.matmul(a, b, bias=bias, gelu=True, result_type=elt), BF16_RTOL
+        elif epi == "f32_acc":
+            out = _dev(c, torch.float32)
+            ops.gemm(da, db, out=out, accumulate_c=True)
+            ref, rtol = orc.matmul(a, b, c=c, accumulate_c=True, result_type="f32"), F32_RTOL
+        else:
+            cr = orc.round_to(c, elt)
+            out = ops.gemm(da, db, _dev(bias, dt), residual=_dev(cr, dt))
+            ref, rtol = orc.matmul(a, b, c=cr, accumulate_c=True, bias=bias, result_type=elt), BF16_RTOL
+        assert_close(_host(out), ref, rtol, f"{elt} gemm {shape} {epi} (split K)")
+
+
 def test_tile_search_and_database(tmp_path):
     """The tuner times every fitting tile for a shape, logs the trials, records the winner, and
     ops.gemm picks the recorded tile up when the database is in use (same results either way)."""
