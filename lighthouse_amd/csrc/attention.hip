@@ -670,8 +670,11 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, h = lane >> 5;
   const int nqb = (a.T + 127) / 128;
-  const int qb = a.causal ? nqb - 1 - (int)blockIdx.x : (int)blockIdx.x;  // causal: heavy blocks first
-  const int bh = blockIdx.y;
+  // Causal work grows with the query block: a 1-D grid lists the blocks heaviest first over ALL
+  // (batch, head) pairs, so that the long ones do not start last.
+  const int bhn = a.Z * a.H;
+  const int qb = a.causal ? nqb - 1 - (int)blockIdx.x / bhn : (int)blockIdx.x;
+  const int bh = a.causal ? (int)blockIdx.x % bhn : (int)blockIdx.y;
   const int z = bh / a.H, hd = bh % a.H;
   const int q0 = qb * 128, wq0 = q0 + 32 * wave;
   const bool wave_valid = wq0 < a.T;
@@ -818,7 +821,9 @@ static int attention16_anyd_launch(const AttnArgs& a, hipStream_t s) {
                                      (int)lds));
     configured = true;
   }
-  hipLaunchKernelGGL(kern, dim3((a.T + 127) / 128, a.Z * a.H), dim3(256), lds, s, a);
+  const int nqb = (a.T + 127) / 128;
+  const dim3 grid = a.causal ? dim3(nqb * a.Z * a.H) : dim3(nqb, a.Z * a.H);
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, a);
   return check_launch("attention16_anyd");
 }
 
