@@ -396,13 +396,30 @@ __device__ __forceinline__ void d8_finish(const GemmArgs& g, const D8Ctx& next, 
 
 // Persistent workgroups, one per CU, each walking the tile list with the grid as stride (tile
 // ids congruent modulo 8 stay on one XCD, which is what xcd_remap assumes).
+// SPLITK: the tile list is g.splits copies of the problem's tiles, copy sp working on its own K
+// columns of A / rows of B and its own f32 block of the output; a second kernel adds the blocks,
+// scales and converts.  For problems with too few tiles for the CUs and a long K.
+template <bool SPLITK>
 __global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
   constexpr int TM = 4, TN = 2, WN = 4, WTN = 64;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_8[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave / WN) * 128, wn0 = (wave % WN) * WTN;
-  const int ntiles = (g.M / 256) * (g.N / 256);
+  const int tiles1 = (g.M / 256) * (g.N / 256);
+  const int ntiles = SPLITK ? tiles1 * g.splits : tiles1;
+  GemmArgs g_cur = g, g_nxt = g;  // (SPLITK) the problem copy of the current / next tile
+  auto select = [&](int t, GemmArgs& ga) -> int {
+    if constexpr (SPLITK) {
+      const int sp = t / tiles1;
+      ga.a = reinterpret_cast<const uint8_t*>(g.a) + (int64_t)sp * g.K;
+      ga.b = reinterpret_cast<const uint8_t*>(g.b) + (int64_t)sp * g.K * g.ldb;
+      ga.out = reinterpret_cast<float*>(g.out) + (int64_t)sp * g.M * g.ldc;
+      ga.c = ga.out;
+      return t - sp * tiles1;
+    }
+    return t;
+  };
 
   D8Ctx c;
   c.ldb = g.ldb;
@@ -425,7 +442,10 @@ __global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
   const int nk = g.K / 64;  // even: K is a multiple of 128
   int t = blockIdx.x;       // < ntiles: the grid is never larger than the tile list
   int m0, n0;
-  d8_place(g, xcd_remap(t, ntiles), c, m0, n0);
+  {
+    const int id = select(t, g_cur);
+    d8_place(SPLITK ? g_cur : g, xcd_remap(id, tiles1), c, m0, n0);
+  }
   d8_prologue(c, nk, smem_8);
   for (;;) {
     f32x16 acc[TN][TM];
@@ -441,13 +461,16 @@ __global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
     D8Ctx cn = c;
     int m1 = 0, n1 = 0;
     uint8_t* const stage = smem_8 + kD8RingBytes;
+    const GemmArgs& ga = SPLITK ? g_cur : g;
     if (more) {
-      d8_place(g, xcd_remap(tn, ntiles), cn, m1, n1);
-      d8_finish<true>(g, cn, nk, smem_8, stage, acc, m0, n0, wm0, wn0);
+      const int idn = select(tn, g_nxt);
+      d8_place(SPLITK ? g_nxt : g, xcd_remap(idn, tiles1), cn, m1, n1);
+      d8_finish<true>(ga, cn, nk, smem_8, stage, acc, m0, n0, wm0, wn0);
     } else {
-      d8_finish<false>(g, cn, nk, smem_8, stage, acc, m0, n0, wm0, wn0);
+      d8_finish<false>(ga, cn, nk, smem_8, stage, acc, m0, n0, wm0, wn0);
     }
     if (!more) break;
+    if constexpr (SPLITK) g_cur = g_nxt;
     c = cn;
     m0 = m1;
     n0 = n1;
@@ -458,13 +481,61 @@ __global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
 static int launch_direct8(const GemmArgs& g, hipStream_t s) {
   static bool configured = false;
   if (!configured) {
-    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_direct),
+    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_direct<false>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kD8LdsBytes));
     configured = true;
   }
   const int ntiles = (g.M / 256) * (g.N / 256), cus = num_cus();
-  hipLaunchKernelGGL(gemm8_direct, dim3(ntiles < cus ? ntiles : cus), dim3(512), kD8LdsBytes, s, g);
+  hipLaunchKernelGGL(gemm8_direct<false>, dim3(ntiles < cus ? ntiles : cus), dim3(512), kD8LdsBytes, s, g);
   return check_launch("gemm8_direct");
+}
+
+// Sum of the split-K blocks ([splits][M][N] f32), scale, conversion: 4 columns per thread.
+__global__ void __launch_bounds__(256) gemm8_splitk_reduce(GemmArgs g, const float* partial, int splits) {
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (idx >= (int64_t)g.M * g.N) return;
+  const int m = (int)(idx / g.N), n = (int)(idx % g.N);
+  f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+  for (int sp = 0; sp < splits; ++sp) {
+    const f32x4 p = *reinterpret_cast<const f32x4*>(partial + ((int64_t)sp * g.M + m) * g.N + n);
+    v[0] += p[0]; v[1] += p[1]; v[2] += p[2]; v[3] += p[3];
+  }
+  epilogue4<LH_BF16>(g, m, n, v[0], v[1], v[2], v[3]);
+}
+
+// Too few 256 x 256 tiles for the CUs and a K long enough to cut.  Returns 1 when the problem does
+// not qualify.
+static int gemm8_splitk(const GemmArgs& g, hipStream_t s) {
+  const int cus = num_cus();
+  const int64_t tiles = (int64_t)(g.M / 256) * (g.N / 256);
+  if (tiles * 2 > cus || g.K < 2048) return 1;
+  int splits = 1;
+  while (splits < 8 && tiles * splits * 2 <= cus && (g.K / (splits * 2)) % kBK8 == 0 && g.K / (splits * 2) >= 1024)
+    splits *= 2;
+  if (splits == 1) return 1;
+  float* partial = static_cast<float*>(splitk_scratch((size_t)splits * g.M * g.N * sizeof(float)));
+  if (!partial) return LH_ERR_RUNTIME;
+  GemmArgs p = g;
+  p.K = g.K / splits;
+  p.splits = splits;
+  p.out = partial;
+  p.c = partial;
+  p.ldc = g.N;
+  p.out_dt = LH_F32;
+  p.alpha = 1.0f;
+  static bool configured = false;
+  if (!configured) {
+    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_direct<true>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kD8LdsBytes));
+    configured = true;
+  }
+  const int64_t total = tiles * splits;
+  hipLaunchKernelGGL(gemm8_direct<true>, dim3((unsigned)(total < cus ? total : cus)), dim3(512), kD8LdsBytes, s, p);
+  int rc = check_launch("gemm8_direct (split K)");
+  if (rc) return rc;
+  const int64_t groups = (int64_t)g.M * g.N / 4;
+  hipLaunchKernelGGL(gemm8_splitk_reduce, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s, g, partial, splits);
+  return check_launch("gemm8_splitk_reduce");
 }
 
 // Any shape: 32 x 32 x 64 tile per wave, one wave per workgroup tile of 32 x 32,
@@ -840,6 +911,11 @@ int gemm8(const GemmArgs& g, hipStream_t s) {
     if (g.M <= 32) return launch_skinny_mt<2>(g, s);
     if (g.M <= 64) return launch_skinny_mt<4>(g, s);
     return launch_skinny_mt<8>(g, s);
+  }
+  if (vec_ok && g.M % 256 == 0 && g.N % 256 == 0 && g.ldb % 16 == 0 && g.ldc % 8 == 0 && g.lda < (1 << 24) &&
+      g.ldb < (1 << 24)) {
+    const int rc = gemm8_splitk(g, s);
+    if (rc <= 0) return rc;
   }
   if (vec_ok && g.M % 256 == 0 && g.N % 256 == 0 && (int64_t)(g.M / 256) * (g.N / 256) >= 128) {
     // the direct kernel addresses a tile's rows with 32-bit byte offsets from the tile's origin

@@ -427,6 +427,8 @@ def test_gemm_fp8_decode_path(shape):
 @pytest.mark.parametrize("shape", [(17, 256, 1024), (32, 1024, 4096), (33, 512, 2048), (48, 256, 384),
                                    (64, 2048, 8192), (64, 8192, 8192), (65, 512, 1024), (100, 1024, 2048),
                                    (128, 8192, 8192),
+                                   # few 256 x 256 tiles, long K: split K of the direct kernel
+                                   (256, 512, 4096), (512, 256, 8192), (768, 1024, 2048),
                                    # M that no tile divides, N a multiple of 128: the fast kernel's M-edge form
                                    (100, 384, 512), (129, 256, 256), (1000, 1024, 1024)])
 def test_gemm_fp8_decode_batches_and_ragged_m(shape):
