@@ -146,13 +146,14 @@ inline int untranspose_operands(GemmArgs& g, int k_multiple, int n_multiple, hip
 // when nothing needs padding, a negative status on failure.
 template <int ELEM_BYTES, typename Run>
 inline int gemm_padded(const GemmArgs& g, int k_multiple, int n_multiple, hipStream_t s, Run run) {
-  if (g.flags & (LH_GEMM_TRANSPOSE_A | LH_GEMM_TRANSPOSE_B)) return 1;
+  const bool ta = g.flags & LH_GEMM_TRANSPOSE_A, tb = g.flags & LH_GEMM_TRANSPOSE_B;
   const int out_bytes = g.out_dt == LH_F32 ? 4 : 2, bias_bytes = g.bias_dt == LH_F32 ? 4 : 2;
   const int Kp = (g.K + k_multiple - 1) / k_multiple * k_multiple;
   const int Np = (g.N + n_multiple - 1) / n_multiple * n_multiple;
   const bool has_bias = g.flags & LH_GEMM_HAS_BIAS, acc = g.flags & LH_GEMM_ACCUMULATE_C;
-  const bool pad_a = Kp != g.K || g.lda % (16 / ELEM_BYTES) != 0 || !aligned16(g.a);
-  const bool pad_b = Kp != g.K || Np != g.N || g.ldb % (16 / ELEM_BYTES) != 0 || !aligned16(g.b);
+  // (a transposed operand is copied in any case: the copy is where it gets untransposed)
+  const bool pad_a = ta || Kp != g.K || g.lda % (16 / ELEM_BYTES) != 0 || !aligned16(g.a);
+  const bool pad_b = tb || Kp != g.K || Np != g.N || g.ldb % (16 / ELEM_BYTES) != 0 || !aligned16(g.b);
   const bool pad_c = Np != g.N || g.ldc % n_multiple != 0 || !aligned16(g.out) || (acc && !aligned16(g.c));
   const bool pad_bias = has_bias && (Np != g.N || !aligned16(g.bias));
   if (!(pad_a || pad_b || pad_c || pad_bias)) return 1;
@@ -167,15 +168,29 @@ inline int gemm_padded(const GemmArgs& g, int k_multiple, int n_multiple, hipStr
   p.K = Kp;
   p.N = Np;
   if (pad_a) {
-    if (int rc = pad_copy_matrix(buf, Kp, g.M, Kp, g.a, g.lda, g.M, g.K, ELEM_BYTES, s)) return rc;
+    if (ta) {  // stored [K, M]: zeros first (the padding), then the transposed matrix on top
+      if (Kp != g.K)
+        if (int rc = pad_copy_matrix(buf, Kp, g.M, Kp, g.a, g.lda, 0, 0, ELEM_BYTES, s)) return rc;
+      if (int rc = transpose_matrix(buf, g.a, g.K, g.M, g.lda, Kp, ELEM_BYTES, s)) return rc;
+    } else if (int rc = pad_copy_matrix(buf, Kp, g.M, Kp, g.a, g.lda, g.M, g.K, ELEM_BYTES, s)) {
+      return rc;
+    }
     p.a = buf;
     p.lda = Kp;
   }
   if (pad_b) {
-    if (int rc = pad_copy_matrix(buf + a_bytes, Np, Kp, Np, g.b, g.ldb, g.K, g.N, ELEM_BYTES, s)) return rc;
-    p.b = buf + a_bytes;
+    char* bp = buf + a_bytes;
+    if (tb) {  // stored [N, K]
+      if (Kp != g.K || Np != g.N)
+        if (int rc = pad_copy_matrix(bp, Np, Kp, Np, g.b, g.ldb, 0, 0, ELEM_BYTES, s)) return rc;
+      if (int rc = transpose_matrix(bp, g.b, g.N, g.K, g.ldb, Np, ELEM_BYTES, s)) return rc;
+    } else if (int rc = pad_copy_matrix(bp, Np, Kp, Np, g.b, g.ldb, g.K, g.N, ELEM_BYTES, s)) {
+      return rc;
+    }
+    p.b = bp;
     p.ldb = Np;
   }
+  p.flags &= ~(uint32_t)(LH_GEMM_TRANSPOSE_A | LH_GEMM_TRANSPOSE_B);
   if (pad_c) {
     char* cp = buf + a_bytes + b_bytes;
     if (acc)

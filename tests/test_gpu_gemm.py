@@ -528,6 +528,27 @@ def test_gemm_16bit_split_k(shape, elt, epi):
         assert_close(_host(out), ref, rtol, f"{elt} gemm {shape} {epi} (split K)")
 
 
+@pytest.mark.parametrize("elt", ["bf16", "f32"])
+@pytest.mark.parametrize("ta,tb", [(True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("shape", [(300, 521, 200), (512, 1000, 1000)])
+def test_gemm_transposed_and_ragged(shape, ta, tb, elt):
+    """Transposed operands of a problem whose K / N need padding: the padded copy is where they
+    get untransposed."""
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K + 2 * ta + tb)
+    dt = {"bf16": torch.bfloat16, "f32": torch.float32}[elt]
+    a = orc.round_to(rng.standard_normal((M, K)).astype(np.float32), elt)
+    b = orc.round_to(rng.standard_normal((K, N)).astype(np.float32) * 0.1, elt)
+    bias = orc.round_to(rng.standard_normal((N,)).astype(np.float32), elt)
+    da = _dev(a.T.copy() if ta else a, dt)
+    db = _dev(b.T.copy() if tb else b, dt)
+    out = ops.gemm(da, db, _dev(bias, dt), relu=True, transpose_a=ta, transpose_b=tb)
+    ref = orc.matmul(a, b, bias=bias, relu=True, result_type=elt)
+    assert_close(_host(out), ref, F32_RTOL if elt == "f32" else BF16_RTOL, f"{elt} gemm {shape} ta={ta} tb={tb}")
+
+
 def test_tile_search_and_database(tmp_path):
     """The tuner times every fitting tile for a shape, logs the trials, records the winner, and
     ops.gemm picks the recorded tile up when the database is in use (same results either way)."""
