@@ -883,6 +883,11 @@ static int launch_skinny_mt(const GemmArgs& g, hipStream_t s) {
 int gemm8(const GemmArgs& g, hipStream_t s) {
   const bool vec_ok = g.K % kBK8 == 0 && g.lda % 16 == 0 && g.ldb % 4 == 0 && g.ldc % 4 == 0 && aligned16(g.a) &&
                       aligned16(g.b) && aligned16(g.out);
+  if (!(vec_ok && g.N % 128 == 0) && (int64_t)g.M * g.N * g.K >= (1 << 22)) {
+    // K that is no multiple of the k-step, N of no tile, unaligned rows: zero-padded copies (code 0 is +0)
+    const int rc = gemm_padded<1>(g, kBK8, 128, s, [&](const GemmArgs& p) { return gemm8(p, s); });
+    if (rc <= 0) return rc;
+  }
   if (vec_ok && g.M <= 16 && g.N % kSkinnyBN == 0 && g.ldb % 16 == 0) {
     // Split K so that about one workgroup per CU streams B (its ring alone keeps 96 KiB in
     // flight) and the A chunk fits its LDS area.

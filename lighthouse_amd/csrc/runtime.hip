@@ -123,6 +123,9 @@ int pad_copy_matrix(void* dst, int64_t ld_dst, int rows_dst, int cols_dst, const
   else if (elem_bytes == 4)
     hipLaunchKernelGGL(pad_copy_kernel<uint32_t>, grid, dim3(256), 0, s, static_cast<uint32_t*>(dst), ld_dst, rows_dst,
                        cols_dst, static_cast<const uint32_t*>(src), ld_src, rows_src, cols_src);
+  else if (elem_bytes == 1)
+    hipLaunchKernelGGL(pad_copy_kernel<uint8_t>, grid, dim3(256), 0, s, static_cast<uint8_t*>(dst), ld_dst, rows_dst,
+                       cols_dst, static_cast<const uint8_t*>(src), ld_src, rows_src, cols_src);
   else
     return fail(LH_ERR_UNSUPPORTED, "pad copy: element size %d", elem_bytes);
   return check_launch("pad_copy");

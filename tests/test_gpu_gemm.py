@@ -430,7 +430,9 @@ def test_gemm_fp8_decode_path(shape):
                                    # few 256 x 256 tiles, long K: split K of the direct kernel
                                    (256, 512, 4096), (512, 256, 8192), (768, 1024, 2048),
                                    # M that no tile divides, N a multiple of 128: the fast kernel's M-edge form
-                                   (100, 384, 512), (129, 256, 256), (1000, 1024, 1024)])
+                                   (100, 384, 512), (129, 256, 256), (1000, 1024, 1024),
+                                   # K no multiple of 128 / N no multiple of 128: zero-padded copies
+                                   (64, 1000, 1000), (300, 520, 777), (16, 8192, 200)])
 def test_gemm_fp8_decode_batches_and_ragged_m(shape):
     """16 < M <= 128: the streaming kernel with 2, 4 or 8 row groups (B still read once; rows past M
     repeat the last row and are not stored); other M: tile kernel with clamped rows.  Run twice
