@@ -813,6 +813,201 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
     }
 }
 
+// Head dimension 128, 16-bit: the kernel above with the key tiles brought in by LDS-DMA
+// (global_load_lds_dwordx4, no registers, no LDS stores) into two unpadded stages, the load of tile
+// j + 1 running under the arithmetic of tile j, one barrier per tile.  Rows are 256 bytes = the 64
+// LDS banks, so the 16-byte chunk a lane fetches is XOR-swizzled with the key's low four bits
+// (LDS chunk p of key row k holds global chunk p ^ (k % 16)); a wave-wide load fills 4 key rows.
+constexpr int kD128TileBytes = kKvTile * 256;          // one tensor's tile
+constexpr int kD128StageBytes = 2 * kD128TileBytes;    // K tile + V tile, 32 KiB
+
+struct Attn128Ctx {
+  const uint16_t* k_src[4];  // lane's source of K load i at key 0 of the tensor
+  const uint16_t* v_src[4];
+  int key_local[4];          // the key of a tile that load i of this lane fetches
+  int64_t k_row, v_row;      // elements per key
+  int wave;
+};
+
+__device__ __forceinline__ void attn128_issue(const Attn128Ctx& c, int jt, int T, uint8_t* __restrict__ stage) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int key = min(jt * kKvTile + c.key_local[i], T - 1);  // keys past the end repeat the last one (masked later)
+    __builtin_amdgcn_global_load_lds(c.k_src[i] + key * c.k_row, (attn_lds_void_t*)(stage + (4 * i + c.wave) * 1024), 16,
+                                     0, 0);
+    __builtin_amdgcn_global_load_lds(c.v_src[i] + key * c.v_row,
+                                     (attn_lds_void_t*)(stage + kD128TileBytes + (4 * i + c.wave) * 1024), 16, 0, 0);
+  }
+}
+
+// One key tile for the wave's 32 query rows.  `rd` holds the tile, `wr` receives the next one
+// meanwhile (separate restrict pointers so that LDS reads do not wait for the asynchronous writes).
+template <int DT>
+__device__ __forceinline__ void attn128_tile(const Attn128Ctx& c, const AttnArgs& a, const u32x4 (&qf)[8],
+                                             f32x16 (&acc_o)[4], float& m_run, float& l_run,
+                                             const uint8_t* __restrict__ rd, uint8_t* __restrict__ wr, int next_jt,
+                                             bool prefetch, int j0, int wq0, bool active, int lane) {
+  if (prefetch) attn128_issue(c, next_jt, a.T, wr);
+  if (!active) return;
+  const int r32 = lane & 31, h = lane >> 5;
+  const uint8_t* ks = rd;
+  const uint8_t* vs = rd + kD128TileBytes;
+  f32x16 s_acc[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s_acc[i][v] = 0.0f;
+#pragma unroll
+    for (int sd = 0; sd < 8; ++sd) {
+      const u32x4 kf = *reinterpret_cast<const u32x4*>(ks + (32 * i + r32) * 256 + (((2 * sd + h) ^ (r32 & 15)) << 4));
+      s_acc[i] = mfma16<DT>(kf, qf[sd], s_acc[i]);
+    }
+  }
+  if ((a.causal && j0 + kKvTile - 1 > wq0) || j0 + kKvTile > a.T) {
+    const int last = a.causal ? min(wq0 + r32, a.T - 1) : a.T - 1;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v)
+        if (j0 + 32 * i + 8 * (v >> 2) + 4 * h + (v & 3) > last) s_acc[i][v] = -INFINITY;
+  }
+  float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
+#pragma unroll
+  for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[0][v]), s_acc[1][v]);
+  mx = halfwave_max(mx);
+  const float m_new = fmaxf(m_run, mx);
+  const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+  const float alpha = exp2_fast(m_run - m_safe);
+  m_run = m_new;
+  float p[2][16];
+  float l_tile = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      p[i][v] = exp2_fast(s_acc[i][v] - m_safe);
+      l_tile += p[i][v];
+    }
+  l_run = l_run * alpha + l_tile;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc_o[j][v] *= alpha;
+  // V^T fragments through the transposing read (lane -> key row 4 h + j16 / 4 of the 16-key step,
+  // +8 for the second read; columns 32 j + 16 (g4 % 2) + 4 (j16 % 4) .. +4).
+  const int tr_row = 4 * h + ((lane & 15) >> 2), tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  const int ch0 = tr_col >> 3, off = (tr_col & 7) * 2;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      u32x4 pf;
+#pragma unroll
+      for (int d = 0; d < 4; ++d) pf[d] = pack2<DT>(p[i][8 * u + 2 * d], p[i][8 * u + 2 * d + 1]);
+      const uint8_t* row0 = vs + (32 * i + 16 * u + tr_row) * 256 + off;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint8_t* p0 = row0 + (((4 * j + ch0) ^ tr_row) << 4);
+        const uint8_t* p1 = row0 + 8 * 256 + (((4 * j + ch0) ^ (tr_row + 8)) << 4);
+        const attn_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) attn_s16x4*)p0);
+        const attn_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) attn_s16x4*)p1);
+        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+        acc_o[j] = mfma16<DT>(u32x4{l2[0], l2[1], h2[0], h2[1]}, pf, acc_o[j]);
+      }
+    }
+}
+
+template <int DT>
+__global__ void __launch_bounds__(256, 2) attention16_d128_kernel(AttnArgs a) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_d128[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r32 = lane & 31, h = lane >> 5;
+  const int nqb = (a.T + 127) / 128;
+  const int bhn = a.Z * a.H;
+  const int qb = a.causal ? nqb - 1 - (int)blockIdx.x / bhn : (int)blockIdx.x;  // causal: heaviest first over all heads
+  const int bh = a.causal ? (int)blockIdx.x % bhn : (int)blockIdx.y;
+  const int z = bh / a.H, hd = bh % a.H;
+  const int q0 = qb * 128, wq0 = q0 + 32 * wave;
+  const bool wave_valid = wq0 < a.T;
+
+  const uint16_t* Q = reinterpret_cast<const uint16_t*>(a.q) + (int64_t)z * a.sq.z + (int64_t)hd * a.sq.h;
+  const uint16_t* K = reinterpret_cast<const uint16_t*>(a.k) + (int64_t)z * a.sk.z + (int64_t)hd * a.sk.h;
+  const uint16_t* V = reinterpret_cast<const uint16_t*>(a.v) + (int64_t)z * a.sv.z + (int64_t)hd * a.sv.h;
+  uint16_t* O = reinterpret_cast<uint16_t*>(a.out) + (int64_t)z * a.so.z + (int64_t)hd * a.so.h;
+
+  Attn128Ctx c;
+  c.wave = wave;
+  c.k_row = a.sk.t;
+  c.v_row = a.sv.t;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int key = (4 * i + wave) * 4 + (lane >> 4);  // the row this lane fills, chunk lane % 16
+    const int gc = (lane & 15) ^ (key & 15);
+    c.key_local[i] = key;
+    c.k_src[i] = K + 8 * gc;
+    c.v_src[i] = V + 8 * gc;
+  }
+  u32x4 qf[8];
+  {
+    const int row = min(wq0 + r32, a.T - 1);
+#pragma unroll
+    for (int sd = 0; sd < 8; ++sd) {
+      const u32x4 raw = *reinterpret_cast<const u32x4*>(Q + (int64_t)row * a.sq.t + 16 * sd + 8 * h);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        qf[sd][e] = pack2<DT>(unpack_lo<DT>(raw[e]) * a.scale_log2e, unpack_hi<DT>(raw[e]) * a.scale_log2e);
+    }
+  }
+  f32x16 acc_o[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc_o[j][v] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  const int kv_end = a.causal ? min(a.T, q0 + 128) : a.T;
+  const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
+  attn128_issue(c, 0, a.T, smem_d128);
+  for (int jt = 0; jt < ntiles; ++jt) {
+    // The tile's 8 loads per lane have had a whole tile's time; one asm block, because a
+    // __syncthreads() would add a fence of its own.
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    const int j0 = jt * kKvTile;
+    const bool active = wave_valid && (!a.causal || j0 <= wq0 + 31);
+    attn128_tile<DT>(c, a, qf, acc_o, m_run, l_run, smem_d128 + (jt & 1) * kD128StageBytes,
+                     smem_d128 + ((jt + 1) & 1) * kD128StageBytes, jt + 1, jt + 1 < ntiles, j0, wq0, active, lane);
+  }
+  if (!wave_valid) return;
+  const float inv_l = 1.0f / halfwave_sum(l_run);
+  if (wq0 + r32 >= a.T) return;
+  uint16_t* orow = O + (int64_t)(wq0 + r32) * a.so.t;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      u32x2 w = {pack2<DT>(acc_o[j][4 * g] * inv_l, acc_o[j][4 * g + 1] * inv_l),
+                 pack2<DT>(acc_o[j][4 * g + 2] * inv_l, acc_o[j][4 * g + 3] * inv_l)};
+      *reinterpret_cast<u32x2*>(orow + 32 * j + 8 * g + 4 * h) = w;
+    }
+}
+
+template <int DT>
+static int attention16_d128_launch(const AttnArgs& a, hipStream_t s) {
+  constexpr size_t lds = 2 * kD128StageBytes;
+  auto kern = attention16_d128_kernel<DT>;
+  static bool configured = false;
+  if (!configured) {
+    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)lds));
+    configured = true;
+  }
+  const int nqb = (a.T + 127) / 128;
+  const dim3 grid = a.causal ? dim3(nqb * a.Z * a.H) : dim3(nqb, a.Z * a.H);
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, a);
+  return check_launch("attention16_d128");
+}
+
 template <int DT, int DB>
 static int attention16_anyd_launch(const AttnArgs& a, hipStream_t s) {
   constexpr int D = 32 * DB;
@@ -836,7 +1031,11 @@ static int attention16_anyd_dispatch(const AttnArgs& a, int d, hipStream_t s) {
   switch (d) {
     case 32: return attention16_anyd_launch<DT, 1>(a, s);
     case 96: return attention16_anyd_launch<DT, 3>(a, s);
+#ifdef LH_ATTN_D128_PADDED
     case 128: return attention16_anyd_launch<DT, 4>(a, s);
+#else
+    case 128: return attention16_d128_launch<DT>(a, s);
+#endif
     case 192: return attention16_anyd_launch<DT, 6>(a, s);
     case 256: return attention16_anyd_launch<DT, 8>(a, s);
     default: return 1;
