@@ -844,7 +844,7 @@ __device__ __forceinline__ void attn128_issue(const Attn128Ctx& c, int jt, int T
 // meanwhile (separate restrict pointers so that LDS reads do not wait for the asynchronous writes).
 template <int DT>
 __device__ __forceinline__ void attn128_tile(const Attn128Ctx& c, const AttnArgs& a, const u32x4 (&qf)[8],
-                                             f32x16 (&acc_o)[4], float& m_run, float& l_run,
+                                             f32x16 (&acc_o)[4], float& m_run, float& l_run, f32x16& neg_m,
                                              const uint8_t* __restrict__ rd, uint8_t* __restrict__ wr, int next_jt,
                                              bool prefetch, int j0, int wq0, bool active, int lane) {
   if (prefetch) attn128_issue(c, next_jt, a.T, wr);
@@ -852,17 +852,18 @@ __device__ __forceinline__ void attn128_tile(const Attn128Ctx& c, const AttnArgs
   const int r32 = lane & 31, h = lane >> 5;
   const uint8_t* ks = rd;
   const uint8_t* vs = rd + kD128TileBytes;
+  // S^T = K Q^T - offset: Q carries scale * log2(e) and the first MFMA of a sub-tile starts from
+  // neg_m (minus the softmax offset of the lane's row, 16 times), so the accumulators are the
+  // exponents; the offset is lazy as in the head-dimension-64 kernel (attn_tile).
   f32x16 s_acc[2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-#pragma unroll
-    for (int v = 0; v < 16; ++v) s_acc[i][v] = 0.0f;
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int sd = 0; sd < 8; ++sd) {
       const u32x4 kf = *reinterpret_cast<const u32x4*>(ks + (32 * i + r32) * 256 + (((2 * sd + h) ^ (r32 & 15)) << 4));
-      s_acc[i] = mfma16<DT>(kf, qf[sd], s_acc[i]);
+      s_acc[i] = mfma16<DT>(kf, qf[sd], sd == 0 ? neg_m : s_acc[i]);
     }
-  }
+  asm volatile("" ::"v"(neg_m));  // (alive past its last MFMA: no accumulator copies)
   if ((a.causal && j0 + kKvTile - 1 > wq0) || j0 + kKvTile > a.T) {
     const int last = a.causal ? min(wq0 + r32, a.T - 1) : a.T - 1;
 #pragma unroll
@@ -871,28 +872,45 @@ __device__ __forceinline__ void attn128_tile(const Attn128Ctx& c, const AttnArgs
       for (int v = 0; v < 16; ++v)
         if (j0 + 32 * i + 8 * (v >> 2) + 4 * h + (v & 3) > last) s_acc[i][v] = -INFINITY;
   }
-  float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
-#pragma unroll
-  for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[0][v]), s_acc[1][v]);
-  mx = halfwave_max(mx);
-  const float m_new = fmaxf(m_run, mx);
-  const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-  const float alpha = exp2_fast(m_run - m_safe);
-  m_run = m_new;
+  const float mc = m_run;
   float p[2][16];
   float l_tile = 0.0f;
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-      p[i][v] = exp2_fast(s_acc[i][v] - m_safe);
+      p[i][v] = exp2_fast(s_acc[i][v]);
       l_tile += p[i][v];
     }
-  l_run = l_run * alpha + l_tile;
+  if (__builtin_amdgcn_ballot_w64(!(l_tile <= kOffsetSlack) || mc == -INFINITY) != 0) {
+    float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
 #pragma unroll
-  for (int j = 0; j < 4; ++j)
+    for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[0][v]), s_acc[1][v]);
+    mx = halfwave_max(mx);  // relative to the offset in use (0 for a row without one)
+    const float m_old = (mc == -INFINITY) ? 0.0f : mc;
+    const float m_new = (mc == -INFINITY) ? mx : mc + fmaxf(mx, 0.0f);
+    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+    const float delta = m_safe - m_old;
+    const float alpha = exp2_fast(mc - m_safe);
+    l_run *= alpha;
+    m_run = m_new;
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc_o[j][v] *= alpha;
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc_o[j][v] *= alpha;
+    l_tile = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        p[i][v] = exp2_fast(s_acc[i][v] - delta);
+        l_tile += p[i][v];
+      }
+#pragma unroll
+    for (int v = 0; v < 16; ++v) neg_m[v] = -m_safe;
+    asm volatile("" : "+v"(neg_m));
+  }
+  l_run += l_tile;
   // V^T fragments through the transposing read (lane -> key row 4 h + j16 / 4 of the 16-key step,
   // +8 for the second read; columns 32 j + 16 (g4 % 2) + 4 (j16 % 4) .. +4).
   const int tr_row = 4 * h + ((lane & 15) >> 2), tr_col = 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
@@ -965,6 +983,10 @@ __global__ void __launch_bounds__(256, 2) attention16_d128_kernel(AttnArgs a) {
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc_o[j][v] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
+  f32x16 neg_m;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) neg_m[v] = 0.0f;
+  asm volatile("" : "+v"(neg_m));
 
   const int kv_end = a.causal ? min(a.T, q0 + 128) : a.T;
   const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
@@ -975,7 +997,7 @@ __global__ void __launch_bounds__(256, 2) attention16_d128_kernel(AttnArgs a) {
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     const int j0 = jt * kKvTile;
     const bool active = wave_valid && (!a.causal || j0 <= wq0 + 31);
-    attn128_tile<DT>(c, a, qf, acc_o, m_run, l_run, smem_d128 + (jt & 1) * kD128StageBytes,
+    attn128_tile<DT>(c, a, qf, acc_o, m_run, l_run, neg_m, smem_d128 + (jt & 1) * kD128StageBytes,
                      smem_d128 + ((jt + 1) & 1) * kD128StageBytes, jt + 1, jt + 1 < ntiles, j0, wq0, active, lane);
   }
   if (!wave_valid) return;

@@ -128,7 +128,7 @@ def test_attention_many_groups(dtype, shape, rtol, causal):
 
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype,elt", [(torch.bfloat16, "bf16"), (torch.float16, "f16")])
-@pytest.mark.parametrize("shape", [(1, 2, 512, 64), (8, 20, 1024, 64)])
+@pytest.mark.parametrize("shape", [(1, 2, 512, 64), (8, 20, 1024, 64), (1, 2, 512, 128), (2, 3, 1024, 128)])
 def test_attention_scores_outgrow_the_offset(shape, dtype, elt, causal):
     """The softmax offset is only raised when a partial row sum of P says so: scores that climb
     from one key tile to the next (by little, by 2^10 and more, and by more than f32 exp can hold)
@@ -137,7 +137,8 @@ def test_attention_scores_outgrow_the_offset(shape, dtype, elt, causal):
 
     Z, H, T, d = shape
     rng = np.random.default_rng(5 + T)
-    # score(q, key t) = 0.125 * 64 * 0.25 * ramp[t] + noise = 2 ramp[t] + noise (natural-log units)
+    # score(q, key t) = 0.125 * 64 * 0.25 * ramp[t] + noise = 2 ramp[t] + noise (natural-log units; 2.8 ramp[t]
+    # at head_dim 128, whose kernel has the same lazy offset)
     steps = np.array([0, 1, 3, 3.5, 9, 9, 30, 31, 90, 90, 91, 160, 40, 0, 161, 161], dtype=np.float32)
     ramp = np.repeat(steps[: T // 64], 64) if T // 64 <= 16 else np.repeat(steps, T // 16)
     q = 0.5 + 0.05 * rng.standard_normal((Z, H, T, d)).astype(np.float32)
@@ -156,10 +157,10 @@ def test_attention_scores_outgrow_the_offset(shape, dtype, elt, causal):
 @pytest.mark.parametrize("shape", [(2, 3, 256, 128), (1, 2, 333, 128), (1, 2, 512, 32), (1, 2, 200, 96), (1, 1, 384, 192),
                                    (1, 2, 257, 256), (1, 1, 1, 128), (2, 2, 64, 32)])
 def test_attention_other_head_dims_on_the_matrix_cores(shape, dtype, elt, causal):
-    """16-bit tensors with head_dim 32, 96, 128, 192 or 256: the matrix-core kernel for head
-    dimensions other than 64 (key tiles copied through registers, V transposed in LDS), at sequence
-    lengths that are and are not multiples of its 64-key tile and 128-row query block; also on
-    head-innermost views ([batch, seq, heads, d] seen as [batch, heads, seq, d])."""
+    """16-bit tensors with head_dim 32, 96, 128, 192 or 256: the matrix-core kernels for head
+    dimensions other than 64 (128: key tiles by LDS-DMA, two stages; the others: copied through
+    registers), at sequence lengths that are and are not multiples of the 64-key tile and 128-row
+    query block; also on head-innermost views ([batch, seq, heads, d] seen as [batch, heads, seq, d])."""
     from lighthouse_amd import ops
 
     Z, H, T, D = shape
