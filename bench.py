@@ -206,6 +206,18 @@ def main() -> int:
         dec_bytes = n8 * n8 + 16 * n8 + 16 * n8 * 2
         extras["gemm_fp8_decode_16x8192x8192_gbs"] = rate(lambda: ops.gemm_fp8(a8d, b8, 0.01, 0.01, out=o8d), dec_bytes) / 1e9
         del a8, b8, o8
+        # Beyond the named configurations: head dimension 128 and a bf16 decode shape.
+        q128, k128, v128 = (torch.randn(4, 16, 2048, 128, device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
+        o128 = torch.empty_like(q128)
+        extras["attention_bf16_d128_noncausal_tflops"] = rate(
+            lambda: ops.attention(q128, k128, v128, out=o128), 4.0 * 4 * 16 * 2048 * 2048 * 128) / 1e12
+        del q128, k128, v128, o128
+        ad = torch.randn(16, n8, device="cuda", generator=g).to(torch.bfloat16)
+        bd = torch.randn(n8, n8, device="cuda", generator=g).to(torch.bfloat16)
+        od = torch.empty(16, n8, device="cuda", dtype=torch.bfloat16)
+        extras["gemm_bf16_decode_16x8192x8192_gbs"] = rate(
+            lambda: ops.gemm(ad, bd, out=od), 2.0 * n8 * n8 + 2 * 2 * 16 * n8) / 1e9
+        del ad, bd, od
         M, C = 8192, 768
         x = torch.randn(M, C, device="cuda", generator=g)
         gam, bet = torch.ones(C, device="cuda"), torch.zeros(C, device="cuda")
