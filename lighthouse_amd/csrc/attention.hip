@@ -628,7 +628,9 @@ static int attention16_launch_ragged(const AttnArgs& a, hipStream_t s) {
 // last tile's loads, masks it and skips rows past the end.
 template <int DT, int NQ, int NS>
 static int attention16_launch_nq(const AttnArgs& a, hipStream_t s) {
-  if (a.T % kKvTile != 0) return attention16_launch_ragged<DT, NQ, NS, true>(a, s);
+  if constexpr (NQ == 1) {
+    if (a.T % kKvTile != 0) return attention16_launch_ragged<DT, NQ, NS, true>(a, s);
+  }
   return attention16_launch_ragged<DT, NQ, NS, false>(a, s);
 }
 
@@ -644,7 +646,9 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
   // Short sequences that do not fill their last 256-row block waste less of a 128-row one
   // ([64,16,257]: 80 -> 57 us, [128,12,300]: 111 -> 82 us).
   const bool short_rows = a.T <= 640 && a.T % kQBlock16 != 0;
-  if (groups64 < limit || short_rows) {
+  // (A partial last key tile also takes the 32-rows-per-wave kernels: the 64-row one has no
+  // registers left for the clamped loads and would spill.)
+  if (groups64 < limit || short_rows || a.T % kKvTile != 0) {
     // With more than one 128-row workgroup per CU a ring of 3 stages (48 KiB) lets three of them
     // share a CU instead of two ([8,12,1024] causal 26.7 -> 25.3 us, [16,16,512] causal 24.2 ->
     // 22.3); a problem that does not fill the CUs is better off with the deeper ring.
@@ -712,6 +716,10 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc_o[j][v] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
+  f32x16 neg_m;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) neg_m[v] = 0.0f;
+  asm volatile("" : "+v"(neg_m));
 
   const int kv_end = a.causal ? min(a.T, q0 + 128) : a.T;
   const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
@@ -730,20 +738,18 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
     }
     __syncthreads();
     if (!wave_valid || (a.causal && j0 > wq0 + 31)) continue;
-    // S^T = K Q^T - nothing: the accumulators are the scores times scale * log2(e).
+    // S^T = K Q^T - offset: the first MFMA of a sub-tile starts from neg_m (minus the lane's softmax
+    // offset, 16 times), so the accumulators are the exponents; lazy offset as in attn_tile.
     f32x16 s_acc[2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-#pragma unroll
-      for (int v = 0; v < 16; ++v) s_acc[i][v] = 0.0f;
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int sd = 0; sd < D / 16; ++sd) {
         const u32x4 kf = *reinterpret_cast<const u32x4*>(Ks + (32 * i + r32) * KROW + 16 * sd + 8 * h);
-        if constexpr (Q_LDS) s_acc[i] = mfma16<DT>(kf, q_lds[sd * 64], s_acc[i]);
-        else s_acc[i] = mfma16<DT>(kf, qf[sd], s_acc[i]);
+        if constexpr (Q_LDS) s_acc[i] = mfma16<DT>(kf, q_lds[sd * 64], sd == 0 ? neg_m : s_acc[i]);
+        else s_acc[i] = mfma16<DT>(kf, qf[sd], sd == 0 ? neg_m : s_acc[i]);
       }
-    }
-    // s_acc[i][v] = score of (query wq0 + r32, key j0 + 32 i + 8 (v / 4) + 4 h + v % 4)
+    asm volatile("" ::"v"(neg_m));  // (alive past its last MFMA: no accumulator copies)
     if ((a.causal && j0 + kKvTile - 1 > wq0) || j0 + kKvTile > a.T) {
       const int last = a.causal ? min(wq0 + r32, a.T - 1) : a.T - 1;
 #pragma unroll
@@ -752,28 +758,45 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
         for (int v = 0; v < 16; ++v)
           if (j0 + 32 * i + 8 * (v >> 2) + 4 * h + (v & 3) > last) s_acc[i][v] = -INFINITY;
     }
-    float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
-#pragma unroll
-    for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[0][v]), s_acc[1][v]);
-    mx = halfwave_max(mx);
-    const float m_new = fmaxf(m_run, mx);
-    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // a row without a visible key so far
-    const float alpha = exp2_fast(m_run - m_safe);
-    m_run = m_new;
+    const float mc = m_run;
     float p[2][16];
     float l_tile = 0.0f;
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        p[i][v] = exp2_fast(s_acc[i][v] - m_safe);
+        p[i][v] = exp2_fast(s_acc[i][v]);
         l_tile += p[i][v];
       }
-    l_run = l_run * alpha + l_tile;
+    if (__builtin_amdgcn_ballot_w64(!(l_tile <= kOffsetSlack) || mc == -INFINITY) != 0) {
+      float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
 #pragma unroll
-    for (int j = 0; j < DB; ++j)
+      for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[0][v]), s_acc[1][v]);
+      mx = halfwave_max(mx);  // relative to the offset in use (0 for a row without one)
+      const float m_old = (mc == -INFINITY) ? 0.0f : mc;
+      const float m_new = (mc == -INFINITY) ? mx : mc + fmaxf(mx, 0.0f);
+      const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+      const float delta = m_safe - m_old;
+      const float alpha = exp2_fast(mc - m_safe);
+      l_run *= alpha;
+      m_run = m_new;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc_o[j][v] *= alpha;
+      for (int j = 0; j < DB; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc_o[j][v] *= alpha;
+      l_tile = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          p[i][v] = exp2_fast(s_acc[i][v] - delta);
+          l_tile += p[i][v];
+        }
+#pragma unroll
+      for (int v = 0; v < 16; ++v) neg_m[v] = -m_safe;
+      asm volatile("" : "+v"(neg_m));
+    }
+    l_run += l_tile;
     // O^T += V^T P^T.  V^T fragments come from the row-major tile through the transposing read:
     // lane (g4 = lane / 16, j16 = lane % 16) addresses key row 4 h + j16 / 4 of the 16-key step
     // (+8 for the second read), columns 32 j + 16 (g4 % 2) + 4 (j16 % 4) .. +4, and receives 8 keys
