@@ -109,7 +109,9 @@ def tune_shape(M: int, N: int, K: int, dtype: str = "bf16", db: TileDB | None = 
     `isolate=False` times in this process (no protection against a hanging or crashing trial)."""
     cands = candidate_tiles(M, N, K) if exhaustive else prefilter(M, N, K)
     best = None
-    for tile in cands:
+    # The library's own choice (tile None: its cost model, split K for decode shapes) is timed first;
+    # a tile enters the database only if it beats that.
+    for tile in [None, *cands] if cands else []:
         if isolate:
             res = run_with_timeout(_time_tile, M, N, K, dtype, tile, nruns, nwarmup, timeout=timeout)
         else:
@@ -118,14 +120,15 @@ def tune_shape(M: int, N: int, K: int, dtype: str = "bf16", db: TileDB | None = 
                 _time_tile(res, M, N, K, dtype, tile, nruns, nwarmup)
             except (ValueError, RuntimeError) as exc:
                 res["error"] = str(exc).split("\n")[0]
-        row = {"dtype": dtype, "M": M, "N": N, "K": K, "tile_m": tile[0], "tile_n": tile[1],
-               "estimate": round(estimate_cost(M, N, K, tile) / 1e6, 3), "time_us": round(res["time"] * 1e6, 3),
+        row = {"dtype": dtype, "M": M, "N": N, "K": K, "tile_m": tile[0] if tile else 0, "tile_n": tile[1] if tile else 0,
+               "estimate": round(estimate_cost(M, N, K, tile) / 1e6, 3) if tile else 0.0,
+               "time_us": round(res["time"] * 1e6, 3),
                "tflops": round(res["throughput"], 2), "error": res["error"]}
         if logger is not None:
             logger.log(row)
         if not res["error"] and res["time"] > 0 and (best is None or row["time_us"] < best["time_us"]):
             best = row
-    if best is not None and db is not None:
+    if best is not None and db is not None and best["tile_m"]:
         db.record(dtype, M, N, K, (best["tile_m"], best["tile_n"]), best["time_us"], best["tflops"])
     return best
 

@@ -552,8 +552,9 @@ def test_gemm_transposed_and_ragged(shape, ta, tb, elt):
 
 
 def test_tile_search_and_database(tmp_path):
-    """The tuner times every fitting tile for a shape, logs the trials, records the winner, and
-    ops.gemm picks the recorded tile up when the database is in use (same results either way)."""
+    """The tuner times the library's own choice and every fitting tile for a shape, logs the trials,
+    records a tile that beats the library's choice, and ops.gemm picks a recorded tile up when the
+    database is in use (same results either way)."""
     from lighthouse_amd import ops
     from lighthouse_amd.tuning import CSVLogger, TileDB, tune_shape, use_db
 
@@ -562,8 +563,13 @@ def test_tile_search_and_database(tmp_path):
     logger = CSVLogger(str(tmp_path / "trials.csv"), echo_stdout=False)
     best = tune_shape(M, N, K, "bf16", db, logger, nruns=5, nwarmup=2, exhaustive=True, isolate=False)
     rows = (tmp_path / "trials.csv").read_text().strip().splitlines()
-    assert len(rows) == 1 + 4 and best is not None and best["error"] == "" and best["tflops"] > 0
-    assert db.lookup("bf16", M, N, K) == (best["tile_m"], best["tile_n"])
+    assert len(rows) == 1 + 1 + 4 and best is not None and best["error"] == "" and best["tflops"] > 0
+    assert rows[1].split(",")[4:6] == ["0", "0"]  # the first trial is the automatic choice
+    if best["tile_m"]:
+        assert db.lookup("bf16", M, N, K) == (best["tile_m"], best["tile_n"])
+    else:
+        assert db.lookup("bf16", M, N, K) is None
+        db.record("bf16", M, N, K, (128, 128), 1.0, 1.0)  # (so that the lookup below has something to find)
     a = torch.randn(M, K, device="cuda").to(torch.bfloat16)
     b = torch.randn(K, N, device="cuda").to(torch.bfloat16)
     plain = ops.gemm(a, b)
