@@ -1076,11 +1076,7 @@ static int attention16_anyd_dispatch(const AttnArgs& a, int d, hipStream_t s) {
   switch (d) {
     case 32: return attention16_anyd_launch<DT, 1>(a, s);
     case 96: return attention16_anyd_launch<DT, 3>(a, s);
-#ifdef LH_ATTN_D128_PADDED
-    case 128: return attention16_anyd_launch<DT, 4>(a, s);
-#else
     case 128: return attention16_d128_launch<DT>(a, s);
-#endif
     case 192: return attention16_anyd_launch<DT, 6>(a, s);
     case 256: return attention16_anyd_launch<DT, 8>(a, s);
     default: return 1;
