@@ -43,7 +43,9 @@ __device__ __forceinline__ void store4(void* p, int64_t i, f32x4 v) {
 // values -> var = that * (1/N); (x - mean) * rsqrt(var + eps) * gamma + beta.
 // A wave takes RPW rows (r, r + rows/RPW ...): all of them, gamma and beta are requested up
 // front, so that the loads of a later row and the stores of an earlier one overlap.
-template <int XDT, int ODT, int VPL, int RPW>
+// GUARD: N is any multiple of 4 up to 256 VPL; element groups past the end are neither loaded,
+// counted nor stored (hidden sizes such as 384, 640 or 1280).
+template <int XDT, int ODT, int VPL, int RPW, bool GUARD = false>
 __global__ void __launch_bounds__(256) layer_norm_vec(void* out, const void* x, const float* gamma, const float* beta,
                                                       int M, int N, float eps, float inv_n) {
   const int lane = threadIdx.x & 63;
@@ -55,13 +57,19 @@ __global__ void __launch_bounds__(256) layer_norm_vec(void* out, const void* x, 
   for (int r = 0; r < RPW; ++r) {
     const int row = min(slot + r * slots, M - 1);  // a row past the end repeats the last one and is not stored
 #pragma unroll
-    for (int i = 0; i < VPL; ++i) v[r][i] = load4<XDT>(x, (int64_t)row * N + (i * 64 + lane) * 4);
+    for (int i = 0; i < VPL; ++i) {
+      v[r][i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      if (!GUARD || (i * 64 + lane) * 4 < N) v[r][i] = load4<XDT>(x, (int64_t)row * N + (i * 64 + lane) * 4);
+    }
   }
   f32x4 g[VPL], b[VPL];
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    g[i] = *reinterpret_cast<const f32x4*>(gamma + (i * 64 + lane) * 4);
-    b[i] = *reinterpret_cast<const f32x4*>(beta + (i * 64 + lane) * 4);
+    g[i] = b[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (!GUARD || (i * 64 + lane) * 4 < N) {
+      g[i] = *reinterpret_cast<const f32x4*>(gamma + (i * 64 + lane) * 4);
+      b[i] = *reinterpret_cast<const f32x4*>(beta + (i * 64 + lane) * 4);
+    }
   }
 #pragma unroll
   for (int r = 0; r < RPW; ++r) {
@@ -73,6 +81,7 @@ __global__ void __launch_bounds__(256) layer_norm_vec(void* out, const void* x, 
     float q = 0.0f;
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
+      if (GUARD && (i * 64 + lane) * 4 >= N) continue;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         float c = v[r][i][e] - mean;
@@ -83,6 +92,7 @@ __global__ void __launch_bounds__(256) layer_norm_vec(void* out, const void* x, 
     if (row < M) {
 #pragma unroll
       for (int i = 0; i < VPL; ++i) {
+        if (GUARD && (i * 64 + lane) * 4 >= N) continue;
         f32x4 o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] = (v[r][i][e] - mean) * inv_std * g[i][e] + b[i][e];
@@ -115,7 +125,7 @@ __global__ void __launch_bounds__(256) layer_norm_generic(void* out, const void*
 
 // Row softmax with the row resident in registers (N = 256 VPL): one read and one write per
 // element, one exp per element.
-template <int DT, int VPL>
+template <int DT, int VPL, bool GUARD = false>
 __global__ void __launch_bounds__(256) softmax_rows_vec(void* out, const void* x, int M, int N) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -125,7 +135,8 @@ __global__ void __launch_bounds__(256) softmax_rows_vec(void* out, const void* x
   float mx = -INFINITY;
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
-    v[i] = load4<DT>(x, base + (i * 64 + lane) * 4);
+    v[i] = f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};  // (GUARD: groups past the end count as exp(-inf) = 0)
+    if (!GUARD || (i * 64 + lane) * 4 < N) v[i] = load4<DT>(x, base + (i * 64 + lane) * 4);
     mx = fmaxf(fmaxf(mx, fmaxf(v[i][0], v[i][1])), fmaxf(v[i][2], v[i][3]));
   }
   mx = wave_max(mx);
@@ -143,7 +154,7 @@ __global__ void __launch_bounds__(256) softmax_rows_vec(void* out, const void* x
     f32x4 o;
 #pragma unroll
     for (int e = 0; e < 4; ++e) o[e] = v[i][e] / s;
-    store4<DT>(out, base + (i * 64 + lane) * 4, o);
+    if (!GUARD || (i * 64 + lane) * 4 < N) store4<DT>(out, base + (i * 64 + lane) * 4, o);
   }
 }
 
@@ -396,6 +407,15 @@ static inline unsigned ew_grid(int64_t work) {
   return (unsigned)(b > cap ? cap : b);
 }
 
+// Smallest instantiated count of 4-element groups per lane that covers a row of N elements.
+static inline int row_groups_rounded(int N) {
+  const int need = (N + 255) / 256;
+  const int have[] = {1, 2, 3, 4, 6, 8, 12, 16};
+  for (int v : have)
+    if (v >= need) return v;
+  return 0;
+}
+
 template <int XDT, int ODT>
 static int layer_norm_launch(void* out, const void* x, const float* gamma, const float* beta, int M, int N, float eps,
                              hipStream_t s) {
@@ -422,6 +442,20 @@ static int layer_norm_launch(void* out, const void* x, const float* gamma, const
   }
 #undef LH_LN_CASE
   const bool vec4 = N % 4 == 0 && aligned16(out) && aligned16(x) && aligned16(gamma) && aligned16(beta);
+  // Any other row of whole 4-element groups up to 4096 elements: the next register count up, guarded.
+  if (vec4 && N >= 64 && N <= 4096) {
+#define LH_LN_GUARD(V)                                                                                                \
+  case V:                                                                                                             \
+    hipLaunchKernelGGL((layer_norm_vec<XDT, ODT, V, 1, true>), grid, block, 0, s, out, x, gamma, beta, M, N, eps,      \
+                       inv_n);                                                                                        \
+    return check_launch("layer_norm_vec (guarded)");
+    switch (row_groups_rounded(N)) {
+      LH_LN_GUARD(1) LH_LN_GUARD(2) LH_LN_GUARD(3) LH_LN_GUARD(4) LH_LN_GUARD(6) LH_LN_GUARD(8) LH_LN_GUARD(12)
+      LH_LN_GUARD(16)
+      default: break;
+    }
+#undef LH_LN_GUARD
+  }
   if (N >= 1024 || (vec4 && N >= 512)) {
     if (vec4 && N <= 1024 * kBlockRegGroups)
       hipLaunchKernelGGL((layer_norm_block_reg<XDT, ODT>), dim3(M), block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);
@@ -501,6 +535,23 @@ int lh_hip_softmax(void* out, const void* x, int64_t M, int64_t N, int32_t dtype
 #undef LH_SM_CASE
   }
   const bool vec = N % 4 == 0 && aligned16(out) && aligned16(x);
+  if (vec && N >= 64 && N <= 4096) {
+#define LH_SM_GUARD(DT, V)                                                                           \
+  case V:                                                                                            \
+    hipLaunchKernelGGL((softmax_rows_vec<DT, V, true>), grid, block, 0, s, out, x, (int)M, (int)N);  \
+    return check_launch("softmax_rows_vec (guarded)");
+#define LH_SM_GUARD_DTYPE(DT)                                                                        \
+  switch (row_groups_rounded((int)N)) {                                                              \
+    LH_SM_GUARD(DT, 1) LH_SM_GUARD(DT, 2) LH_SM_GUARD(DT, 3) LH_SM_GUARD(DT, 4) LH_SM_GUARD(DT, 6)   \
+    LH_SM_GUARD(DT, 8) LH_SM_GUARD(DT, 12) LH_SM_GUARD(DT, 16)                                       \
+    default: break;                                                                                  \
+  }
+    if (dtype == LH_F32) { LH_SM_GUARD_DTYPE(LH_F32) }
+    else if (dtype == LH_BF16) { LH_SM_GUARD_DTYPE(LH_BF16) }
+    else if (dtype == LH_F16) { LH_SM_GUARD_DTYPE(LH_F16) }
+#undef LH_SM_GUARD_DTYPE
+#undef LH_SM_GUARD
+  }
   if (N >= 1024 || (vec && N >= 512)) {
     const dim3 rows((unsigned)M);
 #define LH_SMB_CASE(DT)                                                                                    \

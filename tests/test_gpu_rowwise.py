@@ -55,6 +55,39 @@ def test_long_rows_one_workgroup_per_row(shape, elt):
         assert_close(sm, ref, 2e-2, f"softmax {shape} bf16")
 
 
+@pytest.mark.parametrize(
+    "shape", [(777, 64), (513, 260), (1030, 384), (300, 640), (257, 896), (129, 1000), (66, 1152), (35, 1284),
+              (34, 2560), (9, 3332), (6, 3584), (5, 4092)]
+)
+@pytest.mark.parametrize("elt", ["f32", "bf16"])
+def test_rows_of_whole_vector_groups_stay_in_registers(shape, elt):
+    """Row lengths that are multiples of 4 but not of 256 (or an uncommon multiple): one wave per row
+    with the tail groups masked. Row counts are not multiples of 4 so the last workgroup is partial."""
+    from lighthouse_amd import ops
+
+    rng = np.random.default_rng(shape[0] * 7 + shape[1])
+    dt = torch.float32 if elt == "f32" else torch.bfloat16
+    x = orc.round_to(rng.standard_normal(shape).astype(np.float32) * 2 - 0.75, elt)
+    g = rng.uniform(0.5, 1.5, shape[1:]).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, shape[1:]).astype(np.float32)
+    # The output buffer is one row longer than the result and pre-filled: nothing past the end may change.
+    m, n = shape
+    buf = torch.full((m + 1, n), 123.0, device="cuda", dtype=dt)
+    out = ops.layer_norm(_dev(x, dt), _dev(g), _dev(b), 1e-5, out=buf[:m])
+    rtol = 1e-4 if elt == "f32" else 2e-2
+    assert_close(_host(out), orc.layer_norm(x, g, b, 1e-5, result_type=elt), rtol, f"layer_norm {shape} {elt}")
+    assert torch.all(buf[m] == 123.0)
+    buf.fill_(123.0)
+    sm = _host(ops.softmax(_dev(x, dt), out=buf[:m]))
+    assert torch.all(buf[m] == 123.0)
+    ref = orc.softmax(x, result_type=elt)
+    if elt == "f32":
+        assert np.allclose(sm.sum(1), 1.0, rtol=1e-5, atol=1e-6)
+        assert np.allclose(sm, ref, rtol=1e-4, atol=1e-6)
+    else:
+        assert_close(sm, ref, 2e-2, f"softmax {shape} bf16")
+
+
 def test_layer_norm_bf16_out_and_in():
     from lighthouse_amd import ops
 
