@@ -828,14 +828,10 @@ static int direct_variant(int M, int N, int K) {
 // Sum of the split-K blocks (f32, [splits][M][N]) and the problem's own epilogue, 4 columns per thread.
 template <int DT>
 __global__ void __launch_bounds__(256) gemm16_splitk_reduce(GemmArgs g, const float* partial, int splits) {
-  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (idx >= (int64_t)g.M * g.N) return;
   const int m = (int)(idx / g.N), n = (int)(idx % g.N);
-  f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int sp = 0; sp < splits; ++sp) {
-    const f32x4 p = *reinterpret_cast<const f32x4*>(partial + ((int64_t)sp * g.M + m) * g.N + n);
-    v[0] += p[0]; v[1] += p[1]; v[2] += p[2]; v[3] += p[3];
-  }
+  const f32x4 v = splitk_sum4(partial + (int64_t)m * g.N + n, (int64_t)g.M * g.N, splits, blockDim.x == 64);
   epilogue4<DT>(g, m, n, v[0], v[1], v[2], v[3]);
 }
 
@@ -878,7 +874,8 @@ static int gemm16_splitk(const GemmArgs& g, hipStream_t s) {
                       : launch(gemm16_direct<DT, 2, 1, false, true>, configured_whole);
   if (rc) return rc;
   const int64_t groups = (int64_t)g.M * g.N / 4;
-  hipLaunchKernelGGL(gemm16_splitk_reduce<DT>, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s, g, partial, splits);
+  const int rb = reduce_block(groups);
+  hipLaunchKernelGGL(gemm16_splitk_reduce<DT>, dim3((unsigned)((groups + rb - 1) / rb)), dim3(rb), 0, s, g, partial, splits);
   return check_launch("gemm16_splitk_reduce");
 }
 

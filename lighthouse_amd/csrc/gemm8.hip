@@ -492,14 +492,10 @@ static int launch_direct8(const GemmArgs& g, hipStream_t s) {
 
 // Sum of the split-K blocks ([splits][M][N] f32), scale, conversion: 4 columns per thread.
 __global__ void __launch_bounds__(256) gemm8_splitk_reduce(GemmArgs g, const float* partial, int splits) {
-  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (idx >= (int64_t)g.M * g.N) return;
   const int m = (int)(idx / g.N), n = (int)(idx % g.N);
-  f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
-  for (int sp = 0; sp < splits; ++sp) {
-    const f32x4 p = *reinterpret_cast<const f32x4*>(partial + ((int64_t)sp * g.M + m) * g.N + n);
-    v[0] += p[0]; v[1] += p[1]; v[2] += p[2]; v[3] += p[3];
-  }
+  const f32x4 v = splitk_sum4(partial + (int64_t)m * g.N + n, (int64_t)g.M * g.N, splits, blockDim.x == 64);
   epilogue4<LH_BF16>(g, m, n, v[0], v[1], v[2], v[3]);
 }
 
@@ -534,7 +530,8 @@ static int gemm8_splitk(const GemmArgs& g, hipStream_t s) {
   int rc = check_launch("gemm8_direct (split K)");
   if (rc) return rc;
   const int64_t groups = (int64_t)g.M * g.N / 4;
-  hipLaunchKernelGGL(gemm8_splitk_reduce, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, s, g, partial, splits);
+  const int rb = reduce_block(groups);
+  hipLaunchKernelGGL(gemm8_splitk_reduce, dim3((unsigned)((groups + rb - 1) / rb)), dim3(rb), 0, s, g, partial, splits);
   return check_launch("gemm8_splitk_reduce");
 }
 
@@ -819,13 +816,13 @@ __global__ void __launch_bounds__(256) gemm8_skinny_mt(GemmArgs g, float* partia
   }
 }
 
+// Sum of the split-K blocks partial[split][rows][N] and the epilogue, 4 columns per thread.
 __global__ void __launch_bounds__(256) gemm8_skinny_reduce(GemmArgs g, const float* partial, int splits, int rows) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t idx = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
   if (idx >= (int64_t)g.M * g.N) return;
   const int m = (int)(idx / g.N), n = (int)(idx % g.N);
-  float s = 0.0f;
-  for (int sp = 0; sp < splits; ++sp) s += partial[((int64_t)sp * rows + m) * g.N + n];
-  epilogue1<LH_BF16>(g, m, n, s);
+  const f32x4 v = splitk_sum4(partial + (int64_t)m * g.N + n, (int64_t)rows * g.N, splits, blockDim.x == 64);
+  epilogue4<LH_BF16>(g, m, n, v[0], v[1], v[2], v[3]);
 }
 
 static float* g_partial = nullptr;
@@ -874,8 +871,9 @@ static int launch_skinny_mt(const GemmArgs& g, hipStream_t s) {
                      g.K / splits);
   rc = check_launch("gemm8_skinny_mt");
   if (rc) return rc;
-  const int64_t total = (int64_t)g.M * g.N;
-  hipLaunchKernelGGL(gemm8_skinny_reduce, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, g, g_partial, splits,
+  const int64_t groups = (int64_t)g.M * g.N / 4;
+  const int rb = reduce_block(groups);
+  hipLaunchKernelGGL(gemm8_skinny_reduce, dim3((unsigned)((groups + rb - 1) / rb)), dim3(rb), 0, s, g, g_partial, splits,
                      16 * MT);
   return check_launch("gemm8_skinny_reduce");
 }
@@ -906,8 +904,9 @@ int gemm8(const GemmArgs& g, hipStream_t s) {
       hipLaunchKernelGGL(gemm8_skinny, dim3(nblk, splits), dim3(256), kSkinnyLdsBytes, s, g, g_partial, g.K / splits);
       int rc = check_launch("gemm8_skinny");
       if (rc) return rc;
-      const int64_t total = (int64_t)g.M * g.N;
-      hipLaunchKernelGGL(gemm8_skinny_reduce, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, g, g_partial,
+      const int64_t groups = (int64_t)g.M * g.N / 4;
+      const int rb = reduce_block(groups);
+      hipLaunchKernelGGL(gemm8_skinny_reduce, dim3((unsigned)((groups + rb - 1) / rb)), dim3(rb), 0, s, g, g_partial,
                          splits, 16);
       return check_launch("gemm8_skinny_reduce");
     }

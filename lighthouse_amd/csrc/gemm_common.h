@@ -209,6 +209,40 @@ inline int gemm_padded(const GemmArgs& g, int k_multiple, int n_multiple, hipStr
   return LH_OK;
 }
 
+// Sum over the f32 blocks of a split-K launch for 4 consecutive columns: p + sp * step, sp = 0 ..
+// splits - 1, added in that order.  `deep`: up to 8 loads are in flight before the first add, for the
+// small reductions (a few MiB spread over every CU) that are bound by latency alone; large ones
+// are faster with one block at a time (8 streams several MiB apart: 41 -> 43 us at 256 x 8192 x 8).
+__device__ __forceinline__ f32x4 splitk_sum4(const float* p, int64_t step, int splits, bool deep) {
+  f32x4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+  if (!deep) {
+    for (int sp = 0; sp < splits; ++sp) {
+      const f32x4 t = *reinterpret_cast<const f32x4*>(p + sp * step);
+      v[0] += t[0]; v[1] += t[1]; v[2] += t[2]; v[3] += t[3];
+    }
+    return v;
+  }
+  int sp = 0;
+  for (; sp + 8 <= splits; sp += 8) {
+    f32x4 t[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) t[u] = *reinterpret_cast<const f32x4*>(p + (sp + u) * step);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      v[0] += t[u][0]; v[1] += t[u][1]; v[2] += t[u][2]; v[3] += t[u][3];
+    }
+  }
+  for (; sp < splits; ++sp) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(p + sp * step);
+    v[0] += t[0]; v[1] += t[1]; v[2] += t[2]; v[3] += t[3];
+  }
+  return v;
+}
+
+// Workgroup size of a reduce kernel over `groups` 4-column groups: one wave per workgroup while
+// that still gives every CU only a few of them (decode batches up to 32 rows of 8192), else 256.
+static inline int reduce_block(int64_t groups) { return groups <= 64 * 1024 ? 64 : 256; }
+
 // One output element, any alignment (edge tiles and the generic kernels).
 template <int DT>
 __device__ __forceinline__ void epilogue1(const GemmArgs& g, int m, int n, float x) {
