@@ -843,6 +843,9 @@ static int gemm16_splitk(const GemmArgs& g, hipStream_t s) {
   const int cus = num_cus();
   const int64_t tiles = (int64_t)((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
   if (tiles * 2 > cus || g.K < 2048) return 1;
+  // With more than a quarter of the CUs busy anyway, the second kernel costs more than cutting a
+  // K of 2048 saves (M = 512, N = 4096: 24.1 us cut, 19.7 us whole; at K = 3072 the two are level).
+  if (tiles * 4 > cus && g.K < 3072) return 1;
   int splits = 1;
   while (splits < 8 && tiles * splits * 2 <= 2 * cus && (g.K / (splits * 2)) % kBK == 0 && g.K / (splits * 2) >= 512)
     splits *= 2;
