@@ -504,7 +504,12 @@ __global__ void __launch_bounds__(256) gemm8_splitk_reduce(GemmArgs g, const flo
 static int gemm8_splitk(const GemmArgs& g, hipStream_t s) {
   const int cus = num_cus();
   const int64_t tiles = (int64_t)(g.M / 256) * (g.N / 256);
-  if (tiles * 2 > cus || g.K < 2048) return 1;
+  // Measured against the uncut kernel (M 256 ... 4096, N 1024 ... 8192): cutting pays from K = 8192 on,
+  // and at K = 4096 only when the tiles cover at most an eighth of the CUs (four cuts); below
+  // that the partial blocks and the second kernel cost more than the shorter main loop saves
+  // (512 x 8192 x 2048: 30.3 us cut, 20.9 us whole; 256 x 1024 x 8192: 26 us cut, 62 us whole).
+  if (tiles * 2 > cus || g.K < 4096) return 1;
+  if (g.K < 8192 && tiles * 8 > cus) return 1;
   int splits = 1;
   while (splits < 8 && tiles * splits * 2 <= cus && (g.K / (splits * 2)) % kBK8 == 0 && g.K / (splits * 2) >= 1024)
     splits *= 2;
