@@ -642,7 +642,10 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
   const int64_t groups64 = (int64_t)((a.T + kQBlock16 - 1) / kQBlock16) * a.Z * a.H;
   // Measured on [4,16,2048]: 32 rows per wave 105 us non-causal (64 rows: 99) but 54 us causal
   // (64 rows: 58), hence the different limits.
-  const int64_t limit = a.causal ? 2 * (int64_t)a.cus + 1 : 2 * (int64_t)a.cus;
+  // Causal launches of sequences up to 1024 stay on the 32-row kernel up to four 256-row groups per
+  // CU (the masked diagonal is a larger share of a 256-row block: [1,192,1024] 42.7 vs 44.8 us,
+  // [1,512,512] 41.1 vs 43.3; beyond that the 64-row kernel is ahead again, [1,512,1024] 108 vs 113).
+  const int64_t limit = !a.causal ? 2 * (int64_t)a.cus : (a.T <= 1024 ? 4 : 2) * (int64_t)a.cus + 1;
   // Short sequences that do not fill their last 256-row block waste less of a 128-row one
   // ([64,16,257]: 80 -> 57 us, [128,12,300]: 111 -> 82 us).
   const bool short_rows = a.T <= 640 && a.T % kQBlock16 != 0;
