@@ -26,6 +26,14 @@
  *  - The caller owns every buffer; no entry point allocates results
  *    (lighthouse/dialects/transform/transform_ext/ops/convert_func_results_to_args.py:14-24).
  *  - Matrices are row-major; `ld*` are leading dimensions in elements.
+ *  - Temporary device memory: a few problems need more than their operands (transposed or unaligned
+ *    operands run on copies, short-and-wide "decode" problems are cut along K into f32 blocks that a
+ *    second kernel adds up).  The plain entry points take it from a pool the library keeps per
+ *    (device, stream): calls on different streams never share it, it only grows, and nothing is
+ *    freed inside a call (lh_hip_release_scratch() returns it).  The *_ws entry points and the
+ *    nanoGPT entry points take a caller workspace instead and never allocate
+ *    (lighthouse/dialects/transform/transform_ext/ops/convert_func_results_to_args.py:14-24: the
+ *    callee does not allocate).
  */
 #ifndef LIGHTHOUSE_HIP_H
 #define LIGHTHOUSE_HIP_H
@@ -107,6 +115,10 @@ int lh_hip_memcpy_d2h(void* host_dst, const void* dev_src, size_t bytes);
 int lh_hip_memcpy_d2d(void* dev_dst, const void* dev_src, size_t bytes);
 int lh_hip_memset(void* dev_ptr, int value, size_t bytes);
 int lh_hip_sync(void* stream);
+/* Waits for the current device and frees the library's pool of temporary buffers on it (no
+ * counterpart in the reference, whose JIT'd code frees its temporaries itself:
+ * examples/xegpu/nanoGPT_payload.py:407-408). */
+int lh_hip_release_scratch(void);
 
 /* --------------------------------------------------- plain pointer kernels ---- */
 
@@ -120,6 +132,19 @@ int lh_hip_sync(void* stream);
 int lh_hip_gemm(void* out, const void* a, const void* b, const void* bias, int64_t M, int64_t N, int64_t K,
                 int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype, int32_t out_dtype, uint32_t flags,
                 void* stream);
+
+/*
+ * lh_hip_gemm with its temporary memory in a caller workspace of at least
+ * lh_hip_gemm_workspace_bytes(...) bytes (0 for most problems; the query assumes 16-byte aligned
+ * operands).  No allocation happens inside the call; a workspace that is too small fails with
+ * LH_ERR_INVALID.  Same role as the workspace of lh_hip_nanogpt_block for callers that manage
+ * device memory themselves (GPUMemoryManager, lighthouse/execution/memory_manager.py:97-151).
+ */
+size_t lh_hip_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                   int32_t ab_dtype, int32_t out_dtype, uint32_t flags);
+int lh_hip_gemm_ws(void* out, const void* a, const void* b, const void* bias, int64_t M, int64_t N, int64_t K,
+                   int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype, int32_t out_dtype, uint32_t flags,
+                   void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * lh_hip_gemm whose accumulation starts from a separate matrix: out = epilogue(c + A.B), with
@@ -141,6 +166,12 @@ int lh_hip_gemm_residual(void* out, const void* c, const void* a, const void* b,
  */
 int lh_hip_gemm_fp8(void* out, const void* a_q, const void* b_q, float scale_a, float scale_b, int64_t M,
                     int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int32_t out_dtype, void* stream);
+/* The same with a caller workspace (see lh_hip_gemm_ws); the decode shapes (M <= 128) always need one. */
+size_t lh_hip_gemm_fp8_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                                       int32_t out_dtype);
+int lh_hip_gemm_fp8_ws(void* out, const void* a_q, const void* b_q, float scale_a, float scale_b, int64_t M,
+                       int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int32_t out_dtype,
+                       void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Fused attention forward, the payload of generate_gpu_attention_payload
@@ -163,8 +194,9 @@ int lh_hip_attention(void* out, const void* q, const void* k, const void* v, int
 /*
  * Row LayerNorm, emit_layer_norm_generics
  * (lighthouse/ingress/mlir_gen/gpu_layer_norm_payload.py:15-87): x [M,N] (x_dtype F32 or
- * BF16), gamma/beta [N] f32, statistics in f32, out [M,N] in out_dtype (F32 or BF16; BF16
- * fuses the cast that follows every LayerNorm in examples/xegpu/nanoGPT_payload.py:299-317).
+ * BF16), gamma/beta [N] f32, statistics in f32, out [M,N] in out_dtype (F32, BF16 or, from an
+ * F32 input, F16; a 16-bit output fuses the cast that follows every LayerNorm in
+ * examples/xegpu/nanoGPT_payload.py:299-317).
  */
 int lh_hip_layer_norm(void* out, const void* x, const float* gamma, const float* beta, int64_t M, int64_t N,
                       float eps, int32_t x_dtype, int32_t out_dtype, void* stream);
@@ -184,51 +216,67 @@ int lh_hip_add(void* out, const void* a, const void* b, int64_t n, int32_t dtype
 int lh_hip_cast(void* out, const void* x, int64_t n, int32_t src_dtype, int32_t dst_dtype, void* stream);
 
 /*
- * One pre-LayerNorm GPT-2 block forward (op order of _emit_block_fused,
- * examples/xegpu/nanoGPT_payload.py:299-317, with the benchmark's fused QKV projection,
- * causal mask and tanh-GELU).  x, y: [B*T, C] f32 residual stream.  Weights are stored
- * [in, out] in `dtype` (F32 or BF16) with biases in the same type; LayerNorm parameters
- * are f32.  `workspace` must hold lh_hip_nanogpt_block_workspace_bytes(...) bytes.
+ * One pre-LayerNorm GPT-2 block forward, the op sequence of _emit_block_fused
+ * (examples/xegpu/nanoGPT_payload.py:299-317): ln1 -> q,k,v projections -> fused attention on
+ * (H, T, hs) views -> output projection + bias + residual -> ln2 -> MLP up-projection + bias +
+ * activation -> down-projection + bias + residual.  x, y: [B*T, C] f32 residual stream.  Weights are
+ * stored [in, out] in `dtype` (F32, BF16 or F16: every matmul input is rounded to it, the rounding
+ * points of examples/xegpu/nanoGPT.py:114-126); LayerNorm parameters are f32.
+ *
+ * Two configurations are covered by `opts` and the parameter struct:
+ *  - the benchmark's (opts == NULL): one fused QKV projection [C, 3C] with bias, causal mask,
+ *    tanh-GELU, biases of `dtype`;
+ *  - the reference's own (examples/xegpu/nanoGPT_payload.py:299-317,333-346): separate w_q / w_k /
+ *    w_v [C, C] without bias (w_qkv == NULL), no mask, ReLU, f32 biases.
+ * Any bias pointer may be NULL (no bias).  `workspace` must hold
+ * lh_hip_nanogpt_block_workspace_bytes(...) bytes; the call allocates nothing.
  */
 typedef struct lh_nanogpt_block_params {
   const float* ln1_g;
   const float* ln1_b;
-  const void* w_qkv; /* [C, 3C] */
-  const void* b_qkv; /* [3C]    */
+  const void* w_qkv; /* [C, 3C], or NULL with w_q, w_k, w_v set */
+  const void* b_qkv; /* [3C] (q | k | v), or NULL */
   const void* w_o;   /* [C, C]  */
   const void* b_o;   /* [C]     */
   const float* ln2_g;
   const float* ln2_b;
-  const void* w_fc;   /* [C, 4C] */
-  const void* b_fc;   /* [4C]    */
-  const void* w_proj; /* [4C, C] */
+  const void* w_fc;   /* [C, hidden] */
+  const void* b_fc;   /* [hidden]    */
+  const void* w_proj; /* [hidden, C] */
   const void* b_proj; /* [C]     */
+  const void* w_q;    /* [C, C] each; used when w_qkv is NULL */
+  const void* w_k;
+  const void* w_v;
 } lh_nanogpt_block_params;
-size_t lh_hip_nanogpt_block_workspace_bytes(int64_t B, int64_t T, int64_t C, int32_t dtype);
+typedef enum lh_activation {
+  LH_ACT_GELU_TANH = 0, /* benchmark configuration */
+  LH_ACT_RELU = 1       /* Builder.bias(relu=True), examples/xegpu/nanoGPT_payload.py:311 */
+} lh_activation;
+typedef struct lh_nanogpt_block_opts {
+  int32_t causal;     /* 1: causal mask; 0: none (the reference's fused kernel) */
+  int32_t activation; /* lh_activation */
+  int32_t bias_dtype; /* type of every bias vector: `dtype` or LH_F32 */
+  int32_t hidden;     /* MLP width; 0 selects 4 C */
+} lh_nanogpt_block_opts;
+size_t lh_hip_nanogpt_block_workspace_bytes(int64_t B, int64_t T, int64_t C, int32_t dtype,
+                                            const lh_nanogpt_block_opts* opts);
 int lh_hip_nanogpt_block(float* y, const float* x, const lh_nanogpt_block_params* p, int64_t B, int64_t T,
-                         int64_t C, int64_t n_head, float eps, int32_t dtype, void* workspace,
-                         size_t workspace_bytes, void* stream);
+                         int64_t C, int64_t n_head, float eps, int32_t dtype, const lh_nanogpt_block_opts* opts,
+                         void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * n_layer blocks followed by the final LayerNorm and the lm_head projection with bias, the shape
  * of build_gpt_fused_payload (examples/xegpu/nanoGPT_payload.py:318-407; embeddings stay on the
  * host side there too): logits[B*T, vocab] (f32) = LN_f(block_n(...block_1(x))) W_lm + b_lm.
- * Blocks are lh_hip_nanogpt_block's; lm_w [C, vocab] and lm_b [vocab] have `dtype`.  `workspace`
- * must hold lh_hip_nanogpt_forward_workspace_bytes(...) bytes.
+ * Blocks are lh_hip_nanogpt_block's; lm_w [C, vocab] has `dtype`, lm_b [vocab] (or NULL) the bias
+ * type of `opts`.  `workspace` must hold lh_hip_nanogpt_forward_workspace_bytes(...) bytes.
  */
-size_t lh_hip_nanogpt_forward_workspace_bytes(int64_t B, int64_t T, int64_t C, int32_t dtype);
+size_t lh_hip_nanogpt_forward_workspace_bytes(int64_t B, int64_t T, int64_t C, int64_t vocab, int32_t dtype,
+                                              const lh_nanogpt_block_opts* opts);
 int lh_hip_nanogpt_forward(float* logits, const float* x, const lh_nanogpt_block_params* blocks, int64_t n_layer,
                            const float* lnf_g, const float* lnf_b, const void* lm_w, const void* lm_b, int64_t B,
                            int64_t T, int64_t C, int64_t n_head, int64_t vocab, float eps, int32_t dtype,
-                           void* workspace, size_t workspace_bytes, void* stream);
-
-/*
- * Measurement aid (no counterpart in the reference): TFLOP/s of a register-only MFMA loop of the
- * given element type (LH_BF16, LH_F8E4M3, LH_F32) on every SIMD, with all-zero (random_operands
- * = 0) or random operands.  The matrix-core clock depends on operand bit activity, so this is the
- * rate a GEMM on such data can approach; bench.py reports it beside the published peak.
- */
-int lh_hip_probe_mfma_rate(int32_t dtype, int32_t random_operands, int64_t iters, double* tflops);
+                           const lh_nanogpt_block_opts* opts, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------- packed-argument payloads ---- */
 
@@ -255,8 +303,8 @@ int lh_hip_payload_matmul(void** args, int32_t nargs, const lh_matmul_attrs* att
  * and get the ReLU, the last layer has out_dtype and gets the ReLU only when
  * relu_on_final_layer is set; TRANSPOSE_A applies to the first layer's input only,
  * ACCUMULATE_C to the last layer's output only (the reference accumulates hidden layers into
- * uninitialised tensors, i.e. leaves them undefined).  Hidden activations live in a
- * library-owned device buffer that grows on demand. */
+ * uninitialised tensors, i.e. leaves them undefined).  Hidden activations live in the library's
+ * pool of temporary buffers. */
 typedef struct lh_mlp_attrs {
   int32_t ab_dtype;
   int32_t out_dtype;  /* result type of the last layer: F32 or the A/B type */
@@ -308,15 +356,35 @@ typedef enum lh_elementwise_kind {
 int lh_hip_payload_elementwise(void** args, int32_t nargs, const lh_elementwise_attrs* attrs);
 
 typedef struct lh_nanogpt_block_attrs {
-  int32_t dtype; /* F32 or BF16: type of the weights, biases and matmul inputs */
+  int32_t dtype; /* F32, BF16 or F16: type of the weights and matmul inputs */
   int32_t n_head;
   int32_t B;
   int32_t T;
   float eps;
 } lh_nanogpt_block_attrs;
-/* args: y[B*T,C], x[B*T,C], ln1_g[C], ln1_b[C], w_qkv[C,3C], b_qkv[3C], w_o[C,C], b_o[C], ln2_g[C], ln2_b[C],
- * w_fc[C,4C], b_fc[4C], w_proj[4C,C], b_proj[C], workspace[bytes] (i8). */
+/* The benchmark's block.  args: y[B*T,C], x[B*T,C], ln1_g[C], ln1_b[C], w_qkv[C,3C], b_qkv[3C], w_o[C,C],
+ * b_o[C], ln2_g[C], ln2_b[C], w_fc[C,4C], b_fc[4C], w_proj[4C,C], b_proj[C], workspace[bytes] (i8). */
 int lh_hip_payload_nanogpt_block(void** args, int32_t nargs, const lh_nanogpt_block_attrs* attrs);
+
+/*
+ * The payload of build_gpt_fused_payload (examples/xegpu/nanoGPT_payload.py:318-407) with its own
+ * argument list, so that the reference's nanoGPT driver (examples/xegpu/nanoGPT.py:225-297) can
+ * call it with the buffers it already builds: out[T,vocab] f32, x[T,C] f32, then per layer
+ * g1[C], b1n[C], wq[C,C], wk[C,C], wv[C,C], wp[C,C], bp[C], g2[C], b2n[C], w1[C,hidden], bb1[hidden],
+ * w2[hidden,C], bb2[C] (:333-347), then gf_g[C], gf_b[C], lmw[C,vocab], lmb[vocab], and last a
+ * workspace[bytes] (i8) of lh_hip_nanogpt_forward_workspace_bytes(1, T, C, vocab, dtype, &opts)
+ * with opts = {causal, LH_ACT_RELU, LH_F32, hidden} (the reference frees its temporaries inside the
+ * payload, :407-408; here the caller provides them).  Weights have `dtype` (the reference: F16),
+ * LayerNorm parameters and biases are f32.  Non-causal unless `causal` is set.
+ */
+typedef struct lh_gpt_fused_attrs {
+  int32_t dtype;
+  int32_t n_head;
+  int32_t n_layer;
+  int32_t causal;
+  float eps;
+} lh_gpt_fused_attrs;
+int lh_hip_payload_gpt_fused(void** args, int32_t nargs, const lh_gpt_fused_attrs* attrs);
 
 /*
  * The `__benchmark` wrapper (WrapInBenchingFuncOp, lighthouse/dialects/transform/
@@ -324,7 +392,7 @@ int lh_hip_payload_nanogpt_block(void** args, int32_t nargs, const lh_nanogpt_bl
  * untimed, then `nruns` times, each bracketed by a wall clock read with the device idle
  * on both sides; the durations in seconds go to host_times[0..nruns).  `payload` selects
  * the entry point by its name without the "lh_hip_payload_" prefix ("matmul",
- * "matmul_fp8", "attention", "layer_norm", "elementwise", "nanogpt_block"); `attrs` is that entry point's
+ * "matmul_fp8", "attention", "layer_norm", "elementwise", "nanogpt_block", "mlp", "gpt_fused"); `attrs` is that entry point's
  * attribute struct.
  */
 int lh_hip_payload_benchmark(const char* payload, void** args, int32_t nargs, const void* attrs,

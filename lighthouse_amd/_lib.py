@@ -54,7 +54,17 @@ class DeviceInfo(ctypes.Structure):
 
 class NanoGPTBlockParams(ctypes.Structure):
     _fields_ = [(n, ctypes.c_void_p) for n in (
-        "ln1_g", "ln1_b", "w_qkv", "b_qkv", "w_o", "b_o", "ln2_g", "ln2_b", "w_fc", "b_fc", "w_proj", "b_proj")]
+        "ln1_g", "ln1_b", "w_qkv", "b_qkv", "w_o", "b_o", "ln2_g", "ln2_b", "w_fc", "b_fc", "w_proj", "b_proj",
+        "w_q", "w_k", "w_v")]
+
+
+# lh_activation
+ACT_GELU_TANH, ACT_RELU = 0, 1
+
+
+class NanoGPTBlockOpts(ctypes.Structure):
+    _fields_ = [("causal", ctypes.c_int32), ("activation", ctypes.c_int32), ("bias_dtype", ctypes.c_int32),
+                ("hidden", ctypes.c_int32)]
 
 
 class MatmulAttrs(ctypes.Structure):
@@ -88,6 +98,11 @@ class NanoGPTBlockAttrs(ctypes.Structure):
                 ("eps", ctypes.c_float)]
 
 
+class GptFusedAttrs(ctypes.Structure):
+    _fields_ = [("dtype", ctypes.c_int32), ("n_head", ctypes.c_int32), ("n_layer", ctypes.c_int32),
+                ("causal", ctypes.c_int32), ("eps", ctypes.c_float)]
+
+
 _vp, _i64, _i32, _u32, _f32, _sz = (ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_uint32,
                                     ctypes.c_float, ctypes.c_size_t)
 
@@ -103,9 +118,14 @@ PROTOTYPES = {
     "lh_hip_memcpy_d2d": (_i32, [_vp, _vp, _sz]),
     "lh_hip_memset": (_i32, [_vp, _i32, _sz]),
     "lh_hip_sync": (_i32, [_vp]),
+    "lh_hip_release_scratch": (_i32, []),
     "lh_hip_gemm": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp]),
+    "lh_hip_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32]),
+    "lh_hip_gemm_ws": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp, _sz, _vp]),
     "lh_hip_gemm_residual": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp]),
     "lh_hip_gemm_fp8": (_i32, [_vp, _vp, _vp, _f32, _f32, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _vp]),
+    "lh_hip_gemm_fp8_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64, _i32]),
+    "lh_hip_gemm_fp8_ws": (_i32, [_vp, _vp, _vp, _f32, _f32, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _vp, _sz, _vp]),
     "lh_hip_attention": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, Strides3, Strides3, Strides3, Strides3,
                                 _f32, _i32, _i32, _vp]),
     "lh_hip_layer_norm": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _i32, _i32, _vp]),
@@ -114,13 +134,12 @@ PROTOTYPES = {
     "lh_hip_bias_act": (_i32, [_vp, _vp, _vp, _i64, _i64, _i32, _i32, _vp]),
     "lh_hip_add": (_i32, [_vp, _vp, _vp, _i64, _i32, _vp]),
     "lh_hip_cast": (_i32, [_vp, _vp, _i64, _i32, _i32, _vp]),
-    "lh_hip_nanogpt_block_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+    "lh_hip_nanogpt_block_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32, ctypes.POINTER(NanoGPTBlockOpts)]),
     "lh_hip_nanogpt_block": (_i32, [_vp, _vp, ctypes.POINTER(NanoGPTBlockParams), _i64, _i64, _i64, _i64, _f32, _i32,
-                                    _vp, _sz, _vp]),
-    "lh_hip_nanogpt_forward_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32]),
+                                    ctypes.POINTER(NanoGPTBlockOpts), _vp, _sz, _vp]),
+    "lh_hip_nanogpt_forward_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i32, ctypes.POINTER(NanoGPTBlockOpts)]),
     "lh_hip_nanogpt_forward": (_i32, [_vp, _vp, ctypes.POINTER(NanoGPTBlockParams), _i64, _vp, _vp, _vp, _vp, _i64, _i64,
-                                      _i64, _i64, _i64, _f32, _i32, _vp, _sz, _vp]),
-    "lh_hip_probe_mfma_rate": (_i32, [_i32, _i32, _i64, ctypes.POINTER(ctypes.c_double)]),
+                                      _i64, _i64, _i64, _f32, _i32, ctypes.POINTER(NanoGPTBlockOpts), _vp, _sz, _vp]),
     "lh_hip_payload_matmul": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(MatmulAttrs)]),
     "lh_hip_payload_matmul_fp8": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(MatmulFp8Attrs)]),
     "lh_hip_payload_mlp": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(MlpAttrs)]),
@@ -128,6 +147,7 @@ PROTOTYPES = {
     "lh_hip_payload_layer_norm": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(LayerNormAttrs)]),
     "lh_hip_payload_elementwise": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(ElementwiseAttrs)]),
     "lh_hip_payload_nanogpt_block": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(NanoGPTBlockAttrs)]),
+    "lh_hip_payload_gpt_fused": (_i32, [ctypes.POINTER(_vp), _i32, ctypes.POINTER(GptFusedAttrs)]),
     "lh_hip_payload_benchmark": (_i32, [ctypes.c_char_p, ctypes.POINTER(_vp), _i32, _vp,
                                         ctypes.POINTER(ctypes.c_double), _i64, _i64]),
 }

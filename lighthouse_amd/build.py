@@ -17,9 +17,10 @@ ROOT = Path(__file__).resolve().parent.parent
 CSRC = ROOT / "lighthouse_amd" / "csrc"
 LIB_DIR = ROOT / "lighthouse_amd" / "lib"
 LIB_PATH = LIB_DIR / "liblighthouse_hip.so"
+PROBE_LIB = LIB_DIR / "liblighthouse_probe.so"  # bench.py's MFMA-rate probe, not part of the product library
 ORACLE_LIB = ROOT / "oracle" / "_build" / "libcpu_ref.so"
 
-HIP_SOURCES = ["runtime.hip", "gemm16.hip", "gemm32.hip", "gemm8.hip", "attention.hip", "rowwise.hip", "probe.hip", "api.hip"]
+HIP_SOURCES = ["runtime.hip", "gemm16.hip", "gemm32.hip", "gemm8.hip", "attention.hip", "rowwise.hip", "api.hip"]
 
 HIPCC_FLAGS = [
     "-O3",
@@ -56,9 +57,12 @@ def build_hip(verbose: bool = False) -> Path:
         _run(cmd)
         return str(obj)
 
-    with ThreadPoolExecutor(max_workers=min(8, len(HIP_SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(8, len(HIP_SOURCES) + 1)) as pool:
+        probe = pool.submit(compile_one, "probe.hip")
         objs = list(pool.map(compile_one, HIP_SOURCES))
+        probe_obj = probe.result()
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", str(LIB_PATH)])
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", probe_obj, "-o", str(PROBE_LIB)])
     return LIB_PATH
 
 

@@ -613,14 +613,14 @@ static int attention16_launch_ragged(const AttnArgs& a, hipStream_t s) {
   auto kern = attention16_kernel<DT, NQ, NS, RAGGED>;
   constexpr size_t lds = (size_t)NS * kAttnStageBytes;
   static bool configured = false;
-  if (!configured) {
+  if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds));
     configured = true;
   }
   const int nqb = (a.T + 128 * NQ - 1) / (128 * NQ);
   const dim3 grid = a.causal ? dim3(nqb * a.Z * a.H) : dim3(nqb, a.Z * a.H);
-  hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, a);
+  LH_LAUNCH(kern, grid, dim3(256), lds, s, a);
   return check_launch("attention16");
 }
 
@@ -1045,14 +1045,14 @@ static int attention16_d128_launch(const AttnArgs& a, hipStream_t s) {
   constexpr size_t lds = 2 * kD128StageBytes;
   auto kern = attention16_d128_kernel<DT>;
   static bool configured = false;
-  if (!configured) {
+  if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds));
     configured = true;
   }
   const int nqb = (a.T + 127) / 128;
   const dim3 grid = a.causal ? dim3(nqb * a.Z * a.H) : dim3(nqb, a.Z * a.H);
-  hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, a);
+  LH_LAUNCH(kern, grid, dim3(256), lds, s, a);
   return check_launch("attention16_d128");
 }
 
@@ -1062,14 +1062,14 @@ static int attention16_anyd_launch(const AttnArgs& a, hipStream_t s) {
   constexpr size_t lds = (size_t)2 * kKvTile * (D + 8) * 2 + (DB >= 8 ? 4 * 32 * D * 2 : 0);
   auto kern = attention16_anyd_kernel<DT, DB>;
   static bool configured = false;
-  if (!configured) {
+  if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds));
     configured = true;
   }
   const int nqb = (a.T + 127) / 128;
   const dim3 grid = a.causal ? dim3(nqb * a.Z * a.H) : dim3(nqb, a.Z * a.H);
-  hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, a);
+  LH_LAUNCH(kern, grid, dim3(256), lds, s, a);
   return check_launch("attention16_anyd");
 }
 
@@ -1156,9 +1156,9 @@ __global__ void __launch_bounds__(64) attention_generic_kernel(AttnArgs a, int d
 
 int attention_generic_launch(const AttnArgs& a, int d, int dtype, hipStream_t s) {
   const dim3 grid(a.T, a.Z * a.H);
-  if (dtype == LH_BF16) hipLaunchKernelGGL(attention_generic_kernel<LH_BF16>, grid, dim3(64), 0, s, a, d);
-  else if (dtype == LH_F16) hipLaunchKernelGGL(attention_generic_kernel<LH_F16>, grid, dim3(64), 0, s, a, d);
-  else hipLaunchKernelGGL(attention_generic_kernel<LH_F32>, grid, dim3(64), 0, s, a, d);
+  if (dtype == LH_BF16) LH_LAUNCH(attention_generic_kernel<LH_BF16>, grid, dim3(64), 0, s, a, d);
+  else if (dtype == LH_F16) LH_LAUNCH(attention_generic_kernel<LH_F16>, grid, dim3(64), 0, s, a, d);
+  else LH_LAUNCH(attention_generic_kernel<LH_F32>, grid, dim3(64), 0, s, a, d);
   return check_launch("attention_generic");
 }
 
@@ -1168,12 +1168,12 @@ int attention_launch(const AttnArgs& a, int dtype, hipStream_t s) {
   const int nqb32 = (a.T + kQBlock - 1) / kQBlock;
   const dim3 grid32 = a.causal ? dim3(nqb32 * a.Z * a.H) : dim3(nqb32, a.Z * a.H);
   auto launch = [&](auto kern, bool& configured) -> int {
-    if (!configured) {
+    if (!configured && !planning()) {
       LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        2 * kAttn32StageBytes));
       configured = true;
     }
-    hipLaunchKernelGGL(kern, grid32, dim3(256), 2 * kAttn32StageBytes, s, a);
+    LH_LAUNCH(kern, grid32, dim3(256), 2 * kAttn32StageBytes, s, a);
     return 0;
   };
   static bool configured_whole = false, configured_ragged = false;

@@ -28,7 +28,9 @@ int fail(int code, const char* fmt, ...);
     if (!(cond)) return ::lh::fail(LH_ERR_INVALID, __VA_ARGS__); \
   } while (0)
 
+bool planning();
 inline int check_launch(const char* what) {
+  if (planning()) return LH_OK;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(LH_ERR_RUNTIME, "launch of %s failed: %s", what, hipGetErrorString(e));
   return LH_OK;
@@ -160,15 +162,39 @@ hipStream_t default_stream();
 // out[c][r] = in[r][c] for an R x C matrix of 2- or 4-byte elements (row strides in elements).
 int transpose_matrix(void* out, const void* in, int R, int C, int64_t ld_in, int64_t ld_out, int elem_bytes,
                      hipStream_t s);
-// A library-owned device buffer of at least `bytes` (grown on demand, kept until the process
-// ends); calls that use it on different streams at the same time race.  nullptr on failure
-// (the error message is set).
-void* transpose_scratch(size_t bytes);
 // dst (rows_dst x cols_dst) = src (rows_src x cols_src) padded with zeros or cut; any alignment.
 int pad_copy_matrix(void* dst, int64_t ld_dst, int rows_dst, int cols_dst, const void* src, int64_t ld_src, int rows_src,
                     int cols_src, int elem_bytes, hipStream_t s);
-void* pad_scratch(size_t bytes);
-void* splitk_scratch(size_t bytes);  // f32 partial results of split-K GEMM launches
+
+// ---- temporary device memory of a call ------------------------------------------------------
+// Kernels that need memory beyond their operands (transposed or zero-padded operand copies, the
+// f32 blocks of a launch cut along K, hidden activations of the MLP payload) take it from a Scratch:
+//  * base != nullptr: a workspace the caller handed in, given out front to back in 256-byte
+//    granules; a request that does not fit fails with LH_ERR_INVALID and nothing is allocated;
+//  * base == nullptr (or no Scratch at all): the library's pool, one buffer per purpose ("slot")
+//    and per (device, stream), so that calls on different streams never share memory.  A buffer
+//    that is too small is replaced by a larger one; the old one is kept until
+//    lh_hip_release_scratch() because enqueued work may still use it (no hipFree, hence no
+//    device-wide synchronisation, inside a call).
+// While planning() is true (a *_workspace_bytes query on this thread) nothing is launched or
+// allocated: takes return a dummy address and add their size to `need`.
+enum ScratchSlot { kScratchTranspose = 0, kScratchPad, kScratchSplitK, kScratchSkinny, kScratchMlp, kScratchSlots };
+struct Scratch {
+  char* base = nullptr;
+  size_t bytes = 0;
+  size_t used = 0;
+  size_t need = 0;
+};
+int scratch_take(Scratch* ws, hipStream_t s, int slot, size_t bytes, const char* what, void** out);
+bool planning();
+struct PlanningScope {  // marks the calling thread as running a size query
+  PlanningScope();
+  ~PlanningScope();
+};
+#define LH_LAUNCH(...)                                        \
+  do {                                                        \
+    if (!::lh::planning()) hipLaunchKernelGGL(__VA_ARGS__);   \
+  } while (0)
 // Compute units of the current device (cached; 256 if the query fails).
 int num_cus();
 

@@ -717,14 +717,14 @@ static int launch_direct_edge(const GemmArgs& g, hipStream_t s) {
   auto kern = gemm16_direct<DT, TM, TN, EDGE>;
   constexpr size_t lds = Cfg::kLdsBytes;
   static bool configured = false;
-  if (!configured) {
+  if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds));
     configured = true;
   }
   const int ntiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
   const int resident = num_cus() * (2 * lds <= 160 * 1024 ? 2 : 1);
-  hipLaunchKernelGGL(kern, dim3(ntiles < resident ? ntiles : resident), dim3(512), lds, s, g);
+  LH_LAUNCH(kern, dim3(ntiles < resident ? ntiles : resident), dim3(512), lds, s, g);
   return check_launch("gemm16_direct");
 }
 
@@ -792,13 +792,13 @@ static int launch_fast(const GemmArgs& g, hipStream_t s) {
   auto kern = gemm16_fast<DT, BM, BN, WAVES_M, WAVES_N, B_KC>;
   constexpr size_t lds = gemm16_lds_bytes<BM, BN>();
   static bool configured = false;
-  if (!configured) {
+  if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds));
     configured = true;
   }
   dim3 grid((g.M / BM) * (g.N / BN));
-  hipLaunchKernelGGL(kern, grid, dim3(WAVES_M * WAVES_N * 64), lds, s, g);
+  LH_LAUNCH(kern, grid, dim3(WAVES_M * WAVES_N * 64), lds, s, g);
   return check_launch("gemm16_fast");
 }
 
@@ -850,8 +850,10 @@ static int gemm16_splitk(const GemmArgs& g, hipStream_t s) {
   while (splits < 8 && tiles * splits * 2 <= 2 * cus && (g.K / (splits * 2)) % kBK == 0 && g.K / (splits * 2) >= 512)
     splits *= 2;
   if (splits == 1) return 1;
-  float* partial = static_cast<float*>(splitk_scratch((size_t)splits * g.M * g.N * sizeof(float)));
-  if (!partial) return LH_ERR_RUNTIME;
+  void* taken = nullptr;
+  if (int rc = scratch_take(g.ws, s, kScratchSplitK, (size_t)splits * g.M * g.N * sizeof(float), "gemm (split K)", &taken))
+    return rc;
+  float* partial = static_cast<float*>(taken);
   GemmArgs p = g;
   p.K = g.K / splits;
   p.splits = splits;
@@ -863,13 +865,13 @@ static int gemm16_splitk(const GemmArgs& g, hipStream_t s) {
   p.flags = 0;
   const bool edge = g.M % Cfg::BM != 0 || g.N % Cfg::BN != 0;
   auto launch = [&](auto kern, bool& configured) -> int {
-    if (!configured) {
+    if (!configured && !planning()) {
       LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)Cfg::kLdsBytes));
       configured = true;
     }
     const int64_t total = tiles * splits, resident = 2 * (int64_t)cus;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(total < resident ? total : resident)), dim3(512), Cfg::kLdsBytes, s, p);
+    LH_LAUNCH(kern, dim3((unsigned)(total < resident ? total : resident)), dim3(512), Cfg::kLdsBytes, s, p);
     return check_launch("gemm16_direct (split K)");
   };
   static bool configured_edge = false, configured_whole = false;
@@ -878,7 +880,7 @@ static int gemm16_splitk(const GemmArgs& g, hipStream_t s) {
   if (rc) return rc;
   const int64_t groups = (int64_t)g.M * g.N / 4;
   const int rb = reduce_block(groups);
-  hipLaunchKernelGGL(gemm16_splitk_reduce<DT>, dim3((unsigned)((groups + rb - 1) / rb)), dim3(rb), 0, s, g, partial, splits);
+  LH_LAUNCH(gemm16_splitk_reduce<DT>, dim3((unsigned)((groups + rb - 1) / rb)), dim3(rb), 0, s, g, partial, splits);
   return check_launch("gemm16_splitk_reduce");
 }
 
@@ -931,7 +933,7 @@ static int gemm16_dispatch(const GemmArgs& g_in, hipStream_t s) {
     }
   }
   dim3 grid((g.N + 63) / 64, (g.M + 63) / 64);
-  hipLaunchKernelGGL(gemm16_generic<DT>, grid, dim3(256), 0, s, g);
+  LH_LAUNCH(gemm16_generic<DT>, grid, dim3(256), 0, s, g);
   return check_launch("gemm16_generic");
 }
 

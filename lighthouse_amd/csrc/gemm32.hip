@@ -250,14 +250,14 @@ static int launch_direct32_edge(const GemmArgs& g, hipStream_t s) {
   auto kern = gemm32_direct<TM, TN, NS, NW, EDGE>;
   constexpr size_t lds = (size_t)NS * (64 * TM * 128 + 32 * 64 * TN * 4);
   static bool configured = false;
-  if (!configured) {
+  if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds));
     configured = true;
   }
   const int ntiles = ((g.M + 64 * TM - 1) / (64 * TM)) * ((g.N + 64 * TN - 1) / (64 * TN));
   const int resident = num_cus() * (int)((160 * 1024) / lds);  // workgroups that fit the CUs' LDS together
-  hipLaunchKernelGGL(kern, dim3(ntiles < resident ? ntiles : resident), dim3(NW * 64), lds, s, g);
+  LH_LAUNCH(kern, dim3(ntiles < resident ? ntiles : resident), dim3(NW * 64), lds, s, g);
   return check_launch("gemm32_direct");
 }
 
@@ -351,7 +351,7 @@ int gemm32(const GemmArgs& g_in, hipStream_t s) {
     return launch_direct32<1, 1, 3>(g, s);
   }
   dim3 grid((g.N + 63) / 64, (g.M + 63) / 64);
-  hipLaunchKernelGGL(gemm32_generic, grid, dim3(256), 0, s, g);
+  LH_LAUNCH(gemm32_generic, grid, dim3(256), 0, s, g);
   return check_launch("gemm32_generic");
 }
 

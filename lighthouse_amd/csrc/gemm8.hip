@@ -480,13 +480,13 @@ __global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
 
 static int launch_direct8(const GemmArgs& g, hipStream_t s) {
   static bool configured = false;
-  if (!configured) {
+  if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_direct<false>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kD8LdsBytes));
     configured = true;
   }
   const int ntiles = (g.M / 256) * (g.N / 256), cus = num_cus();
-  hipLaunchKernelGGL(gemm8_direct<false>, dim3(ntiles < cus ? ntiles : cus), dim3(512), kD8LdsBytes, s, g);
+  LH_LAUNCH(gemm8_direct<false>, dim3(ntiles < cus ? ntiles : cus), dim3(512), kD8LdsBytes, s, g);
   return check_launch("gemm8_direct");
 }
 
@@ -514,8 +514,10 @@ static int gemm8_splitk(const GemmArgs& g, hipStream_t s) {
   while (splits < 8 && tiles * splits * 2 <= cus && (g.K / (splits * 2)) % kBK8 == 0 && g.K / (splits * 2) >= 1024)
     splits *= 2;
   if (splits == 1) return 1;
-  float* partial = static_cast<float*>(splitk_scratch((size_t)splits * g.M * g.N * sizeof(float)));
-  if (!partial) return LH_ERR_RUNTIME;
+  void* taken = nullptr;
+  if (int rc = scratch_take(g.ws, s, kScratchSplitK, (size_t)splits * g.M * g.N * sizeof(float), "fp8 gemm (split K)", &taken))
+    return rc;
+  float* partial = static_cast<float*>(taken);
   GemmArgs p = g;
   p.K = g.K / splits;
   p.splits = splits;
@@ -525,18 +527,18 @@ static int gemm8_splitk(const GemmArgs& g, hipStream_t s) {
   p.out_dt = LH_F32;
   p.alpha = 1.0f;
   static bool configured = false;
-  if (!configured) {
+  if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_direct<true>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, kD8LdsBytes));
     configured = true;
   }
   const int64_t total = tiles * splits;
-  hipLaunchKernelGGL(gemm8_direct<true>, dim3((unsigned)(total < cus ? total : cus)), dim3(512), kD8LdsBytes, s, p);
+  LH_LAUNCH(gemm8_direct<true>, dim3((unsigned)(total < cus ? total : cus)), dim3(512), kD8LdsBytes, s, p);
   int rc = check_launch("gemm8_direct (split K)");
   if (rc) return rc;
   const int64_t groups = (int64_t)g.M * g.N / 4;
   const int rb = reduce_block(groups);
-  hipLaunchKernelGGL(gemm8_splitk_reduce, dim3((unsigned)((groups + rb - 1) / rb)), dim3(rb), 0, s, g, partial, splits);
+  LH_LAUNCH(gemm8_splitk_reduce, dim3((unsigned)((groups + rb - 1) / rb)), dim3(rb), 0, s, g, partial, splits);
   return check_launch("gemm8_splitk_reduce");
 }
 
@@ -830,31 +832,25 @@ __global__ void __launch_bounds__(256) gemm8_skinny_reduce(GemmArgs g, const flo
   epilogue4<LH_BF16>(g, m, n, v[0], v[1], v[2], v[3]);
 }
 
-static float* g_partial = nullptr;
-static size_t g_partial_bytes = 0;
-
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool EDGE_M = false>
 static int launch_fast8(const GemmArgs& g, hipStream_t s) {
   auto kern = gemm8_fast<BM, BN, WAVES_M, WAVES_N, EDGE_M>;
   constexpr size_t lds = (size_t)2 * (BM + BN) * kStride8;
   static bool configured = false;
-  if (!configured) {
+  if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                      (int)lds));
     configured = true;
   }
-  hipLaunchKernelGGL(kern, dim3(((g.M + BM - 1) / BM) * (g.N / BN)), dim3(WAVES_M * WAVES_N * 64), lds, s, g);
+  LH_LAUNCH(kern, dim3(((g.M + BM - 1) / BM) * (g.N / BN)), dim3(WAVES_M * WAVES_N * 64), lds, s, g);
   return check_launch("gemm8_fast");
 }
 
-static int skinny_partial_buffer(size_t need) {
-  if (need > g_partial_bytes) {
-    if (g_partial) LH_HIP_CHECK(hipFree(g_partial));
-    g_partial = nullptr;
-    g_partial_bytes = 0;
-    LH_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&g_partial), need));
-    g_partial_bytes = need;
-  }
+// f32 partial blocks of the decode kernels, [splits][rows][N].
+static int skinny_partial_buffer(const GemmArgs& g, hipStream_t s, size_t need, float** partial) {
+  void* taken = nullptr;
+  if (int rc = scratch_take(g.ws, s, kScratchSkinny, need, "fp8 gemm (decode partial sums)", &taken)) return rc;
+  *partial = static_cast<float*>(taken);
   return LH_OK;
 }
 
@@ -864,21 +860,22 @@ static int launch_skinny_mt(const GemmArgs& g, hipStream_t s) {
   const int nblk = g.N / kSkinnyBN;
   int splits = 1;
   while (nblk * splits < num_cus() && (g.K / kBK8) % (splits * 2) == 0) splits *= 2;
-  int rc = skinny_partial_buffer((size_t)splits * 16 * MT * g.N * sizeof(float));
+  float* g_partial = nullptr;
+  int rc = skinny_partial_buffer(g, s, (size_t)splits * 16 * MT * g.N * sizeof(float), &g_partial);
   if (rc) return rc;
   static bool configured = false;
-  if (!configured) {
+  if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_skinny_mt<MT>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, SkinnyMt<MT>::kLdsBytes));
     configured = true;
   }
-  hipLaunchKernelGGL(gemm8_skinny_mt<MT>, dim3(nblk, splits), dim3(256), SkinnyMt<MT>::kLdsBytes, s, g, g_partial,
+  LH_LAUNCH(gemm8_skinny_mt<MT>, dim3(nblk, splits), dim3(256), SkinnyMt<MT>::kLdsBytes, s, g, g_partial,
                      g.K / splits);
   rc = check_launch("gemm8_skinny_mt");
   if (rc) return rc;
   const int64_t groups = (int64_t)g.M * g.N / 4;
   const int rb = reduce_block(groups);
-  hipLaunchKernelGGL(gemm8_skinny_reduce, dim3((unsigned)((groups + rb - 1) / rb)), dim3(rb), 0, s, g, g_partial, splits,
+  LH_LAUNCH(gemm8_skinny_reduce, dim3((unsigned)((groups + rb - 1) / rb)), dim3(rb), 0, s, g, g_partial, splits,
                      16 * MT);
   return check_launch("gemm8_skinny_reduce");
 }
@@ -898,20 +895,21 @@ int gemm8(const GemmArgs& g, hipStream_t s) {
     int splits = 1;
     while ((nblk * splits < num_cus() || g.K / splits > kSkinnyMaxChunk) && (g.K / kBK8) % (splits * 2) == 0) splits *= 2;
     if (g.K / splits <= kSkinnyMaxChunk) {
-      int prc = skinny_partial_buffer((size_t)splits * 16 * g.N * sizeof(float));
+      float* g_partial = nullptr;
+      int prc = skinny_partial_buffer(g, s, (size_t)splits * 16 * g.N * sizeof(float), &g_partial);
       if (prc) return prc;
       static bool configured = false;
-      if (!configured) {
+      if (!configured && !planning()) {
         LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm8_skinny),
                                          hipFuncAttributeMaxDynamicSharedMemorySize, kSkinnyLdsBytes));
         configured = true;
       }
-      hipLaunchKernelGGL(gemm8_skinny, dim3(nblk, splits), dim3(256), kSkinnyLdsBytes, s, g, g_partial, g.K / splits);
+      LH_LAUNCH(gemm8_skinny, dim3(nblk, splits), dim3(256), kSkinnyLdsBytes, s, g, g_partial, g.K / splits);
       int rc = check_launch("gemm8_skinny");
       if (rc) return rc;
       const int64_t groups = (int64_t)g.M * g.N / 4;
       const int rb = reduce_block(groups);
-      hipLaunchKernelGGL(gemm8_skinny_reduce, dim3((unsigned)((groups + rb - 1) / rb)), dim3(rb), 0, s, g, g_partial,
+      LH_LAUNCH(gemm8_skinny_reduce, dim3((unsigned)((groups + rb - 1) / rb)), dim3(rb), 0, s, g, g_partial,
                          splits, 16);
       return check_launch("gemm8_skinny_reduce");
     }
@@ -934,7 +932,7 @@ int gemm8(const GemmArgs& g, hipStream_t s) {
   if (vec_ok && g.M % 128 == 0 && g.N % 128 == 0) return launch_fast8<128, 128, 2, 2>(g, s);
   if (vec_ok && g.N % 128 == 0) return launch_fast8<128, 128, 2, 2, true>(g, s);  // any M
   dim3 grid((g.N + 31) / 32, (g.M + 31) / 32);
-  hipLaunchKernelGGL(gemm8_generic, grid, dim3(64), 0, s, g);
+  LH_LAUNCH(gemm8_generic, grid, dim3(64), 0, s, g);
   return check_launch("gemm8_generic");
 }
 

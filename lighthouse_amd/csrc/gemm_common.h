@@ -20,6 +20,8 @@ struct GemmArgs {
   // Split-K launches of the 16-bit direct kernel: `splits` problems of K columns each, problem sp reads
   // A from column sp K, B from row sp K and writes its own M x ldc block of `out`.
   int splits = 1;
+  // Source of the call's temporary device memory; nullptr: the library's pool of the stream.
+  Scratch* ws = nullptr;
 };
 
 // Epilogue for 4 consecutive columns of one row.
@@ -113,7 +115,7 @@ __device__ __forceinline__ u32x2 epilogue4_pack(const GemmArgs& g, int n, float 
 }
 
 // Transposed operands (A stored [K,M], B stored [N,K]) of a problem the direct kernels would
-// otherwise take are first transposed into a library-owned buffer (one extra pass over that
+// otherwise take are first transposed into temporary memory (one extra pass over that
 // operand, about a tenth of a 4096^3 problem's time) instead of running the slower kernels that
 // read them in place.  Returns 0 and rewrites `g` on success, 1 when the problem does not qualify.
 template <int ELEM_BYTES>
@@ -122,8 +124,9 @@ inline int untranspose_operands(GemmArgs& g, int k_multiple, int n_multiple, hip
   if (!(ta || tb) || g.K % k_multiple != 0 || g.N % n_multiple != 0) return 1;
   const size_t a_bytes = ta ? ((size_t)g.M * g.K * ELEM_BYTES + 255) / 256 * 256 : 0;
   const size_t b_bytes = tb ? (size_t)g.K * g.N * ELEM_BYTES : 0;
-  char* buf = static_cast<char*>(transpose_scratch(a_bytes + b_bytes));
-  if (!buf) return LH_ERR_RUNTIME;
+  void* taken = nullptr;
+  if (int rc = scratch_take(g.ws, s, kScratchTranspose, a_bytes + b_bytes, "gemm (transposed operands)", &taken)) return rc;
+  char* buf = static_cast<char*>(taken);
   if (ta) {  // stored [K, M] -> [M, K]
     if (int rc = transpose_matrix(buf, g.a, g.K, g.M, g.lda, g.K, ELEM_BYTES, s)) return rc;
     g.a = buf;
@@ -140,7 +143,7 @@ inline int untranspose_operands(GemmArgs& g, int k_multiple, int n_multiple, hip
 
 // A problem whose K or N the direct kernels cannot take (K not a multiple of the k-step, N not a
 // multiple of the vector width, or rows that are not 16-byte aligned) runs on them all the same:
-// A and B are copied into library-owned matrices padded with zeros, the kernel writes a padded
+// A and B are copied into temporary matrices padded with zeros, the kernel writes a padded
 // result, and that is copied back (bf16 4096 x 4100 x 4096: 2012 -> about 200 us; the generic
 // kernel it replaces reads element by element).  `run` launches the padded problem.  Returns 1
 // when nothing needs padding, a negative status on failure.
@@ -162,8 +165,11 @@ inline int gemm_padded(const GemmArgs& g, int k_multiple, int n_multiple, hipStr
   const size_t b_bytes = pad_b ? round256((size_t)Kp * Np * ELEM_BYTES) : 0;
   const size_t c_bytes = pad_c ? round256((size_t)g.M * Np * out_bytes) : 0;
   const size_t bias_bytes_total = pad_bias ? round256((size_t)Np * bias_bytes) : 0;
-  char* buf = static_cast<char*>(pad_scratch(a_bytes + b_bytes + c_bytes + bias_bytes_total));
-  if (!buf) return LH_ERR_RUNTIME;
+  void* taken = nullptr;
+  if (int rc = scratch_take(g.ws, s, kScratchPad, a_bytes + b_bytes + c_bytes + bias_bytes_total, "gemm (padded operands)",
+                            &taken))
+    return rc;
+  char* buf = static_cast<char*>(taken);
   GemmArgs p = g;
   p.K = Kp;
   p.N = Np;

@@ -1,3 +1,5 @@
+// Benchmark-side helper, built into a library of its own (liblighthouse_probe.so) that only
+// bench.py loads; it is not part of liblighthouse_hip.so or of its C ABI.
 // Measurement aid: the rate of a register-only MFMA loop (no LDS, no global traffic in the timed
 // part) on every SIMD of the device, with all-zero or random operands.  The matrix cores' clock
 // under load depends on how much the operand bits toggle, so this is the ceiling a GEMM of the same
@@ -56,12 +58,19 @@ __global__ void __launch_bounds__(512) mfma_rate_kernel(float* out, const u32x4*
 
 using namespace lh;
 
-extern "C" int lh_hip_probe_mfma_rate(int32_t dtype, int32_t random_operands, int64_t iters, double* tflops) {
-  LH_REQUIRE(tflops && iters > 0 && iters < (1ll << 30), "lh_hip_probe_mfma_rate: bad arguments");
-  LH_REQUIRE(dtype == LH_BF16 || dtype == LH_F8E4M3 || dtype == LH_F32, "lh_hip_probe_mfma_rate: dtype %d", dtype);
+// Self-contained error handling: this file links against nothing of the main library.
+#define PROBE_CHECK(expr)                  \
+  do {                                     \
+    if ((expr) != hipSuccess) return -3;   \
+  } while (0)
+
+// Returns 0, -1 (bad arguments) or -3 (HIP runtime failure).
+extern "C" int lh_probe_mfma_rate(int32_t dtype, int32_t random_operands, int64_t iters, double* tflops) {
+  if (!(tflops && iters > 0 && iters < (1ll << 30))) return -1;
+  if (!(dtype == LH_BF16 || dtype == LH_F8E4M3 || dtype == LH_F32)) return -1;
   int dev = 0, cus = 0;
-  LH_HIP_CHECK(hipGetDevice(&dev));
-  LH_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  PROBE_CHECK(hipGetDevice(&dev));
+  PROBE_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
   const size_t nfrag = 8 * 512;
   std::vector<uint32_t> host(nfrag * 4, 0u);
   if (random_operands) {
@@ -88,31 +97,31 @@ extern "C" int lh_hip_probe_mfma_rate(int32_t dtype, int32_t random_operands, in
   }
   u32x4* frag = nullptr;
   float* out = nullptr;
-  LH_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&frag), nfrag * 16));
-  LH_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&out), (size_t)cus * 512 * sizeof(float)));
-  LH_HIP_CHECK(hipMemcpy(frag, host.data(), nfrag * 16, hipMemcpyHostToDevice));
+  PROBE_CHECK(hipMalloc(reinterpret_cast<void**>(&frag), nfrag * 16));
+  PROBE_CHECK(hipMalloc(reinterpret_cast<void**>(&out), (size_t)cus * 512 * sizeof(float)));
+  PROBE_CHECK(hipMemcpy(frag, host.data(), nfrag * 16, hipMemcpyHostToDevice));
   hipEvent_t e0, e1;
-  LH_HIP_CHECK(hipEventCreate(&e0));
-  LH_HIP_CHECK(hipEventCreate(&e1));
+  PROBE_CHECK(hipEventCreate(&e0));
+  PROBE_CHECK(hipEventCreate(&e1));
   auto launch = [&]() {
     if (dtype == LH_BF16) hipLaunchKernelGGL(mfma_rate_kernel<LH_BF16>, dim3(cus), dim3(512), 0, nullptr, out, frag, (int)iters);
     else if (dtype == LH_F8E4M3) hipLaunchKernelGGL(mfma_rate_kernel<LH_F8E4M3>, dim3(cus), dim3(512), 0, nullptr, out, frag, (int)iters);
     else hipLaunchKernelGGL(mfma_rate_kernel<LH_F32>, dim3(cus), dim3(512), 0, nullptr, out, frag, (int)iters);
   };
   launch();  // warm-up
-  LH_HIP_CHECK(hipEventRecord(e0, nullptr));
+  PROBE_CHECK(hipEventRecord(e0, nullptr));
   launch();
-  LH_HIP_CHECK(hipEventRecord(e1, nullptr));
-  LH_HIP_CHECK(hipEventSynchronize(e1));
-  int rc = check_launch("mfma_rate_kernel");
+  PROBE_CHECK(hipEventRecord(e1, nullptr));
+  PROBE_CHECK(hipEventSynchronize(e1));
+  const int rc = hipGetLastError() == hipSuccess ? 0 : -3;
   float ms = 0.0f;
-  LH_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
-  LH_HIP_CHECK(hipEventDestroy(e0));
-  LH_HIP_CHECK(hipEventDestroy(e1));
-  LH_HIP_CHECK(hipFree(frag));
-  LH_HIP_CHECK(hipFree(out));
+  PROBE_CHECK(hipEventElapsedTime(&ms, e0, e1));
+  PROBE_CHECK(hipEventDestroy(e0));
+  PROBE_CHECK(hipEventDestroy(e1));
+  PROBE_CHECK(hipFree(frag));
+  PROBE_CHECK(hipFree(out));
   if (rc) return rc;
   const double flop_per_mfma = dtype == LH_BF16 ? 32768.0 : dtype == LH_F8E4M3 ? 131072.0 : 4096.0;
   *tflops = (double)iters * 8.0 * flop_per_mfma * 8.0 * cus / ((double)ms * 1e-3) / 1e12;
-  return LH_OK;
+  return 0;
 }

@@ -429,10 +429,10 @@ static int layer_norm_launch(void* out, const void* x, const float* gamma, const
 #define LH_LN_CASE(V)                                                                                                 \
   case V:                                                                                                             \
     if (two && V <= 4)                                                                                                \
-      hipLaunchKernelGGL((layer_norm_vec<XDT, ODT, V, V <= 4 ? 2 : 1>), grid2, block, 0, s, out, x, gamma, beta, M, N, eps, \
+      LH_LAUNCH((layer_norm_vec<XDT, ODT, V, V <= 4 ? 2 : 1>), grid2, block, 0, s, out, x, gamma, beta, M, N, eps, \
                          inv_n);                                                                                      \
     else                                                                                                              \
-      hipLaunchKernelGGL((layer_norm_vec<XDT, ODT, V, 1>), grid, block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);  \
+      LH_LAUNCH((layer_norm_vec<XDT, ODT, V, 1>), grid, block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);  \
     return check_launch("layer_norm_vec");
   if (vec) {
     switch (N / 256) {
@@ -446,7 +446,7 @@ static int layer_norm_launch(void* out, const void* x, const float* gamma, const
   if (vec4 && N >= 64 && N <= 4096) {
 #define LH_LN_GUARD(V)                                                                                                \
   case V:                                                                                                             \
-    hipLaunchKernelGGL((layer_norm_vec<XDT, ODT, V, 1, true>), grid, block, 0, s, out, x, gamma, beta, M, N, eps,      \
+    LH_LAUNCH((layer_norm_vec<XDT, ODT, V, 1, true>), grid, block, 0, s, out, x, gamma, beta, M, N, eps,      \
                        inv_n);                                                                                        \
     return check_launch("layer_norm_vec (guarded)");
     switch (row_groups_rounded(N)) {
@@ -458,15 +458,15 @@ static int layer_norm_launch(void* out, const void* x, const float* gamma, const
   }
   if (N >= 1024 || (vec4 && N >= 512)) {
     if (vec4 && N <= 1024 * kBlockRegGroups)
-      hipLaunchKernelGGL((layer_norm_block_reg<XDT, ODT>), dim3(M), block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);
+      LH_LAUNCH((layer_norm_block_reg<XDT, ODT>), dim3(M), block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);
     else if (vec4)
-      hipLaunchKernelGGL((layer_norm_block<XDT, ODT, true>), dim3(M), block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);
+      LH_LAUNCH((layer_norm_block<XDT, ODT, true>), dim3(M), block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);
     else
-      hipLaunchKernelGGL((layer_norm_block<XDT, ODT, false>), dim3(M), block, 0, s, out, x, gamma, beta, M, N, eps,
+      LH_LAUNCH((layer_norm_block<XDT, ODT, false>), dim3(M), block, 0, s, out, x, gamma, beta, M, N, eps,
                          inv_n);
     return check_launch("layer_norm_block");
   }
-  hipLaunchKernelGGL((layer_norm_generic<XDT, ODT>), grid, block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);
+  LH_LAUNCH((layer_norm_generic<XDT, ODT>), grid, block, 0, s, out, x, gamma, beta, M, N, eps, inv_n);
   return check_launch("layer_norm_generic");
 }
 
@@ -474,8 +474,8 @@ template <int DT, int KIND>
 static int ew_launch(void* out, const void* a, const void* b, int64_t n, int N, hipStream_t s) {
   const bool vec = n % 4 == 0 && (KIND < EW_BIAS || N % 4 == 0) && aligned16(out) && aligned16(a) &&
                    (b == nullptr || aligned16(b));
-  if (vec) hipLaunchKernelGGL((elementwise4<DT, KIND>), dim3(ew_grid(n / 4)), dim3(256), 0, s, out, a, b, n / 4, N);
-  else hipLaunchKernelGGL((elementwise1<DT, KIND>), dim3(ew_grid(n)), dim3(256), 0, s, out, a, b, n, N);
+  if (vec) LH_LAUNCH((elementwise4<DT, KIND>), dim3(ew_grid(n / 4)), dim3(256), 0, s, out, a, b, n / 4, N);
+  else LH_LAUNCH((elementwise1<DT, KIND>), dim3(ew_grid(n)), dim3(256), 0, s, out, a, b, n, N);
   return check_launch("elementwise");
 }
 
@@ -505,6 +505,8 @@ int lh_hip_layer_norm(void* out, const void* x, const float* gamma, const float*
     return layer_norm_launch<LH_F32, LH_F32>(out, x, gamma, beta, (int)M, (int)N, eps, s);
   if (x_dtype == LH_F32 && out_dtype == LH_BF16)
     return layer_norm_launch<LH_F32, LH_BF16>(out, x, gamma, beta, (int)M, (int)N, eps, s);
+  if (x_dtype == LH_F32 && out_dtype == LH_F16)
+    return layer_norm_launch<LH_F32, LH_F16>(out, x, gamma, beta, (int)M, (int)N, eps, s);
   if (x_dtype == LH_BF16 && out_dtype == LH_BF16)
     return layer_norm_launch<LH_BF16, LH_BF16>(out, x, gamma, beta, (int)M, (int)N, eps, s);
   if (x_dtype == LH_BF16 && out_dtype == LH_F32)
@@ -520,7 +522,7 @@ int lh_hip_softmax(void* out, const void* x, int64_t M, int64_t N, int32_t dtype
   if (N % 256 == 0 && N <= 4096 && aligned16(out) && aligned16(x)) {
 #define LH_SM_CASE(DT, V)                                                                            \
   case V:                                                                                            \
-    hipLaunchKernelGGL((softmax_rows_vec<DT, V>), grid, block, 0, s, out, x, (int)M, (int)N);        \
+    LH_LAUNCH((softmax_rows_vec<DT, V>), grid, block, 0, s, out, x, (int)M, (int)N);        \
     return check_launch("softmax_rows_vec");
 #define LH_SM_DTYPE(DT)                                                                              \
   switch (N / 256) {                                                                                 \
@@ -538,7 +540,7 @@ int lh_hip_softmax(void* out, const void* x, int64_t M, int64_t N, int32_t dtype
   if (vec && N >= 64 && N <= 4096) {
 #define LH_SM_GUARD(DT, V)                                                                           \
   case V:                                                                                            \
-    hipLaunchKernelGGL((softmax_rows_vec<DT, V, true>), grid, block, 0, s, out, x, (int)M, (int)N);  \
+    LH_LAUNCH((softmax_rows_vec<DT, V, true>), grid, block, 0, s, out, x, (int)M, (int)N);  \
     return check_launch("softmax_rows_vec (guarded)");
 #define LH_SM_GUARD_DTYPE(DT)                                                                        \
   switch (row_groups_rounded((int)N)) {                                                              \
@@ -557,9 +559,9 @@ int lh_hip_softmax(void* out, const void* x, int64_t M, int64_t N, int32_t dtype
 #define LH_SMB_CASE(DT)                                                                                    \
   case DT:                                                                                                 \
     if (vec && N <= 1024 * kBlockRegGroups)                                                                \
-      hipLaunchKernelGGL((softmax_block_reg<DT>), rows, block, 0, s, out, x, (int)M, (int)N);              \
-    else if (vec) hipLaunchKernelGGL((softmax_block<DT, true>), rows, block, 0, s, out, x, (int)M, (int)N); \
-    else hipLaunchKernelGGL((softmax_block<DT, false>), rows, block, 0, s, out, x, (int)M, (int)N);        \
+      LH_LAUNCH((softmax_block_reg<DT>), rows, block, 0, s, out, x, (int)M, (int)N);              \
+    else if (vec) LH_LAUNCH((softmax_block<DT, true>), rows, block, 0, s, out, x, (int)M, (int)N); \
+    else LH_LAUNCH((softmax_block<DT, false>), rows, block, 0, s, out, x, (int)M, (int)N);        \
     return check_launch("softmax_block");
     switch (dtype) {
       LH_SMB_CASE(LH_F32) LH_SMB_CASE(LH_BF16) LH_SMB_CASE(LH_F16)
@@ -568,9 +570,9 @@ int lh_hip_softmax(void* out, const void* x, int64_t M, int64_t N, int32_t dtype
 #undef LH_SMB_CASE
   }
   switch (dtype) {
-    case LH_F32: hipLaunchKernelGGL(softmax_rows<LH_F32>, grid, block, 0, s, out, x, (int)M, (int)N); break;
-    case LH_BF16: hipLaunchKernelGGL(softmax_rows<LH_BF16>, grid, block, 0, s, out, x, (int)M, (int)N); break;
-    case LH_F16: hipLaunchKernelGGL(softmax_rows<LH_F16>, grid, block, 0, s, out, x, (int)M, (int)N); break;
+    case LH_F32: LH_LAUNCH(softmax_rows<LH_F32>, grid, block, 0, s, out, x, (int)M, (int)N); break;
+    case LH_BF16: LH_LAUNCH(softmax_rows<LH_BF16>, grid, block, 0, s, out, x, (int)M, (int)N); break;
+    case LH_F16: LH_LAUNCH(softmax_rows<LH_F16>, grid, block, 0, s, out, x, (int)M, (int)N); break;
     default: return fail(LH_ERR_UNSUPPORTED, "lh_hip_softmax: unsupported dtype %d", dtype);
   }
   return check_launch("softmax_rows");
@@ -602,7 +604,7 @@ int lh_hip_cast(void* out, const void* x, int64_t n, int32_t src, int32_t dst, v
   dim3 grid(ew_grid(n / 4 + 1)), block(256);
 #define LH_CAST(S, D)                                                         \
   if (src == S && dst == D) {                                                 \
-    hipLaunchKernelGGL((cast_kernel<S, D>), grid, block, 0, s, out, x, n);    \
+    LH_LAUNCH((cast_kernel<S, D>), grid, block, 0, s, out, x, n);    \
     return check_launch("cast_kernel");                                       \
   }
   LH_CAST(LH_F32, LH_BF16) LH_CAST(LH_F32, LH_F16) LH_CAST(LH_BF16, LH_F32) LH_CAST(LH_F16, LH_F32)

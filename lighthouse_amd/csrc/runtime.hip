@@ -1,5 +1,9 @@
 // Runtime part of the C ABI: error state, device info, device memory helpers.
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <utility>
+#include <vector>
 
 #include "common.h"
 
@@ -83,13 +87,13 @@ int transpose_matrix(void* out, const void* in, int R, int C, int64_t ld_in, int
                      hipStream_t s) {
   const dim3 grid((C + 63) / 64, (R + 63) / 64);
   if (elem_bytes == 2 && R % 8 == 0 && C % 8 == 0 && ld_in % 8 == 0 && ld_out % 8 == 0 && aligned16(out) && aligned16(in))
-    hipLaunchKernelGGL(transpose_tiles16, grid, dim3(256), 0, s, static_cast<uint16_t*>(out),
+    LH_LAUNCH(transpose_tiles16, grid, dim3(256), 0, s, static_cast<uint16_t*>(out),
                        static_cast<const uint16_t*>(in), R, C, ld_in, ld_out);
   else if (elem_bytes == 2)
-    hipLaunchKernelGGL(transpose_tiles<uint16_t>, grid, dim3(256), 0, s, static_cast<uint16_t*>(out),
+    LH_LAUNCH(transpose_tiles<uint16_t>, grid, dim3(256), 0, s, static_cast<uint16_t*>(out),
                        static_cast<const uint16_t*>(in), R, C, ld_in, ld_out);
   else if (elem_bytes == 4)
-    hipLaunchKernelGGL(transpose_tiles<uint32_t>, grid, dim3(256), 0, s, static_cast<uint32_t*>(out),
+    LH_LAUNCH(transpose_tiles<uint32_t>, grid, dim3(256), 0, s, static_cast<uint32_t*>(out),
                        static_cast<const uint32_t*>(in), R, C, ld_in, ld_out);
   else
     return fail(LH_ERR_UNSUPPORTED, "transpose: element size %d", elem_bytes);
@@ -118,54 +122,113 @@ int pad_copy_matrix(void* dst, int64_t ld_dst, int rows_dst, int cols_dst, const
   if (rows_dst <= 0 || cols_dst <= 0) return LH_OK;
   const dim3 grid((cols_dst + 2047) / 2048, rows_dst);
   if (elem_bytes == 2)
-    hipLaunchKernelGGL(pad_copy_kernel<uint16_t>, grid, dim3(256), 0, s, static_cast<uint16_t*>(dst), ld_dst, rows_dst,
+    LH_LAUNCH(pad_copy_kernel<uint16_t>, grid, dim3(256), 0, s, static_cast<uint16_t*>(dst), ld_dst, rows_dst,
                        cols_dst, static_cast<const uint16_t*>(src), ld_src, rows_src, cols_src);
   else if (elem_bytes == 4)
-    hipLaunchKernelGGL(pad_copy_kernel<uint32_t>, grid, dim3(256), 0, s, static_cast<uint32_t*>(dst), ld_dst, rows_dst,
+    LH_LAUNCH(pad_copy_kernel<uint32_t>, grid, dim3(256), 0, s, static_cast<uint32_t*>(dst), ld_dst, rows_dst,
                        cols_dst, static_cast<const uint32_t*>(src), ld_src, rows_src, cols_src);
   else if (elem_bytes == 1)
-    hipLaunchKernelGGL(pad_copy_kernel<uint8_t>, grid, dim3(256), 0, s, static_cast<uint8_t*>(dst), ld_dst, rows_dst,
+    LH_LAUNCH(pad_copy_kernel<uint8_t>, grid, dim3(256), 0, s, static_cast<uint8_t*>(dst), ld_dst, rows_dst,
                        cols_dst, static_cast<const uint8_t*>(src), ld_src, rows_src, cols_src);
   else
     return fail(LH_ERR_UNSUPPORTED, "pad copy: element size %d", elem_bytes);
   return check_launch("pad_copy");
 }
 
-static char* g_transpose_scratch = nullptr;
-static size_t g_transpose_scratch_bytes = 0;
+// ---- temporary device memory (see common.h) ------------------------------------------------
+static thread_local int g_planning = 0;
+bool planning() { return g_planning > 0; }
+PlanningScope::PlanningScope() { ++g_planning; }
+PlanningScope::~PlanningScope() { --g_planning; }
 
-// Library-owned buffers that only grow (hipFree waits for the work that may still use the old one).
-static void* grow_buffer(char*& buf, size_t& have, size_t bytes, const char* what) {
-  if (bytes > have) {
-    if (buf && hipFree(buf) != hipSuccess) (void)hipGetLastError();
-    buf = nullptr;
-    have = 0;
-    const hipError_t e = hipMalloc(reinterpret_cast<void**>(&buf), bytes);
+namespace {
+struct PoolBuffer {
+  char* p = nullptr;
+  size_t bytes = 0;
+};
+struct StreamPool {
+  PoolBuffer slot[kScratchSlots];
+};
+std::mutex g_pool_mutex;
+std::map<std::pair<int, hipStream_t>, StreamPool> g_pools;
+std::vector<std::pair<int, void*>> g_retired;  // (device, buffer) replaced by a larger one
+constexpr size_t kGranule = 256;
+size_t round_granule(size_t b) { return (b + kGranule - 1) / kGranule * kGranule; }
+}  // namespace
+
+int scratch_take(Scratch* ws, hipStream_t s, int slot, size_t bytes, const char* what, void** out) {
+  *out = nullptr;
+  if (bytes == 0) bytes = kGranule;
+  if (planning()) {
+    if (ws) ws->need += round_granule(bytes);
+    *out = reinterpret_cast<void*>(uintptr_t(1) << 20);  // aligned, never dereferenced
+    return LH_OK;
+  }
+  if (ws && ws->base) {
+    const size_t at = round_granule(ws->used);
+    if (at + bytes > ws->bytes)
+      return fail(LH_ERR_INVALID, "%s: workspace too small: %zu more bytes needed, %zu of %zu in use", what, bytes, at,
+                  ws->bytes);
+    ws->used = at + bytes;
+    *out = ws->base + at;
+    return LH_OK;
+  }
+  int dev = 0;
+  LH_HIP_CHECK(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  PoolBuffer& b = g_pools[{dev, s}].slot[slot];
+  if (bytes > b.bytes) {
+    // At least double, so that the buffers left behind add up to less than the live one.
+    size_t want = round_granule(bytes > 2 * b.bytes ? bytes : 2 * b.bytes);
+    char* p = nullptr;
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&p), want);
+    if (e != hipSuccess && want > round_granule(bytes)) {
+      (void)hipGetLastError();
+      want = round_granule(bytes);
+      e = hipMalloc(reinterpret_cast<void**>(&p), want);
+    }
     if (e != hipSuccess) {
       (void)hipGetLastError();
-      set_error("%s: hipMalloc of %zu bytes failed: %s", what, bytes, hipGetErrorString(e));
-      buf = nullptr;
-      return nullptr;
+      return fail(LH_ERR_RUNTIME, "%s: hipMalloc of %zu bytes failed: %s", what, want, hipGetErrorString(e));
     }
-    have = bytes;
+    if (b.p) g_retired.emplace_back(dev, b.p);
+    b.p = p;
+    b.bytes = want;
   }
-  return buf;
+  *out = b.p;
+  return LH_OK;
 }
 
-void* transpose_scratch(size_t bytes) {
-  return grow_buffer(g_transpose_scratch, g_transpose_scratch_bytes, bytes, "transpose scratch");
-}
-
-static char* g_pad_scratch = nullptr;
-static size_t g_pad_scratch_bytes = 0;
-
-void* pad_scratch(size_t bytes) { return grow_buffer(g_pad_scratch, g_pad_scratch_bytes, bytes, "padding scratch"); }
-
-static char* g_splitk_scratch = nullptr;
-static size_t g_splitk_scratch_bytes = 0;
-
-void* splitk_scratch(size_t bytes) {
-  return grow_buffer(g_splitk_scratch, g_splitk_scratch_bytes, bytes, "split-K scratch");
+static int release_pool_of_current_device() {
+  int dev = 0;
+  LH_HIP_CHECK(hipGetDevice(&dev));
+  LH_HIP_CHECK(hipDeviceSynchronize());
+  std::lock_guard<std::mutex> lock(g_pool_mutex);
+  hipError_t first = hipSuccess;
+  auto release = [&](void* p) {
+    const hipError_t e = hipFree(p);
+    if (e != hipSuccess && first == hipSuccess) first = e;
+  };
+  for (auto it = g_pools.begin(); it != g_pools.end();) {
+    if (it->first.first != dev) {
+      ++it;
+      continue;
+    }
+    for (PoolBuffer& b : it->second.slot)
+      if (b.p) release(b.p);
+    it = g_pools.erase(it);
+  }
+  std::vector<std::pair<int, void*>> keep;
+  for (auto& r : g_retired) {
+    if (r.first == dev) release(r.second);
+    else keep.push_back(r);
+  }
+  g_retired.swap(keep);
+  if (first != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(LH_ERR_RUNTIME, "lh_hip_release_scratch: hipFree failed: %s", hipGetErrorString(first));
+  }
+  return LH_OK;
 }
 
 }  // namespace lh
@@ -248,6 +311,8 @@ int lh_hip_memset(void* dev_ptr, int value, size_t bytes) {
   LH_HIP_CHECK(hipMemset(dev_ptr, value, bytes));
   return LH_OK;
 }
+
+int lh_hip_release_scratch(void) { return release_pool_of_current_device(); }
 
 int lh_hip_sync(void* stream) {
   LH_HIP_CHECK(hipStreamSynchronize(reinterpret_cast<hipStream_t>(stream)));

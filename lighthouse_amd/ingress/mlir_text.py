@@ -12,7 +12,9 @@ rejects everything else with ``ValueError``:
   mulf+addf contraction, addf of a 1-D operand, maximumf against a zero constant.
 
 The matmul accumulates into its ``outs`` operand when that is a function argument (the in-place
-result of bufferisation) and starts from zero when it is a zero ``linalg.fill`` / ``tensor.empty``.
+result of bufferisation) and starts from zero when it is a zero ``linalg.fill`` / ``tensor.empty``,
+also when that fill is itself an in-place operation on the argument buffer (memref form, where
+operations have no results and a buffer's contents depend on the program order).
 The function's argument order is kept: callers pass buffers in signature order.
 """
 
@@ -107,12 +109,19 @@ def parse_function(text: str, name: str, maps: dict[str, tuple[str, ...]]) -> Pa
         arg_names.append(nm.strip())
         arg_types.append(_parse_type(ty))
     env: dict[str, _Value] = {n: _Value("arg", (i,)) for i, n in enumerate(arg_names)}
+    # A buffer (memref) is rewritten in place by operations that have no SSA result.  Each such
+    # write makes a new version of the buffer's name, and operands are read through `cur`, so a
+    # value always refers to the contents its operands had at that point of the program.
+    cur: dict[str, str] = {}
+    versions: dict[str, int] = {}
     returned = None
     for stmt in _split_statements(_function_body(text, m.end())):
         res = re.match(r"(%[\w.#-]+)(?::\d+)?\s*=\s*(.*)", stmt)
         result, rest = (res.group(1), res.group(2)) if res else (None, stmt)
         op = rest.split()[0].split("(")[0]
-        ins, outs = _operands(rest, "ins"), _operands(rest, "outs")
+        raw_outs = _operands(rest, "outs")
+        ins = [cur.get(x, x) for x in _operands(rest, "ins")]
+        outs = [cur.get(x, x) for x in raw_outs]
         val = None
         if op == "arith.constant":
             c = re.search(r"arith\.constant\s+(dense<)?([-+0-9.eE]+|true|false)", rest)
@@ -150,11 +159,18 @@ def parse_function(text: str, name: str, maps: dict[str, tuple[str, ...]]) -> Pa
         elif op in ("return", "func.return"):
             ops_ = [o.strip() for o in rest.split(":")[0].split()[1:]]
             returned = ops_[0].rstrip(",") if ops_ else None
+            returned = cur.get(returned, returned) if returned else None
             continue
         else:
             raise ValueError(f"unsupported operation '{op}' in @{name}; this target runs matmul(+bias)(+relu) payloads")
         if result is not None:
             env[result] = val
+        elif raw_outs and op.startswith("linalg."):
+            # in-place write to a buffer: later reads of raw_outs[0] see this value
+            versions[raw_outs[0]] = versions.get(raw_outs[0], 0) + 1
+            versioned = f"{raw_outs[0]}@{versions[raw_outs[0]]}"
+            env[versioned] = val
+            cur[raw_outs[0]] = versioned
         last = val if val.kind in ("matmul", "bias", "relu") else None
         if last is not None:
             env["__last__"] = val

@@ -254,9 +254,9 @@ def generate_nanogpt_block_payload(
     workspace)``: one pre-LayerNorm GPT-2 block (op order of ``_emit_block_fused``,
     examples/xegpu/nanoGPT_payload.py:299-317; fused QKV, causal, tanh-GELU)."""
     dt = elem_name(dtype)
-    if dt not in ("f32", "bf16"):
-        raise ValueError("nanoGPT block dtype must be f32 or bf16")
-    ws = int(_lib.load().lh_hip_nanogpt_block_workspace_bytes(B, T, C, lh_dtype(dt)))
+    if dt not in ("f32", "bf16", "f16"):
+        raise ValueError("nanoGPT block dtype must be f32, bf16 or f16")
+    ws = int(_lib.load().lh_hip_nanogpt_block_workspace_bytes(B, T, C, lh_dtype(dt), None))
     args = [
         ArgSpec((B * T, C), "f32", writable=True), ArgSpec((B * T, C), "f32"),
         ArgSpec((C,), "f32"), ArgSpec((C,), "f32"),
@@ -271,6 +271,35 @@ def generate_nanogpt_block_payload(
     rows, hs = B * T, C // n_head
     flops = 2 * rows * C * 3 * C + 2 * B * n_head * T * T * hs + 2 * rows * C * C + 4 * rows * C * 4 * C
     return _single(PayloadFunction(func_name, "nanogpt_block", attrs, args, flops, 0))
+
+
+def build_gpt_fused_payload(
+    func_name: str, T: int, C: int, hidden: int, vocab: int, n_layer: int, H: int, eps: float = 1e-5,
+    dtype: str = "f16", causal: bool = False,
+) -> PayloadModule:
+    """The reference's full nanoGPT forward, ``build_gpt_fused_payload``
+    examples/xegpu/nanoGPT_payload.py:318-407, with its argument list: ``payload(out, x, per layer
+    [g1, b1n, wq, wk, wv, wp, bp, g2, b2n, w1, bb1, w2, bb2], gf_g, gf_b, lmw, lmb)`` plus a trailing
+    workspace (the reference allocates and frees its intermediates inside the payload, :407-408;
+    here the caller's memory manager owns them).  Weights are 16-bit (``dtype``), LayerNorm
+    parameters and biases f32, attention non-causal, MLP activation ReLU."""
+    dt = elem_name(dtype)
+    if dt not in ("f32", "bf16", "f16"):
+        raise ValueError("nanoGPT dtype must be f32, bf16 or f16")
+    opts = _lib.NanoGPTBlockOpts(1 if causal else 0, _lib.ACT_RELU, _lib.F32, int(hidden))
+    ws = int(_lib.load().lh_hip_nanogpt_forward_workspace_bytes(1, T, C, vocab, lh_dtype(dt), ctypes.byref(opts)))
+    per_layer = [ArgSpec((C,), "f32"), ArgSpec((C,), "f32"), ArgSpec((C, C), dt), ArgSpec((C, C), dt), ArgSpec((C, C), dt),
+                 ArgSpec((C, C), dt), ArgSpec((C,), "f32"), ArgSpec((C,), "f32"), ArgSpec((C,), "f32"),
+                 ArgSpec((C, hidden), dt), ArgSpec((hidden,), "f32"), ArgSpec((hidden, C), dt), ArgSpec((C,), "f32")]
+    args = [ArgSpec((T, vocab), "f32", writable=True), ArgSpec((T, C), "f32")]
+    for _ in range(n_layer):
+        args += [ArgSpec(a.shape, a.elem) for a in per_layer]
+    args += [ArgSpec((C,), "f32"), ArgSpec((C,), "f32"), ArgSpec((C, vocab), dt), ArgSpec((vocab,), "f32"),
+             ArgSpec((ws,), "i8")]
+    attrs = _lib.GptFusedAttrs(lh_dtype(dt), int(H), int(n_layer), 1 if causal else 0, float(eps))
+    hs = C // H
+    flops = n_layer * (2 * T * C * 3 * C + 4 * H * T * T * hs + 2 * T * C * C + 4 * T * C * hidden) + 2 * T * C * vocab
+    return _single(PayloadFunction(func_name, "gpt_fused", attrs, args, flops, 0))
 
 
 def _size(elem: str) -> int:

@@ -109,6 +109,94 @@ int lhref_matmul_bf16(uint16_t* out, const uint16_t* a, const uint16_t* b, const
   return 0;
 }
 
+/*
+ * The same two payloads cache-tiled: the CPU analogue of the reference's optimising matmul
+ * pipeline (pack, tile, register-tile, vectorise: lighthouse/pipeline/descriptors/x86_64/matmul/
+ * f32.yaml:1-17) with the OpenMP stage of x86_64/lower.yaml:6 over row blocks.  Each thread takes
+ * blocks of TM rows; for a block and a strip of TN columns the f32 accumulators live in a
+ * thread-private tile and K is walked in chunks of TK (the TK x TN piece of B stays in the cache
+ * across the block's rows; the innermost loop runs along columns and vectorises).  Every output
+ * element still adds its products one at a time in increasing k, multiply and add separate, so the
+ * results equal the plain loop nests' bit for bit.
+ */
+#define LHREF_TM 32
+#define LHREF_TN 512
+#define LHREF_TK 128
+
+int lhref_matmul_f32_tiled(float* out, const float* a, const float* b, const float* bias, int64_t M, int64_t N,
+                           int64_t K, uint32_t flags, int threads) {
+#pragma omp parallel for num_threads(threads) schedule(dynamic, 1)
+  for (int64_t i0 = 0; i0 < M; i0 += LHREF_TM) {
+    float acc[LHREF_TM][LHREF_TN];
+    const int64_t mi = (M - i0 < LHREF_TM) ? M - i0 : LHREF_TM;
+    for (int64_t j0 = 0; j0 < N; j0 += LHREF_TN) {
+      const int64_t nj = (N - j0 < LHREF_TN) ? N - j0 : LHREF_TN;
+      for (int64_t i = 0; i < mi; ++i)
+        for (int64_t j = 0; j < nj; ++j) acc[i][j] = (flags & LHREF_ACCUMULATE_C) ? out[(i0 + i) * N + j0 + j] : 0.0f;
+      for (int64_t k0 = 0; k0 < K; k0 += LHREF_TK) {
+        const int64_t nk = (K - k0 < LHREF_TK) ? K - k0 : LHREF_TK;
+        for (int64_t i = 0; i < mi; ++i)
+          for (int64_t k = 0; k < nk; ++k) {
+            const float av = a[(i0 + i) * K + k0 + k];
+            const float* brow = b + (k0 + k) * N + j0;
+            for (int64_t j = 0; j < nj; ++j) {
+              float p = av * brow[j];
+              acc[i][j] = acc[i][j] + p;
+            }
+          }
+      }
+      for (int64_t i = 0; i < mi; ++i)
+        for (int64_t j = 0; j < nj; ++j) {
+          float v = acc[i][j];
+          if (flags & LHREF_BIAS) v = bias[j0 + j] + v;
+          if (flags & LHREF_GELU) v = gelu_tanh_f32(v);
+          if (flags & LHREF_RELU) v = v > 0.0f ? v : (v != v ? v : 0.0f);
+          out[(i0 + i) * N + j0 + j] = v;
+        }
+    }
+  }
+  return 0;
+}
+
+int lhref_matmul_bf16_tiled(uint16_t* out, const uint16_t* a, const uint16_t* b, const uint16_t* bias, int64_t M,
+                            int64_t N, int64_t K, uint32_t flags, int threads) {
+#pragma omp parallel for num_threads(threads) schedule(dynamic, 1)
+  for (int64_t i0 = 0; i0 < M; i0 += LHREF_TM) {
+    float acc[LHREF_TM][LHREF_TN];
+    float bt[LHREF_TK][LHREF_TN]; /* the B piece extended to f32 once per block */
+    const int64_t mi = (M - i0 < LHREF_TM) ? M - i0 : LHREF_TM;
+    for (int64_t j0 = 0; j0 < N; j0 += LHREF_TN) {
+      const int64_t nj = (N - j0 < LHREF_TN) ? N - j0 : LHREF_TN;
+      for (int64_t i = 0; i < mi; ++i)
+        for (int64_t j = 0; j < nj; ++j)
+          acc[i][j] = (flags & LHREF_ACCUMULATE_C) ? bf16_to_f32(out[(i0 + i) * N + j0 + j]) : 0.0f;
+      for (int64_t k0 = 0; k0 < K; k0 += LHREF_TK) {
+        const int64_t nk = (K - k0 < LHREF_TK) ? K - k0 : LHREF_TK;
+        for (int64_t k = 0; k < nk; ++k)
+          for (int64_t j = 0; j < nj; ++j) bt[k][j] = bf16_to_f32(b[(k0 + k) * N + j0 + j]);
+        for (int64_t i = 0; i < mi; ++i)
+          for (int64_t k = 0; k < nk; ++k) {
+            const float av = bf16_to_f32(a[(i0 + i) * K + k0 + k]);
+            for (int64_t j = 0; j < nj; ++j) {
+              float p = av * bt[k][j];
+              acc[i][j] = acc[i][j] + p;
+            }
+          }
+      }
+      for (int64_t i = 0; i < mi; ++i)
+        for (int64_t j = 0; j < nj; ++j) {
+          float v = acc[i][j];
+          if (flags & LHREF_BIAS) v = bf16_to_f32(bias[j0 + j]) + v;
+          if (flags & LHREF_GELU) v = gelu_tanh_f32(v);
+          uint16_t r = f32_to_bf16(v);
+          if ((flags & LHREF_RELU) && (r & 0x8000) && (r & 0x7fff) <= 0x7f80) r = 0;
+          out[(i0 + i) * N + j0 + j] = r;
+        }
+    }
+  }
+  return 0;
+}
+
 /* fp8 e4m3 GEMM with per-tensor scales: bf16((Aq.Bq)_f32 * (sa*sb)). */
 int lhref_matmul_fp8(uint16_t* out, const uint8_t* a, const uint8_t* b, float scale_a, float scale_b, int64_t M,
                      int64_t N, int64_t K, int threads) {

@@ -22,6 +22,11 @@ Parity status of each function (what pins it, see tests/test_oracle_*.py):
   layer_norm, softmax, gelu_tanh  : pinned by torch.nn.functional routines.
   nanogpt_block                   : pinned by an independent torch nn.Module
       restating the block of the benchmark configuration.
+  nanogpt_forward                 : pinned by the same module stacked n times, then
+      torch LayerNorm and Linear with non-trivial final gamma / beta / bias.
+  ref_block_fused, ref_gpt_fused  : the reference's own checker restated
+      (examples/xegpu/nanoGPT.py:84-135); pinned by an independent torch module
+      (separate q/k/v projections, non-causal SDPA, ReLU MLP) in float64.
 """
 
 from __future__ import annotations
@@ -422,7 +427,8 @@ def residual_add(a, b, result_type: str = "f32"):
 # ----------------------------------------------------------------------------
 
 
-def nanogpt_block(x, p: dict, n_head: int, *, mode: str = "f32", eps: float = 1e-5, causal: bool = True):
+def nanogpt_block(x, p: dict, n_head: int, *, mode: str = "f32", eps: float = 1e-5, causal: bool = True,
+                  activation: str = "gelu_tanh", bias_f32: bool = False):
     """Forward of one pre-LayerNorm GPT-2 block.
 
     Op order follows ``_emit_block_fused`` examples/xegpu/nanoGPT_payload.py:299-317
@@ -435,22 +441,34 @@ def nanogpt_block(x, p: dict, n_head: int, *, mode: str = "f32", eps: float = 1e
       ln2 = LN(a) ; h = gelu(ln2 W1 + b1) ; y = a + h W2 + b2
 
     ``mode="f32"``: every tensor float32 (float64 arithmetic here as arbiter).
-    ``mode="bf16"``: residual stream, LayerNorm statistics and all accumulators
+    ``mode="bf16"`` / ``"f16"``: residual stream, LayerNorm statistics and all accumulators
     in float32; every matmul input (ln1, ln2, weights, q, k, v, attention
-    probabilities, attention output, GELU output) rounded to bfloat16, i.e. the
-    rounding points of examples/xegpu/nanoGPT.py:114-126 with bf16 for f16.
+    probabilities, attention output, MLP hidden activations) rounded to the 16-bit type, i.e. the
+    rounding points of examples/xegpu/nanoGPT.py:114-126.
+
+    The reference's own block is reached with ``causal=False, activation="relu", bias_f32=True``
+    and separate projections ``w_q / w_k / w_v`` in place of ``w_qkv`` (any bias may be None).
 
     x: [B, T, C].  p keys: ln1_g ln1_b w_qkv b_qkv w_o b_o ln2_g ln2_b w_fc b_fc w_proj b_proj,
     weights stored [in, out].  Returns float32 [B, T, C].
     """
-    elt = "f32" if mode == "f32" else "bf16"
-    r = (lambda t: np.asarray(t, dtype=np.float32)) if elt == "f32" else (lambda t: round_bf16(np.asarray(t, dtype=np.float32)))
+    elt = mode
+    r = lambda t: round_to(np.asarray(t, dtype=np.float32), elt)
+    rb = (lambda t: None if t is None else np.asarray(t, dtype=np.float32)) if bias_f32 else (
+        lambda t: None if t is None else r(t))
+    gelu, relu = activation == "gelu_tanh", activation == "relu"
+    if not (gelu or relu):
+        raise ValueError(f"unknown activation {activation}")
     x = np.asarray(x, dtype=np.float32)
     bsz, t, c = x.shape
     hs = c // n_head
     x2 = x.reshape(bsz * t, c)
     ln1 = layer_norm(x2, p["ln1_g"], p["ln1_b"], eps, elt)
-    qkv = matmul(ln1, r(p["w_qkv"]), bias=r(p["b_qkv"]), result_type=elt)
+    if "w_qkv" in p:
+        qkv = matmul(ln1, r(p["w_qkv"]), bias=rb(p.get("b_qkv")), result_type=elt)
+    else:
+        qkv = np.concatenate([matmul(ln1, r(p[k]), bias=rb(p.get("b" + k[1:])), result_type=elt)
+                              for k in ("w_q", "w_k", "w_v")], axis=1)
     qkv = qkv.reshape(bsz, t, 3, n_head, hs)
     q = qkv[:, :, 0].transpose(0, 2, 1, 3)
     k = qkv[:, :, 1].transpose(0, 2, 1, 3)
@@ -460,26 +478,80 @@ def nanogpt_block(x, p: dict, n_head: int, *, mode: str = "f32", eps: float = 1e
     else:
         att = _attention_rounded_p(q, k, v, causal=causal, elt=elt)
     att = att.transpose(0, 2, 1, 3).reshape(bsz * t, c)
-    proj = matmul(att, r(p["w_o"]), bias=r(p["b_o"]), result_type="f32")
+    proj = matmul(att, r(p["w_o"]), bias=rb(p.get("b_o")), result_type="f32")
     a = x2 + proj
     ln2 = layer_norm(a, p["ln2_g"], p["ln2_b"], eps, elt)
-    h = matmul(ln2, r(p["w_fc"]), bias=r(p["b_fc"]), gelu=True, result_type=elt)
-    o = matmul(h, r(p["w_proj"]), bias=r(p["b_proj"]), result_type="f32")
+    h = matmul(ln2, r(p["w_fc"]), bias=rb(p.get("b_fc")), gelu=gelu, relu=relu, result_type=elt)
+    o = matmul(h, r(p["w_proj"]), bias=rb(p.get("b_proj")), result_type="f32")
     return (a + o).astype(np.float32).reshape(bsz, t, c)
 
 
-def nanogpt_forward(x, layers, lnf_g, lnf_b, lm_w, lm_b, n_head: int, *, mode: str = "f32", eps: float = 1e-5):
+def nanogpt_forward(x, layers, lnf_g, lnf_b, lm_w, lm_b, n_head: int, *, mode: str = "f32", eps: float = 1e-5,
+                    causal: bool = True, activation: str = "gelu_tanh", bias_f32: bool = False):
     """n blocks, final LayerNorm, lm_head with bias: the tail of ``build_gpt_fused_payload``
     examples/xegpu/nanoGPT_payload.py:401-407 (``hf = LN(h)``, cast to the matmul input type,
     ``logits = hf W + b`` in float32) after ``nanogpt_block`` applied per layer (:399-400)."""
-    elt = "f32" if mode == "f32" else "bf16"
+    elt = mode
     h = np.asarray(x, dtype=np.float32)
     for p in layers:
-        h = nanogpt_block(h, p, n_head, mode=mode, eps=eps)
+        h = nanogpt_block(h, p, n_head, mode=mode, eps=eps, causal=causal, activation=activation, bias_f32=bias_f32)
     bsz, t, c = h.shape
     hf = layer_norm(h.reshape(bsz * t, c), lnf_g, lnf_b, eps, elt)
-    logits = matmul(hf, round_to(lm_w, elt), bias=None if lm_b is None else round_to(lm_b, elt), result_type="f32")
+    lm_bias = None if lm_b is None else (np.asarray(lm_b, dtype=np.float32) if bias_f32 else round_to(lm_b, elt))
+    logits = matmul(hf, round_to(lm_w, elt), bias=lm_bias, result_type="f32")
     return logits.reshape(bsz, t, -1)
+
+
+def ref_block_fused(x, w: dict, n_head: int, eps: float = 1e-5, causal: bool = False, elt: str = "f16"):
+    """The reference's own block checker, ``numpy_ref_block_fused`` examples/xegpu/nanoGPT.py:112-126,
+    for the block of ``_emit_block_fused`` examples/xegpu/nanoGPT_payload.py:299-317: separate
+    ``wq/wk/wv`` projections without bias, non-causal attention by default, ReLU MLP, float32 biases
+    and LayerNorm parameters, 16-bit weights.  x: [T, C] float32.  ``w`` keys as in the reference:
+    g1 b1n wq wk wv wp bp g2 b2n w1 bb1 w2 bb2.
+
+    Rounding points (``_f16`` there, ``elt`` here): ln1, q, k, v, the normalised attention weights
+    (``_mha`` :95-109), the attention output, ln2, the MLP hidden activations; everything else float32
+    (float64 sums here)."""
+    r = lambda t: round_to(np.asarray(t, dtype=np.float32), elt)
+    f64 = lambda t: np.asarray(t, dtype=np.float64)
+    x = np.asarray(x, dtype=np.float32)
+    t, c = x.shape
+    hs = c // n_head
+
+    def ln(v, g, b):  # _ln :85-88: population variance, division by sqrt
+        v = f64(v)
+        mu = v.mean(-1, keepdims=True)
+        var = ((v - mu) ** 2).mean(-1, keepdims=True)
+        return ((v - mu) / np.sqrt(var + eps) * f64(g) + f64(b)).astype(np.float32)
+
+    ln1 = r(ln(x, w["g1"], w["b1n"]))
+    q = r((f64(ln1) @ f64(w["wq"])).astype(np.float32))
+    k = r((f64(ln1) @ f64(w["wk"])).astype(np.float32))
+    v = r((f64(ln1) @ f64(w["wv"])).astype(np.float32))
+    attn = np.zeros((t, c), np.float32)
+    mask = np.triu(np.full((t, t), -np.inf), k=1) if causal else 0.0
+    for h in range(n_head):  # _mha :95-109
+        sl = slice(h * hs, (h + 1) * hs)
+        s = (f64(q[:, sl]) @ f64(k[:, sl]).T) * (1.0 / hs**0.5) + mask
+        e = np.exp(s - s.max(-1, keepdims=True))
+        p = r((e / e.sum(-1, keepdims=True)).astype(np.float32))
+        attn[:, sl] = (f64(p) @ f64(v[:, sl])).astype(np.float32)
+    proj = (f64(r(attn)) @ f64(w["wp"]) + f64(w["bp"])).astype(np.float32)
+    a = x + proj
+    ln2 = r(ln(a, w["g2"], w["b2n"]))
+    hh = np.maximum((f64(ln2) @ f64(w["w1"]) + f64(w["bb1"])).astype(np.float32), np.float32(0))
+    o = (f64(r(hh)) @ f64(w["w2"]) + f64(w["bb2"])).astype(np.float32)
+    return a + o
+
+
+def ref_gpt_fused(x, layer_w, gf_g, gf_b, lmw, lmb, n_head: int, eps: float = 1e-5, elt: str = "f16"):
+    """``numpy_ref_gpt_fused`` examples/xegpu/nanoGPT.py:128-135: the blocks above, the final
+    LayerNorm rounded to the 16-bit type, ``logits = hf W + b`` in float32."""
+    h = np.asarray(x, dtype=np.float32)
+    for w in layer_w:
+        h = ref_block_fused(h, w, n_head, eps, elt=elt)
+    hf = layer_norm(h, gf_g, gf_b, eps, elt)
+    return (hf.astype(np.float64) @ np.asarray(lmw, dtype=np.float64) + np.asarray(lmb, dtype=np.float64)).astype(np.float32)
 
 
 def _attention_rounded_p(q, k, v, *, causal: bool, elt: str):

@@ -40,7 +40,7 @@ def test_gemm_f32(shape, epi):
     has = epi == "bias_relu"
     out = ops.gemm(_dev(a, torch.float32), _dev(b, torch.float32), _dev(bias, torch.float32) if has else None, relu=has)
     ref = orc.matmul(a, b, bias=bias if has else None, relu=has)
-    assert_close(_host(out), ref, F32_RTOL, f"f32 gemm {shape} {epi}")
+    assert_close(_host(out), ref, F32_RTOL, f"f32 gemm {shape} {epi}", report=shape == (1024, 1024, 1024) and epi != "none")
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -316,9 +316,24 @@ def test_gemm_bf16_4096_properties():
     a_h = a[rows].float().cpu().numpy()
     b_h = b[:, cols].float().cpu().numpy()
     ref = orc.matmul(a_h, b_h, result_type="bf16")
-    assert_close(_host(out[rows][:, cols]), ref, BF16_RTOL, "bf16 4096 sample")
+    assert_close(_host(out[rows][:, cols]), ref, BF16_RTOL, "bf16 GEMM 4096^3 (sampled)", report=True)
     ref_epi = orc.matmul(a_h, b_h, bias=bias[cols].float().cpu().numpy(), relu=True, result_type="bf16")
-    assert_close(_host(out_epi[rows][:, cols]), ref_epi, BF16_RTOL, "bf16 4096 epilogue sample")
+    assert_close(_host(out_epi[rows][:, cols]), ref_epi, BF16_RTOL, "bf16 GEMM 4096^3 + bias + ReLU (sampled)",
+                 report=True)
+    # The same samples far inside the benchmark tolerance: the result is the float64 sum rounded to
+    # bf16, up to one more bf16 step where the f32 accumulation error crosses a rounding boundary
+    # (|err| <= 2^-7 |ref| + 0.02).  An element is ~N(0, 64^2) here, a lost 16-wide k-slice ~N(0, 4^2).
+    for got, want in ((_host(out[rows][:, cols]), ref), (_host(out_epi[rows][:, cols]), ref_epi)):
+        assert (np.abs(got - want) <= 2.0**-7 * np.abs(want) + 0.02).all()
+    # Whole sampled rows of an integer problem at the same size, exact against numpy: any wrong,
+    # missing or doubled product changes an integer.
+    ai = torch.randint(-3, 4, (n, n), device="cuda", generator=g).to(torch.bfloat16)
+    bint = torch.randint(-3, 4, (n, n), device="cuda", generator=g).to(torch.bfloat16)
+    exact = ops.gemm(ai, bint, out_dtype=torch.float32)
+    want = ai[rows].float().cpu().numpy().astype(np.int64) @ bint.float().cpu().numpy().astype(np.int64)
+    np.testing.assert_array_equal(_host(exact[rows]).astype(np.int64), want)
+    cols_want = ai.float().cpu().numpy().astype(np.int64) @ bint[:, cols].float().cpu().numpy().astype(np.int64)
+    np.testing.assert_array_equal(_host(exact[:, cols]).astype(np.int64), cols_want)
     # Small-integer matrices: every partial sum is exact, so linearity must hold bit for bit.
     a1 = torch.randint(-2, 3, (n, n), device="cuda", generator=g).to(torch.bfloat16)
     a2 = torch.randint(-2, 3, (n, n), device="cuda", generator=g).to(torch.bfloat16)
@@ -393,7 +408,7 @@ def test_gemm_fp8_8192_properties():
     a_codes = a.view(torch.uint8)[rows].cpu().numpy()
     b_codes = b.view(torch.uint8).cpu().numpy()
     ref = orc.matmul_fp8(a_codes, b_codes, 0.5, 0.25)
-    assert_close(_host(out[rows]), ref, FP8_RTOL, "fp8 8192^3 sampled rows")
+    assert_close(_host(out[rows]), ref, FP8_RTOL, "fp8 GEMM 8192^3 (sampled rows)", report=True)
     eye = torch.eye(n, device="cuda").to(torch.float8_e4m3fn)
     out_id = ops.gemm_fp8(a, eye, 0.5, 0.25)
     expect = (a.float() * 0.125).to(torch.bfloat16)
@@ -417,7 +432,7 @@ def test_gemm_fp8_decode_path(shape):
     first = None
     for _ in range(3):
         out = ops.gemm_fp8(da, db, float(sa), float(sb))
-        assert_close(_host(out), ref, FP8_RTOL, f"fp8 decode {shape}")
+        assert_close(_host(out), ref, FP8_RTOL, f"fp8 decode {shape}", report=shape == (16, 8192, 8192))
         first = out if first is None else first
         assert torch.equal(out, first)
     out32 = ops.gemm_fp8(da, db, float(sa), float(sb), out_dtype=torch.float32)
@@ -603,3 +618,89 @@ def test_gemm_residual_input(shape, elt, out_elt):
     assert_close(_host(out), ref, rtol, f"{elt}->{out_elt} gemm {shape} + residual")
     assert np.array_equal(_host(d_res), res), "the residual input was modified"
     assert out.data_ptr() != d_res.data_ptr()
+
+
+# ---- temporary memory: caller workspaces and the per-stream pool -------------------------------------
+
+
+@pytest.mark.parametrize("case", ["split_k", "padded", "transposed", "plain"])
+def test_gemm_with_caller_workspace(case):
+    """lh_hip_gemm_ws: same kernels, temporaries from the caller's buffer; results equal the pooled
+    call bit for bit, a short workspace is refused before anything runs."""
+    from lighthouse_amd import ops
+
+    shapes = {"split_k": (16, 2048, 8192), "padded": (300, 520, 776), "transposed": (512, 512, 512), "plain": (512, 512, 512)}
+    M, N, K = shapes[case]
+    tb = case == "transposed"
+    rng = np.random.default_rng(11)
+    a = _dev(orc.round_bf16(rng.standard_normal((M, K)).astype(np.float32)), torch.bfloat16)
+    b_h = orc.round_bf16(rng.standard_normal((K, N)).astype(np.float32))
+    b = _dev(b_h.T.copy() if tb else b_h, torch.bfloat16)
+    bias = _dev(orc.round_bf16(rng.standard_normal(N).astype(np.float32)), torch.bfloat16)
+    need = ops.gemm_workspace_bytes(M, N, K, torch.bfloat16, bias=True, relu=True, transpose_b=tb)
+    assert (need > 0) == (case != "plain")
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    want = ops.gemm(a, b, bias, relu=True, transpose_b=tb)
+    got = ops.gemm(a, b, bias, relu=True, transpose_b=tb, workspace=ws)
+    assert torch.equal(got, want)
+    ref = orc.matmul(_host(a), b_h, bias=_host(bias), relu=True, result_type="bf16")
+    assert_close(_host(got), ref, BF16_RTOL, f"bf16 gemm {case} with a caller workspace")
+    if need:
+        sentinel = torch.full((M, N), 7.0, device="cuda", dtype=torch.bfloat16)
+        with pytest.raises(ValueError, match="workspace too small"):
+            ops.gemm(a, b, bias, relu=True, transpose_b=tb, workspace=ws[: need - 256], out=sentinel)
+        with pytest.raises(ValueError, match="workspace too small"):
+            ops.gemm(a, b, bias, relu=True, transpose_b=tb, workspace=ws[:0], out=sentinel)
+
+
+def test_gemm_fp8_with_caller_workspace():
+    from lighthouse_amd import ops
+
+    rng = np.random.default_rng(12)
+    for M, N, K in ((16, 2048, 4096), (64, 1024, 2048), (256, 512, 8192), (512, 512, 512)):
+        aq = _dev(rng.integers(0, 256, (M, K), dtype=np.uint8) & 0x77, torch.uint8).view(torch.float8_e4m3fn)
+        bq = _dev(rng.integers(0, 256, (K, N), dtype=np.uint8) & 0x77, torch.uint8).view(torch.float8_e4m3fn)
+        need = ops.gemm_fp8_workspace_bytes(M, N, K)
+        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        want = ops.gemm_fp8(aq, bq, 0.5, 0.25)
+        got = ops.gemm_fp8(aq, bq, 0.5, 0.25, workspace=ws)
+        assert torch.equal(got, want), (M, N, K)
+        if need:
+            with pytest.raises(ValueError, match="workspace too small"):
+                ops.gemm_fp8(aq, bq, 0.5, 0.25, workspace=ws[: need // 2])
+
+
+def test_split_k_gemms_on_two_streams():
+    """Two streams run decode-shaped GEMMs of different shapes (both cut along K, so both use f32
+    partial blocks) at the same time, many times over: each stream has its own temporaries, so
+    every result equals the one computed alone and matches the oracle."""
+    from lighthouse_amd import ops
+
+    rng = np.random.default_rng(13)
+    problems = []
+    for M, N, K in ((16, 4096, 8192), (32, 1024, 4096)):
+        a_h = rng.integers(-3, 4, (M, K)).astype(np.float32)
+        b_h = rng.integers(-3, 4, (K, N)).astype(np.float32)
+        assert ops.gemm_workspace_bytes(M, N, K, torch.bfloat16, torch.float32) > 0
+        problems.append((_dev(a_h, torch.bfloat16), _dev(b_h, torch.bfloat16), a_h @ b_h))
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[], []]
+    torch.cuda.synchronize()
+    for _ in range(20):
+        for i, (a, b, _) in enumerate(problems):
+            with torch.cuda.stream(streams[i]):
+                outs[i].append(ops.gemm(a, b, out_dtype=torch.float32))
+    torch.cuda.synchronize()
+    for i, (_, _, want) in enumerate(problems):
+        for o in outs[i]:
+            np.testing.assert_array_equal(_host(o), want)  # small integers: exact whatever the K cut
+    # growing a pool buffer mid-stream leaves the work already enqueued intact
+    ops.release_scratch()
+    a, b, want = problems[1]
+    small = ops.gemm(a, b, out_dtype=torch.float32)
+    a2, b2, want2 = problems[0]
+    big = ops.gemm(a2, b2, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(_host(small), want)
+    np.testing.assert_array_equal(_host(big), want2)
+    ops.release_scratch()

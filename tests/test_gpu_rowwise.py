@@ -102,6 +102,21 @@ def test_layer_norm_bf16_out_and_in():
     assert_close(_host(out), orc.layer_norm(xb, g, b, result_type="bf16"), 2e-2, "ln bf16->bf16")
 
 
+def test_layer_norm_f16_out():
+    """f32 rows to f16: the LayerNorm + cast_f16 pair of the reference's block
+    (examples/xegpu/nanoGPT_payload.py:305-306)."""
+    from lighthouse_amd import ops
+
+    rng = np.random.default_rng(2)
+    for M, N in ((256, 256), (100, 768), (33, 1000)):
+        x = rng.standard_normal((M, N)).astype(np.float32)
+        g = rng.uniform(0.5, 1.5, N).astype(np.float32)
+        b = rng.uniform(-0.1, 0.1, N).astype(np.float32)
+        out = ops.layer_norm(_dev(x), _dev(g), _dev(b), out_dtype=torch.float16)
+        assert out.dtype == torch.float16
+        assert_close(_host(out), orc.layer_norm(x, g, b, result_type="f16"), 2e-3, f"ln f32->f16 {M}x{N}")
+
+
 def test_layer_norm_special_cases():
     from lighthouse_amd import ops
 

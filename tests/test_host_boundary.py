@@ -216,7 +216,7 @@ def test_c_abi_argument_validation_without_gpu():
     assert lib.lh_hip_attention(p, p, p, p, 1, 1, 100, 64, z, z, z, z, 1.0, 0, _lib.BF16, None) == _lib.LH_ERR_INVALID  # row stride 0
     assert lib.lh_hip_attention(p, p, p, p, 0, 1, 100, 64, z, z, z, z, 1.0, 0, _lib.BF16, None) == _lib.LH_ERR_INVALID
     assert lib.lh_hip_layer_norm(p, p, p, p, 0, 8, 1e-5, _lib.F32, _lib.F32, None) == _lib.LH_ERR_INVALID
-    assert lib.lh_hip_nanogpt_block(p, p, None, 1, 1, 8, 2, 1e-5, _lib.F32, p, 0, None) == _lib.LH_ERR_INVALID
+    assert lib.lh_hip_nanogpt_block(p, p, None, 1, 1, 8, 2, 1e-5, _lib.F32, None, p, 0, None) == _lib.LH_ERR_INVALID
     with pytest.raises(ValueError):
         _lib.check(_lib.LH_ERR_INVALID, "x")
     with pytest.raises(RuntimeError):

@@ -70,6 +70,47 @@ def test_zero_fill_means_no_accumulation():
     assert fn.attrs.flags == 0 and fn.arg_order == [2, 0, 1]
 
 
+MEMREF = """
+module {
+  func.func @mm(%a: memref<8x24xf32>, %b: memref<24x16xf32>, %bias: memref<16xf32>, %c: memref<8x16xf32>) {
+    %zero = arith.constant 0.000000e+00 : f32
+    linalg.fill ins(%zero : f32) outs(%c : memref<8x16xf32>)
+    linalg.matmul ins(%a, %b : memref<8x24xf32>, memref<24x16xf32>) outs(%c : memref<8x16xf32>)
+    %bc = memref.alloc() : memref<8x16xf32>
+    linalg.broadcast ins(%bias : memref<16xf32>) outs(%bc : memref<8x16xf32>) dimensions = [0]
+    linalg.add ins(%c, %bc : memref<8x16xf32>, memref<8x16xf32>) outs(%c : memref<8x16xf32>)
+    %zeros = memref.alloc() : memref<8x16xf32>
+    linalg.fill ins(%zero : f32) outs(%zeros : memref<8x16xf32>)
+    linalg.max ins(%c, %zeros : memref<8x16xf32>, memref<8x16xf32>) outs(%c : memref<8x16xf32>)
+    return
+  }
+}
+"""
+
+
+def test_bufferised_form_follows_program_order():
+    """Operations on memrefs have no results: a zero fill of the output buffer BEFORE the matmul
+    means the product does not accumulate into what the caller passed; without the fill, or with
+    the fill after the matmul's read, it does."""
+    fn = parse_payload_module(MEMREF).lookup("mm")
+    assert fn.arg_order == [3, 0, 1, 2]
+    assert fn.attrs.flags == _lib.GEMM_HAS_BIAS | _lib.GEMM_HAS_RELU
+    no_fill = MEMREF.replace("    linalg.fill ins(%zero : f32) outs(%c : memref<8x16xf32>)\n", "")
+    assert parse_payload_module(no_fill).lookup("mm").attrs.flags == (
+        _lib.GEMM_HAS_BIAS | _lib.GEMM_HAS_RELU | _lib.GEMM_ACCUMULATE_C)
+    plain = """
+    func.func @mm(%a: memref<8x24xf32>, %b: memref<24x16xf32>, %c: memref<8x16xf32>) {
+      %zero = arith.constant 0.0 : f32
+      linalg.fill ins(%zero : f32) outs(%c : memref<8x16xf32>)
+      linalg.matmul ins(%a, %b : memref<8x24xf32>, memref<24x16xf32>) outs(%c : memref<8x16xf32>)
+      return
+    }"""
+    assert parse_payload_module(plain).lookup("mm").attrs.flags == 0
+    one = plain.replace("arith.constant 0.0", "arith.constant 1.0")
+    with pytest.raises(ValueError, match="non-zero fill"):
+        parse_payload_module(one)
+
+
 def test_generic_chain_with_bias_and_relu():
     fn = parse_payload_module(GENERIC, ["layer"]).lookup("layer")
     assert fn.arg_order == [3, 0, 1, 2]

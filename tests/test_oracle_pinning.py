@@ -346,19 +346,184 @@ def test_nanogpt_block_against_torch_module():
     p = _block_params(C, rng)
     x = rng.standard_normal((B, T, C)).astype(np.float32)
     blk = _TorchBlock(C, H).double()
+    _load_block(blk, p)
     with torch.no_grad():
-        t = lambda a: torch.from_numpy(a).double()
+        ref = blk(torch.from_numpy(x).double()).numpy()
+    np.testing.assert_allclose(orc.nanogpt_block(x, p, H, mode="f32"), ref, rtol=2e-5, atol=2e-5)
+    bf = orc.nanogpt_block(x, p, H, mode="bf16")
+    assert np.abs(bf - ref).max() <= 2e-2 * np.abs(ref).max()
+    assert np.abs(bf - ref).max() > 0  # the bf16 rounding points are really applied
+
+
+def _load_block(blk, p):
+    t = lambda a: torch.from_numpy(np.asarray(a)).double()
+    with torch.no_grad():
         blk.ln_1.weight.copy_(t(p["ln1_g"])); blk.ln_1.bias.copy_(t(p["ln1_b"]))
         blk.c_attn.weight.copy_(t(p["w_qkv"]).T); blk.c_attn.bias.copy_(t(p["b_qkv"]))
         blk.c_proj.weight.copy_(t(p["w_o"]).T); blk.c_proj.bias.copy_(t(p["b_o"]))
         blk.ln_2.weight.copy_(t(p["ln2_g"])); blk.ln_2.bias.copy_(t(p["ln2_b"]))
         blk.c_fc.weight.copy_(t(p["w_fc"]).T); blk.c_fc.bias.copy_(t(p["b_fc"]))
         blk.mlp_proj.weight.copy_(t(p["w_proj"]).T); blk.mlp_proj.bias.copy_(t(p["b_proj"]))
+
+
+def test_nanogpt_forward_against_torch_stack():
+    """n blocks, final LayerNorm, lm_head with bias (examples/xegpu/nanoGPT_payload.py:399-407) against an
+    independent float64 torch stack.  The final gamma / beta and the lm_head bias are non-trivial, the
+    vocabulary is ragged, and a variant of the torch model with one piece left out must NOT match, so a
+    skipped LayerNorm, bias or layer in the oracle cannot pass."""
+    rng = np.random.default_rng(29)
+    B, T, C, H, V, L = 2, 20, 32, 4, 45, 3
+    layers = [_block_params(C, rng) for _ in range(L)]
+    lnf_g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    lnf_b = rng.uniform(-0.3, 0.3, C).astype(np.float32)
+    lm_w = (rng.standard_normal((C, V)) * 0.1).astype(np.float32)
+    lm_b = rng.uniform(-0.5, 0.5, V).astype(np.float32)
+    x = rng.standard_normal((B, T, C)).astype(np.float32)
+
+    blocks = [_TorchBlock(C, H).double() for _ in range(L)]
+    for blk, p in zip(blocks, layers):
+        _load_block(blk, p)
+    ln_f = torch.nn.LayerNorm(C, eps=1e-5).double()
+    head = torch.nn.Linear(C, V).double()
+    with torch.no_grad():
+        ln_f.weight.copy_(torch.from_numpy(lnf_g).double()); ln_f.bias.copy_(torch.from_numpy(lnf_b).double())
+        head.weight.copy_(torch.from_numpy(lm_w).double().T); head.bias.copy_(torch.from_numpy(lm_b).double())
+
+        def run(skip_ln=False, skip_bias=False, n=L):
+            h = torch.from_numpy(x).double()
+            for blk in blocks[:n]:
+                h = blk(h)
+            if not skip_ln:
+                h = ln_f(h)
+            out = h @ head.weight.T
+            return (out if skip_bias else out + head.bias).numpy()
+
+        ref = run()
+        wrong = [run(skip_ln=True), run(skip_bias=True), run(n=L - 1)]
+    got = orc.nanogpt_forward(x, layers, lnf_g, lnf_b, lm_w, lm_b, H, mode="f32")
+    assert got.shape == (B, T, V)
+    np.testing.assert_allclose(got, ref, rtol=2e-5, atol=2e-5)
+    for w in wrong:
+        assert np.abs(got - w).max() > 1e-2
+    no_bias = orc.nanogpt_forward(x, layers, lnf_g, lnf_b, lm_w, None, H, mode="f32")
+    np.testing.assert_allclose(no_bias, wrong[1], rtol=2e-5, atol=2e-5)
+    bf = orc.nanogpt_forward(x, layers, lnf_g, lnf_b, lm_w, lm_b, H, mode="bf16")
+    err = np.abs(bf - ref).max()
+    assert 0 < err <= 2e-2 * np.abs(ref).max()
+
+
+class _TorchRefBlock(torch.nn.Module):
+    """Independent statement of the reference's own block (examples/xegpu/nanoGPT_payload.py:299-317):
+    separate bias-free q/k/v projections, non-causal attention, ReLU MLP."""
+
+    def __init__(self, C, H, hidden, causal=False):
+        super().__init__()
+        self.H, self.causal = H, causal
+        self.ln_1 = torch.nn.LayerNorm(C, eps=1e-5)
+        self.q = torch.nn.Linear(C, C, bias=False)
+        self.k = torch.nn.Linear(C, C, bias=False)
+        self.v = torch.nn.Linear(C, C, bias=False)
+        self.proj = torch.nn.Linear(C, C)
+        self.ln_2 = torch.nn.LayerNorm(C, eps=1e-5)
+        self.fc1 = torch.nn.Linear(C, hidden)
+        self.fc2 = torch.nn.Linear(hidden, C)
+
+    def forward(self, x):  # x: [T, C]
+        T, C = x.shape
+        h = self.ln_1(x)
+        q, k, v = (m(h).view(T, self.H, C // self.H).transpose(0, 1) for m in (self.q, self.k, self.v))
+        y = F.scaled_dot_product_attention(q, k, v, is_causal=self.causal).transpose(0, 1).reshape(T, C)
+        x = x + self.proj(y)
+        return x + self.fc2(F.relu(self.fc1(self.ln_2(x))))
+
+
+def _ref_block_weights(C, hidden, rng, sc=0.05):
+    """Weights shaped and typed as the reference's driver makes them (examples/xegpu/nanoGPT.py:243-258),
+    with non-trivial LayerNorm parameters and biases so that a dropped one shows."""
+    f16 = lambda a: a.astype(np.float16)
+    return dict(
+        g1=rng.uniform(0.5, 1.5, C).astype(np.float32), b1n=rng.uniform(-0.1, 0.1, C).astype(np.float32),
+        wq=f16(rng.standard_normal((C, C)) * sc), wk=f16(rng.standard_normal((C, C)) * sc),
+        wv=f16(rng.standard_normal((C, C)) * sc), wp=f16(rng.standard_normal((C, C)) * sc),
+        bp=(rng.standard_normal(C) * sc).astype(np.float32),
+        g2=rng.uniform(0.5, 1.5, C).astype(np.float32), b2n=rng.uniform(-0.1, 0.1, C).astype(np.float32),
+        w1=f16(rng.standard_normal((C, hidden)) * sc), bb1=(rng.standard_normal(hidden) * sc).astype(np.float32),
+        w2=f16(rng.standard_normal((hidden, C)) * sc), bb2=(rng.standard_normal(C) * sc).astype(np.float32),
+    )
+
+
+def _load_ref_block(blk, w):
+    t = lambda a: torch.from_numpy(np.asarray(a, dtype=np.float32)).double()
+    with torch.no_grad():
+        blk.ln_1.weight.copy_(t(w["g1"])); blk.ln_1.bias.copy_(t(w["b1n"]))
+        blk.q.weight.copy_(t(w["wq"]).T); blk.k.weight.copy_(t(w["wk"]).T); blk.v.weight.copy_(t(w["wv"]).T)
+        blk.proj.weight.copy_(t(w["wp"]).T); blk.proj.bias.copy_(t(w["bp"]))
+        blk.ln_2.weight.copy_(t(w["g2"])); blk.ln_2.bias.copy_(t(w["b2n"]))
+        blk.fc1.weight.copy_(t(w["w1"]).T); blk.fc1.bias.copy_(t(w["bb1"]))
+        blk.fc2.weight.copy_(t(w["w2"]).T); blk.fc2.bias.copy_(t(w["bb2"]))
+
+
+def _ref_to_block_params(w):
+    """The reference's weight names -> the parameter names of orc.nanogpt_block (separate projections)."""
+    return dict(ln1_g=w["g1"], ln1_b=w["b1n"], w_q=w["wq"], w_k=w["wk"], w_v=w["wv"], w_o=w["wp"], b_o=w["bp"],
+                ln2_g=w["g2"], ln2_b=w["b2n"], w_fc=w["w1"], b_fc=w["bb1"], w_proj=w["w2"], b_proj=w["bb2"])
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_reference_block_checker_against_torch_module(causal):
+    """orc.ref_block_fused (the reference's numpy checker restated, f16 rounding points) and
+    orc.nanogpt_block in the reference's configuration (the kernels' rounding points) against the
+    float64 torch module: both within f16 rounding of it, neither equal to it, and within the
+    reference's own pass criterion max|diff| / max|ref| < 5e-2 (examples/xegpu/nanoGPT.py:298-302)
+    of each other by a wide margin."""
+    rng = np.random.default_rng(31)
+    T, C, hidden, H = 48, 64, 256, 4
+    w = _ref_block_weights(C, hidden, rng)
+    x = (rng.standard_normal((T, C)) * 0.5).astype(np.float32)
+    blk = _TorchRefBlock(C, H, hidden, causal).double()
+    _load_ref_block(blk, w)
+    with torch.no_grad():
         ref = blk(torch.from_numpy(x).double()).numpy()
-    np.testing.assert_allclose(orc.nanogpt_block(x, p, H, mode="f32"), ref, rtol=2e-5, atol=2e-5)
-    bf = orc.nanogpt_block(x, p, H, mode="bf16")
-    assert np.abs(bf - ref).max() <= 2e-2 * np.abs(ref).max()
-    assert np.abs(bf - ref).max() > 0  # the bf16 rounding points are really applied
+    got = orc.ref_block_fused(x, w, H, causal=causal)
+    scale = np.abs(ref).max()
+    assert 0 < np.abs(got - ref).max() <= 4e-3 * scale
+    # f32 "rounding": the restatement is the torch module to float32 accuracy
+    np.testing.assert_allclose(orc.ref_block_fused(x, w, H, causal=causal, elt="f32"), ref, rtol=2e-5, atol=2e-5)
+    mine = orc.nanogpt_block(x[None], _ref_to_block_params(w), H, mode="f16", causal=causal, activation="relu",
+                             bias_f32=True)[0]
+    assert 0 < np.abs(mine - ref).max() <= 4e-3 * scale
+    assert np.abs(mine - got).max() <= 4e-3 * scale
+    exact = orc.nanogpt_block(x[None], _ref_to_block_params(w), H, mode="f32", causal=causal, activation="relu",
+                              bias_f32=True)[0]
+    np.testing.assert_allclose(exact, ref, rtol=2e-5, atol=2e-5)
+
+
+def test_reference_gpt_checker_against_torch_stack():
+    """orc.ref_gpt_fused (examples/xegpu/nanoGPT.py:128-135) and orc.nanogpt_forward in the reference's
+    configuration against two float64 torch blocks + LayerNorm + Linear."""
+    rng = np.random.default_rng(37)
+    T, C, hidden, H, V, L = 32, 64, 128, 4, 40, 2
+    ws = [_ref_block_weights(C, hidden, rng) for _ in range(L)]
+    gf_g = rng.uniform(0.5, 1.5, C).astype(np.float32)
+    gf_b = rng.uniform(-0.3, 0.3, C).astype(np.float32)
+    lmw = (rng.standard_normal((C, V)) * 0.05).astype(np.float16)
+    lmb = rng.uniform(-0.5, 0.5, V).astype(np.float32)
+    x = (rng.standard_normal((T, C)) * 0.5).astype(np.float32)
+    with torch.no_grad():
+        h = torch.from_numpy(x).double()
+        for w in ws:
+            blk = _TorchRefBlock(C, H, hidden).double()
+            _load_ref_block(blk, w)
+            h = blk(h)
+        h = F.layer_norm(h, (C,), torch.from_numpy(gf_g).double(), torch.from_numpy(gf_b).double(), 1e-5)
+        ref = (h @ torch.from_numpy(lmw.astype(np.float32)).double() + torch.from_numpy(lmb).double()).numpy()
+    scale = np.abs(ref).max()
+    got = orc.ref_gpt_fused(x, ws, gf_g, gf_b, lmw, lmb, H)
+    assert 0 < np.abs(got - ref).max() <= 4e-3 * scale
+    np.testing.assert_allclose(orc.ref_gpt_fused(x, ws, gf_g, gf_b, lmw, lmb, H, elt="f32"), ref, rtol=2e-5, atol=2e-5)
+    mine = orc.nanogpt_forward(x[None], [_ref_to_block_params(w) for w in ws], gf_g, gf_b, lmw, lmb, H, mode="f16",
+                               causal=False, activation="relu", bias_f32=True)[0]
+    assert 0 < np.abs(mine - ref).max() <= 4e-3 * scale
 
 
 def test_complexity_formulas():
