@@ -147,6 +147,23 @@ int lh_hip_gemm_ws(void* out, const void* a, const void* b, const void* bias, in
                    void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * lh_hip_gemm for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments, kernels and results as lh_hip_gemm; the temporary memory of the problems that need
+ * any (f32 blocks of decode shapes cut along K, copies of transposed or unaligned operands) is a
+ * device array of LH_STATIC_SCRATCH_BYTES that is part of the library's device image, so the call
+ * performs no hipMalloc / hipFree and uses no allocating library routine.  A problem whose
+ * temporaries exceed that size is refused with LH_ERR_INVALID before anything is launched.
+ * Nothing in the array needs clearing between calls (every kernel writes what it later reads).
+ * All calls on one GPU share the array: calls that overlap in time on one GPU (different streams
+ * or threads) race; calls on one stream are safe.
+ */
+#define LH_STATIC_SCRATCH_BYTES (16u << 20)
+int lh_hip_gemm_static(void* out, const void* a, const void* b, const void* bias, int64_t M, int64_t N, int64_t K,
+                       int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype, int32_t out_dtype, uint32_t flags,
+                       void* stream);
+
+/*
  * lh_hip_gemm whose accumulation starts from a separate matrix: out = epilogue(c + A.B), with
  * `c` [M,N] of out_dtype and row stride ldc (ACCUMULATE_C is implied; c may be `out`, which is
  * lh_hip_gemm with the flag).  This is emit_mlp_layer's `acc_tensor` argument in its general

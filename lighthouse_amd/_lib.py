@@ -122,6 +122,7 @@ PROTOTYPES = {
     "lh_hip_gemm": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp]),
     "lh_hip_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32]),
     "lh_hip_gemm_ws": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp, _sz, _vp]),
+    "lh_hip_gemm_static": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp]),
     "lh_hip_gemm_residual": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp]),
     "lh_hip_gemm_fp8": (_i32, [_vp, _vp, _vp, _f32, _f32, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _vp]),
     "lh_hip_gemm_fp8_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64, _i32]),

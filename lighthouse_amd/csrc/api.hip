@@ -155,6 +155,24 @@ int lh_hip_gemm_ws(void* out, const void* a, const void* b, const void* bias, in
                   reinterpret_cast<hipStream_t>(stream), &ws);
 }
 
+int lh_hip_gemm_static(void* out, const void* a, const void* b, const void* bias, int64_t M, int64_t N, int64_t K,
+                       int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype, int32_t out_dtype, uint32_t flags,
+                       void* stream) {
+  int rc = gemm_common_checks("lh_hip_gemm_static", out, a, b, bias, M, N, K, lda, ldb, ldc, flags);
+  if (rc) return rc;
+  if ((rc = gemm_dtype_checks("lh_hip_gemm_static", ab_dtype, out_dtype))) return rc;
+  // What the dispatch would take for aligned operands, known before anything is launched.
+  const size_t need = gemm_need(M, N, K, lda, ldb, ldc, ab_dtype, out_dtype, out_dtype, flags);
+  LH_REQUIRE(need <= LH_STATIC_SCRATCH_BYTES,
+             "lh_hip_gemm_static: this problem needs %zu bytes of temporary memory, the static scratch holds %zu "
+             "(use lh_hip_gemm_ws with a workspace of that size)",
+             need, (size_t)LH_STATIC_SCRATCH_BYTES);
+  Scratch ws;
+  if ((rc = static_scratch(&ws.base, &ws.bytes))) return rc;
+  return gemm_run(out, out, a, b, bias, M, N, K, lda, ldb, ldc, ab_dtype, out_dtype, out_dtype, flags,
+                  reinterpret_cast<hipStream_t>(stream), &ws);
+}
+
 int lh_hip_gemm_residual(void* out, const void* c, const void* a, const void* b, const void* bias, int64_t M, int64_t N,
                          int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype, int32_t out_dtype,
                          uint32_t flags, void* stream) {

@@ -195,6 +195,8 @@ struct PlanningScope {  // marks the calling thread as running a size query
   do {                                                        \
     if (!::lh::planning()) hipLaunchKernelGGL(__VA_ARGS__);   \
   } while (0)
+// The current device's statically allocated scratch array (runtime.hip): its device address and size.
+int static_scratch(char** base, size_t* bytes);
 // Compute units of the current device (cached; 256 if the query fails).
 int num_cus();
 

@@ -199,6 +199,33 @@ int scratch_take(Scratch* ws, hipStream_t s, int slot, size_t bytes, const char*
   return LH_OK;
 }
 
+// ---- statically allocated scratch ------------------------------------------------------------
+// Temporary memory for the one entry point that must not allocate (lh_hip_gemm_static): an array
+// in the library's device image, so every GPU the library runs on holds its own copy from the
+// moment the code object is loaded until the process ends.  In host code the array's name is only
+// a handle for the runtime; the address kernels may use comes from hipGetSymbolAddress, asked once
+// per device with that device current, and kept.
+static __device__ __align__(256) unsigned char scratch[LH_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+static std::mutex g_static_mutex;
+static char* g_static_ptr[kMaxDevices] = {};
+
+int static_scratch(char** base, size_t* bytes) {
+  int dev = 0;
+  LH_HIP_CHECK(hipGetDevice(&dev));
+  LH_REQUIRE(dev >= 0 && dev < kMaxDevices, "static scratch: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_static_mutex);
+  if (g_static_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    LH_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    LH_REQUIRE(p != nullptr && (reinterpret_cast<uintptr_t>(p) & 255u) == 0, "static scratch: bad device address %p", p);
+    g_static_ptr[dev] = static_cast<char*>(p);
+  }
+  *base = g_static_ptr[dev];
+  *bytes = LH_STATIC_SCRATCH_BYTES;
+  return LH_OK;
+}
+
 static int release_pool_of_current_device() {
   int dev = 0;
   LH_HIP_CHECK(hipGetDevice(&dev));

@@ -1,0 +1,91 @@
+"""lh_hip_gemm_static: the GEMM entry point that allocates nothing (temporaries in a device array
+that is part of the library's image), called through the C ABI and compared bit for bit with
+lh_hip_gemm on the same inputs: a decode shape that is cut along K, then a smaller one (the array
+keeps the first call's contents), then problems with padded and transposed operands, then one whose
+temporaries exceed the array."""
+
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from lighthouse_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+STATIC_BYTES = 16 << 20
+
+
+def _call(fn, out, a, b, bias, M, N, K, flags, stream=None):
+    return fn(out.data_ptr(), a.data_ptr(), b.data_ptr(), bias.data_ptr() if bias is not None else None, M, N, K,
+              a.stride(0), b.stride(0), out.stride(0), _lib.BF16, _lib.F32 if out.dtype == torch.float32 else _lib.BF16,
+              flags, stream)
+
+
+def _problem(M, N, K, seed, transpose_b=False):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    a = torch.randn(M, K, device="cuda", generator=g).to(torch.bfloat16)
+    b = torch.randn((N, K) if transpose_b else (K, N), device="cuda", generator=g).to(torch.bfloat16)
+    bias = torch.randn(N, device="cuda", generator=g).to(torch.bfloat16)
+    return a, b, bias
+
+
+def test_static_scratch_gemm_matches_the_pooled_entry_point():
+    lib = _lib.load()
+    flags = _lib.GEMM_HAS_BIAS | _lib.GEMM_HAS_RELU
+    # (M, N, K, extra flags): cut along K (4 MiB of partial sums); smaller, cut along K; ragged N and K
+    # (padded copies); transposed B (untransposed copy); no temporaries at all
+    cases = [(16, 8192, 8192, 0), (16, 1024, 4096, 0), (300, 520, 776, 0), (512, 512, 512, _lib.GEMM_TRANSPOSE_B),
+             (512, 512, 512, 0)]
+    # The array itself becomes resident on the device when the runtime is first asked for its
+    # address; one call up front keeps that out of the memory readings below.
+    a, b, bias = _problem(256, 256, 256, 99)
+    first = torch.empty(256, 256, device="cuda", dtype=torch.bfloat16)
+    _lib.check(_call(lib.lh_hip_gemm_static, first, a, b, bias, 256, 256, 256, flags), "lh_hip_gemm_static")
+    torch.cuda.synchronize()
+    for i, (M, N, K, extra) in enumerate(cases):
+        tb = bool(extra & _lib.GEMM_TRANSPOSE_B)
+        a, b, bias = _problem(M, N, K, 100 + i, tb)
+        need = lib.lh_hip_gemm_workspace_bytes(M, N, K, a.stride(0), b.stride(0), N, _lib.BF16, _lib.BF16, flags | extra)
+        assert need <= STATIC_BYTES and (need > 0) == (i < 4)
+        want = torch.full((M, N), 3.0, device="cuda", dtype=torch.bfloat16)
+        got = torch.full((M, N), 5.0, device="cuda", dtype=torch.bfloat16)
+        _lib.check(_call(lib.lh_hip_gemm, want, a, b, bias, M, N, K, flags | extra), "lh_hip_gemm")
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        _lib.check(_call(lib.lh_hip_gemm_static, got, a, b, bias, M, N, K, flags | extra), "lh_hip_gemm_static")
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] >= free_before  # the call took no device memory
+        assert torch.equal(got, want), (M, N, K)
+        ref = torch.relu(a.float() @ (b.float().T if tb else b.float()) + bias.float())
+        assert (got.float() - ref).abs().max() <= 2e-2 * ref.abs().max()
+    # the two decode shapes again in the opposite order, back to back on one stream without a
+    # synchronisation in between: the second call's kernels run after the first call's
+    (a1, b1, bias1), (a2, b2, bias2) = _problem(16, 1024, 4096, 101), _problem(16, 8192, 8192, 100)
+    o1 = torch.empty(16, 1024, device="cuda", dtype=torch.bfloat16)
+    o2 = torch.empty(16, 8192, device="cuda", dtype=torch.bfloat16)
+    w1, w2 = torch.empty_like(o1), torch.empty_like(o2)
+    _lib.check(_call(lib.lh_hip_gemm_static, o1, a1, b1, bias1, 16, 1024, 4096, flags), "static")
+    _lib.check(_call(lib.lh_hip_gemm_static, o2, a2, b2, bias2, 16, 8192, 8192, flags), "static")
+    _lib.check(_call(lib.lh_hip_gemm, w1, a1, b1, bias1, 16, 1024, 4096, flags), "pooled")
+    _lib.check(_call(lib.lh_hip_gemm, w2, a2, b2, bias2, 16, 8192, 8192, flags), "pooled")
+    torch.cuda.synchronize()
+    assert torch.equal(o1, w1) and torch.equal(o2, w2)
+
+
+def test_static_scratch_gemm_refuses_what_does_not_fit():
+    lib = _lib.load()
+    M, N, K = 128, 8192, 8192  # eight f32 blocks of 128 x 8192: 32 MiB
+    assert lib.lh_hip_gemm_workspace_bytes(M, N, K, K, N, N, _lib.BF16, _lib.BF16, 0) > STATIC_BYTES
+    a, b, _ = _problem(M, N, K, 7)
+    out = torch.full((M, N), 9.0, device="cuda", dtype=torch.bfloat16)
+    rc = _call(lib.lh_hip_gemm_static, out, a, b, None, M, N, K, 0)
+    assert rc == _lib.LH_ERR_INVALID
+    assert b"static scratch holds" in lib.lh_hip_last_error()
+    torch.cuda.synchronize()
+    assert bool((out == 9.0).all())  # nothing ran
+    with pytest.raises(ValueError):
+        _lib.check(rc, "lh_hip_gemm_static")
+    # argument validation is the plain entry point's
+    assert _call(lib.lh_hip_gemm_static, out, a, b, None, 0, N, K, 0) == _lib.LH_ERR_INVALID
