@@ -83,6 +83,19 @@ typedef enum lh_dtype {
 #define LH_GEMM_TILE_256x128 0x200u
 #define LH_GEMM_TILE_128x256 0x300u
 #define LH_GEMM_TILE_128x128 0x400u
+/* Cut along K for the 16-bit GEMM ("split K": `splits` workgroup sets each take K / splits columns
+ * of A and rows of B and write an f32 block; a second kernel adds the blocks and runs the
+ * epilogue), for problems with too few tiles to fill the CUs; the k-dimension counterpart of the
+ * tile request above (lighthouse/schedule/xegpu/matmul_params.json holds such per-shape choices).
+ * AUTO lets the library decide; NONE forbids the cut; 2 / 4 / 8 request it and need untransposed
+ * aligned operands and K / splits a multiple of 64 (runs on 128 x 128 tiles, so it excludes a tile
+ * request). */
+#define LH_GEMM_SPLITK_MASK 0x3800u
+#define LH_GEMM_SPLITK_AUTO 0x0000u
+#define LH_GEMM_SPLITK_NONE 0x0800u
+#define LH_GEMM_SPLITK_2 0x1000u
+#define LH_GEMM_SPLITK_4 0x1800u
+#define LH_GEMM_SPLITK_8 0x2000u
 
 /* ---------------------------------------------------------------- runtime ---- */
 
@@ -201,6 +214,20 @@ int lh_hip_gemm_fp8_ws(void* out, const void* a_q, const void* b_q, float scale_
  * dtype in {BF16, F16, F32}; d <= 256.  The matrix-core kernels take d = 64 with 16-byte aligned
  * rows at any T; every other problem runs on a generic kernel.
  */
+/* `causal` is a word of flags: bit 0 selects the causal mask; the other bits request a kernel
+ * variant for 16-bit tensors with head dimension 64, the counterpart of the wg_rows / sg_rows
+ * parameters of the reference's fused-attention schedule (examples/xegpu/fused_attention.py:109-145,
+ * lighthouse/schedule/xegpu/fused_attention_schedule.py): query rows per wave (64: two 32-row
+ * sub-tiles share every K/V fragment, 256-row workgroups; 32: 128-row workgroups, twice as many)
+ * and, for the 32-row kernel, the depth of the K/V ring (3 stages: three workgroups per CU; 4: two).
+ * 0 lets the library choose by shape.  A request that does not apply fails with LH_ERR_INVALID. */
+#define LH_ATTN_CAUSAL 0x1
+#define LH_ATTN_ROWS_MASK 0x300
+#define LH_ATTN_ROWS_32 0x100
+#define LH_ATTN_ROWS_64 0x200
+#define LH_ATTN_STAGES_MASK 0xC00
+#define LH_ATTN_STAGES_3 0x400
+#define LH_ATTN_STAGES_4 0x800
 typedef struct lh_strides3 {
   int64_t z, h, t;
 } lh_strides3;
@@ -343,7 +370,7 @@ int lh_hip_payload_matmul_fp8(void** args, int32_t nargs, const lh_matmul_fp8_at
 
 typedef struct lh_attention_attrs {
   int32_t dtype;
-  int32_t causal;
+  int32_t causal; /* LH_ATTN_CAUSAL | variant request bits, as for lh_hip_attention */
   float scale; /* <= 0 selects 1/sqrt(d) */
 } lh_attention_attrs;
 /* args: out, Q, K, V, each rank-4 [Z,H,T,d] */

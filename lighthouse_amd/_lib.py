@@ -25,6 +25,14 @@ GEMM_TRANSPOSE_B = 16
 GEMM_HAS_GELU = 32
 GEMM_TILE_AUTO = 0
 GEMM_TILES = {(256, 256): 0x100, (256, 128): 0x200, (128, 256): 0x300, (128, 128): 0x400}
+GEMM_TILE_MASK = 0x700
+# LH_GEMM_SPLITK_*: 0 = the library decides, 1 = never cut, 2 / 4 / 8 = cut K that many times
+GEMM_SPLITK = {0: 0x0000, 1: 0x0800, 2: 0x1000, 4: 0x1800, 8: 0x2000}
+GEMM_SPLITK_MASK = 0x3800
+# LH_ATTN_*: bit 0 causal; query rows per wave and K/V ring depth requests (0 = the library decides)
+ATTN_CAUSAL = 1
+ATTN_ROWS = {0: 0, 32: 0x100, 64: 0x200}
+ATTN_STAGES = {0: 0, 3: 0x400, 4: 0x800}
 
 # lh_elementwise_kind
 EW_SOFTMAX, EW_GELU, EW_BIAS, EW_ADD, EW_CAST = range(5)

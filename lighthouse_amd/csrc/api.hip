@@ -21,10 +21,14 @@ static int gemm_common_checks(const char* who, const void* out, const void* a, c
   LH_REQUIRE(!(flags & LH_GEMM_HAS_BIAS) || bias != nullptr, "%s: HAS_BIAS set but bias is null", who);
   LH_REQUIRE(!((flags & LH_GEMM_HAS_RELU) && (flags & LH_GEMM_HAS_GELU)), "%s: RELU and GELU are exclusive", who);
   const uint32_t known = LH_GEMM_HAS_BIAS | LH_GEMM_HAS_RELU | LH_GEMM_ACCUMULATE_C | LH_GEMM_TRANSPOSE_A |
-                         LH_GEMM_TRANSPOSE_B | LH_GEMM_HAS_GELU | LH_GEMM_TILE_MASK;
+                         LH_GEMM_TRANSPOSE_B | LH_GEMM_HAS_GELU | LH_GEMM_TILE_MASK | LH_GEMM_SPLITK_MASK;
   LH_REQUIRE((flags & ~known) == 0, "%s: unknown flag bits 0x%x", who, flags & ~known);
   LH_REQUIRE((flags & LH_GEMM_TILE_MASK) <= LH_GEMM_TILE_128x128, "%s: unknown tile request 0x%x", who,
              flags & LH_GEMM_TILE_MASK);
+  LH_REQUIRE((flags & LH_GEMM_SPLITK_MASK) <= LH_GEMM_SPLITK_8, "%s: unknown split-K request 0x%x", who,
+             flags & LH_GEMM_SPLITK_MASK);
+  LH_REQUIRE((flags & LH_GEMM_SPLITK_MASK) <= LH_GEMM_SPLITK_NONE || (flags & LH_GEMM_TILE_MASK) == LH_GEMM_TILE_AUTO,
+             "%s: a split-K request runs on 128 x 128 tiles and excludes a tile request", who);
   return LH_OK;
 }
 
@@ -40,7 +44,8 @@ int gemm_run(void* out, const void* c, const void* a, const void* b, const void*
   g.ws = ws;
   if (ws) ws->used = 0;  // temporaries of an earlier call on the stream are dead once this one runs
   if (ab_dtype == LH_F32) {
-    LH_REQUIRE((flags & LH_GEMM_TILE_MASK) == LH_GEMM_TILE_AUTO, "gemm: tile requests apply to 16-bit inputs only");
+    LH_REQUIRE((flags & (LH_GEMM_TILE_MASK | LH_GEMM_SPLITK_MASK)) == 0,
+               "gemm: tile and split-K requests apply to 16-bit inputs only");
     return gemm32(g, s);
   }
   return gemm16(g, ab_dtype, s);

@@ -32,6 +32,7 @@ struct AttnArgs {
   float scale;
   int causal;
   int cus;  // compute units of the device (causal launch order)
+  int request = 0;  // LH_ATTN_ROWS_* | LH_ATTN_STAGES_* bits of the call (0: the library chooses)
 };
 
 template <int DT>
@@ -651,6 +652,19 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
   const bool short_rows = a.T <= 640 && a.T % kQBlock16 != 0;
   // (A partial last key tile also takes the 32-rows-per-wave kernels: the 64-row one has no
   // registers left for the clamped loads and would spill.)
+  const int rows_req = a.request & LH_ATTN_ROWS_MASK, stages_req = a.request & LH_ATTN_STAGES_MASK;
+  if (rows_req == LH_ATTN_ROWS_64) {
+    LH_REQUIRE(a.T % kKvTile == 0, "attention: 64 query rows per wave need a sequence length that is a multiple of %d",
+               kKvTile);
+    LH_REQUIRE(stages_req != LH_ATTN_STAGES_3, "attention: the 64-rows-per-wave kernel has a 4-stage ring only");
+    return attention16_launch_nq<DT, 2, 4>(a, s);
+  }
+  if (rows_req == LH_ATTN_ROWS_32 || stages_req) {
+    const int64_t groups32 = (int64_t)((a.T + 127) / 128) * a.Z * a.H;
+    const bool three = stages_req ? stages_req == LH_ATTN_STAGES_3 : groups32 > a.cus;
+    if (three) return attention16_launch_nq<DT, 1, 3>(a, s);
+    return attention16_launch_nq<DT, 1, 4>(a, s);
+  }
   if (groups64 < limit || short_rows || a.T % kKvTile != 0) {
     // With more than one 128-row workgroup per CU a ring of 3 stages (48 KiB) lets three of them
     // share a CU instead of two ([8,12,1024] causal 26.7 -> 25.3 us, [16,16,512] causal 24.2 ->
@@ -1215,7 +1229,14 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   a.so = so; a.sq = sq; a.sk = sk; a.sv = sv;
   a.scale = scale;
   a.scale_log2e = scale * 1.4426950408889634f;
-  a.causal = causal ? 1 : 0;
+  LH_REQUIRE((causal & ~(int32_t)(LH_ATTN_CAUSAL | LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK)) == 0 &&
+                 (causal & LH_ATTN_ROWS_MASK) != LH_ATTN_ROWS_MASK && (causal & LH_ATTN_STAGES_MASK) != LH_ATTN_STAGES_MASK,
+             "lh_hip_attention: unknown bits 0x%x in the causal / request word", causal);
+  a.causal = (causal & LH_ATTN_CAUSAL) ? 1 : 0;
+  a.request = causal & (LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK);
+  LH_REQUIRE(a.request == 0 || (fast && dtype != LH_F32),
+             "lh_hip_attention: query-row / ring-depth requests apply to 16-bit tensors with head_dim %d and aligned rows",
+             kHeadDim);
   a.cus = num_cus();
   if (!fast) {
     if (vec_ok) {  // 16-bit tensors with another head dimension the matrix-core kernel takes

@@ -837,19 +837,28 @@ __global__ void __launch_bounds__(256) gemm16_splitk_reduce(GemmArgs g, const fl
 
 // Decode shapes: so few 128 x 128 tiles that most CUs would idle, and a K long enough to cut.
 // Returns 1 when the problem does not qualify.
+// `request`: LH_GEMM_SPLITK_* bits of the call; an explicit 2 / 4 / 8 bypasses the criteria.
 template <int DT>
-static int gemm16_splitk(const GemmArgs& g, hipStream_t s) {
+static int gemm16_splitk(const GemmArgs& g, uint32_t request, hipStream_t s) {
   using Cfg = DirectCfg<2, 1>;
   const int cus = num_cus();
   const int64_t tiles = (int64_t)((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
-  if (tiles * 2 > cus || g.K < 2048) return 1;
-  // With more than a quarter of the CUs busy anyway, the second kernel costs more than cutting a
-  // K of 2048 saves (M = 512, N = 4096: 24.1 us cut, 19.7 us whole; at K = 3072 the two are level).
-  if (tiles * 4 > cus && g.K < 3072) return 1;
   int splits = 1;
-  while (splits < 8 && tiles * splits * 2 <= 2 * cus && (g.K / (splits * 2)) % kBK == 0 && g.K / (splits * 2) >= 512)
-    splits *= 2;
-  if (splits == 1) return 1;
+  if (request == LH_GEMM_SPLITK_NONE) return 1;
+  if (request != LH_GEMM_SPLITK_AUTO) {
+    splits = request == LH_GEMM_SPLITK_2 ? 2 : request == LH_GEMM_SPLITK_4 ? 4 : 8;
+    LH_REQUIRE(g.K % (splits * kBK) == 0 && g.K / splits >= 2 * kBK,
+               "gemm: a cut of K = %d into %d needs K / %d to be a multiple of %d and at least %d", g.K, splits, splits,
+               kBK, 2 * kBK);
+  } else {
+    if (tiles * 2 > cus || g.K < 2048) return 1;
+    // With more than a quarter of the CUs busy anyway, the second kernel costs more than cutting a
+    // K of 2048 saves (M = 512, N = 4096: 24.1 us cut, 19.7 us whole; at K = 3072 the two are level).
+    if (tiles * 4 > cus && g.K < 3072) return 1;
+    while (splits < 8 && tiles * splits * 2 <= 2 * cus && (g.K / (splits * 2)) % kBK == 0 && g.K / (splits * 2) >= 512)
+      splits *= 2;
+    if (splits == 1) return 1;
+  }
   void* taken = nullptr;
   if (int rc = scratch_take(g.ws, s, kScratchSplitK, (size_t)splits * g.M * g.N * sizeof(float), "gemm (split K)", &taken))
     return rc;
@@ -897,7 +906,9 @@ static int gemm16_dispatch(const GemmArgs& g_in, hipStream_t s) {
                       aligned16(g.a) && aligned16(g.b) && aligned16(g.out) &&
                       (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias));
   const uint32_t tile = g.flags & LH_GEMM_TILE_MASK;
-  if (tile == LH_GEMM_TILE_AUTO && !(vec_ok && !tb && g.ldc % 8 == 0 && g.N % 8 == 0) &&
+  const uint32_t splitk = g.flags & LH_GEMM_SPLITK_MASK;
+  const bool cut_requested = splitk > LH_GEMM_SPLITK_NONE;
+  if (tile == LH_GEMM_TILE_AUTO && !cut_requested && !(vec_ok && !tb && g.ldc % 8 == 0 && g.N % 8 == 0) &&
       (int64_t)g.M * g.N * g.K >= (1 << 22)) {
     // not a shape for the direct kernels as it stands: run it on padded copies of the operands
     const int rc = gemm_padded<2>(g, kBK, 8, s, [&](const GemmArgs& p) { return gemm16_dispatch<DT>(p, s); });
@@ -911,10 +922,14 @@ static int gemm16_dispatch(const GemmArgs& g_in, hipStream_t s) {
                "K %% 64 == 0 and 16-byte aligned rows (M=%d N=%d K=%d)",
                bm[v], bn[v], bm[v], bn[v], g.M, g.N, g.K);
   }
+  if (cut_requested)
+    LH_REQUIRE(vec_ok && !tb && g.ldc % 8 == 0 && g.N % 8 == 0,
+               "gemm: a split-K request needs untransposed operands, K %% 64 == 0, N %% 8 == 0 and 16-byte aligned rows "
+               "(M=%d N=%d K=%d)", g.M, g.N, g.K);
   if (vec_ok) {
     if (!tb && g.ldc % 8 == 0 && g.N % 8 == 0) {
       if (tile == LH_GEMM_TILE_AUTO) {
-        const int rc = gemm16_splitk<DT>(g, s);
+        const int rc = gemm16_splitk<DT>(g, splitk, s);
         if (rc <= 0) return rc;
       }
       const int v = tile != LH_GEMM_TILE_AUTO ? (int)(tile >> 8) - 1 : direct_variant(g.M, g.N, g.K);

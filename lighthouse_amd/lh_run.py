@@ -6,7 +6,8 @@ Same command line as lighthouse/lh_run.py:14-145 (``payload_module --entry-point
 ``Output: <array>``) and exit codes (1 on FileNotFoundError / OSError / ValueError, 130 on
 Ctrl-C).  The payload module is MLIR text of one of the matmul forms this target has a kernel for
 (see ingress/mlir_text.py).  A ``--stage`` that names a pipeline descriptor with a ``kernel:`` stage
-(descriptors/gfx950/<pipeline>/<dtype>.yaml) selects that kernel's parameters; MLIR pass /
+(descriptors/gfx950/<pipeline>/<dtype>.yaml) sets that kernel's request flags (every parameter of
+such a stage acts; an unknown one is an error); MLIR pass /
 transform stages have no counterpart here (the kernels are already lowered) and are skipped with a
 note on stderr, so the reference's own RUN lines work unchanged.
 """
@@ -27,6 +28,57 @@ from .ingress.payloads import PayloadModule
 from .pipeline.descriptor import Descriptor, PipelineDescriptor
 
 
+# Parameters a `kernel:` stage may carry, per payload kind: each one changes what runs (a request
+# flag of the C entry point).  Anything else in a stage is an error, so a descriptor cannot
+# describe a kernel it does not select.
+KERNEL_PARAMETERS = {
+    "matmul": {"tile_m", "tile_n", "split_k"},
+    "attention": {"q_rows_per_wave", "kv_stages"},
+    "matmul_fp8": set(), "mlp": set(), "layer_norm": set(), "elementwise": set(), "nanogpt_block": set(),
+    "gpt_fused": set(),
+}
+
+
+def _apply_matmul(fn, params: dict, notes: list[str]) -> None:
+    if not params:
+        return
+    out_shape = fn.args[fn.arg_order[0] if fn.arg_order else 0].shape
+    if fn.attrs.ab_dtype == _lib.F32:
+        notes.append(f"stage 'matmul': tile / split-K requests apply to 16-bit operands, not to @{fn.name}; the library chooses")
+        return
+    flags = fn.attrs.flags
+    if "tile_m" in params or "tile_n" in params:
+        tile = (params.get("tile_m"), params.get("tile_n"))
+        if tile not in _lib.GEMM_TILES:
+            raise ValueError(f"stage 'matmul': unsupported tile {tile[0]}x{tile[1]}; choose from {sorted(_lib.GEMM_TILES)}")
+        if out_shape[0] % tile[0] == 0 and out_shape[1] % tile[1] == 0:
+            flags = (flags & ~_lib.GEMM_TILE_MASK) | _lib.GEMM_TILES[tile]
+        else:
+            notes.append(f"stage 'matmul': tile {tile[0]}x{tile[1]} does not apply to @{fn.name} "
+                         f"({out_shape[0]}x{out_shape[1]}); the library chooses")
+    if "split_k" in params:
+        sp = params["split_k"]
+        if sp not in _lib.GEMM_SPLITK:
+            raise ValueError(f"stage 'matmul': unsupported split_k {sp}; choose from {sorted(_lib.GEMM_SPLITK)}")
+        if sp > 1 and flags & _lib.GEMM_TILE_MASK:
+            raise ValueError("stage 'matmul': a cut along K runs on 128x128 tiles and excludes tile_m / tile_n")
+        flags = (flags & ~_lib.GEMM_SPLITK_MASK) | _lib.GEMM_SPLITK[sp]
+    fn.attrs.flags = flags
+
+
+def _apply_attention(fn, params: dict, notes: list[str]) -> None:
+    rows, stages = params.get("q_rows_per_wave", 0), params.get("kv_stages", 0)
+    if rows not in _lib.ATTN_ROWS or stages not in _lib.ATTN_STAGES:
+        raise ValueError(f"stage 'attention': q_rows_per_wave must be 32 or 64 and kv_stages 3 or 4, got {rows} / {stages}")
+    if not (rows or stages):
+        return
+    if fn.attrs.dtype == _lib.F32 or fn.args[0].shape[-1] != 64:
+        notes.append(f"stage 'attention': variant requests apply to 16-bit tensors with head dimension 64, not to "
+                     f"@{fn.name}; the library chooses")
+        return
+    fn.attrs.causal = (fn.attrs.causal & _lib.ATTN_CAUSAL) | _lib.ATTN_ROWS[rows] | _lib.ATTN_STAGES[stages]
+
+
 def apply_stage(module: PayloadModule, stage: str, notes: list[str]) -> None:
     """Apply one ``--stage`` to every function of the module."""
     desc = Descriptor(stage)
@@ -39,19 +91,21 @@ def apply_stage(module: PayloadModule, stage: str, notes: list[str]) -> None:
             notes.append(f"stage '{st}': MLIR {st.type or 'pass'} stage skipped (the HIP kernels are already lowered)")
             continue
         params = {**st.args, **st.opts}
+        if st.basename not in KERNEL_PARAMETERS:
+            raise ValueError(f"kernel stage '{st.basename}': no such payload kind; known: {sorted(KERNEL_PARAMETERS)}")
+        unknown = sorted(set(params) - KERNEL_PARAMETERS[st.basename])
+        if unknown:
+            raise ValueError(f"kernel stage '{st.basename}': unknown parameter(s) {unknown}; "
+                             f"it takes {sorted(KERNEL_PARAMETERS[st.basename]) or 'none'}")
         matched = False
         for fn in module.functions.values():
             if fn.entry != st.basename:
                 continue
             matched = True
-            tile = (params.get("tile_m"), params.get("tile_n"))
-            if fn.entry == "matmul" and tuple(tile) in _lib.GEMM_TILES:
-                out_shape = fn.args[fn.arg_order[0] if fn.arg_order else 0].shape
-                if out_shape[0] % tile[0] == 0 and out_shape[1] % tile[1] == 0 and fn.attrs.ab_dtype != _lib.F32:
-                    fn.attrs.flags = (fn.attrs.flags & ~0x700) | _lib.GEMM_TILES[tuple(tile)]
-                else:
-                    notes.append(f"stage '{st.basename}': tile {tile[0]}x{tile[1]} does not apply to @{fn.name} "
-                                 f"({out_shape[0]}x{out_shape[1]}); the library chooses")
+            if fn.entry == "matmul":
+                _apply_matmul(fn, params, notes)
+            elif fn.entry == "attention":
+                _apply_attention(fn, params, notes)
         if not matched:
             notes.append(f"stage '{st.basename}': no function of this kind in the module")
 

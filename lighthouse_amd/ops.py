@@ -36,6 +36,17 @@ def _require(cond: bool, msg: str) -> None:
         raise ValueError(msg)
 
 
+def _rows_aligned16(*tensors) -> bool:
+    """Base address and every stride but the innermost are multiples of 16 bytes."""
+    for t in tensors:
+        if t is None:
+            continue
+        per = 16 // t.element_size()
+        if t.data_ptr() % 16 or any(s % per for s in t.stride()[:-1]):
+            return False
+    return True
+
+
 def _is_matrix(t, rows, cols, what: str) -> None:
     _require(t.dim() == 2 and tuple(t.shape) == (rows, cols), f"{what} must have shape [{rows}, {cols}], got {tuple(t.shape)}")
     _require(t.stride(1) == 1 or cols == 1, f"{what}: innermost stride must be 1")
@@ -66,8 +77,10 @@ def device_info() -> dict:
 
 
 def gemm(a, b, bias=None, *, out=None, out_dtype=None, relu=False, gelu=False, accumulate_c=False,
-         transpose_a=False, transpose_b=False, tile=None, residual=None, workspace=None):
-    """out = epilogue(A @ B); see lh_hip_gemm.  `tile=(bm, bn)` requests a workgroup tile;
+         transpose_a=False, transpose_b=False, tile=None, split_k=None, residual=None, workspace=None):
+    """out = epilogue(A @ B); see lh_hip_gemm.  `tile=(bm, bn)` requests a workgroup tile and
+    `split_k` (1 = never, 2 / 4 / 8) a cut along K for the 16-bit kernels; with neither given the
+    tuned-parameter database is asked, then the library's own choice applies;
     `residual` [M, N] is added to A @ B before the epilogue (lh_hip_gemm_residual) and is left intact;
     `workspace` (uint8, see gemm_workspace_bytes) makes the call take its temporary memory from
     there instead of the library's pool (lh_hip_gemm_ws)."""
@@ -106,16 +119,21 @@ def gemm(a, b, bias=None, *, out=None, out_dtype=None, relu=False, gelu=False, a
     flags = ((_lib.GEMM_HAS_BIAS if bias is not None else 0) | (_lib.GEMM_HAS_RELU if relu else 0)
              | (_lib.GEMM_HAS_GELU if gelu else 0) | (_lib.GEMM_ACCUMULATE_C if accumulate_c else 0)
              | (_lib.GEMM_TRANSPOSE_A if transpose_a else 0) | (_lib.GEMM_TRANSPOSE_B if transpose_b else 0))
-    if tile is None and a.dtype in (torch.bfloat16, torch.float16) and not (transpose_a or transpose_b):
-        from .tuning.tile_db import active_db  # a tuned tile for this shape, if a database is in use
+    if tile is None and split_k is None and a.dtype in (torch.bfloat16, torch.float16) and not (transpose_a or transpose_b) \
+            and _rows_aligned16(a, b, out, bias):  # (a request needs aligned rows; tuned entries assume them)
+        from .tuning.tile_db import active_db  # tuned parameters for this shape, if the database has any
 
         db = active_db()
         if db is not None:
-            tile = db.lookup("bf16" if a.dtype == torch.bfloat16 else "f16", M, N, K)
+            tile, split_k = db.lookup_gemm("bf16" if a.dtype == torch.bfloat16 else "f16", M, N, K)
     if tile is not None:
         if tuple(tile) not in _lib.GEMM_TILES:
             raise ValueError(f"unsupported tile {tile}; choose from {sorted(_lib.GEMM_TILES)}")
         flags |= _lib.GEMM_TILES[tuple(tile)]
+    if split_k is not None:
+        if split_k not in _lib.GEMM_SPLITK:
+            raise ValueError(f"unsupported split_k {split_k}; choose from {sorted(_lib.GEMM_SPLITK)}")
+        flags |= _lib.GEMM_SPLITK[split_k]
     bias_ptr = bias.data_ptr() if bias is not None else None
     if residual is not None:
         _lib.check(_lib.load().lh_hip_gemm_residual(
@@ -185,8 +203,11 @@ def _strides3(t) -> _lib.Strides3:
     return _lib.Strides3(t.stride(0), t.stride(1), t.stride(2))
 
 
-def attention(q, k, v, *, causal=False, scale=None, out=None):
-    """Fused attention forward on [Z,H,T,d] tensors (any strides with unit stride along d)."""
+def attention(q, k, v, *, causal=False, scale=None, out=None, rows_per_wave=None, stages=None):
+    """Fused attention forward on [Z,H,T,d] tensors (any strides with unit stride along d).
+    `rows_per_wave` (32 or 64) and `stages` (3 or 4, K/V ring of the 32-row kernel) request a
+    kernel variant for 16-bit tensors with head dimension 64; with neither given the
+    tuned-parameter database is asked, then the library chooses by shape."""
     if q.dim() != 4 or q.shape != k.shape or q.shape != v.shape:
         raise ValueError("attention expects Q, K, V of equal 4-D shape [Z,H,T,d]")
     _require(q.dtype in _FLOATS and k.dtype == q.dtype and v.dtype == q.dtype,
@@ -199,10 +220,19 @@ def attention(q, k, v, *, causal=False, scale=None, out=None):
             raise ValueError("innermost stride must be 1")
     _need_cuda(q, k, v, out)
     Z, H, T, d = q.shape
+    if rows_per_wave is None and stages is None and d == 64 and q.dtype != torch.float32 and _rows_aligned16(q, k, v, out):
+        from .tuning.tile_db import active_db
+
+        db = active_db()
+        if db is not None:
+            rows_per_wave, stages = db.lookup_attention("bf16" if q.dtype == torch.bfloat16 else "f16", Z * H, T, d, causal)
+    _require((rows_per_wave or 0) in _lib.ATTN_ROWS and (stages or 0) in _lib.ATTN_STAGES,
+             f"rows_per_wave must be one of {sorted(_lib.ATTN_ROWS)[1:]}, stages one of {sorted(_lib.ATTN_STAGES)[1:]}")
+    word = (_lib.ATTN_CAUSAL if causal else 0) | _lib.ATTN_ROWS[rows_per_wave or 0] | _lib.ATTN_STAGES[stages or 0]
     _lib.check(_lib.load().lh_hip_attention(
         out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), Z, H, T, d,
         _strides3(out), _strides3(q), _strides3(k), _strides3(v),
-        float(scale) if scale is not None else 1.0 / math.sqrt(d), 1 if causal else 0, lh_dtype(q.dtype), _stream()),
+        float(scale) if scale is not None else 1.0 / math.sqrt(d), word, lh_dtype(q.dtype), _stream()),
         "attention")
     return out
 

@@ -1,5 +1,7 @@
-"""Tile search for the 16-bit GEMM: enumerate the tiles that fit a shape, drop the ones a cost
-model already rules out, time the rest in child processes, log every trial and keep the winner.
+"""Parameter search for the 16-bit GEMM (workgroup tile, cut along K) and the head-dimension-64
+attention kernel (query rows per wave, K/V ring depth): enumerate the settings that fit a shape,
+drop the ones a cost model already rules out, time the rest in child processes, log every trial
+and keep the winner when it beats the library's own choice.
 
 The structure follows the reference's tuner for the XeGPU matmul: candidate generation and the
 roofline pre-filter of examples/xegpu/tune_matmul_costmodel.py, crash- and hang-isolated trials of
@@ -7,6 +9,9 @@ examples/xegpu/tune_utils.py:35-85 (`run_with_timeout`), CSV logging of csv_logg
 per-shape JSON parameters.  Usage:
 
     python -m lighthouse_amd.tuning.tune_gemm --sizes 8192,2304,768 --dtype bf16 --db tiles.json --csv tune.csv
+    python -m lighthouse_amd.tuning.tune_gemm --attention 64,2048,causal --db tiles.json
+
+Without --db the packaged database (gfx950_tuned.json, the one `ops` consults by default) is updated.
 """
 
 from __future__ import annotations
@@ -48,27 +53,71 @@ def prefilter(M: int, N: int, K: int, slack: float = 1.35) -> list[tuple[int, in
     return [t for t in cands if estimate_cost(M, N, K, t) <= slack * best]
 
 
-def _time_tile(res, M, N, K, dtype, tile, nruns, nwarmup):
+SPLITS = (2, 4, 8)
+
+
+def candidate_splits(M: int, N: int, K: int) -> list[int]:
+    """Cuts of K worth timing: the problem's 128 x 128 tiles leave CUs idle and every piece of K is
+    a multiple of the k-step, at least 256 long."""
+    tiles = -(-M // 128) * -(-N // 128)
+    if K % 64 or N % 8 or tiles >= _CUS:
+        return []
+    return [sp for sp in SPLITS if K % (64 * sp) == 0 and K // sp >= 256 and tiles * sp <= 4 * _CUS]
+
+
+def candidate_settings(M: int, N: int, K: int, exhaustive: bool = False) -> list[tuple]:
+    """(tile or None, split_k or None) pairs to time after the library's own choice (None, None)."""
+    tiles = candidate_tiles(M, N, K) if exhaustive else prefilter(M, N, K)
+    return [(t, None) for t in tiles] + [(None, sp) for sp in candidate_splits(M, N, K)]
+
+
+def _time_tile(res, M, N, K, dtype, tile, nruns, nwarmup, split_k=None):
     import torch
 
     from .. import ops
+    from .tile_db import use_db
 
+    use_db(None)  # the baseline trial must be the library's own choice, not an earlier database entry
     tdt = {"bf16": torch.bfloat16, "f16": torch.float16}[dtype]
     a = torch.randn(M, K, device="cuda").to(tdt)
     b = torch.randn(K, N, device="cuda").to(tdt)
     out = torch.empty(M, N, device="cuda", dtype=tdt)
     for _ in range(nwarmup):
-        ops.gemm(a, b, out=out, tile=tile)
+        ops.gemm(a, b, out=out, tile=tile, split_k=split_k)
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(nruns):
-        ops.gemm(a, b, out=out, tile=tile)
+        ops.gemm(a, b, out=out, tile=tile, split_k=split_k)
     stop.record()
     torch.cuda.synchronize()
     seconds = start.elapsed_time(stop) * 1e-3 / nruns
     res["time"] = seconds
     res["throughput"] = 2.0 * M * N * K / seconds / 1e12
+
+
+def _time_attention(res, BH, T, d, causal, dtype, rows_per_wave, stages, nruns, nwarmup):
+    import torch
+
+    from .. import ops
+    from .tile_db import use_db
+
+    use_db(None)
+    tdt = {"bf16": torch.bfloat16, "f16": torch.float16}[dtype]
+    q, k, v = (torch.randn(1, BH, T, d, device="cuda").to(tdt) for _ in range(3))
+    out = torch.empty_like(q)
+    for _ in range(nwarmup):
+        ops.attention(q, k, v, causal=causal, out=out, rows_per_wave=rows_per_wave, stages=stages)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(nruns):
+        ops.attention(q, k, v, causal=causal, out=out, rows_per_wave=rows_per_wave, stages=stages)
+    stop.record()
+    torch.cuda.synchronize()
+    seconds = start.elapsed_time(stop) * 1e-3 / nruns
+    res["time"] = seconds
+    res["throughput"] = 4.0 * BH * T * T * d * (0.5 if causal else 1.0) / seconds / 1e12
 
 
 def run_with_timeout(experiment_func, *args, timeout: float = 60.0, **kwargs) -> dict:
@@ -102,48 +151,97 @@ def run_with_timeout(experiment_func, *args, timeout: float = 60.0, **kwargs) ->
         return out
 
 
+def _trial(fn, args, isolate, timeout):
+    if isolate:
+        return run_with_timeout(fn, *args, timeout=timeout)
+    res = {"time": 0.0, "throughput": 0.0, "error": ""}
+    try:
+        fn(res, *args)
+    except (ValueError, RuntimeError) as exc:
+        res["error"] = str(exc).split("\n")[0]
+    return res
+
+
+# A setting enters the database only if it beats the library's own choice by this factor
+# (two timings of one kernel in different child processes differ by up to 4 %).
+MIN_GAIN = 1.05
+
+
 def tune_shape(M: int, N: int, K: int, dtype: str = "bf16", db: TileDB | None = None, logger: CSVLogger | None = None,
-               nruns: int = 50, nwarmup: int = 20, timeout: float = 60.0, exhaustive: bool = False,
+               nruns: int = 300, nwarmup: int = 200, timeout: float = 60.0, exhaustive: bool = False,
                isolate: bool = True) -> dict | None:
-    """Time the (pre-filtered) tiles for one shape; record the fastest in `db`.  Returns its row.
-    `isolate=False` times in this process (no protection against a hanging or crashing trial)."""
-    cands = candidate_tiles(M, N, K) if exhaustive else prefilter(M, N, K)
-    best = None
-    # The library's own choice (tile None: its cost model, split K for decode shapes) is timed first;
-    # a tile enters the database only if it beats that.
-    for tile in [None, *cands] if cands else []:
-        if isolate:
-            res = run_with_timeout(_time_tile, M, N, K, dtype, tile, nruns, nwarmup, timeout=timeout)
-        else:
-            res = {"time": 0.0, "throughput": 0.0, "error": ""}
-            try:
-                _time_tile(res, M, N, K, dtype, tile, nruns, nwarmup)
-            except (ValueError, RuntimeError) as exc:
-                res["error"] = str(exc).split("\n")[0]
+    """Time the (pre-filtered) tiles and K cuts for one shape; record the fastest in `db` if it beats
+    the library's own choice.  Returns the fastest row.  `isolate=False` times in this process (no
+    protection against a hanging or crashing trial)."""
+    cands = candidate_settings(M, N, K, exhaustive)
+    best = base = None
+    # The library's own choice (no request: its cost model, its own split-K criterion) is timed first.
+    for tile, split_k in [(None, None), *cands] if cands else []:
+        res = _trial(_time_tile, (M, N, K, dtype, tile, nruns, nwarmup, split_k), isolate, timeout)
         row = {"dtype": dtype, "M": M, "N": N, "K": K, "tile_m": tile[0] if tile else 0, "tile_n": tile[1] if tile else 0,
+               "split_k": split_k or 0,
                "estimate": round(estimate_cost(M, N, K, tile) / 1e6, 3) if tile else 0.0,
                "time_us": round(res["time"] * 1e6, 3),
                "tflops": round(res["throughput"], 2), "error": res["error"]}
         if logger is not None:
             logger.log(row)
-        if not res["error"] and res["time"] > 0 and (best is None or row["time_us"] < best["time_us"]):
+        ok = not res["error"] and res["time"] > 0
+        if ok and tile is None and split_k is None:
+            base = row
+        if ok and (best is None or row["time_us"] < best["time_us"]):
             best = row
-    if best is not None and db is not None and best["tile_m"]:
-        db.record(dtype, M, N, K, (best["tile_m"], best["tile_n"]), best["time_us"], best["tflops"])
+    if best is not None and db is not None and (best["tile_m"] or best["split_k"]) and (
+            base is None or best["time_us"] * MIN_GAIN <= base["time_us"]):
+        db.record(dtype, M, N, K, (best["tile_m"], best["tile_n"]) if best["tile_m"] else None, best["time_us"],
+                  best["tflops"], split_k=best["split_k"] or None)
+    return best
+
+
+ATTENTION_SETTINGS = ((64, None), (32, 3), (32, 4))
+
+
+def tune_attention(BH: int, T: int, causal: bool, dtype: str = "bf16", db: TileDB | None = None,
+                   logger: CSVLogger | None = None, nruns: int = 300, nwarmup: int = 200, timeout: float = 60.0,
+                   isolate: bool = True, d: int = 64) -> dict | None:
+    """The same for the head-dimension-64 attention kernel: query rows per wave x K/V ring depth."""
+    best = base = None
+    settings = [s for s in ATTENTION_SETTINGS if s[0] != 64 or T % 64 == 0]
+    for rows, stages in [(None, None), *settings]:
+        res = _trial(_time_attention, (BH, T, d, causal, dtype, rows, stages, nruns, nwarmup), isolate, timeout)
+        row = {"dtype": dtype, "BH": BH, "T": T, "d": d, "causal": int(causal), "rows_per_wave": rows or 0,
+               "stages": stages or 0, "time_us": round(res["time"] * 1e6, 3), "tflops": round(res["throughput"], 2),
+               "error": res["error"]}
+        if logger is not None:
+            logger.log(row)
+        ok = not res["error"] and res["time"] > 0
+        if ok and rows is None:
+            base = row
+        if ok and (best is None or row["time_us"] < best["time_us"]):
+            best = row
+    if best is not None and db is not None and best["rows_per_wave"] and (
+            base is None or best["time_us"] * MIN_GAIN <= base["time_us"]):
+        db.record_attention(dtype, BH, T, d, causal, best["rows_per_wave"], best["stages"] or None, best["time_us"],
+                            best["tflops"])
     return best
 
 
 def main(argv: list[str] | None = None) -> int:
-    ap = argparse.ArgumentParser(description="Tile search for the 16-bit HIP GEMM.")
-    ap.add_argument("--sizes", action="append", required=True, help="M,N,K (repeatable)")
+    from .tile_db import DEFAULT_DB_PATH
+
+    ap = argparse.ArgumentParser(description="Parameter search for the 16-bit HIP GEMM and the attention kernel.")
+    ap.add_argument("--sizes", action="append", default=[], help="GEMM M,N,K (repeatable)")
+    ap.add_argument("--attention", action="append", default=[], help="attention BH,T[,causal] (repeatable; head_dim 64)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16"])
-    ap.add_argument("--db", default="gemm_tiles.json", help="JSON tile database to update")
-    ap.add_argument("--csv", default=None, help="CSV log of every trial")
-    ap.add_argument("--nruns", type=int, default=50)
-    ap.add_argument("--nwarmup", type=int, default=20)
+    ap.add_argument("--db", default=str(DEFAULT_DB_PATH), help="JSON database to update (default: the packaged one)")
+    ap.add_argument("--csv", default=None, help="CSV log of every GEMM trial (attention trials: <name>_attention.csv)")
+    ap.add_argument("--nruns", type=int, default=300)
+    ap.add_argument("--nwarmup", type=int, default=200, help="untimed launches first (the clocks need ~100 to settle)")
     ap.add_argument("--timeout", type=float, default=60.0)
     ap.add_argument("--exhaustive", action="store_true", help="skip the cost-model pre-filter")
     args = ap.parse_args(argv)
+    if not args.sizes and not args.attention:
+        print("Error: nothing to tune (give --sizes and / or --attention)", file=sys.stderr)
+        return 1
     db = TileDB(args.db)
     logger = CSVLogger(args.csv)
     for spec in args.sizes:
@@ -154,7 +252,17 @@ def main(argv: list[str] | None = None) -> int:
             return 1
         best = tune_shape(M, N, K, args.dtype, db, logger, args.nruns, args.nwarmup, args.timeout, args.exhaustive)
         if best is None:
-            print(f"{spec}: no tile of the direct kernel fits (or every trial failed)", file=sys.stderr)
+            print(f"{spec}: no setting of the direct kernel fits (or every trial failed)", file=sys.stderr)
+    alog = CSVLogger(args.csv.replace(".csv", "_attention.csv") if args.csv else None)
+    for spec in args.attention:
+        parts = spec.split(",")
+        try:
+            BH, T = int(parts[0]), int(parts[1])
+            causal = len(parts) > 2 and parts[2] == "causal"
+        except (ValueError, IndexError):
+            print(f"Error: --attention expects BH,T[,causal], got '{spec}'", file=sys.stderr)
+            return 1
+        tune_attention(BH, T, causal, args.dtype, db, alog, args.nruns, args.nwarmup, args.timeout)
     db.save()
     return 0
 

@@ -230,3 +230,41 @@ def test_attention_errors():
     z = torch.zeros(1, 1, 64, 64, device="cuda", dtype=torch.bfloat16)
     with pytest.raises(ValueError):
         ops.attention(z, z[:, :, :32], z)
+
+
+@pytest.mark.parametrize("rows,stages", [(64, None), (32, 3), (32, 4), (32, None), (None, 3)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_variant_requests(rows, stages, causal):
+    """LH_ATTN_ROWS_* / LH_ATTN_STAGES_*: every variant of the head-dimension-64 kernel computes the
+    same attention (oracle on one head, equality of all heads with the library's own choice up to
+    the rounding of a different summation order)."""
+    from lighthouse_amd import ops
+
+    shape = (2, 3, 512, 64)
+    g = torch.Generator(device="cuda").manual_seed(21)
+    q, k, v = (torch.randn(shape, device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
+    out = ops.attention(q, k, v, causal=causal, rows_per_wave=rows, stages=stages)
+    ref = orc.attention(q[1, 2].float().cpu().numpy(), k[1, 2].float().cpu().numpy(), v[1, 2].float().cpu().numpy(),
+                        causal=causal)
+    assert_close(out[1, 2].float().cpu().numpy(), orc.round_bf16(ref), 2e-2, f"attention rows={rows} stages={stages} causal={causal}")
+    auto = ops.attention(q, k, v, causal=causal)
+    assert (out.float() - auto.float()).abs().max() <= 2e-2 * auto.float().abs().max()
+
+
+def test_attention_variant_request_errors():
+    from lighthouse_amd import ops
+
+    q = torch.zeros(1, 2, 256, 64, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="rows_per_wave"):
+        ops.attention(q, q, q, rows_per_wave=48)
+    with pytest.raises(ValueError, match="4-stage ring only"):
+        ops.attention(q, q, q, rows_per_wave=64, stages=3)
+    q100 = torch.zeros(1, 2, 100, 64, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="multiple of 64"):
+        ops.attention(q100, q100, q100, rows_per_wave=64)
+    q32 = torch.zeros(1, 2, 256, 64, device="cuda")
+    with pytest.raises(ValueError, match="16-bit"):
+        ops.attention(q32, q32, q32, rows_per_wave=32)
+    q128 = torch.zeros(1, 2, 256, 128, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="head_dim 64"):
+        ops.attention(q128, q128, q128, rows_per_wave=32)

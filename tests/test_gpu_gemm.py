@@ -704,3 +704,40 @@ def test_split_k_gemms_on_two_streams():
     np.testing.assert_array_equal(_host(small), want)
     np.testing.assert_array_equal(_host(big), want2)
     ops.release_scratch()
+
+
+@pytest.mark.parametrize("shape,split_k", [((16, 2048, 4096), 2), ((16, 2048, 4096), 8), ((100, 520, 1024), 4),
+                                           ((512, 512, 2048), 2), ((256, 256, 512), 1), ((16, 8192, 8192), 1)])
+def test_gemm_split_k_request(shape, split_k):
+    """LH_GEMM_SPLITK_*: an explicit cut (or its prohibition) computes the same product; small
+    integers make every summation order exact."""
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K + split_k)
+    a_h = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    b_h = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    bias_h = rng.integers(-3, 4, N).astype(np.float32)
+    out = ops.gemm(_dev(a_h, torch.bfloat16), _dev(b_h, torch.bfloat16), _dev(bias_h, torch.float32), relu=True,
+                   out_dtype=torch.float32, split_k=split_k)
+    np.testing.assert_array_equal(_host(out), np.maximum(a_h @ b_h + bias_h, 0))
+    a = _dev(orc.round_bf16(rng.standard_normal((M, K)).astype(np.float32)), torch.bfloat16)
+    b = _dev(orc.round_bf16(rng.standard_normal((K, N)).astype(np.float32)), torch.bfloat16)
+    got = ops.gemm(a, b, split_k=split_k)
+    assert_close(_host(got), orc.matmul(_host(a), _host(b), result_type="bf16"), BF16_RTOL, f"bf16 gemm {shape} split_k={split_k}")
+
+
+def test_gemm_split_k_request_errors():
+    from lighthouse_amd import ops
+
+    a = torch.zeros(128, 192, device="cuda", dtype=torch.bfloat16)
+    b = torch.zeros(192, 128, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="cut of K"):
+        ops.gemm(a, b, split_k=2)                       # 96 is no multiple of the k-step
+    with pytest.raises(ValueError, match="excludes a tile"):
+        ops.gemm(torch.zeros(128, 256, device="cuda", dtype=torch.bfloat16),
+                 torch.zeros(256, 128, device="cuda", dtype=torch.bfloat16), split_k=2, tile=(128, 128))
+    with pytest.raises(ValueError, match="16-bit"):
+        ops.gemm(torch.zeros(128, 256, device="cuda"), torch.zeros(256, 128, device="cuda"), split_k=2)
+    with pytest.raises(ValueError, match="unsupported split_k"):
+        ops.gemm(a, b, split_k=3)

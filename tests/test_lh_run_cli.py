@@ -152,6 +152,48 @@ def test_stage_application(tmp_path):
     assert "does not apply" in notes[-1]
 
 
+def test_stage_parameters_all_act_or_fail(tmp_path):
+    """Every parameter of a `kernel:` stage sets a request flag; an unknown one is an error, so a
+    descriptor cannot carry text that selects nothing."""
+    from lighthouse_amd.ingress import generate_gpu_attention_payload
+    from lighthouse_amd.pipeline.finder import find_pipeline_file
+    from lighthouse_amd.execution.target import TargetInfo
+
+    text = GENERIC.replace("32x", "256x").replace("x128", "x384").replace("<128x", "<384x")
+    module = parse_payload_module(text)
+    notes = []
+    y = tmp_path / "s.yaml"
+    y.write_text('Pipeline:\n  - kernel: "matmul{split_k=4}"\n')
+    apply_stage(module, str(y), notes)
+    assert module.lookup("layer").attrs.flags & _lib.GEMM_SPLITK_MASK == _lib.GEMM_SPLITK[4]
+    y.write_text('Pipeline:\n  - kernel: "matmul{split_k=1}"\n')
+    apply_stage(module, str(y), notes)
+    assert module.lookup("layer").attrs.flags & _lib.GEMM_SPLITK_MASK == _lib.GEMM_SPLITK[1]
+    for bad, match in (('matmul{tile_m=256 tile_n=128 wave_m=128}', "unknown parameter"), ('matmul{split_k=3}', "split_k"),
+                       ('matmul{tile_m=96 tile_n=128}', "unsupported tile"), ('conv{tile=1}', "no such payload kind"),
+                       ('matmul{tile_m=128 tile_n=128 split_k=2}', "excludes"), ('attention{rescale=lazy}', "unknown parameter"),
+                       ('layer_norm{rows_per_wg=4}', "unknown parameter")):
+        y.write_text(f'Pipeline:\n  - kernel: "{bad}"\n')
+        with pytest.raises(ValueError, match=match):
+            apply_stage(parse_payload_module(text), str(y), notes)
+    att = generate_gpu_attention_payload("payload", 4, 16, 2048, 64, "bf16", causal=True)
+    y.write_text('Pipeline:\n  - kernel: "attention{q_rows_per_wave=32 kv_stages=3}"\n')
+    apply_stage(att, str(y), notes)
+    assert att.lookup("payload").attrs.causal == _lib.ATTN_CAUSAL | _lib.ATTN_ROWS[32] | _lib.ATTN_STAGES[3]
+    y.write_text('Pipeline:\n  - kernel: "attention{q_rows_per_wave=48}"\n')
+    with pytest.raises(ValueError, match="q_rows_per_wave"):
+        apply_stage(att, str(y), notes)
+    # every packaged descriptor parses and applies: none carries a parameter that does nothing
+    target = TargetInfo("gfx950", [])
+    for pipeline, dtypes in {"matmul": ["bf16", "f16", "f32", "f8E4M3FN"], "attention": ["bf16", "f16", "f32"],
+                             "layer_norm": ["f32", "bf16"], "softmax": ["f32", "bf16"], "element_wise": ["f32", "bf16"],
+                             "nanogpt_block": ["f32", "bf16"]}.items():
+        for dt in dtypes:
+            path = find_pipeline_file(target, pipeline, dt)
+            assert path is not None, (pipeline, dt)
+            apply_stage(parse_payload_module(text), str(path), [])
+
+
 def test_cli_error_codes(tmp_path, capsys):
     missing = main([str(tmp_path / "nope.mlir"), "--entry-point", "mm", "--input-shape", "8x24xf32x1", "--stage", "cse"])
     assert missing == 1 and "Error:" in capsys.readouterr().err

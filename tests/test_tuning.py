@@ -5,8 +5,8 @@ import time
 
 import pytest
 
-from lighthouse_amd.tuning import CSVLogger, TileDB, active_db, candidate_tiles, estimate_cost, prefilter, \
-    run_with_timeout, use_db
+from lighthouse_amd.tuning import CSVLogger, TileDB, active_db, candidate_settings, candidate_tiles, estimate_cost, \
+    prefilter, run_with_timeout, use_db, use_default_db
 
 
 def test_candidates_and_prefilter():
@@ -67,6 +67,31 @@ def test_tile_db_round_trip(tmp_path):
         TileDB(str(tmp_path / "bad.json"))
     try:
         assert use_db(again) is again and active_db() is again
-    finally:
         use_db(None)
-    assert active_db() is None
+        assert active_db() is None
+    finally:
+        use_default_db()
+
+
+def test_settings_and_database_kinds(tmp_path):
+    """Cuts along K are offered where the tiles leave CUs idle; the database keeps tile, cut and the
+    attention variant apart and the packaged one loads by default."""
+    assert ((None, 8) in candidate_settings(16, 8192, 8192)) and ((None, 2) in candidate_settings(16, 8192, 8192))
+    assert all(sp is None for _, sp in candidate_settings(4096, 4096, 4096))      # 1024 tiles: nothing to cut for
+    assert all(sp != 8 for _, sp in candidate_settings(128, 1024, 1024))           # K / 8 = 128 is too short a piece
+    db = TileDB(str(tmp_path / "t.json"))
+    db.record("bf16", 16, 8192, 8192, None, 25.0, 86.0, split_k=8)
+    db.record("bf16", 8192, 768, 768, (128, 128), 20.0, 480.0)
+    db.record_attention("bf16", 64, 2048, 64, True, 32, 3, 50.0, 690.0)
+    db.save()
+    again = TileDB(str(tmp_path / "t.json"))
+    assert again.lookup_gemm("bf16", 16, 8192, 8192) == (None, 8)
+    assert again.lookup_gemm("bf16", 8192, 768, 768) == ((128, 128), None)
+    assert again.lookup_gemm("bf16", 1, 1, 1) == (None, None)
+    assert again.lookup_attention("bf16", 64, 2048, 64, True) == (32, 3)
+    assert again.lookup_attention("bf16", 64, 2048, 64, False) == (None, None)
+    default = use_default_db()
+    assert default is None or isinstance(default, TileDB)
+    if default is not None:
+        for key, entry in default.entries.items():
+            assert key.split(":")[0] in ("bf16", "f16", "attn") and entry["time_us"] > 0
