@@ -76,11 +76,23 @@ __device__ __forceinline__ float halfwave_sum(float x) {
   return a + b;
 }
 
+// 16 bytes per lane from a buffer resource (base + per-lane byte offset) straight into LDS, 1 KiB per
+// wave from lds_wave_base.  The buffer form of the LDS-DMA load, not the global (flat-encoded) one:
+// while a flat-encoded LDS access is in flight the compiler has to assume LDS operations complete
+// out of order and waits for ALL of a wave's LDS reads (lgkmcnt(0)) before the first use of any;
+// with the buffer form it counts them, and an MFMA waits for its own fragments only.
+__device__ __forceinline__ void attn_dma16(const void* base, int lane_bytes, uint8_t* lds_wave_base) {
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0xffffffff, 0x00020000);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (attn_lds_void_t*)lds_wave_base, 16, lane_bytes, 0, 0, 0);
+}
+
 struct AttnCtx {
-  const uint16_t* k_src[2];  // lane's source of K load i at key 0
-  const uint16_t* v_src[2];
+  const uint16_t* k_base;    // K and V of the workgroup's (batch, head), key 0 (uniform)
+  const uint16_t* v_base;
+  int k_src[2];              // lane's byte offset within a key tile for load i
+  int v_src[2];
   int64_t k_step, v_step;    // elements per key tile
-  int64_t k_row, v_row;      // elements per key (row strides), for the clamped loads of a partial tile
+  int k_row, v_row;          // bytes per key (row strides), for the clamped loads of a partial tile
   int key_local[2];          // the key of the tile that load i of this lane fetches
   int wave, r32, h;
   int k_off[2], k_swz[2];    // K fragment: byte offset of the lane's row, its swizzle, per key sub-tile
@@ -92,17 +104,19 @@ struct AttnCtx {
 // and a template parameter, so that the loads of the common case stay one addition each.
 template <bool RAGGED>
 __device__ __forceinline__ void attn_issue_loads(const AttnCtx& c, int jt, int T, uint8_t* __restrict__ stage) {
+  // The resources start at the tile's first key, so lane offsets stay within 64 key rows.
+  const uint16_t* kt = c.k_base + jt * c.k_step;
+  const uint16_t* vt = c.v_base + jt * c.v_step;
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    int64_t k_off = jt * c.k_step, v_off = jt * c.v_step;
+    int k_off = c.k_src[i], v_off = c.v_src[i];
     if constexpr (RAGGED) {
       const int back = max(jt * kKvTile + c.key_local[i] - (T - 1), 0);  // keys past the last one
       k_off -= back * c.k_row;
       v_off -= back * c.v_row;
     }
-    __builtin_amdgcn_global_load_lds(c.k_src[i] + k_off, (attn_lds_void_t*)(stage + (4 * i + c.wave) * 1024), 16, 0, 0);
-    __builtin_amdgcn_global_load_lds(c.v_src[i] + v_off, (attn_lds_void_t*)(stage + 8192 + (4 * i + c.wave) * 1024), 16,
-                                     0, 0);
+    attn_dma16(kt, k_off, stage + (4 * i + c.wave) * 1024);
+    attn_dma16(vt, v_off, stage + 8192 + (4 * i + c.wave) * 1024);
   }
 }
 
@@ -262,7 +276,7 @@ __device__ __forceinline__ void causal_block_of(int L, int G, int R, int nqb, in
 
 // 16-bit kernel.  A workgroup owns 256 query rows of one (batch, head): 4 waves x 64 rows (two
 // 32-row sub-tiles per wave share every K and V fragment).  K/V tiles of 64 keys go global ->
-// LDS with global_load_lds_dwordx4 through a ring of NS stages; K fragments are 16-byte LDS
+// LDS with buffer_load_dwordx4 ... lds through a ring of NS stages; K fragments are 16-byte LDS
 // reads, V^T fragments come from ds_read_b64_tr_b16 on the row-major V tile.  Rows of a tile
 // are 128 bytes and cannot be padded (a wave-wide load writes 1 KiB contiguous), so the
 // 16-byte chunk a lane fetches is XOR-swizzled: K chunk ^ ((key / 2) % 8), V chunk ^ 4 ((key / 2) % 2).
@@ -296,10 +310,12 @@ __global__ void __launch_bounds__(256, (NQ == 1 && NS == 3 ? 3 : 2)) attention16
 
   AttnCtx c;
   c.wave = wave; c.r32 = r32; c.h = h;
+  c.k_base = K;
+  c.v_base = V;
   c.k_step = (int64_t)kKvTile * a.sk.t;
   c.v_step = (int64_t)kKvTile * a.sv.t;
-  c.k_row = a.sk.t;
-  c.v_row = a.sv.t;
+  c.k_row = (int)a.sk.t * 2;
+  c.v_row = (int)a.sv.t * 2;
   // Loader: load i of wave w fills keys (4 i + w) 8 .. +8 of the tile; lane -> key += lane / 8,
   // LDS chunk p = lane % 8 holds global chunk p ^ swizzle(key).
 #pragma unroll
@@ -307,8 +323,8 @@ __global__ void __launch_bounds__(256, (NQ == 1 && NS == 3 ? 3 : 2)) attention16
     const int key = (4 * i + wave) * 8 + (lane >> 3);
     const int p = lane & 7;
     c.key_local[i] = key;
-    c.k_src[i] = K + (int64_t)key * a.sk.t + ((p ^ ((key >> 1) & 7)) << 3);
-    c.v_src[i] = V + (int64_t)key * a.sv.t + ((p ^ (4 * ((key >> 1) & 1))) << 3);
+    c.k_src[i] = key * c.k_row + ((p ^ ((key >> 1) & 7)) << 4);
+    c.v_src[i] = key * c.v_row + ((p ^ (4 * ((key >> 1) & 1))) << 4);
   }
   // K fragment (first MFMA operand of S^T): key 32 i + r32, logical chunk 2 sd + h.
 #pragma unroll
@@ -1220,7 +1236,8 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   // (the kernels mask a partial last key tile and skip rows past the end themselves)
   bool vec_ok = true;
   for (int i = 0; i < 4 && vec_ok; ++i)
-    vec_ok = ss[i]->t % vec == 0 && ss[i]->h % vec == 0 && ss[i]->z % vec == 0 && aligned16(ps[i]);
+    vec_ok = ss[i]->t % vec == 0 && ss[i]->h % vec == 0 && ss[i]->z % vec == 0 && aligned16(ps[i]) &&
+             ss[i]->t < (1 << 24);  // (a key tile's rows are addressed with 32-bit byte offsets)
   const bool fast = vec_ok && d == kHeadDim;
   if (scale <= 0.0f) scale = 1.0f / sqrtf((float)d);
   AttnArgs a;

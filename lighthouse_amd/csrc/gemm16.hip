@@ -196,7 +196,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm16_fast(GemmArgs g)
 // ---- direct-to-LDS kernels --------------------------------------------------------------
 // Workgroup tile (64 TM) x (128 TN), 8 waves as 2 x 4, (32 TM) x (32 TN) per wave; TM x TN is
 // 4 x 2 (256 x 256), 4 x 1 (256 x 128), 2 x 2 (128 x 256) or 2 x 1 (128 x 128).  Both panels go
-// global -> LDS with global_load_lds_dwordx4 (no register staging, no LDS store instructions) in
+// global -> LDS with buffer_load_dwordx4 ... lds (no register staging, no LDS store instructions) in
 // their GLOBAL orientation.  The k-contiguous A fragment is one 16-byte LDS read; the
 // n-contiguous B panel is read with ds_read_b64_tr_b16, which hands each lane 4 k-values of one
 // column, i.e. the MFMA operand layout, transposing in the LDS crossbar.
@@ -207,7 +207,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm16_fast(GemmArgs g)
 // fragment reads always overlap MFMAs of the previous k-half and the buffer a step has finished
 // reading is refilled right away (B: 3 stages ahead, A: on odd steps, one 64-k stage ahead).
 //
-// A wave-wide global_load_lds writes 64 x 16 contiguous LDS bytes, so rows cannot be padded;
+// A wave-wide load into LDS writes 64 x 16 contiguous LDS bytes, so rows cannot be padded;
 // bank conflicts are avoided by XOR-swizzling which 16-byte chunk of a row each lane fetches
 // (A: chunk ^ ((row / 2) % 8); B: chunk ^ 4 (k % 4)).
 template <int TM, int TN>
@@ -232,17 +232,35 @@ struct DirectCfg {
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ void async_copy16(const void* gsrc, uint8_t* lds_wave_base) {
-  __builtin_amdgcn_global_load_lds(gsrc, (lds_void_t*)lds_wave_base, 16, 0, 0);
+// 16 bytes per lane from a buffer resource (base + per-lane byte offset + scalar byte offset)
+// straight into LDS, 1 KiB per wave starting at lds_wave_base.  The buffer form of the LDS-DMA
+// load, not the global (flat-encoded) one: with a flat-encoded LDS access in flight the compiler
+// must assume that LDS operations complete out of order and turns every s_waitcnt on an LDS read
+// into lgkmcnt(0); with the buffer form it counts, so a fragment read issued a few MFMAs ago is
+// not waited for behind the ones issued last.
+__device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t rsrc, int lane_bytes, int scalar_bytes,
+                                      uint8_t* lds_wave_base) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_t*)lds_wave_base, 16, lane_bytes, scalar_bytes, 0, 0);
+}
+// A resource over [base, base + 4 GiB): raw (unstructured) addressing, offsets in bytes.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t panel_resource(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0xffffffff, 0x00020000);
+}
+// The direct kernels address a tile's operand panels with 32-bit byte offsets from the panel's
+// first element: 256 rows of A, K rows of B.
+static inline bool direct_offsets_fit(const GemmArgs& g) {
+  return g.lda < (1ll << 22) && (int64_t)g.K * g.ldb < (1ll << 30);
 }
 
 template <int TM, int TN>
 struct DirectCtx {
-  const uint16_t* a_src[TM];  // lane's source of A load i at k = 0
-  const uint16_t* b_src[TN];
+  const uint16_t* a_base;     // the tile's A row panel and B column panel (uniform; the buffer
+  const uint16_t* b_base;     // resources are made from them at each load: four scalar moves)
+  int a_src[TM];              // lane's byte offset in the A panel for load i at k = 0
+  int b_src[TN];
+  int b_step;                 // bytes between B stages (32 k rows)
   int a_off[TM];              // byte offset of the lane's A row in a stage, per m-subtile
   int a_swz[TM];
-  int64_t ldb;
   int wave, h, b_off, b_chunk, b_swz;
 };
 
@@ -255,14 +273,16 @@ struct DirectFrags {
 // A stage `sa` (k = 64 sa .. +64): TM loads per lane.
 template <int TM, int TN>
 __device__ __forceinline__ void direct_load_a(const DirectCtx<TM, TN>& c, int sa, uint8_t* __restrict__ abuf) {
+  const __amdgpu_buffer_rsrc_t rsrc = panel_resource(c.a_base);
 #pragma unroll
-  for (int i = 0; i < TM; ++i) async_copy16(c.a_src[i] + sa * 64, abuf + (8 * i + c.wave) * 1024);
+  for (int i = 0; i < TM; ++i) dma16(rsrc, c.a_src[i], sa * 128, abuf + (8 * i + c.wave) * 1024);
 }
 // B stage `sb` (k = 32 sb .. +32): TN loads per lane.
 template <int TM, int TN>
 __device__ __forceinline__ void direct_load_b(const DirectCtx<TM, TN>& c, int sb, uint8_t* __restrict__ bbuf) {
+  const __amdgpu_buffer_rsrc_t rsrc = panel_resource(c.b_base);
 #pragma unroll
-  for (int i = 0; i < TN; ++i) async_copy16(c.b_src[i] + (int64_t)(sb * 32) * c.ldb, bbuf + (8 * i + c.wave) * 1024);
+  for (int i = 0; i < TN; ++i) dma16(rsrc, c.b_src[i], sb * c.b_step, bbuf + (8 * i + c.wave) * 1024);
 }
 
 // Fragments of 16 k: A chunk pair `kc` (0..3: which 16 of the stage's 64 k), B k-step `ks`
@@ -272,18 +292,23 @@ __device__ __forceinline__ void direct_read_frags(const DirectCtx<TM, TN>& c, co
                                                   const uint8_t* __restrict__ bs, int kc, int ks,
                                                   DirectFrags<TM, TN>& f) {
   constexpr int row = DirectCfg<TM, TN>::kBRow;
-#pragma unroll
-  for (int j = 0; j < TM; ++j)
-    f.a[j] = *reinterpret_cast<const u32x4*>(as + c.a_off[j] + (((2 * kc + c.h) ^ c.a_swz[j]) << 4));
-#pragma unroll
-  for (int i = 0; i < TN; ++i) {
+  auto read_b = [&](int i) {
     const int p = (c.b_chunk + 4 * i) ^ c.b_swz;
     const uint8_t* p0 = bs + ks * 16 * row + c.b_off + p * 16;
     s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p0);
     s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p0 + 4 * row));
     u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
     f.b[i] = u32x4{l2[0], l2[1], h2[0], h2[1]};
-  }
+  };
+  // In the order direct_mfma consumes them (B fragment 0 with every A fragment, then B fragment 1 ...):
+  // LDS reads return in order and the waits in front of the MFMAs count, so the fragment wanted
+  // first must be the oldest request.
+  read_b(0);
+#pragma unroll
+  for (int j = 0; j < TM; ++j)
+    f.a[j] = *reinterpret_cast<const u32x4*>(as + c.a_off[j] + (((2 * kc + c.h) ^ c.a_swz[j]) << 4));
+#pragma unroll
+  for (int i = 1; i < TN; ++i) read_b(i);
 }
 
 template <int DT, int TM, int TN>
@@ -306,7 +331,6 @@ template <int TM, int TN>
 __device__ __forceinline__ void direct_interleave_hint() {
   direct_interleave_step<0, TM * TN, TM + 2 * TN>();
 }
-
 // Wait until at most N of this wave's loads are still in flight and all its LDS reads have
 // returned, then barrier.  One asm block: a __syncthreads() would add a release fence, i.e. a
 // wait for ALL outstanding loads, and drain the rings.
@@ -376,14 +400,18 @@ __device__ __forceinline__ void direct_place(const GemmArgs& g, int id, DirectCt
   n0 = ((id % group_size) / gm) * BN;
   const uint16_t* A = reinterpret_cast<const uint16_t*>(g.a);
   const uint16_t* B = reinterpret_cast<const uint16_t*>(g.b);
+  const int lda = (int)g.lda, ldb = (int)g.ldb;
+  c.a_base = A + (int64_t)m0 * g.lda;
+  c.b_base = B + n0;
+  c.b_step = 64 * ldb;
   // A: load i of wave w fills rows (8 i + w) 8 .. +8 (1024 bytes); lane -> row += lane / 8, LDS
   // chunk p = lane % 8 holds global chunk p ^ ((row / 2) % 8).
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int ar = (8 * i + c.wave) * 8 + (lane >> 3);
     const int ac = (lane & 7) ^ ((ar >> 1) & 7);
-    const int arow = EDGE ? min(m0 + ar, g.M - 1) : m0 + ar;
-    c.a_src[i] = A + (int64_t)arow * g.lda + ac * 8;
+    const int arow = EDGE ? min(ar, g.M - 1 - m0) : ar;  // row within the panel
+    c.a_src[i] = (arow * lda + ac * 8) * 2;
   }
   // B: load i of wave w fills k rows (8 i + w) R .. +R with R = 1024 / row bytes; lane ->
   // row += lane / chunks-per-row, LDS chunk p holds global chunk p ^ 4 (k % 4).
@@ -391,8 +419,8 @@ __device__ __forceinline__ void direct_place(const GemmArgs& g, int id, DirectCt
   for (int i = 0; i < TN; ++i) {
     const int bk = (8 * i + c.wave) * Cfg::kBRowsPerLoad + lane / Cfg::kBChunks;
     const int bc = (lane % Cfg::kBChunks) ^ (4 * (bk & 3));
-    const int bcol = EDGE ? min(n0 + bc * 8, g.N - 8) : n0 + bc * 8;
-    c.b_src[i] = B + (int64_t)bk * g.ldb + bcol;
+    const int bcol = EDGE ? min(bc * 8, g.N - 8 - n0) : bc * 8;  // column within the panel
+    c.b_src[i] = (bk * ldb + bcol) * 2;
   }
 }
 
@@ -644,7 +672,6 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
   const int r32 = lane & 31, h = lane >> 5;
 
   DirectCtx<TM, TN> c;
-  c.ldb = g.ldb;
   c.wave = wave;
   c.h = h;
   // A fragment (second MFMA operand): row wm0 + 32 j + r32, logical chunk 2 kc + h.
@@ -917,17 +944,17 @@ static int gemm16_dispatch(const GemmArgs& g_in, hipStream_t s) {
   if (tile != LH_GEMM_TILE_AUTO) {
     static const int bm[4] = {256, 256, 128, 128}, bn[4] = {256, 128, 256, 128};
     const int v = (int)(tile >> 8) - 1;
-    LH_REQUIRE(vec_ok && !tb && g.ldc % 8 == 0 && g.M % bm[v] == 0 && g.N % bn[v] == 0,
+    LH_REQUIRE(vec_ok && !tb && g.ldc % 8 == 0 && g.M % bm[v] == 0 && g.N % bn[v] == 0 && direct_offsets_fit(g),
                "gemm: the requested %d x %d tile needs untransposed operands, M %% %d == 0, N %% %d == 0, "
                "K %% 64 == 0 and 16-byte aligned rows (M=%d N=%d K=%d)",
                bm[v], bn[v], bm[v], bn[v], g.M, g.N, g.K);
   }
   if (cut_requested)
-    LH_REQUIRE(vec_ok && !tb && g.ldc % 8 == 0 && g.N % 8 == 0,
+    LH_REQUIRE(vec_ok && !tb && g.ldc % 8 == 0 && g.N % 8 == 0 && direct_offsets_fit(g),
                "gemm: a split-K request needs untransposed operands, K %% 64 == 0, N %% 8 == 0 and 16-byte aligned rows "
                "(M=%d N=%d K=%d)", g.M, g.N, g.K);
   if (vec_ok) {
-    if (!tb && g.ldc % 8 == 0 && g.N % 8 == 0) {
+    if (!tb && g.ldc % 8 == 0 && g.N % 8 == 0 && direct_offsets_fit(g)) {
       if (tile == LH_GEMM_TILE_AUTO) {
         const int rc = gemm16_splitk<DT>(g, splitk, s);
         if (rc <= 0) return rc;
