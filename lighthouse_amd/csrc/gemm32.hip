@@ -17,7 +17,7 @@ constexpr int kBK32 = 32;
 // ---- direct-to-LDS kernel ---------------------------------------------------------------
 // Workgroup tile (64 TM) x (64 TN) x 32 with NW = 4 waves (2 x 2) or 8 waves (4 x 2, two per
 // SIMD: one wave's waits and barriers are covered by the other's MFMAs).  Both panels go global -> LDS with
-// global_load_lds_dwordx4 in their global orientation through a ring of NS stages, NS - 1 of
+// buffer_load_dwordx4 ... lds in their global orientation through a ring of NS stages, NS - 1 of
 // them in flight: at f32 rates a k-step lasts about as long as a global load takes, so a
 // register-staged double buffer stalls on every step.  A wave-wide load writes 1 KiB
 // contiguously, so rows cannot be padded; which 16-byte chunk of a row a lane fetches is
@@ -25,8 +25,18 @@ constexpr int kBK32 = 32;
 // k rows with (k / 4) odd, which are the rows the upper half wave reads).
 typedef __attribute__((address_space(3))) void lds32_void_t;
 
-__device__ __forceinline__ void async_copy16_f32(const float* gsrc, uint8_t* lds_wave_base) {
-  __builtin_amdgcn_global_load_lds(gsrc, (lds32_void_t*)lds_wave_base, 16, 0, 0);
+// 16 bytes per lane from a buffer resource over [base, base + 4 GiB) (+ per-lane and scalar byte
+// offsets) straight into LDS, 1 KiB per wave.  The buffer form of the LDS-DMA load: with the global
+// (flat-encoded) form in flight the compiler must assume LDS operations complete out of order and
+// waits for all of a wave's LDS reads before the first use of any; with this form it counts them.
+__device__ __forceinline__ void dma16_f32(const float* base, int lane_bytes, int scalar_bytes, uint8_t* lds_wave_base) {
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(base), 0, 0xffffffff, 0x00020000);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds32_void_t*)lds_wave_base, 16, lane_bytes, scalar_bytes, 0, 0);
+}
+// The tile's operand panels (64 TM rows of A, K rows of B) are addressed with 32-bit byte offsets.
+static inline bool direct32_offsets_fit(const GemmArgs& g) {
+  return g.lda < (1ll << 21) && (int64_t)g.K * g.ldb < (1ll << 29);
 }
 
 template <int TM, int TN, int NW_>
@@ -36,9 +46,11 @@ struct Direct32Ctx {
   static constexpr int LA = 8 * TM / NW;       // A loads per lane and stage
   static constexpr int LB = 8 * TN / NW;       // B loads per lane and stage
   static_assert(WTM >= 1 && LA >= 1 && LB >= 1, "tile too small for the wave count");
-  const float* a_src[LA];
-  const float* b_src[LB];
-  int64_t ldb;
+  const float* a_base;  // the tile's first A row and first B column (uniform)
+  const float* b_base;
+  int a_src[LA];        // the lane's byte offsets within the panels at k = 0
+  int b_src[LB];
+  int b_step;           // bytes between B stages (32 k rows)
   int wave, h;
   int a_off[WTM], a_swz[WTM];  // byte offset of the lane's A row, its swizzle
   int b_off[TN];               // byte offset of the lane's B column inside a k row (swizzle applied)
@@ -49,10 +61,10 @@ __device__ __forceinline__ void direct32_issue(const Direct32Ctx<TM, TN, NW>& c,
   using C = Direct32Ctx<TM, TN, NW>;
   constexpr int a_bytes = 64 * TM * 128;
 #pragma unroll
-  for (int i = 0; i < C::LA; ++i) async_copy16_f32(c.a_src[i] + kt * 32, stage + (C::NW * i + c.wave) * 1024);
+  for (int i = 0; i < C::LA; ++i) dma16_f32(c.a_base, c.a_src[i], kt * 128, stage + (C::NW * i + c.wave) * 1024);
 #pragma unroll
   for (int i = 0; i < C::LB; ++i)
-    async_copy16_f32(c.b_src[i] + (int64_t)(kt * 32) * c.ldb, stage + a_bytes + (C::NW * i + c.wave) * 1024);
+    dma16_f32(c.b_base, c.b_src[i], kt * c.b_step, stage + a_bytes + (C::NW * i + c.wave) * 1024);
 }
 
 // One k-step: refill `wr` (if `prefetch`) and multiply the stage in `rd`.
@@ -121,12 +133,16 @@ __device__ __forceinline__ void direct32_place(const GemmArgs& g, int id, Direct
   n0 = (id % tiles_n) * BN;
   const float* A = reinterpret_cast<const float*>(g.a);
   const float* B = reinterpret_cast<const float*>(g.b);
+  const int lda = (int)g.lda, ldb = (int)g.ldb;
+  c.a_base = A + (int64_t)m0 * g.lda;
+  c.b_base = B + n0;
+  c.b_step = 128 * ldb;
   // A: load i of wave w fills rows (NW i + w) 8 .. +8; lane -> row += lane / 8, LDS chunk lane % 8.
 #pragma unroll
   for (int i = 0; i < C::LA; ++i) {
     const int row = (C::NW * i + c.wave) * 8 + (lane >> 3);
     const int gc = (lane & 7) ^ ((row >> 1) & 7);
-    c.a_src[i] = A + (int64_t)(EDGE ? min(m0 + row, g.M - 1) : m0 + row) * g.lda + gc * 4;
+    c.a_src[i] = ((EDGE ? min(row, g.M - 1 - m0) : row) * lda + gc * 4) * 4;
   }
   // B: a k row is 16 TN chunks; load i of wave w fills k rows (NW i + w) (4 / TN) .. ; lane ->
   // row += lane / (16 TN), LDS chunk lane % (16 TN).
@@ -135,7 +151,7 @@ __device__ __forceinline__ void direct32_place(const GemmArgs& g, int id, Direct
     constexpr int chunks = 16 * TN;
     const int k = (C::NW * i + c.wave) * (64 / chunks) + lane / chunks;
     const int gc = (lane % chunks) ^ (8 * ((k >> 2) & 1));
-    c.b_src[i] = B + (int64_t)k * g.ldb + (EDGE ? min(n0 + gc * 4, g.N - 4) : n0 + gc * 4);
+    c.b_src[i] = (k * ldb + (EDGE ? min(gc * 4, g.N - 4 - n0) : gc * 4)) * 4;
   }
 }
 
@@ -159,8 +175,7 @@ __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
   const int r32 = lane & 31, h = lane >> 5;
 
   C c;
-  c.ldb = g.ldb;
-  c.wave = wave;
+    c.wave = wave;
   c.h = h;
 #pragma unroll
   for (int j = 0; j < WTM; ++j) {
@@ -333,7 +348,7 @@ int gemm32(const GemmArgs& g_in, hipStream_t s) {
     const int rc = gemm_padded<4>(g, kBK32, 4, s, [&](const GemmArgs& p) { return gemm32(p, s); });
     if (rc <= 0) return rc;
   }
-  if (vec_ok && g.N % 4 == 0) {
+  if (vec_ok && g.N % 4 == 0 && direct32_offsets_fit(g)) {
     // Tiles are counted with edge tiles in full (M, N need not be multiples of a tile).
     const int cus = num_cus();
     const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);

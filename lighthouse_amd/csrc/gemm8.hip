@@ -157,7 +157,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm8_fast(GemmArgs g) 
 
 // ---- direct-to-LDS kernel ---------------------------------------------------------------
 // Same structure as the 16-bit direct kernel: 256 x 256 workgroup tile, 8 waves (2 x 4, 128 x 64
-// per wave), panels global -> LDS with global_load_lds_dwordx4 in their global orientation, A ring
+// per wave), panels global -> LDS with buffer_load_dwordx4 ... lds in their global orientation, A ring
 // 2 stages x 128 k (256 rows x 128 bytes), B ring 4 stages x 64 k (64 rows x 256 bytes), one
 // v_mfma_f32_32x32x64_f8f6f4 k-step (64 k) per main-loop step with the barrier in the middle.
 // The k-contiguous A fragment (32 bytes per lane) is two 16-byte LDS reads; the n-contiguous B
@@ -175,6 +175,16 @@ typedef int i32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ void async8_copy16(const void* gsrc, uint8_t* lds_wave_base) {
   __builtin_amdgcn_global_load_lds(gsrc, (lds8_void_t*)lds_wave_base, 16, 0, 0);
+}
+// The buffer form of the same load (base + per-lane + scalar byte offsets).  The direct kernel uses
+// it: with the global (flat-encoded) form in flight the compiler must assume LDS operations complete
+// out of order and waits for all of a wave's LDS reads before the first use of any; with the buffer
+// form it counts them, and an MFMA waits for its own fragments only.
+__device__ __forceinline__ void dma8_16(const void* base, uint32_t lane_bytes, uint32_t scalar_bytes,
+                                        uint8_t* lds_wave_base) {
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0xffffffff, 0x00020000);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds8_void_t*)lds_wave_base, 16, (int)lane_bytes, (int)scalar_bytes, 0, 0);
 }
 
 struct D8Ctx {
@@ -197,11 +207,13 @@ struct D8Frags {
 
 __device__ __forceinline__ void d8_load_a(const D8Ctx& c, int sa, uint8_t* __restrict__ abuf) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) async8_copy16(c.a_base + (c.a_voff[i] + (uint32_t)(sa * 128)), abuf + (8 * i + c.wave) * 1024);
+  for (int i = 0; i < 4; ++i) dma8_16(c.a_base, c.a_voff[i], (uint32_t)(sa * 128), abuf + (8 * i + c.wave) * 1024);
 }
 __device__ __forceinline__ void d8_load_b(const D8Ctx& c, int sb, uint8_t* __restrict__ bbuf) {
+  // (the resource starts at the stage's first k row: lane offsets stay within 64 rows)
+  const uint8_t* stage_base = c.b_base + (int64_t)(sb * 64) * c.ldb;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) async8_copy16(c.b_base + (int64_t)(sb * 64) * c.ldb + c.b_voff[i], bbuf + (8 * i + c.wave) * 1024);
+  for (int i = 0; i < 2; ++i) dma8_16(stage_base, c.b_voff[i], 0u, bbuf + (8 * i + c.wave) * 1024);
 }
 
 // Fragments of one 64-k step: A bytes 64 kb .. +64 of the stage's rows (kb = 0 / 1), B stage bs.
