@@ -354,3 +354,62 @@ def test_nanogpt_small_batch_and_ragged_vocab_use_only_the_workspace():
     fixed = B * T * (C * (2 + 6 + 2 + 4) + 4 * C * 2) + 2 * B * T * C * 4
     assert need > fixed + C * 50264 * 2  # at least the padded lm_head weight on top of the fixed buffers
     del before
+
+
+def test_generic_form_module_at_the_fixture_size():
+    """The linalg.generic chain of test/opt/pipeline-check.mlir:27-46 at that fixture's own shapes
+    (256x1024 . 1024x2048, f32): the product accumulates into the passed C, then bias, then
+    max(., 0).  The module text is generated here, parsed by the MLIR-text front end and run
+    through the Runner; integer-valued operands make the f32 result exact in any summation order."""
+    from lighthouse_amd.execution import Runner
+    from lighthouse_amd.ingress.mlir_text import parse_payload_module
+
+    M, K, N = 256, 1024, 2048
+    t = lambda *dims: "tensor<" + "x".join(str(d) for d in dims) + "xf32>"
+    text = f"""
+#lhs = affine_map<(i, j, k) -> (i, k)>
+#rhs = affine_map<(i, j, k) -> (k, j)>
+#acc = affine_map<(i, j, k) -> (i, j)>
+#vec = affine_map<(i, j) -> (j)>
+#mat = affine_map<(i, j) -> (i, j)>
+module {{
+  func.func @entry(%a: {t(M, K)}, %b: {t(K, N)}, %bias: {t(N)}, %c: {t(M, N)}) -> {t(M, N)} {{
+    %p = linalg.generic {{indexing_maps = [#lhs, #rhs, #acc], iterator_types = ["parallel", "parallel", "reduction"]}} ins(%a, %b : {t(M, K)}, {t(K, N)}) outs(%c : {t(M, N)}) {{
+    ^bb0(%x: f32, %y: f32, %o: f32):
+      %m = arith.mulf %x, %y : f32
+      %s = arith.addf %m, %o : f32
+      linalg.yield %s : f32
+    }} -> {t(M, N)}
+    %q = linalg.generic {{indexing_maps = [#vec, #mat], iterator_types = ["parallel", "parallel"]}} ins(%bias : {t(N)}) outs(%p : {t(M, N)}) {{
+    ^bb0(%x: f32, %o: f32):
+      %s = arith.addf %x, %o : f32
+      linalg.yield %s : f32
+    }} -> {t(M, N)}
+    %zero = arith.constant 0.000000e+00 : f32
+    %r = linalg.generic {{indexing_maps = [#mat], iterator_types = ["parallel", "parallel"]}} outs(%q : {t(M, N)}) {{
+    ^bb0(%o: f32):
+      %s = arith.maximumf %o, %zero : f32
+      linalg.yield %s : f32
+    }} -> {t(M, N)}
+    return %r : {t(M, N)}
+  }}
+}}
+"""
+    module = parse_payload_module(text, ["entry"])
+    rng = np.random.default_rng(77)
+    a = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    bias = rng.integers(-40, 41, N).astype(np.float32)
+    c0 = rng.integers(-50, 51, (M, N)).astype(np.float32)
+    c = c0.copy()
+    Runner(module).execute("entry", [a, b, bias, c])
+    want = np.maximum(a.astype(np.float64) @ b.astype(np.float64) + c0 + bias[None, :], 0.0)
+    assert (want > 0).any() and (want == 0).any()
+    np.testing.assert_array_equal(c, want.astype(np.float32))
+    # Real-valued operands: the benchmark's f32 tolerance against the f64 product.
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    b = rng.standard_normal((K, N)).astype(np.float32)
+    c = c0.copy()
+    Runner(module).execute("entry", [a, b, bias, c])
+    assert_close(c, orc.matmul(a, b, c=c0, bias=bias, relu=True, accumulate_c=True), 1e-4,
+                 what="generic-form fixture 256x1024x2048 f32")
