@@ -209,6 +209,41 @@ class _Lowering:
 
         self._emit(node.name, "hip.gemm", run, bias=b_arg is not None, activation=act, residual=add_node is not None)
 
+    def _matmul(self, node, a_arg, b_arg, bias_arg=None):
+        """torch.matmul / mm / `@` with a 2-D right operand (and addmm with a vector bias): one GEMM.
+        A transposed view of a row-major matrix (`w.t()`) goes to the kernel as a transpose flag, not
+        as a copy; a following ReLU / tanh-GELU with no other user is fused into the epilogue."""
+        act, act_node = self._single_user_activation(node)
+        if act_node is not None:
+            self.fused[act_node.name] = node.name
+        a_f, b_f, bias_f = _resolver(a_arg), _resolver(b_arg), _resolver(bias_arg)
+
+        def operand(t):
+            """-> (matrix with unit inner stride, transposed?)"""
+            if t.stride(1) == 1 and t.stride(0) >= t.shape[1]:
+                return t, False
+            if t.stride(0) == 1 and t.stride(1) >= t.shape[0]:
+                return t.t(), True
+            return t.contiguous(), False
+
+        def run(env, act=act):
+            a, b, bias = a_f(env), b_f(env), bias_f(env)
+            if not (isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor)) or a.dim() < 2 or b.dim() != 2:
+                raise ValueError(f"{node.name}: matmul needs a [..., K] left and a [K, N] right operand "
+                                 "(batched right operands are not supported)")
+            if a.dtype != b.dtype:
+                raise ValueError(f"{node.name}: mixed-type matmul ({a.dtype} @ {b.dtype}) is not supported")
+            if bias is not None and (bias.dim() != 1 or bias.shape[0] != b.shape[1] or bias.dtype != a.dtype):
+                raise ValueError(f"{node.name}: addmm needs a vector bias of the result's width and type")
+            shape = (*a.shape[:-1], b.shape[1])
+            a2, ta = operand(a) if a.dim() == 2 else (_as_2d(a), False)
+            b2, tb = operand(b)
+            out = ops.gemm(a2, b2, bias.detach().contiguous() if bias is not None else None, relu=act == "relu",
+                           gelu=act == "gelu", transpose_a=ta, transpose_b=tb)
+            return out.view(shape)
+
+        self._emit(node.name, "hip.gemm", run, bias=bias_arg is not None, activation=act, residual=False)
+
     def _layer_norm(self, node, x_arg, shape, w_arg, b_arg, eps):
         if len(tuple(shape)) != 1:
             raise ValueError(f"{node.name}: LayerNorm over {tuple(shape)}: only the last dimension is supported")
@@ -363,6 +398,12 @@ class _Lowering:
         t = node.target
         if t in (torch._C._nn.linear, F.linear):
             return self._linear(node, node.args[0], node.args[1], self._kwarg(node, "bias", 2))
+        if t in (torch.matmul, operator.matmul, torch.mm):
+            return self._matmul(node, node.args[0], node.args[1])
+        if t is torch.addmm:
+            if self._kwarg(node, "beta", 3, 1) != 1 or self._kwarg(node, "alpha", 4, 1) != 1:
+                return self._fallback(node, "addmm(alpha, beta)")
+            return self._matmul(node, node.args[1], node.args[2], node.args[0])
         if t is F.layer_norm:
             return self._layer_norm(node, node.args[0], node.args[1], self._kwarg(node, "weight", 2),
                                     self._kwarg(node, "bias", 3), self._kwarg(node, "eps", 4, 1e-5))
@@ -394,6 +435,8 @@ class _Lowering:
             return self._unary(node, "relu", node.args[0])
         if node.target in ("add", "__add__"):
             return self._binary_add(node)
+        if node.target in ("matmul", "mm", "__matmul__"):
+            return self._matmul(node, node.args[0], node.args[1])
         return self._fallback(node, f"Tensor.{node.target}")
 
     def _call_module(self, node):

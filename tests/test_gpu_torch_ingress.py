@@ -105,3 +105,40 @@ def test_jit_function_benchmark_protocol():
     assert times.shape == (5,) and times.dtype == np.float64 and (times > 0).all()
     with pytest.raises(ValueError):
         jit(x.cpu())
+
+
+@pytest.mark.parametrize("dtype,rtol", [(torch.float32, 1e-4), (torch.bfloat16, 2e-2)])
+def test_compiled_matmul_nodes(dtype, rtol):
+    """Plain matmul graph nodes (torch.matmul, `@` on a transposed weight view, addmm, a 3-D left
+    operand): each runs as one GEMM, transposed views as transpose flags; integer-valued operands make
+    the f32 chain exact."""
+    from lighthouse_amd.ingress.torch import gpu_backend
+
+    class M(nn.Module):
+        def __init__(self, w, b):
+            super().__init__()
+            self.w, self.b = nn.Parameter(w), nn.Parameter(b)
+
+        def forward(self, x, y):
+            h = torch.relu(torch.matmul(x, y))            # [3, 40, 96] @ [96, 64], ReLU fused
+            h = h @ self.w.t()                             # w [128, 64] read as its transpose
+            return torch.addmm(self.b, h.flatten(0, 1), self.w)   # [120, 128] @ [128, 64] + b
+
+    g = torch.Generator().manual_seed(5)
+    ints = lambda *shape: torch.randint(-2, 3, shape, generator=g).float()  # noqa: E731
+    x, y, w, b = ints(3, 40, 96), ints(96, 64), ints(128, 64), ints(64)
+    model = M(w.clone(), b.clone()).cuda().to(dtype)
+    backend = gpu_backend()
+    compiled = torch.compile(model, backend=backend, dynamic=False)
+    with torch.no_grad():
+        out = compiled(x.cuda().to(dtype), y.cuda().to(dtype))
+    assert backend.last_jit_function.kinds == ["hip.gemm", "hip.gemm", "hip.gemm"]
+    assert out.shape == (120, 64) and out.dtype == dtype
+    rt = "f32" if dtype == torch.float32 else "bf16"
+    h = orc.matmul(_np(x).reshape(120, 96), _np(y), relu=True, result_type=rt)
+    h = orc.matmul(h, _np(w).T, result_type=rt)
+    ref = orc.matmul(h, _np(w), bias=_np(b), result_type=rt)
+    if dtype == torch.float32:
+        np.testing.assert_array_equal(_np(out), ref)
+    else:
+        assert_close(_np(out), ref, rtol, "compiled matmul nodes bf16")

@@ -132,3 +132,34 @@ def test_argument_resolvers_follow_nested_structures():
     const = (1, [2, 3], {"k": None}, slice(0, 4))
     assert _resolver(const)(env) is const  # no node inside: returned without a walk
     assert _resolver(None)(env) is None
+
+
+def test_plain_matmul_nodes_become_gemms():
+    """torch.matmul / `@` / mm / addmm with a 2-D right operand (the form of the KernelBench level-1
+    problems the reference's backend is driven with, tools/kernel-bench:443-452): one GEMM each,
+    a following ReLU fused; a batched right operand is refused when the plan runs."""
+
+    class M(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.w = nn.Parameter(torch.randn(16, 8))
+            self.b = nn.Parameter(torch.randn(16))
+
+        def forward(self, x, y):
+            h = torch.relu(torch.matmul(x, y))   # [4, 8] @ [8, 8]
+            h = h @ self.w.t()                   # transposed view of a row-major weight
+            h = torch.addmm(self.b, h, torch.mm(self.w, self.w.t()))
+            return h.matmul(self.w)
+
+    jit = gpu_backend()(torch.fx.symbolic_trace(M()), [torch.randn(4, 8), torch.randn(8, 8)])
+    assert jit.kinds == ["hip.gemm"] * 5
+    gemms = [s for s in jit.plan if s.kind == "hip.gemm"]
+    assert [g.detail["activation"] for g in gemms] == ["relu", None, None, None, None]
+    assert [g.detail["bias"] for g in gemms] == [False, False, False, True, False]
+
+    class Scaled(nn.Module):
+        def forward(self, x, y):
+            return torch.addmm(x, x, y, beta=0.5)
+
+    with pytest.raises(ValueError, match="addmm"):
+        gpu_backend()(torch.fx.symbolic_trace(Scaled()), [torch.randn(4, 4), torch.randn(4, 4)])
