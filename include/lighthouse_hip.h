@@ -219,7 +219,9 @@ int lh_hip_gemm_fp8_ws(void* out, const void* a_q, const void* b_q, float scale_
  * parameters of the reference's fused-attention schedule (examples/xegpu/fused_attention.py:109-145,
  * lighthouse/schedule/xegpu/fused_attention_schedule.py): query rows per wave (64: two 32-row
  * sub-tiles share every K/V fragment, 256-row workgroups; 32: 128-row workgroups, twice as many)
- * and, for the 32-row kernel, the depth of the K/V ring (3 stages: three workgroups per CU; 4: two).
+ * and, for the 32-row kernel, the depth of the K/V ring (3 stages: three workgroups per CU; 4: two);
+ * LH_ATTN_KSPLIT_2 gives a workgroup of the 64-row kernel two groups of four waves that walk the two
+ * halves of the key range side by side and are combined at the end (LH_ATTN_KSPLIT_1: never).
  * 0 lets the library choose by shape.  A request that does not apply fails with LH_ERR_INVALID. */
 #define LH_ATTN_CAUSAL 0x1
 #define LH_ATTN_ROWS_MASK 0x300
@@ -228,6 +230,9 @@ int lh_hip_gemm_fp8_ws(void* out, const void* a_q, const void* b_q, float scale_
 #define LH_ATTN_STAGES_MASK 0xC00
 #define LH_ATTN_STAGES_3 0x400
 #define LH_ATTN_STAGES_4 0x800
+#define LH_ATTN_KSPLIT_MASK 0x3000
+#define LH_ATTN_KSPLIT_1 0x1000
+#define LH_ATTN_KSPLIT_2 0x2000
 typedef struct lh_strides3 {
   int64_t z, h, t;
 } lh_strides3;

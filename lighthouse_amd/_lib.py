@@ -33,6 +33,7 @@ GEMM_SPLITK_MASK = 0x3800
 ATTN_CAUSAL = 1
 ATTN_ROWS = {0: 0, 32: 0x100, 64: 0x200}
 ATTN_STAGES = {0: 0, 3: 0x400, 4: 0x800}
+ATTN_KSPLIT = {0: 0, 1: 0x1000, 2: 0x2000}
 
 # lh_elementwise_kind
 EW_SOFTMAX, EW_GELU, EW_BIAS, EW_ADD, EW_CAST = range(5)

@@ -123,7 +123,8 @@ __device__ __forceinline__ void attn_issue_loads(const AttnCtx& c, int jt, int T
 // One key tile (64 keys) for the wave's two 32-row query sub-tiles.  `rd` holds the tile, `wr`
 // is the ring slot that receives a later tile meanwhile (separate restrict pointers so that LDS
 // reads do not wait for the asynchronous writes).
-template <int DT, int NQ, bool RAGGED, bool AHEAD>
+// (KS only separates the instantiations of the two kernels that share the other parameters.)
+template <int DT, int NQ, bool RAGGED, bool AHEAD, int KS = 1>
 __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, const u32x4 (&qf)[NQ][4],
                                           f32x16 (&acc_o)[NQ][2], float (&m_run)[NQ], float (&l_run)[NQ],
                                           f32x16 (&neg_m)[NQ], const uint8_t* __restrict__ rd,
@@ -280,17 +281,25 @@ __device__ __forceinline__ void causal_block_of(int L, int G, int R, int nqb, in
 // reads, V^T fragments come from ds_read_b64_tr_b16 on the row-major V tile.  Rows of a tile
 // are 128 bytes and cannot be padded (a wave-wide load writes 1 KiB contiguous), so the
 // 16-byte chunk a lane fetches is XOR-swizzled: K chunk ^ ((key / 2) % 8), V chunk ^ 4 ((key / 2) % 2).
-template <int DT, int NQ, int NS, bool RAGGED>
-__global__ void __launch_bounds__(256, (NQ == 1 && NS == 3 ? 3 : 2)) attention16_kernel(AttnArgs a) {
+// KS = 2: the workgroup has two such groups of 4 waves on the SAME 256 query rows, each with a ring
+// of its own and its own half of the key tiles; at the end the second group hands its (unnormalised
+// output, offset, row sum) over through LDS and the first combines the two.  Same waves per CU as
+// two workgroups of 4, but the two halves of a query block's key range run side by side and end
+// together: the chain of key tiles a causal problem's heaviest query block has to walk is half as long.
+template <int DT, int NQ, int NS, bool RAGGED, int KS = 1>
+__global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attention16_kernel(AttnArgs a) {
   constexpr int kRowsPerWave = 32 * NQ, kRowsPerGroup = 4 * kRowsPerWave;
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn[];
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn_all[];
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_wg = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave = wave_wg & 3, ksplit = wave_wg >> 2;  // row group within the 256 rows, key half
+  uint8_t* const smem_attn = smem_attn_all + ksplit * (NS * kAttnStageBytes);
   const int r32 = lane & 31, h = lane >> 5;
   const int nqb = (a.T + kRowsPerGroup - 1) / kRowsPerGroup;
   int qb, bh;
   if (a.causal) {
-    causal_block_of(blockIdx.x, gridDim.x, a.cus, nqb, a.Z * a.H, qb, bh);
+    // (KS = 2: one workgroup per CU at a time, the others start as CUs free up: plainly heaviest first.)
+    causal_block_of(blockIdx.x, gridDim.x, KS == 2 ? (int)gridDim.x : a.cus, nqb, a.Z * a.H, qb, bh);
   } else {
     qb = blockIdx.x;
     bh = blockIdx.y;
@@ -378,25 +387,75 @@ __global__ void __launch_bounds__(256, (NQ == 1 && NS == 3 ? 3 : 2)) attention16
   }
 
   const int kv_end = a.causal ? min(a.T, q0 + kRowsPerGroup) : a.T;
-  const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
+  const int ntiles_all = (kv_end + kKvTile - 1) / kKvTile;
+  // This group's key tiles are t_first .. t_first + ntiles - 1; every wave of the workgroup walks
+  // `steps` iterations (the larger of the two counts), because the barrier in the loop is the
+  // workgroup's: a group that has run out of tiles neither loads nor computes in the rest.
+  const int steps = KS == 2 ? (ntiles_all + 1) / 2 : ntiles_all;
+  const int t_first = ksplit * steps;
+  const int ntiles = KS == 2 ? (ksplit ? ntiles_all - steps : steps) : ntiles_all;
   constexpr int kAttnStages = NS;  // K/V ring depth, 3 or 4
 #pragma unroll
   for (int st = 0; st < kAttnStages - 1; ++st)
-    if (st < ntiles) attn_issue_loads<RAGGED>(c, st, a.T, smem_attn + st * kAttnStageBytes);
+    if (st < ntiles) attn_issue_loads<RAGGED>(c, t_first + st, a.T, smem_attn + st * kAttnStageBytes);
 
-  for (int jt = 0; jt < ntiles; ++jt) {
+  for (int it = 0; it < steps; ++it) {
     // 4 loads per lane and stage; the NS - 2 younger stages may stay in flight.  One asm block: a
     // __syncthreads() would add a fence that waits for ALL outstanding loads.
-    const int younger = min(ntiles - 1 - jt, kAttnStages - 2);
+    const int younger = min(ntiles - 1 - it, kAttnStages - 2);
     if (younger >= 2) asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
     else if (younger == 1) asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    const int jt = t_first + it;
     const int j0 = jt * kKvTile;
-    const bool active = wave_valid && (!a.causal || (j0 <= wq0 + kRowsPerWave - 1));
+    const bool active = wave_valid && (KS == 1 || it < ntiles) && (!a.causal || (j0 <= wq0 + kRowsPerWave - 1));
     const bool need_mask = (a.causal && (j0 + kKvTile - 1 > wq0)) || (RAGGED && j0 + kKvTile > a.T);
-    const int nxt = jt + kAttnStages - 1;
-    attn_tile<DT, NQ, RAGGED, !(NQ == 1 && NS == 3) && !(NQ == 2 && RAGGED)>(c, a, qf, acc_o, m_run, l_run, neg_m, smem_attn + (jt % kAttnStages) * kAttnStageBytes,
-                  smem_attn + (nxt % kAttnStages) * kAttnStageBytes, nxt, nxt < ntiles, j0, wq0, active, need_mask);
+    const int nxt = it + kAttnStages - 1;
+    attn_tile<DT, NQ, RAGGED, !(NQ == 1 && NS == 3) && !(NQ == 2 && RAGGED), KS>(c, a, qf, acc_o, m_run, l_run, neg_m, smem_attn + (it % kAttnStages) * kAttnStageBytes,
+                  smem_attn + (nxt % kAttnStages) * kAttnStageBytes, t_first + nxt, nxt < ntiles, j0, wq0, active, need_mask);
+  }
+
+  if constexpr (KS == 2) {
+    // Hand-over through the (now idle) rings: block (wave, qt, j), four 16-byte groups of 64 lanes each,
+    // then the offsets and row sums.  Every wave of the workgroup passes both barriers.
+    f32x4* const xo = reinterpret_cast<f32x4*>(smem_attn_all);
+    float* const xs = reinterpret_cast<float*>(smem_attn_all + 4 * NQ * 2 * 4 * 64 * 16);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (ksplit == 1 && wave_valid) {
+#pragma unroll
+      for (int qt = 0; qt < NQ; ++qt) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            xo[(((wave * NQ + qt) * 2 + j) * 4 + g) * 64 + lane] =
+                f32x4{acc_o[qt][j][4 * g], acc_o[qt][j][4 * g + 1], acc_o[qt][j][4 * g + 2], acc_o[qt][j][4 * g + 3]};
+        xs[((wave * NQ + qt) * 2 + 0) * 64 + lane] = m_run[qt];
+        xs[((wave * NQ + qt) * 2 + 1) * 64 + lane] = l_run[qt];
+      }
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (ksplit == 1 || !wave_valid) return;
+#pragma unroll
+    for (int qt = 0; qt < NQ; ++qt) {
+      // Offsets are per query row (equal in the two lanes that share it), sums per lane.  A side that
+      // saw no visible key has offset -inf, sum 0 and a zero accumulator, and gets the factor 0.
+      const float m_b = xs[((wave * NQ + qt) * 2 + 0) * 64 + lane];
+      const float l_b = xs[((wave * NQ + qt) * 2 + 1) * 64 + lane];
+      const float m_a = m_run[qt];
+      const float m_ab = fmaxf(m_a, m_b);
+      const float f_a = (m_a == -INFINITY) ? 0.0f : exp2_fast(m_a - m_ab);
+      const float f_b = (m_b == -INFINITY) ? 0.0f : exp2_fast(m_b - m_ab);
+      l_run[qt] = l_run[qt] * f_a + l_b * f_b;
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 o_b = xo[(((wave * NQ + qt) * 2 + j) * 4 + g) * 64 + lane];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc_o[qt][j][4 * g + e] = acc_o[qt][j][4 * g + e] * f_a + o_b[e] * f_b;
+        }
+    }
   }
 
   // acc_o[qt][j][v] = O[q = wq0 + 32 qt + r32][d = 32 j + 8 (v/4) + 4 h + v%4] * l
@@ -625,10 +684,10 @@ __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
     }
 }
 
-template <int DT, int NQ, int NS, bool RAGGED>
+template <int DT, int NQ, int NS, bool RAGGED, int KS = 1>
 static int attention16_launch_ragged(const AttnArgs& a, hipStream_t s) {
-  auto kern = attention16_kernel<DT, NQ, NS, RAGGED>;
-  constexpr size_t lds = (size_t)NS * kAttnStageBytes;
+  auto kern = attention16_kernel<DT, NQ, NS, RAGGED, KS>;
+  constexpr size_t lds = (size_t)KS * NS * kAttnStageBytes;
   static bool configured = false;
   if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -637,7 +696,7 @@ static int attention16_launch_ragged(const AttnArgs& a, hipStream_t s) {
   }
   const int nqb = (a.T + 128 * NQ - 1) / (128 * NQ);
   const dim3 grid = a.causal ? dim3(nqb * a.Z * a.H) : dim3(nqb, a.Z * a.H);
-  LH_LAUNCH(kern, grid, dim3(256), lds, s, a);
+  LH_LAUNCH(kern, grid, dim3(256 * KS), lds, s, a);
   return check_launch("attention16");
 }
 
@@ -669,24 +728,42 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
   // (A partial last key tile also takes the 32-rows-per-wave kernels: the 64-row one has no
   // registers left for the clamped loads and would spill.)
   const int rows_req = a.request & LH_ATTN_ROWS_MASK, stages_req = a.request & LH_ATTN_STAGES_MASK;
-  if (rows_req == LH_ATTN_ROWS_64) {
+  const int ksplit_req = a.request & LH_ATTN_KSPLIT_MASK;
+  if (rows_req == LH_ATTN_ROWS_64 && ksplit_req != LH_ATTN_KSPLIT_2) {
     LH_REQUIRE(a.T % kKvTile == 0, "attention: 64 query rows per wave need a sequence length that is a multiple of %d",
                kKvTile);
     LH_REQUIRE(stages_req != LH_ATTN_STAGES_3, "attention: the 64-rows-per-wave kernel has a 4-stage ring only");
     return attention16_launch_nq<DT, 2, 4>(a, s);
   }
+  if (ksplit_req == LH_ATTN_KSPLIT_2) {
+    // Two groups of four waves per workgroup, each on half of the key tiles (64 rows per wave, 4 stages).
+    LH_REQUIRE(rows_req != LH_ATTN_ROWS_32 && stages_req != LH_ATTN_STAGES_3,
+               "attention: the split key range exists for 64 query rows per wave and a 4-stage ring only");
+    LH_REQUIRE(a.T % kKvTile == 0, "attention: 64 query rows per wave need a sequence length that is a multiple of %d",
+               kKvTile);
+    return attention16_launch_ragged<DT, 2, 4, false, 2>(a, s);
+  }
+  // Unasked, the split pays where at most one 256-row workgroup falls on a CU but more than half
+  // the CUs get one: a lone group of four waves leaves each SIMD with a single wave, and splitting the
+  // rows instead (the 32-row kernel) halves the reuse of every K/V fragment.  Non-causal
+  // [1,16,4096] 77 -> 72 us, [1,8,8192] 152 -> 132 us.  Causal problems are bound by the
+  // total of their key tiles, not by the longest chain ([4,16,2048] 47 -> 53 us with the split).
+  if (!ksplit_req && !rows_req && !stages_req && !a.causal && a.T % kKvTile == 0 && groups64 <= a.cus &&
+      2 * groups64 > a.cus)
+    return attention16_launch_ragged<DT, 2, 4, false, 2>(a, s);
   if (rows_req == LH_ATTN_ROWS_32 || stages_req) {
     const int64_t groups32 = (int64_t)((a.T + 127) / 128) * a.Z * a.H;
-    const bool three = stages_req ? stages_req == LH_ATTN_STAGES_3 : groups32 > a.cus;
+    const bool three = stages_req ? stages_req == LH_ATTN_STAGES_3 : groups32 >= 3 * (int64_t)a.cus;
     if (three) return attention16_launch_nq<DT, 1, 3>(a, s);
     return attention16_launch_nq<DT, 1, 4>(a, s);
   }
   if (groups64 < limit || short_rows || a.T % kKvTile != 0) {
-    // With more than one 128-row workgroup per CU a ring of 3 stages (48 KiB) lets three of them
+    // With three 128-row workgroups or more per CU a ring of 3 stages (48 KiB) lets three of them
     // share a CU instead of two ([8,12,1024] causal 26.7 -> 25.3 us, [16,16,512] causal 24.2 ->
-    // 22.3); a problem that does not fill the CUs is better off with the deeper ring.
+    // 22.3); a problem that cannot put a third one there is better off with the deeper ring
+    // (causal [1,16,4096] 57.9 -> 53.9 us, [1,8,8192] 108 -> 98.8, [2,16,2048] 32.7 -> 30.6, [1,40,2048] 36.2 -> 33.7).
     const int64_t groups32 = (int64_t)((a.T + 127) / 128) * a.Z * a.H;
-    if (groups32 > a.cus) return attention16_launch_nq<DT, 1, 3>(a, s);
+    if (groups32 >= 3 * (int64_t)a.cus) return attention16_launch_nq<DT, 1, 3>(a, s);
     return attention16_launch_nq<DT, 1, 4>(a, s);
   }
   return attention16_launch_nq<DT, 2, 4>(a, s);
@@ -1250,11 +1327,12 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   a.so = so; a.sq = sq; a.sk = sk; a.sv = sv;
   a.scale = scale;
   a.scale_log2e = scale * 1.4426950408889634f;
-  LH_REQUIRE((causal & ~(int32_t)(LH_ATTN_CAUSAL | LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK)) == 0 &&
-                 (causal & LH_ATTN_ROWS_MASK) != LH_ATTN_ROWS_MASK && (causal & LH_ATTN_STAGES_MASK) != LH_ATTN_STAGES_MASK,
+  LH_REQUIRE((causal & ~(int32_t)(LH_ATTN_CAUSAL | LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK | LH_ATTN_KSPLIT_MASK)) == 0 &&
+                 (causal & LH_ATTN_ROWS_MASK) != LH_ATTN_ROWS_MASK && (causal & LH_ATTN_STAGES_MASK) != LH_ATTN_STAGES_MASK &&
+                 (causal & LH_ATTN_KSPLIT_MASK) != LH_ATTN_KSPLIT_MASK,
              "lh_hip_attention: unknown bits 0x%x in the causal / request word", causal);
   a.causal = (causal & LH_ATTN_CAUSAL) ? 1 : 0;
-  a.request = causal & (LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK);
+  a.request = causal & (LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK | LH_ATTN_KSPLIT_MASK);
   LH_REQUIRE(a.request == 0 || (fast && dtype != LH_F32),
              "lh_hip_attention: query-row / ring-depth requests apply to 16-bit tensors with head_dim %d and aligned rows",
              kHeadDim);

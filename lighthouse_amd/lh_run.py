@@ -33,7 +33,7 @@ from .pipeline.descriptor import Descriptor, PipelineDescriptor
 # describe a kernel it does not select.
 KERNEL_PARAMETERS = {
     "matmul": {"tile_m", "tile_n", "split_k"},
-    "attention": {"q_rows_per_wave", "kv_stages"},
+    "attention": {"q_rows_per_wave", "kv_stages", "kv_split"},
     "matmul_fp8": set(), "mlp": set(), "layer_norm": set(), "elementwise": set(), "nanogpt_block": set(),
     "gpt_fused": set(),
 }
@@ -67,16 +67,18 @@ def _apply_matmul(fn, params: dict, notes: list[str]) -> None:
 
 
 def _apply_attention(fn, params: dict, notes: list[str]) -> None:
-    rows, stages = params.get("q_rows_per_wave", 0), params.get("kv_stages", 0)
-    if rows not in _lib.ATTN_ROWS or stages not in _lib.ATTN_STAGES:
-        raise ValueError(f"stage 'attention': q_rows_per_wave must be 32 or 64 and kv_stages 3 or 4, got {rows} / {stages}")
-    if not (rows or stages):
+    rows, stages, split = params.get("q_rows_per_wave", 0), params.get("kv_stages", 0), params.get("kv_split", 0)
+    if rows not in _lib.ATTN_ROWS or stages not in _lib.ATTN_STAGES or split not in _lib.ATTN_KSPLIT:
+        raise ValueError(f"stage 'attention': q_rows_per_wave must be 32 or 64, kv_stages 3 or 4 and kv_split 1 or 2, "
+                         f"got {rows} / {stages} / {split}")
+    if not (rows or stages or split):
         return
     if fn.attrs.dtype == _lib.F32 or fn.args[0].shape[-1] != 64:
         notes.append(f"stage 'attention': variant requests apply to 16-bit tensors with head dimension 64, not to "
                      f"@{fn.name}; the library chooses")
         return
-    fn.attrs.causal = (fn.attrs.causal & _lib.ATTN_CAUSAL) | _lib.ATTN_ROWS[rows] | _lib.ATTN_STAGES[stages]
+    fn.attrs.causal = ((fn.attrs.causal & _lib.ATTN_CAUSAL) | _lib.ATTN_ROWS[rows] | _lib.ATTN_STAGES[stages]
+                       | _lib.ATTN_KSPLIT[split])
 
 
 def apply_stage(module: PayloadModule, stage: str, notes: list[str]) -> None:

@@ -203,10 +203,11 @@ def _strides3(t) -> _lib.Strides3:
     return _lib.Strides3(t.stride(0), t.stride(1), t.stride(2))
 
 
-def attention(q, k, v, *, causal=False, scale=None, out=None, rows_per_wave=None, stages=None):
+def attention(q, k, v, *, causal=False, scale=None, out=None, rows_per_wave=None, stages=None, kv_split=None):
     """Fused attention forward on [Z,H,T,d] tensors (any strides with unit stride along d).
-    `rows_per_wave` (32 or 64) and `stages` (3 or 4, K/V ring of the 32-row kernel) request a
-    kernel variant for 16-bit tensors with head dimension 64; with neither given the
+    `rows_per_wave` (32 or 64), `stages` (3 or 4, K/V ring of the 32-row kernel) and `kv_split`
+    (2: two wave groups per workgroup on halves of the key range, 1: never) request a
+    kernel variant for 16-bit tensors with head dimension 64; with none given the
     tuned-parameter database is asked, then the library chooses by shape."""
     if q.dim() != 4 or q.shape != k.shape or q.shape != v.shape:
         raise ValueError("attention expects Q, K, V of equal 4-D shape [Z,H,T,d]")
@@ -220,15 +221,18 @@ def attention(q, k, v, *, causal=False, scale=None, out=None, rows_per_wave=None
             raise ValueError("innermost stride must be 1")
     _need_cuda(q, k, v, out)
     Z, H, T, d = q.shape
-    if rows_per_wave is None and stages is None and d == 64 and q.dtype != torch.float32 and _rows_aligned16(q, k, v, out):
+    if rows_per_wave is None and stages is None and kv_split is None and d == 64 and q.dtype != torch.float32 and _rows_aligned16(q, k, v, out):
         from .tuning.tile_db import active_db
 
         db = active_db()
         if db is not None:
-            rows_per_wave, stages = db.lookup_attention("bf16" if q.dtype == torch.bfloat16 else "f16", Z * H, T, d, causal)
-    _require((rows_per_wave or 0) in _lib.ATTN_ROWS and (stages or 0) in _lib.ATTN_STAGES,
-             f"rows_per_wave must be one of {sorted(_lib.ATTN_ROWS)[1:]}, stages one of {sorted(_lib.ATTN_STAGES)[1:]}")
-    word = (_lib.ATTN_CAUSAL if causal else 0) | _lib.ATTN_ROWS[rows_per_wave or 0] | _lib.ATTN_STAGES[stages or 0]
+            rows_per_wave, stages, kv_split = db.lookup_attention("bf16" if q.dtype == torch.bfloat16 else "f16", Z * H, T, d, causal)
+    _require((rows_per_wave or 0) in _lib.ATTN_ROWS and (stages or 0) in _lib.ATTN_STAGES
+             and (kv_split or 0) in _lib.ATTN_KSPLIT,
+             f"rows_per_wave must be one of {sorted(_lib.ATTN_ROWS)[1:]}, stages one of {sorted(_lib.ATTN_STAGES)[1:]}, "
+             f"kv_split one of {sorted(_lib.ATTN_KSPLIT)[1:]}")
+    word = ((_lib.ATTN_CAUSAL if causal else 0) | _lib.ATTN_ROWS[rows_per_wave or 0] | _lib.ATTN_STAGES[stages or 0]
+            | _lib.ATTN_KSPLIT[kv_split or 0])
     _lib.check(_lib.load().lh_hip_attention(
         out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), Z, H, T, d,
         _strides3(out), _strides3(q), _strides3(k), _strides3(v),

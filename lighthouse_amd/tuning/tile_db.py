@@ -63,19 +63,22 @@ class TileDB:
         return f"attn:{dtype}:{BH}x{T}x{d}:{'causal' if causal else 'full'}"
 
     def lookup_attention(self, dtype: str, BH: int, T: int, d: int, causal: bool):
-        """(rows_per_wave or None, stages or None) for this problem (BH = batch x heads)."""
+        """(rows_per_wave, stages, kv_split), each None where the entry leaves the choice to the
+        library, for this problem (BH = batch x heads)."""
         entry = self.entries.get(self.attention_key(dtype, BH, T, d, causal))
         if not entry:
-            return None, None
-        return entry.get("rows_per_wave"), entry.get("stages")
+            return None, None, None
+        return entry.get("rows_per_wave"), entry.get("stages"), entry.get("kv_split")
 
     def record_attention(self, dtype: str, BH: int, T: int, d: int, causal: bool, rows_per_wave, stages, time_us: float,
-                         tflops: float) -> None:
+                         tflops: float, kv_split=None) -> None:
         entry = {"time_us": round(float(time_us), 3), "tflops": round(float(tflops), 2)}
         if rows_per_wave:
             entry["rows_per_wave"] = int(rows_per_wave)
         if stages:
             entry["stages"] = int(stages)
+        if kv_split:
+            entry["kv_split"] = int(kv_split)
         self.entries[self.attention_key(dtype, BH, T, d, causal)] = entry
 
     def save(self, path: str | None = None) -> str:

@@ -96,7 +96,7 @@ def _time_tile(res, M, N, K, dtype, tile, nruns, nwarmup, split_k=None):
     res["throughput"] = 2.0 * M * N * K / seconds / 1e12
 
 
-def _time_attention(res, BH, T, d, causal, dtype, rows_per_wave, stages, nruns, nwarmup):
+def _time_attention(res, BH, T, d, causal, dtype, rows_per_wave, stages, kv_split, nruns, nwarmup):
     import torch
 
     from .. import ops
@@ -107,12 +107,12 @@ def _time_attention(res, BH, T, d, causal, dtype, rows_per_wave, stages, nruns, 
     q, k, v = (torch.randn(1, BH, T, d, device="cuda").to(tdt) for _ in range(3))
     out = torch.empty_like(q)
     for _ in range(nwarmup):
-        ops.attention(q, k, v, causal=causal, out=out, rows_per_wave=rows_per_wave, stages=stages)
+        ops.attention(q, k, v, causal=causal, out=out, rows_per_wave=rows_per_wave, stages=stages, kv_split=kv_split)
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(nruns):
-        ops.attention(q, k, v, causal=causal, out=out, rows_per_wave=rows_per_wave, stages=stages)
+        ops.attention(q, k, v, causal=causal, out=out, rows_per_wave=rows_per_wave, stages=stages, kv_split=kv_split)
     stop.record()
     torch.cuda.synchronize()
     seconds = start.elapsed_time(stop) * 1e-3 / nruns
@@ -194,23 +194,26 @@ def tune_shape(M: int, N: int, K: int, dtype: str = "bf16", db: TileDB | None = 
             base is None or best["time_us"] * MIN_GAIN <= base["time_us"]):
         db.record(dtype, M, N, K, (best["tile_m"], best["tile_n"]) if best["tile_m"] else None, best["time_us"],
                   best["tflops"], split_k=best["split_k"] or None)
+    elif best is not None and db is not None:
+        db.entries.pop(db.key(dtype, M, N, K), None)  # an older entry no longer beats the library
     return best
 
 
-ATTENTION_SETTINGS = ((64, None), (32, 3), (32, 4))
+ATTENTION_SETTINGS = ((64, None, 1), (64, None, 2), (32, 3, None), (32, 4, None))
 
 
 def tune_attention(BH: int, T: int, causal: bool, dtype: str = "bf16", db: TileDB | None = None,
                    logger: CSVLogger | None = None, nruns: int = 300, nwarmup: int = 200, timeout: float = 60.0,
                    isolate: bool = True, d: int = 64) -> dict | None:
-    """The same for the head-dimension-64 attention kernel: query rows per wave x K/V ring depth."""
+    """The same for the head-dimension-64 attention kernel: query rows per wave x K/V ring depth x
+    split of the key range between two wave groups."""
     best = base = None
     settings = [s for s in ATTENTION_SETTINGS if s[0] != 64 or T % 64 == 0]
-    for rows, stages in [(None, None), *settings]:
-        res = _trial(_time_attention, (BH, T, d, causal, dtype, rows, stages, nruns, nwarmup), isolate, timeout)
+    for rows, stages, split in [(None, None, None), *settings]:
+        res = _trial(_time_attention, (BH, T, d, causal, dtype, rows, stages, split, nruns, nwarmup), isolate, timeout)
         row = {"dtype": dtype, "BH": BH, "T": T, "d": d, "causal": int(causal), "rows_per_wave": rows or 0,
-               "stages": stages or 0, "time_us": round(res["time"] * 1e6, 3), "tflops": round(res["throughput"], 2),
-               "error": res["error"]}
+               "stages": stages or 0, "kv_split": split or 0, "time_us": round(res["time"] * 1e6, 3),
+               "tflops": round(res["throughput"], 2), "error": res["error"]}
         if logger is not None:
             logger.log(row)
         ok = not res["error"] and res["time"] > 0
@@ -221,7 +224,9 @@ def tune_attention(BH: int, T: int, causal: bool, dtype: str = "bf16", db: TileD
     if best is not None and db is not None and best["rows_per_wave"] and (
             base is None or best["time_us"] * MIN_GAIN <= base["time_us"]):
         db.record_attention(dtype, BH, T, d, causal, best["rows_per_wave"], best["stages"] or None, best["time_us"],
-                            best["tflops"])
+                            best["tflops"], kv_split=best["kv_split"] or None)
+    elif best is not None and db is not None:
+        db.entries.pop(db.attention_key(dtype, BH, T, d, causal), None)  # an older entry no longer beats the library
     return best
 
 

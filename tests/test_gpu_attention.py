@@ -251,6 +251,31 @@ def test_attention_variant_requests(rows, stages, causal):
     assert (out.float() - auto.float()).abs().max() <= 2e-2 * auto.float().abs().max()
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(2, 3, 512, 64), (1, 2, 64, 64), (1, 2, 192, 64), (1, 3, 320, 64), (2, 2, 1088, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_attention_split_key_range(shape, causal, dtype):
+    """LH_ATTN_KSPLIT_2: two groups of four waves per workgroup walk the two halves of a query block's
+    key tiles and are combined at the end.  Sequence lengths with an odd tile count, a single tile (the
+    second group has nothing to do), a last query block that is partly past the end, strided views
+    (the [B, T, 3C] projection buffer of a transformer block): every head against the oracle."""
+    from lighthouse_amd import ops
+
+    Z, H, T, d = shape
+    g = torch.Generator(device="cuda").manual_seed(33)
+    qkv = torch.randn(Z, T, 3, H, d, device="cuda", generator=g).to(dtype)
+    q, k, v = (qkv[:, :, i].transpose(1, 2) for i in range(3))       # [Z, H, T, d] views, row stride 3 H d
+    out = ops.attention(q, k, v, causal=causal, kv_split=2)
+    rnd = orc.round_bf16 if dtype == torch.bfloat16 else orc.round_f16
+    for z in range(Z):
+        for h in range(H):
+            ref = orc.attention(*(t[z, h].float().cpu().numpy() for t in (q, k, v)), causal=causal)
+            assert_close(out[z, h].float().cpu().numpy(), rnd(ref), 2e-2 if dtype == torch.bfloat16 else 5e-3,
+                         f"attention kv_split=2 {shape} causal={causal} head ({z},{h})")
+    whole = ops.attention(q, k, v, causal=causal, kv_split=1, rows_per_wave=64)
+    assert (out.float() - whole.float()).abs().max() <= (2e-2 if dtype == torch.bfloat16 else 5e-3) * whole.float().abs().max()
+
+
 def test_attention_variant_request_errors():
     from lighthouse_amd import ops
 
@@ -259,6 +284,10 @@ def test_attention_variant_request_errors():
         ops.attention(q, q, q, rows_per_wave=48)
     with pytest.raises(ValueError, match="4-stage ring only"):
         ops.attention(q, q, q, rows_per_wave=64, stages=3)
+    with pytest.raises(ValueError, match="kv_split"):
+        ops.attention(q, q, q, kv_split=3)
+    with pytest.raises(ValueError, match="split key range"):
+        ops.attention(q, q, q, kv_split=2, rows_per_wave=32)
     q100 = torch.zeros(1, 2, 100, 64, device="cuda", dtype=torch.bfloat16)
     with pytest.raises(ValueError, match="multiple of 64"):
         ops.attention(q100, q100, q100, rows_per_wave=64)

@@ -180,6 +180,9 @@ def test_stage_parameters_all_act_or_fail(tmp_path):
     y.write_text('Pipeline:\n  - kernel: "attention{q_rows_per_wave=32 kv_stages=3}"\n')
     apply_stage(att, str(y), notes)
     assert att.lookup("payload").attrs.causal == _lib.ATTN_CAUSAL | _lib.ATTN_ROWS[32] | _lib.ATTN_STAGES[3]
+    y.write_text('Pipeline:\n  - kernel: "attention{kv_split=2}"\n')
+    apply_stage(att, str(y), notes)
+    assert att.lookup("payload").attrs.causal == _lib.ATTN_CAUSAL | _lib.ATTN_KSPLIT[2]
     y.write_text('Pipeline:\n  - kernel: "attention{q_rows_per_wave=48}"\n')
     with pytest.raises(ValueError, match="q_rows_per_wave"):
         apply_stage(att, str(y), notes)

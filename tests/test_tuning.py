@@ -88,8 +88,8 @@ def test_settings_and_database_kinds(tmp_path):
     assert again.lookup_gemm("bf16", 16, 8192, 8192) == (None, 8)
     assert again.lookup_gemm("bf16", 8192, 768, 768) == ((128, 128), None)
     assert again.lookup_gemm("bf16", 1, 1, 1) == (None, None)
-    assert again.lookup_attention("bf16", 64, 2048, 64, True) == (32, 3)
-    assert again.lookup_attention("bf16", 64, 2048, 64, False) == (None, None)
+    assert again.lookup_attention("bf16", 64, 2048, 64, True) == (32, 3, None)
+    assert again.lookup_attention("bf16", 64, 2048, 64, False) == (None, None, None)
     default = use_default_db()
     assert default is None or isinstance(default, TileDB)
     if default is not None:
