@@ -275,6 +275,21 @@ __device__ __forceinline__ void causal_block_of(int L, int G, int R, int nqb, in
   bh = r % bhn;
 }
 
+// Launch order of a non-causal problem.  Workgroups are dealt to the 8 XCDs in turn (linear id
+// modulo 8), and each XCD has an L2 of its own: the query blocks of one (batch, head), which all read
+// that head's K and V, are given ids that agree modulo 8, so that a K/V tile comes from memory once
+// per head and not once per query block.  (With the plain (query block, head) grid and 8 query
+// blocks, every block of a head sat on a different XCD.)
+__device__ __forceinline__ void xcd_block_of(int L, int nqb, int bhn, int& qb, int& bh) {
+  if (bhn % 8 == 0) {
+    bh = (L % 8) + 8 * (L / (8 * nqb));
+    qb = (L / 8) % nqb;
+  } else {
+    qb = L % nqb;
+    bh = L / nqb;
+  }
+}
+
 // 16-bit kernel.  A workgroup owns 256 query rows of one (batch, head): 4 waves x 64 rows (two
 // 32-row sub-tiles per wave share every K and V fragment).  K/V tiles of 64 keys go global ->
 // LDS with buffer_load_dwordx4 ... lds through a ring of NS stages; K fragments are 16-byte LDS
@@ -301,8 +316,7 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
     // (KS = 2: one workgroup per CU at a time, the others start as CUs free up: plainly heaviest first.)
     causal_block_of(blockIdx.x, gridDim.x, KS == 2 ? (int)gridDim.x : a.cus, nqb, a.Z * a.H, qb, bh);
   } else {
-    qb = blockIdx.x;
-    bh = blockIdx.y;
+    xcd_block_of((int)(blockIdx.y * gridDim.x + blockIdx.x), nqb, a.Z * a.H, qb, bh);
   }
   const int z = bh / a.H, hd = bh % a.H;
   const int q0 = qb * kRowsPerGroup;
@@ -406,6 +420,18 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
     if (younger >= 2) asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
     else if (younger == 1) asm volatile("s_waitcnt vmcnt(4)\n\ts_barrier" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    if constexpr (NQ == 2 && KS == 1) {
+      // Two workgroups share a CU, one wave of each per SIMD, and at equal priority the older wave
+      // wins every contested issue slot: the workgroup that started first runs ahead (its 32 key
+      // tiles of a [4,16,2048] launch in 51 us against 65 us for its partner, which then finishes
+      // alone at a lone workgroup's lower rate).  Taking turns at the higher priority, tile by tile
+      // and in opposite phase on the two wave slots, keeps the pair closer together (0.8 % of the
+      // launch; 3.5 % before the query blocks of a head shared an XCD).  The 32-row kernels, three
+      // workgroups per CU or long causal chains, lost 3-5 % with it.
+      const unsigned slot = __builtin_amdgcn_s_getreg((3u << 11) | (0u << 6) | 4u);  // HW_ID: wave slot within its SIMD
+      if (((unsigned)it ^ slot) & 1u) __builtin_amdgcn_s_setprio(1);
+      else __builtin_amdgcn_s_setprio(0);
+    }
     const int jt = t_first + it;
     const int j0 = jt * kKvTile;
     const bool active = wave_valid && (KS == 1 || it < ntiles) && (!a.causal || (j0 <= wq0 + kRowsPerWave - 1));
@@ -603,8 +629,9 @@ __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, h = lane >> 5;
   const int nqb = (a.T + kQBlock - 1) / kQBlock;
-  int qb = blockIdx.x, bh = blockIdx.y;
+  int qb, bh;
   if (a.causal) causal_block_of(blockIdx.x, gridDim.x, a.cus, nqb, a.Z * a.H, qb, bh);
+  else xcd_block_of((int)(blockIdx.y * gridDim.x + blockIdx.x), nqb, a.Z * a.H, qb, bh);
   const int z = bh / a.H, hd = bh % a.H;
   const int q0 = qb * kQBlock;
   const int wq0 = q0 + wave * 32;
@@ -790,8 +817,8 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
   // Causal work grows with the query block: a 1-D grid lists the blocks heaviest first over ALL
   // (batch, head) pairs, so that the long ones do not start last.
   const int bhn = a.Z * a.H;
-  const int qb = a.causal ? nqb - 1 - (int)blockIdx.x / bhn : (int)blockIdx.x;
-  const int bh = a.causal ? (int)blockIdx.x % bhn : (int)blockIdx.y;
+  int qb = nqb - 1 - (int)blockIdx.x / bhn, bh = (int)blockIdx.x % bhn;
+  if (!a.causal) xcd_block_of((int)(blockIdx.y * gridDim.x + blockIdx.x), nqb, bhn, qb, bh);
   const int z = bh / a.H, hd = bh % a.H;
   const int q0 = qb * 128, wq0 = q0 + 32 * wave;
   const bool wave_valid = wq0 < a.T;
@@ -1079,8 +1106,8 @@ __global__ void __launch_bounds__(256, 2) attention16_d128_kernel(AttnArgs a) {
   const int r32 = lane & 31, h = lane >> 5;
   const int nqb = (a.T + 127) / 128;
   const int bhn = a.Z * a.H;
-  const int qb = a.causal ? nqb - 1 - (int)blockIdx.x / bhn : (int)blockIdx.x;  // causal: heaviest first over all heads
-  const int bh = a.causal ? (int)blockIdx.x % bhn : (int)blockIdx.y;
+  int qb = nqb - 1 - (int)blockIdx.x / bhn, bh = (int)blockIdx.x % bhn;  // causal: heaviest first over all heads
+  if (!a.causal) xcd_block_of((int)(blockIdx.y * gridDim.x + blockIdx.x), nqb, bhn, qb, bh);
   const int z = bh / a.H, hd = bh % a.H;
   const int q0 = qb * 128, wq0 = q0 + 32 * wave;
   const bool wave_valid = wq0 < a.T;
