@@ -129,7 +129,7 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
                                           f32x16 (&acc_o)[NQ][2], float (&m_run)[NQ], float (&l_run)[NQ],
                                           f32x16 (&neg_m)[NQ], const uint8_t* __restrict__ rd,
                                           uint8_t* __restrict__ wr, int next_jt,
-                                          bool prefetch, int j0, int wq0, bool active, bool need_mask) {
+                                          bool prefetch, int j0, int wq0, bool active, bool need_mask, bool first) {
   if (prefetch) attn_issue_loads<RAGGED>(c, next_jt, a.T, wr);
   if (!active) return;
   const uint8_t* ks = rd;
@@ -183,17 +183,24 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
     // slow path, so that its first visible maximum becomes the offset and l >= 1 from then on.
     // Only there is the row maximum computed, the offset raised, l and acc rescaled and P
     // recomputed, for the whole wave.
+    // `first` (the workgroup's first key tile: no row has an offset yet, l and acc are zero) goes
+    // straight to the slow path, without the pass that would only find that out and without
+    // rescaling zeros.
     const float mc = m_run[qt];
     float p[2][16];
     float l_tile = 0.0f;
+    bool move_offset = true;
+    if (!first) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        p[i][v] = exp2_fast(s_acc[qt][i][v]);
-        l_tile += p[i][v];
-      }
-    if (__builtin_amdgcn_ballot_w64(!(l_tile <= kOffsetSlack) || mc == -INFINITY) != 0) {
+        for (int v = 0; v < 16; ++v) {
+          p[i][v] = exp2_fast(s_acc[qt][i][v]);
+          l_tile += p[i][v];
+        }
+      move_offset = __builtin_amdgcn_ballot_w64(!(l_tile <= kOffsetSlack) || mc == -INFINITY) != 0;
+    }
+    if (move_offset) {
       float mx = fmaxf(s_acc[qt][0][0], s_acc[qt][1][0]);
 #pragma unroll
       for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[qt][0][v]), s_acc[qt][1][v]);
@@ -204,12 +211,14 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
       const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
       const float delta = m_safe - m_old;
       const float alpha = exp2_fast(mc - m_safe);
-      l_run[qt] *= alpha;
       m_run[qt] = m_new;
+      if (!first) {
+        l_run[qt] *= alpha;
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc_o[qt][j][v] *= alpha;
+          for (int v = 0; v < 16; ++v) acc_o[qt][j][v] *= alpha;
+      }
       l_tile = 0.0f;
 #pragma unroll
       for (int i = 0; i < 2; ++i)
@@ -438,7 +447,7 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
     const bool need_mask = (a.causal && (j0 + kKvTile - 1 > wq0)) || (RAGGED && j0 + kKvTile > a.T);
     const int nxt = it + kAttnStages - 1;
     attn_tile<DT, NQ, RAGGED, !(NQ == 1 && NS == 3) && !(NQ == 2 && RAGGED), KS>(c, a, qf, acc_o, m_run, l_run, neg_m, smem_attn + (it % kAttnStages) * kAttnStageBytes,
-                  smem_attn + (nxt % kAttnStages) * kAttnStageBytes, t_first + nxt, nxt < ntiles, j0, wq0, active, need_mask);
+                  smem_attn + (nxt % kAttnStages) * kAttnStageBytes, t_first + nxt, nxt < ntiles, j0, wq0, active, need_mask, it == 0);
   }
 
   if constexpr (KS == 2) {
