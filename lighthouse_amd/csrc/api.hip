@@ -301,7 +301,7 @@ int lh_hip_nanogpt_block(float* y, const float* x, const lh_nanogpt_block_params
   auto bias_flag = [](const void* b) -> uint32_t { return b ? LH_GEMM_HAS_BIAS : 0u; };
   int rc;
   // ln1 = LN(x), rounded to the matmul input type.
-  if ((rc = lh_hip_layer_norm(ln, x, p->ln1_g, p->ln1_b, rows, C, eps, LH_F32, dtype, s))) return rc;
+  if ((rc = layer_norm(ln, x, p->ln1_g, p->ln1_b, rows, C, eps, LH_F32, dtype, false, s))) return rc;
   if (p->w_qkv) {
     // qkv = ln1 Wqkv + bqkv
     if ((rc = gemm_run(qkv, nullptr, ln, p->w_qkv, p->b_qkv, rows, 3 * C, C, C, 3 * C, 3 * C, dtype, dtype, bdt,
@@ -331,7 +331,7 @@ int lh_hip_nanogpt_block(float* y, const float* x, const lh_nanogpt_block_params
                      bias_flag(p->b_o) | LH_GEMM_ACCUMULATE_C, s, &ws)))
     return rc;
   // ln2 = LN(a)
-  if ((rc = lh_hip_layer_norm(ln, a, p->ln2_g, p->ln2_b, rows, C, eps, LH_F32, dtype, s))) return rc;
+  if ((rc = layer_norm(ln, a, p->ln2_g, p->ln2_b, rows, C, eps, LH_F32, dtype, false, s))) return rc;
   // h = act(ln2 W1 + b1)
   const uint32_t act = cfg.activation == LH_ACT_RELU ? LH_GEMM_HAS_RELU : LH_GEMM_HAS_GELU;
   if ((rc = gemm_run(hid, nullptr, ln, p->w_fc, p->b_fc, rows, hidden, C, C, hidden, hidden, dtype, dtype, bdt,
@@ -383,7 +383,7 @@ int lh_hip_nanogpt_forward(float* logits, const float* x, const lh_nanogpt_block
     cur = nxt;
   }
   // hf = LN_f(h) rounded to the matmul input type (first area of the block workspace), then lm_head.
-  int rc = lh_hip_layer_norm(workspace, cur, lnf_g, lnf_b, rows, C, eps, LH_F32, dtype, s);
+  int rc = layer_norm(workspace, cur, lnf_g, lnf_b, rows, C, eps, LH_F32, dtype, false, s);
   if (rc) return rc;
   Scratch ws;
   ws.base = w + block_ws + 2 * align256((size_t)rows * C * 4);

@@ -197,6 +197,10 @@ struct PlanningScope {  // marks the calling thread as running a size query
   } while (0)
 // The current device's statically allocated scratch array (runtime.hip): its device address and size.
 int static_scratch(char** base, size_t* bytes);
+// lh_hip_layer_norm with the choice of store: `streaming` (what the public entry point uses) writes
+// the rows with non-temporal stores; a caller whose next kernel reads them at once passes false.
+int layer_norm(void* out, const void* x, const float* gamma, const float* beta, int64_t M, int64_t N, float eps,
+               int32_t x_dtype, int32_t out_dtype, bool streaming, void* stream);
 // Compute units of the current device (cached; 256 if the query fails).
 int num_cus();
 
