@@ -33,6 +33,7 @@ struct AttnArgs {
   int causal;
   int cus;  // compute units of the device (causal launch order)
   int request = 0;  // LH_ATTN_ROWS_* | LH_ATTN_STAGES_* bits of the call (0: the library chooses)
+  int d = 0;        // head dimension of the call (the padded kernels mask the columns from d on)
 };
 
 template <int DT>
@@ -805,16 +806,20 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
   return attention16_launch_nq<DT, 2, 4>(a, s);
 }
 
-// 16-bit tensors, head dimension D = 32 DB other than 64 (32, 96, 128, 192, 256): the same
+// 16-bit tensors, head dimension D = 32 DB (32, 96, 128, 192, 256; 64 and 128 for padded calls): the same
 // transposed formulation on the matrix cores (S^T = K Q^T, O^T = V^T P^T, a lane owns a query row)
 // without the streaming machinery of the head-dimension-64 kernel.  A workgroup owns 128 query
 // rows (4 waves x 32); a tile of 64 keys is copied through registers into LDS, K and V row-major
 // with rows padded by 16 bytes (V^T fragments through ds_read_b64_tr_b16), two barriers per tile.  Row statistics follow the plain online-softmax recurrence (maximum per
 // tile).  Any sequence length: keys past the end are loaded from the last key and masked, rows
 // past the end are computed on the last row and not stored.
-template <int DT, int DB>
+// PAD: the head dimension a.d is a multiple of 8 below D.  The 16-byte chunks of Q, K and V from
+// column a.d on are zeros in registers and LDS (they add nothing to S, and their output columns
+// are not stored), so the result is that of head dimension a.d exactly.
+template <int DT, int DB, bool PAD>
 __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kernel(AttnArgs a) {
   constexpr int D = 32 * DB;
+  const int d_real = PAD ? a.d : D;
   constexpr int KROW = D + 8;  // elements per LDS row
   extern __shared__ __attribute__((aligned(16))) uint8_t smem_anyd[];
   uint16_t* Ks = reinterpret_cast<uint16_t*>(smem_anyd);  // [64][KROW]
@@ -847,7 +852,9 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
     const int row = min(wq0 + r32, a.T - 1);
 #pragma unroll
     for (int sd = 0; sd < D / 16; ++sd) {
-      const u32x4 raw = *reinterpret_cast<const u32x4*>(Q + (int64_t)row * a.sq.t + 16 * sd + 8 * h);
+      const bool inside = !PAD || 16 * sd + 8 * h < d_real;
+      u32x4 raw = *reinterpret_cast<const u32x4*>(Q + (int64_t)row * a.sq.t + (inside ? 16 * sd + 8 * h : 0));
+      if (PAD && !inside) raw = u32x4{0u, 0u, 0u, 0u};
       u32x4 scaled;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
@@ -877,8 +884,12 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
     for (int i = 0; i < DB; ++i) {
       const int c = tid + 256 * i, key = c / (D / 8), ch = c % (D / 8);
       const int kg = min(j0 + key, a.T - 1);
-      const u32x4 kv = *reinterpret_cast<const u32x4*>(K + (int64_t)kg * a.sk.t + 8 * ch);
-      const u32x4 vv = *reinterpret_cast<const u32x4*>(V + (int64_t)kg * a.sv.t + 8 * ch);
+      // (a masked chunk loads the row's first chunk and drops it: no branch around the loads)
+      const bool inside = !PAD || 8 * ch < d_real;
+      const int col = inside ? 8 * ch : 0;
+      u32x4 kv = *reinterpret_cast<const u32x4*>(K + (int64_t)kg * a.sk.t + col);
+      u32x4 vv = *reinterpret_cast<const u32x4*>(V + (int64_t)kg * a.sv.t + col);
+      if (PAD && !inside) kv = vv = u32x4{0u, 0u, 0u, 0u};
       *reinterpret_cast<u32x4*>(Ks + key * KROW + 8 * ch) = kv;
       *reinterpret_cast<u32x4*>(Vs + key * KROW + 8 * ch) = vv;
     }
@@ -978,7 +989,7 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
     for (int g = 0; g < 4; ++g) {
       u32x2 w = {pack2<DT>(acc_o[j][4 * g] * inv_l, acc_o[j][4 * g + 1] * inv_l),
                  pack2<DT>(acc_o[j][4 * g + 2] * inv_l, acc_o[j][4 * g + 3] * inv_l)};
-      *reinterpret_cast<u32x2*>(orow + 32 * j + 8 * g + 4 * h) = w;
+      if (!PAD || 32 * j + 8 * g + 4 * h < d_real) *reinterpret_cast<u32x2*>(orow + 32 * j + 8 * g + 4 * h) = w;
     }
 }
 
@@ -1203,11 +1214,11 @@ static int attention16_d128_launch(const AttnArgs& a, hipStream_t s) {
   return check_launch("attention16_d128");
 }
 
-template <int DT, int DB>
+template <int DT, int DB, bool PAD = false>
 static int attention16_anyd_launch(const AttnArgs& a, hipStream_t s) {
   constexpr int D = 32 * DB;
   constexpr size_t lds = (size_t)2 * kKvTile * (D + 8) * 2 + (DB >= 8 ? 4 * 32 * D * 2 : 0);
-  auto kern = attention16_anyd_kernel<DT, DB>;
+  auto kern = attention16_anyd_kernel<DT, DB, PAD>;
   static bool configured = false;
   if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1229,8 +1240,17 @@ static int attention16_anyd_dispatch(const AttnArgs& a, int d, hipStream_t s) {
     case 128: return attention16_d128_launch<DT>(a, s);
     case 192: return attention16_anyd_launch<DT, 6>(a, s);
     case 256: return attention16_anyd_launch<DT, 8>(a, s);
-    default: return 1;
+    default: break;
   }
+  // Other multiples of 8: the next instantiated width, the columns from d on masked.
+  if (d % 8 != 0) return 1;
+  if (d < 32) return attention16_anyd_launch<DT, 1, true>(a, s);
+  if (d < 64) return attention16_anyd_launch<DT, 2, true>(a, s);
+  if (d < 96) return attention16_anyd_launch<DT, 3, true>(a, s);
+  if (d < 128) return attention16_anyd_launch<DT, 4, true>(a, s);
+  if (d < 192) return attention16_anyd_launch<DT, 6, true>(a, s);
+  if (d < 256) return attention16_anyd_launch<DT, 8, true>(a, s);
+  return 1;
 }
 
 int attention16_anyd(const AttnArgs& a, int d, int dtype, hipStream_t s) {
@@ -1363,6 +1383,7 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   a.so = so; a.sq = sq; a.sk = sk; a.sv = sv;
   a.scale = scale;
   a.scale_log2e = scale * 1.4426950408889634f;
+  a.d = (int)d;
   LH_REQUIRE((causal & ~(int32_t)(LH_ATTN_CAUSAL | LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK | LH_ATTN_KSPLIT_MASK)) == 0 &&
                  (causal & LH_ATTN_ROWS_MASK) != LH_ATTN_ROWS_MASK && (causal & LH_ATTN_STAGES_MASK) != LH_ATTN_STAGES_MASK &&
                  (causal & LH_ATTN_KSPLIT_MASK) != LH_ATTN_KSPLIT_MASK,

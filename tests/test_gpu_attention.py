@@ -177,12 +177,45 @@ def test_attention_other_head_dims_on_the_matrix_cores(shape, dtype, elt, causal
 
 
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype,elt", [(torch.bfloat16, "bf16"), (torch.float16, "f16")])
+@pytest.mark.parametrize("shape", [(1, 2, 200, 8), (2, 2, 130, 24), (1, 3, 257, 40), (1, 2, 64, 56), (2, 1, 300, 72),
+                                   (1, 2, 129, 80), (1, 1, 200, 104), (1, 2, 192, 120), (1, 1, 140, 160),
+                                   (1, 1, 131, 224), (1, 1, 70, 248)])
+def test_attention_padded_head_dims_on_the_matrix_cores(shape, dtype, elt, causal):
+    """16-bit tensors whose head dimension is a multiple of 8 without a kernel width of its own run
+    on the next wider matrix-core kernel with the columns from head_dim on masked.  The tensors are
+    views into wider buffers whose other columns hold NaN (inputs) or a marker (output): the result
+    is that of the head dimension itself and nothing outside it is written."""
+    from lighthouse_amd import ops
+
+    Z, H, T, D = shape
+    W = D + 8 * (1 + (T + D) % 3)  # row stride of the buffers
+    rng = np.random.default_rng(sum(shape) + 5 * causal)
+    q, k, v = (orc.round_to(rng.standard_normal(shape).astype(np.float32), elt) for _ in range(3))
+    ref = orc.attention(q, k, v, causal=causal, result_type=elt)
+
+    def widened(x):
+        buf = torch.full((Z, H, T, W), float("nan"), dtype=dtype, device="cuda")
+        buf[..., :D] = _dev(x, dtype)
+        return buf[..., :D]
+
+    out_buf = torch.full((Z, H, T, W), 7.0, dtype=dtype, device="cuda")
+    out = out_buf[..., :D]
+    ops.attention(widened(q), widened(k), widened(v), causal=causal, out=out)
+    assert_close(_host(out), ref, 2e-2, f"attention {shape} {elt} causal={causal}")
+    assert torch.all(out_buf[..., D:] == 7.0), "columns past head_dim were written"
+    # contiguous tensors give the same bits
+    out_c = ops.attention(_dev(q, dtype), _dev(k, dtype), _dev(v, dtype), causal=causal)
+    assert torch.equal(out_c, out)
+
+
+@pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype,elt,rtol", [(torch.bfloat16, "bf16", 2e-2), (torch.float32, "f32", 1e-4)])
 @pytest.mark.parametrize("shape", [(1, 2, 100, 40), (2, 1, 77, 64), (1, 1, 130, 128), (1, 3, 64, 64), (1, 1, 1, 8),
-                                   (1, 1, 200, 256)])
+                                   (1, 1, 200, 256), (1, 2, 100, 36), (1, 1, 70, 100), (1, 1, 33, 3)])
 def test_attention_any_shape(shape, dtype, elt, rtol, causal):
     """Head dimensions (and element types) the MFMA kernels do not take run on the generic kernel
-    with the same rounding points (16-bit head_dim 32 / 64 / 96 / 128 / 192 / 256 and f32 head_dim 64
+    with the same rounding points (16-bit head dimensions that are multiples of 8 and f32 head_dim 64
     take the MFMA kernels at any sequence length)."""
     from lighthouse_amd import ops
 
