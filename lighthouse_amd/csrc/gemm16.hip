@@ -392,7 +392,9 @@ __device__ __forceinline__ void direct_place(const GemmArgs& g, int id, DirectCt
   constexpr int BM = Cfg::BM, BN = Cfg::BN;
   const int lane = lane_now();
   const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-  constexpr int GROUP_M = 4;
+  // Tiles are walked in groups of GROUP_M tile rows: 1024 rows of A.  For the 128-row tiles that
+  // is 8 up to K = 1536 (1-3 % faster than 4 there; 0.3-1.4 % slower from K = 3072 on).
+  const int GROUP_M = (BM == 128 && g.K <= 1536) ? 8 : 4;
   const int group_size = GROUP_M * tiles_n;
   const int first_m = (id / group_size) * GROUP_M;
   const int gm = min(tiles_m - first_m, GROUP_M);
