@@ -339,6 +339,7 @@ __device__ __forceinline__ void direct_wait_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
+
 // Steps kt (even) and kt + 1 of the main loop; both have a successor step.  On entry f0 holds
 // the fragments of (step kt, first k-half).  a_cur = A stage kt / 2, a_nxt = the next A stage,
 // b0 / b1 / b2 = B stages kt, kt + 1, kt + 2.  The refill pointers alias a_cur, b0 and b1: every
@@ -426,6 +427,38 @@ __device__ __forceinline__ void direct_place(const GemmArgs& g, int id, DirectCt
   }
 }
 
+// The same two steps with ONE barrier, in the middle of the odd step: the rings work as two halves
+// of 64 k.  At the barrier every read of this pair's stages has returned and the next pair's
+// stages (issued at the previous barrier, 64 k ago) are awaited in full; the pair after that is
+// then requested into this pair's buffers.
+template <int DT, int TM, int TN>
+__device__ __forceinline__ void direct_step_pair_1b(const DirectCtx<TM, TN>& c, f32x16 (&acc)[TN][TM],
+                                                    DirectFrags<TM, TN>& f0, const uint8_t* __restrict__ a_cur,
+                                                    const uint8_t* __restrict__ a_nxt, const uint8_t* __restrict__ b0,
+                                                    const uint8_t* __restrict__ b1, const uint8_t* __restrict__ b2,
+                                                    uint8_t* __restrict__ a_refill, uint8_t* __restrict__ b_refill0,
+                                                    uint8_t* __restrict__ b_refill1, int kt, int nk) {
+  DirectFrags<TM, TN> f1;
+  direct_read_frags(c, a_cur, b0, 1, 1, f1);
+  direct_mfma<DT>(acc, f0);
+  direct_interleave_hint<TM, TN>();
+  direct_read_frags(c, a_cur, b1, 2, 0, f0);
+  direct_mfma<DT>(acc, f1);
+  direct_interleave_hint<TM, TN>();
+  direct_read_frags(c, a_cur, b1, 3, 1, f1);
+  direct_mfma<DT>(acc, f0);
+  direct_interleave_hint<TM, TN>();
+  direct_wait_barrier<0>();
+  if (kt + 4 < nk) {
+    direct_load_a(c, kt / 2 + 2, a_refill);
+    direct_load_b(c, kt + 4, b_refill0);
+    direct_load_b(c, kt + 5, b_refill1);
+  }
+  direct_read_frags(c, a_nxt, b2, 0, 0, f0);
+  direct_mfma<DT>(acc, f1);
+  direct_interleave_hint<TM, TN>();
+}
+
 // First loads of a tile: A stages 0, 1 and B stages 0 .. 3 (nk = K / 32 >= 2).
 template <int TM, int TN>
 __device__ __forceinline__ void direct_prologue(const DirectCtx<TM, TN>& c, int nk, uint8_t* __restrict__ ring) {
@@ -466,6 +499,9 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
                                                 uint8_t* smem_d, int nk, bool stores_behind, bool staged, int n_base,
                                                 u32x2 (&bias)[TN][4]) {
   using Cfg = DirectCfg<TM, TN>;
+  // The 256 x 256 tile, whose 64 k last about 1.7 us, runs with one barrier per 64 k (4096^3 109.8 ->
+  // 108.3 us); for the smaller tiles 64 k of look-ahead is too short (2048^3 21.4 -> 24.5 us).
+  constexpr bool kOneBarrier = TM == 4 && TN == 2;
   uint8_t* const abuf = smem_d;
   uint8_t* const bbuf = smem_d + Cfg::kBBase;
   if (stores_behind) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(Cfg::kStagedStores) : "memory");
@@ -479,7 +515,8 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
     uint8_t* b0 = bbuf + (kt & 3) * Cfg::kBBytes;
     uint8_t* b1 = bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
     uint8_t* b2 = bbuf + ((kt + 2) & 3) * Cfg::kBBytes;
-    direct_step_pair<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
+    if constexpr (kOneBarrier) direct_step_pair_1b<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
+    else direct_step_pair<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
   }
   {
     // Last two steps: nothing left to load; stage nk - 1 of B must have landed.
@@ -490,7 +527,7 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
     if (staged) direct_load_bias<TN, EDGE>(g, n_base, bias);
     direct_read_frags(c, a_cur, b0, 1, 1, f1);
     direct_mfma<DT>(acc, f0);
-    direct_wait_barrier<0>();
+    if constexpr (!kOneBarrier) direct_wait_barrier<0>();  // (one barrier per pair: awaited at the pair before)
     direct_read_frags(c, a_cur, b1, 2, 0, f0);
     direct_mfma<DT>(acc, f1);
     direct_read_frags(c, a_cur, b1, 3, 1, f1);
