@@ -12,6 +12,8 @@
 //
 // Generic kernel: any shape, stride and transpose combination, 64 x 64 x 32 tiles with
 // bounds-checked scalar loads.
+#include <type_traits>
+
 #include "gemm_common.h"
 
 namespace lh {
@@ -499,9 +501,12 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
                                                 uint8_t* smem_d, int nk, bool stores_behind, bool staged, int n_base,
                                                 u32x2 (&bias)[TN][4]) {
   using Cfg = DirectCfg<TM, TN>;
-  // The 256 x 256 tile, whose 64 k last about 1.7 us, runs with one barrier per 64 k (4096^3 109.8 ->
-  // 108.3 us); for the smaller tiles 64 k of look-ahead is too short (2048^3 21.4 -> 24.5 us).
-  constexpr bool kOneBarrier = TM == 4 && TN == 2;
+  // One barrier per 64 k (loads one 64-k half of the rings ahead) or two (B three 32-k stages
+  // ahead).  One is 1-3 % faster for every tile with a 256 side (4096^3 109.8 -> 108.3 us) and, when
+  // two workgroups share a compute unit, 2-7 % for the 128 x 128 tile (M = 8192, N = 768, K = 3072:
+  // 46.0 -> 42.9 us); a lone 128 x 128 workgroup has nobody to cover the shorter look-ahead
+  // (2048^3 22.7 -> 24.2 us) and keeps two.
+  const bool one_barrier = TM * TN > 2 || g.one_barrier;
   uint8_t* const abuf = smem_d;
   uint8_t* const bbuf = smem_d + Cfg::kBBase;
   if (stores_behind) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(Cfg::kStagedStores) : "memory");
@@ -509,14 +514,21 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
   DirectFrags<TM, TN> f0;
   direct_read_frags(c, abuf, bbuf, 0, 0, f0);
   int kt = 0;
-  for (; kt + 2 < nk; kt += 2) {
+  auto pair = [&](auto one) {
     uint8_t* a_cur = abuf + ((kt >> 1) & 1) * Cfg::kABytes;
     uint8_t* a_nxt = abuf + (((kt >> 1) + 1) & 1) * Cfg::kABytes;
     uint8_t* b0 = bbuf + (kt & 3) * Cfg::kBBytes;
     uint8_t* b1 = bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
     uint8_t* b2 = bbuf + ((kt + 2) & 3) * Cfg::kBBytes;
-    if constexpr (kOneBarrier) direct_step_pair_1b<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
+    if constexpr (decltype(one)::value) direct_step_pair_1b<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
     else direct_step_pair<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
+  };
+  if constexpr (TM * TN > 2) {
+    for (; kt + 2 < nk; kt += 2) pair(std::true_type{});
+  } else if (one_barrier) {
+    for (; kt + 2 < nk; kt += 2) pair(std::true_type{});
+  } else {
+    for (; kt + 2 < nk; kt += 2) pair(std::false_type{});
   }
   {
     // Last two steps: nothing left to load; stage nk - 1 of B must have landed.
@@ -527,7 +539,7 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
     if (staged) direct_load_bias<TN, EDGE>(g, n_base, bias);
     direct_read_frags(c, a_cur, b0, 1, 1, f1);
     direct_mfma<DT>(acc, f0);
-    if constexpr (!kOneBarrier) direct_wait_barrier<0>();  // (one barrier per pair: awaited at the pair before)
+    if (!one_barrier) direct_wait_barrier<0>();  // (one barrier per pair: awaited at the pair before)
     direct_read_frags(c, a_cur, b1, 2, 0, f0);
     direct_mfma<DT>(acc, f1);
     direct_read_frags(c, a_cur, b1, 3, 1, f1);
@@ -790,7 +802,9 @@ static int launch_direct_edge(const GemmArgs& g, hipStream_t s) {
   }
   const int ntiles = ((g.M + Cfg::BM - 1) / Cfg::BM) * ((g.N + Cfg::BN - 1) / Cfg::BN);
   const int resident = num_cus() * (2 * lds <= 160 * 1024 ? 2 : 1);
-  LH_LAUNCH(kern, dim3(ntiles < resident ? ntiles : resident), dim3(512), lds, s, g);
+  GemmArgs ga = g;
+  ga.one_barrier = ntiles > num_cus();
+  LH_LAUNCH(kern, dim3(ntiles < resident ? ntiles : resident), dim3(512), lds, s, ga);
   return check_launch("gemm16_direct");
 }
 
@@ -938,6 +952,7 @@ static int gemm16_splitk(const GemmArgs& g, uint32_t request, hipStream_t s) {
   p.out_dt = LH_F32;
   p.bias = nullptr;
   p.flags = 0;
+  p.one_barrier = 0;  // B is streamed from memory here: the deeper look-ahead wins (M = 16, N = K = 8192: 26.7 against 27.4 us)
   const bool edge = g.M % Cfg::BM != 0 || g.N % Cfg::BN != 0;
   auto launch = [&](auto kern, bool& configured) -> int {
     if (!configured && !planning()) {

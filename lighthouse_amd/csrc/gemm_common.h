@@ -22,6 +22,9 @@ struct GemmArgs {
   int splits = 1;
   // Source of the call's temporary device memory; nullptr: the library's pool of the stream.
   Scratch* ws = nullptr;
+  // 16-bit direct kernel, 128 x 128 tile: main loop with one barrier per 64 k (set by the launcher
+  // when more than one workgroup falls on a compute unit).
+  int one_barrier = 0;
 };
 
 // Epilogue for 4 consecutive columns of one row.
