@@ -159,7 +159,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm8_fast(GemmArgs g) 
 // Same structure as the 16-bit direct kernel: 256 x 256 workgroup tile, 8 waves (2 x 4, 128 x 64
 // per wave), panels global -> LDS with buffer_load_dwordx4 ... lds in their global orientation, A ring
 // 2 stages x 128 k (256 rows x 128 bytes), B ring 4 stages x 64 k (64 rows x 256 bytes), one
-// v_mfma_f32_32x32x64_f8f6f4 k-step (64 k) per main-loop step with the barrier in the middle.
+// v_mfma_f32_32x32x64_f8f6f4 k-step (64 k) per main-loop step, one barrier per two steps.
 // The k-contiguous A fragment (32 bytes per lane) is two 16-byte LDS reads; the n-contiguous B
 // panel is read with ds_read_b64_tr_b8, which hands a lane 8 k-values of one column (16 lanes
 // cover 8 k-rows x 16 columns), four reads per fragment.  Swizzles: A chunk ^ ((row / 2) % 8),
@@ -253,37 +253,35 @@ __device__ __forceinline__ void d8_interleave_hint() {
   }
 }
 
-__device__ __forceinline__ void d8_wait_barrier(int allowed) {
-  if (allowed >= 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  else if (allowed >= 4) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+// All loads of this wave have landed and all its LDS reads have returned, then barrier.  One asm
+// block: a __syncthreads() would add a release fence.
+__device__ __forceinline__ void d8_wait_barrier() {
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
 // Steps kt (even) and kt + 1.  f holds the fragments of step kt on entry and of step kt + 2 on
-// exit.  Unlike the 16-bit kernel a step is a single MFMA k-step, so the fragments of the next
-// step are read (into g) while the current ones are multiplied; the barrier that makes the next
-// B stage visible therefore comes BEFORE the step's MFMAs:
-//   barrier(kt): B(kt+1) landed (and A for odd -> even transitions); refill B slot of kt-1...
-// To keep the LDS-DMA accounting identical to the 16-bit kernel the refills are issued for the
-// stage that was finished one step earlier (its reads completed before this barrier).
+// exit; a step is a single MFMA k-step, so the fragments of the next step are read while the
+// current ones are multiplied.  ONE barrier per pair, between the two steps: the rings work as two
+// halves of 128 k.  At the barrier both fragment sets of this pair are in registers and the next
+// pair's stages (requested at the previous barrier, 128 k ago) are awaited in full; the pair after
+// that is then requested into this pair's buffers.  (Two barriers per pair with B requested three
+// stages ahead, as in the small tiles of the 16-bit kernel, measured 2-2.5 % slower: 8192^3 426 ->
+// 416 us.)
 __device__ __forceinline__ void d8_step_pair(const D8Ctx& c, f32x16 (&acc)[2][4], D8Frags& f,
-                                             const uint8_t* __restrict__ a_cur, const uint8_t* __restrict__ a_nxt,
-                                             const uint8_t* __restrict__ b1, const uint8_t* __restrict__ b2,
-                                             uint8_t* __restrict__ a_refill, uint8_t* __restrict__ b_refill0,
-                                             uint8_t* __restrict__ b_refill1, int kt, int nk) {
+                                                const uint8_t* __restrict__ a_cur, const uint8_t* __restrict__ a_nxt,
+                                                const uint8_t* __restrict__ b1, const uint8_t* __restrict__ b2,
+                                                uint8_t* __restrict__ a_refill, uint8_t* __restrict__ b_refill0,
+                                                uint8_t* __restrict__ b_refill1, int kt, int nk) {
   D8Frags g;
-  const bool steady = kt + 6 < nk;
-  // ---- even step kt: fragments f (read earlier).  Stage kt of B and the first half of a_cur are
-  // no longer needed by this wave once f is in registers.
-  d8_wait_barrier(steady ? 8 : 0);   // B(kt+1) landed for everyone; everyone holds step kt in registers
-  if (kt + 4 < nk) d8_load_b(c, kt + 4, b_refill0);
   d8_read_frags(c, a_cur, b1, 1, g);  // step kt + 1
   d8_mfma(acc, f);
   d8_interleave_hint();
-  // ---- odd step kt + 1: fragments g.
-  d8_wait_barrier(steady ? 4 : 0);   // A stage kt/2 + 1 and B(kt+2) landed; a_cur and B(kt+1) are free
-  if (kt + 4 < nk) d8_load_a(c, kt / 2 + 2, a_refill);
-  if (kt + 5 < nk) d8_load_b(c, kt + 5, b_refill1);
+  d8_wait_barrier();
+  if (kt + 4 < nk) {
+    d8_load_a(c, kt / 2 + 2, a_refill);
+    d8_load_b(c, kt + 4, b_refill0);
+    d8_load_b(c, kt + 5, b_refill1);
+  }
   d8_read_frags(c, a_nxt, b2, 0, f);  // step kt + 2
   d8_mfma(acc, g);
   d8_interleave_hint();
@@ -344,8 +342,7 @@ __device__ __forceinline__ void d8_mainloop(const D8Ctx& c, f32x16 (&acc)[2][4],
   {
     const uint8_t* a_cur = abuf + ((kt >> 1) & 1) * kD8ABytes;
     const uint8_t* b1 = bbuf + ((kt + 1) & 3) * kD8BBytes;
-    D8Frags gfr;
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    D8Frags gfr;  // (the last pair's stages were awaited at the barrier of the pair before, or at the start)
     d8_read_frags(c, a_cur, b1, 1, gfr);
     d8_mfma(acc, f);
     d8_mfma(acc, gfr);
