@@ -208,6 +208,8 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm16_fast(GemmArgs g)
 // MIDDLE of a step, after the LDS reads of the step's second k-half have been issued, so
 // fragment reads always overlap MFMAs of the previous k-half and the buffer a step has finished
 // reading is refilled right away (B: 3 stages ahead, A: on odd steps, one 64-k stage ahead).
+// The large tiles (and the 128 x 128 tile when workgroups share a compute unit) run a second form
+// with one barrier per 64 k, the rings as two halves: direct_step_pair_1b.
 //
 // A wave-wide load into LDS writes 64 x 16 contiguous LDS bytes, so rows cannot be padded;
 // bank conflicts are avoided by XOR-swizzling which 16-byte chunk of a row each lane fetches
