@@ -885,20 +885,34 @@ static int launch_fast(const GemmArgs& g, hipStream_t s) {
 }
 
 // Tile choice for the direct kernels: 0 = 256 x 256, 1 = 256 x 128, 2 = 128 x 256, 3 = 128 x 128.
-// Cost model: rounds of one workgroup per CU times the tile area (edge tiles count in
-// full), with a penalty for the smaller tiles' extra operand traffic per flop.  For short K a
-// tile's prologue and epilogue weigh as much as its main loop, and the 128 x 128 tile, of which
-// two share a CU and cover each other's, costs little more per flop than the large ones
-// (measured at M = 8192, K = 768: N = 768 24 vs 28 us, N = 2304 38 vs 46, N = 3072 50 vs 51).
-static int direct_variant(int M, int N, int K) {
+// Cost model: rounds of resident workgroups times the tile area (edge tiles count in full) times a
+// measured cost per flop relative to the 256 x 256 tile (one round of 256 tiles each at K = 2048 and
+// 4096: 256 x 128 1.155, 128 x 256 1.135; 128 x 128 1.2 with two workgroups on a CU, 1.37 alone).
+// The 128 x 128 tile runs two workgroups per CU, which share the CU's rate: a round is 2 CUs' worth
+// of tiles at twice a tile's cost, except when no CU gets a second tile.  For short K a tile's
+// prologue and epilogue weigh as much as its main loop, and the 128 x 128 tile, whose two
+// co-resident workgroups cover each other's, costs little more per flop than the large ones
+// (M = 8192, K = 768: N = 768 19 vs 22 us, N = 2304 39 vs 46, N = 3072 51 vs 53).  `slow_epilogue`:
+// an accumulator input or an f32 output is staged block by block, which the tiles with a 256 side
+// pay more for (M = 8192, N = 768, K = 3072 + residual: 49.1 / 49.6 us against 46.6 us for 128 x 128;
+// without the residual 42.6 / 43.3 against 43.0).
+static int direct_variant(int M, int N, int K, bool slow_epilogue) {
   static const int bm[4] = {256, 256, 128, 128}, bn[4] = {256, 128, 256, 128};
-  const double penalty[4] = {1.0, 1.1, 1.1, K <= 1536 ? 1.08 : 1.25};
+  const int cus = num_cus();
+  const double big = slow_epilogue ? 1.08 : 1.0;
   int best = -1;
   double best_cost = 0.0;
-  const int cus = num_cus();
   for (int v = 0; v < 4; ++v) {
     const int64_t tiles = (int64_t)((M + bm[v] - 1) / bm[v]) * ((N + bn[v] - 1) / bn[v]);
-    const double cost = (double)((tiles + cus - 1) / cus) * bm[v] * bn[v] * penalty[v];
+    double cost;
+    if (v < 3) {
+      const double per_flop = v == 0 ? 1.0 : v == 1 ? 1.155 : 1.135;
+      cost = (double)((tiles + cus - 1) / cus) * bm[v] * bn[v] * per_flop * big;
+    } else if (tiles <= cus) {
+      cost = 128.0 * 128.0 * (K <= 1536 ? 1.08 : 1.37);
+    } else {
+      cost = (double)((tiles + 2 * cus - 1) / (2 * cus)) * 2.0 * 128.0 * 128.0 * (K <= 1536 ? 1.08 : 1.2);
+    }
     if (best < 0 || cost < best_cost) {
       best = v;
       best_cost = cost;
@@ -1015,7 +1029,7 @@ static int gemm16_dispatch(const GemmArgs& g_in, hipStream_t s) {
         const int rc = gemm16_splitk<DT>(g, splitk, s);
         if (rc <= 0) return rc;
       }
-      const int v = tile != LH_GEMM_TILE_AUTO ? (int)(tile >> 8) - 1 : direct_variant(g.M, g.N, g.K);
+      const int v = tile != LH_GEMM_TILE_AUTO ? (int)(tile >> 8) - 1 : direct_variant(g.M, g.N, g.K, g.out_dt == LH_F32 || (g.flags & LH_GEMM_ACCUMULATE_C) != 0);
       if (v == 0) return launch_direct<DT, 4, 2>(g, s);
       if (v == 1) return launch_direct<DT, 4, 1>(g, s);
       if (v == 2) return launch_direct<DT, 2, 2>(g, s);
