@@ -36,6 +36,20 @@ def _require(cond: bool, msg: str) -> None:
         raise ValueError(msg)
 
 
+def _tuned_db():
+    """The active tuned-parameter database (None when there is none); the import is deferred so that
+    loading this module does not read the database file."""
+    global _active_db
+    if _active_db is None:
+        from .tuning.tile_db import active_db
+
+        _active_db = active_db
+    return _active_db()
+
+
+_active_db = None
+
+
 def _rows_aligned16(*tensors) -> bool:
     """Base address and every stride but the innermost are multiples of 16 bytes."""
     for t in tensors:
@@ -119,13 +133,13 @@ def gemm(a, b, bias=None, *, out=None, out_dtype=None, relu=False, gelu=False, a
     flags = ((_lib.GEMM_HAS_BIAS if bias is not None else 0) | (_lib.GEMM_HAS_RELU if relu else 0)
              | (_lib.GEMM_HAS_GELU if gelu else 0) | (_lib.GEMM_ACCUMULATE_C if accumulate_c else 0)
              | (_lib.GEMM_TRANSPOSE_A if transpose_a else 0) | (_lib.GEMM_TRANSPOSE_B if transpose_b else 0))
-    if tile is None and split_k is None and a.dtype in (torch.bfloat16, torch.float16) and not (transpose_a or transpose_b) \
-            and _rows_aligned16(a, b, out, bias):  # (a request needs aligned rows; tuned entries assume them)
-        from .tuning.tile_db import active_db  # tuned parameters for this shape, if the database has any
-
-        db = active_db()
+    if tile is None and split_k is None and a.dtype in (torch.bfloat16, torch.float16) and not (transpose_a or transpose_b):
+        db = _tuned_db()  # tuned parameters for this shape, if the database has any
         if db is not None:
             tile, split_k = db.lookup_gemm("bf16" if a.dtype == torch.bfloat16 else "f16", M, N, K)
+            # (a request needs aligned rows; tuned entries assume them)
+            if (tile is not None or split_k is not None) and not _rows_aligned16(a, b, out, bias):
+                tile = split_k = None
     if tile is not None:
         if tuple(tile) not in _lib.GEMM_TILES:
             raise ValueError(f"unsupported tile {tile}; choose from {sorted(_lib.GEMM_TILES)}")
@@ -221,12 +235,12 @@ def attention(q, k, v, *, causal=False, scale=None, out=None, rows_per_wave=None
             raise ValueError("innermost stride must be 1")
     _need_cuda(q, k, v, out)
     Z, H, T, d = q.shape
-    if rows_per_wave is None and stages is None and kv_split is None and d == 64 and q.dtype != torch.float32 and _rows_aligned16(q, k, v, out):
-        from .tuning.tile_db import active_db
-
-        db = active_db()
+    if rows_per_wave is None and stages is None and kv_split is None and d == 64 and q.dtype != torch.float32:
+        db = _tuned_db()
         if db is not None:
             rows_per_wave, stages, kv_split = db.lookup_attention("bf16" if q.dtype == torch.bfloat16 else "f16", Z * H, T, d, causal)
+            if (rows_per_wave or stages or kv_split) and not _rows_aligned16(q, k, v, out):
+                rows_per_wave = stages = kv_split = None
     _require((rows_per_wave or 0) in _lib.ATTN_ROWS and (stages or 0) in _lib.ATTN_STAGES
              and (kv_split or 0) in _lib.ATTN_KSPLIT,
              f"rows_per_wave must be one of {sorted(_lib.ATTN_ROWS)[1:]}, stages one of {sorted(_lib.ATTN_STAGES)[1:]}, "
