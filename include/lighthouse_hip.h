@@ -73,16 +73,20 @@ typedef enum lh_dtype {
 #define LH_GEMM_TRANSPOSE_A 8u
 #define LH_GEMM_TRANSPOSE_B 16u
 #define LH_GEMM_HAS_GELU 32u /* tanh-GELU on the accumulator instead of ReLU (nanoGPT MLP) */
-/* Workgroup-tile request for the 16-bit GEMM, the counterpart of the wg_m / wg_n schedule
- * parameters (lighthouse/schedule/xegpu/mlp_schedule.py:72-78,142).  AUTO lets the library pick by
- * shape; an explicit tile must divide M and N and needs untransposed operands, K % 64 == 0 and
- * 16-byte aligned rows, otherwise the call fails with LH_ERR_INVALID. */
+/* Workgroup-tile request, the counterpart of the wg_m / wg_n schedule parameters
+ * (lighthouse/schedule/xegpu/mlp_schedule.py:72-78,142).  AUTO lets the library pick by shape.
+ * 16-bit inputs take 256x256, 256x128, 128x256 and 128x128: the tile must divide M and N and
+ * needs untransposed operands, K % 64 == 0 and 16-byte aligned rows.  f32 inputs take 128x128,
+ * 128x64 and 64x64 (M and N need not be multiples): untransposed operands, K % 32 == 0, N % 4 == 0
+ * and 16-byte aligned rows.  A request the problem does not meet fails with LH_ERR_INVALID. */
 #define LH_GEMM_TILE_MASK 0x700u
 #define LH_GEMM_TILE_AUTO 0x000u
 #define LH_GEMM_TILE_256x256 0x100u
 #define LH_GEMM_TILE_256x128 0x200u
 #define LH_GEMM_TILE_128x256 0x300u
 #define LH_GEMM_TILE_128x128 0x400u
+#define LH_GEMM_TILE_128x64 0x500u
+#define LH_GEMM_TILE_64x64 0x600u
 /* Cut along K for the 16-bit GEMM ("split K": `splits` workgroup sets each take K / splits columns
  * of A and rows of B and write an f32 block; a second kernel adds the blocks and runs the
  * epilogue), for problems with too few tiles to fill the CUs; the k-dimension counterpart of the

@@ -24,7 +24,9 @@ GEMM_TRANSPOSE_A = 8
 GEMM_TRANSPOSE_B = 16
 GEMM_HAS_GELU = 32
 GEMM_TILE_AUTO = 0
-GEMM_TILES = {(256, 256): 0x100, (256, 128): 0x200, (128, 256): 0x300, (128, 128): 0x400}
+GEMM_TILES = {(256, 256): 0x100, (256, 128): 0x200, (128, 256): 0x300, (128, 128): 0x400, (128, 64): 0x500, (64, 64): 0x600}
+GEMM_TILES_16BIT = ((256, 256), (256, 128), (128, 256), (128, 128))  # what bf16 / f16 inputs take
+GEMM_TILES_F32 = ((128, 128), (128, 64), (64, 64))                   # what f32 inputs take
 GEMM_TILE_MASK = 0x700
 # LH_GEMM_SPLITK_*: 0 = the library decides, 1 = never cut, 2 / 4 / 8 = cut K that many times
 GEMM_SPLITK = {0: 0x0000, 1: 0x0800, 2: 0x1000, 4: 0x1800, 8: 0x2000}

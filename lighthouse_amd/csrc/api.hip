@@ -23,7 +23,7 @@ static int gemm_common_checks(const char* who, const void* out, const void* a, c
   const uint32_t known = LH_GEMM_HAS_BIAS | LH_GEMM_HAS_RELU | LH_GEMM_ACCUMULATE_C | LH_GEMM_TRANSPOSE_A |
                          LH_GEMM_TRANSPOSE_B | LH_GEMM_HAS_GELU | LH_GEMM_TILE_MASK | LH_GEMM_SPLITK_MASK;
   LH_REQUIRE((flags & ~known) == 0, "%s: unknown flag bits 0x%x", who, flags & ~known);
-  LH_REQUIRE((flags & LH_GEMM_TILE_MASK) <= LH_GEMM_TILE_128x128, "%s: unknown tile request 0x%x", who,
+  LH_REQUIRE((flags & LH_GEMM_TILE_MASK) <= LH_GEMM_TILE_64x64, "%s: unknown tile request 0x%x", who,
              flags & LH_GEMM_TILE_MASK);
   LH_REQUIRE((flags & LH_GEMM_SPLITK_MASK) <= LH_GEMM_SPLITK_8, "%s: unknown split-K request 0x%x", who,
              flags & LH_GEMM_SPLITK_MASK);
@@ -44,10 +44,14 @@ int gemm_run(void* out, const void* c, const void* a, const void* b, const void*
   g.ws = ws;
   if (ws) ws->used = 0;  // temporaries of an earlier call on the stream are dead once this one runs
   if (ab_dtype == LH_F32) {
-    LH_REQUIRE((flags & (LH_GEMM_TILE_MASK | LH_GEMM_SPLITK_MASK)) == 0,
-               "gemm: tile and split-K requests apply to 16-bit inputs only");
+    const uint32_t tile = flags & LH_GEMM_TILE_MASK;
+    LH_REQUIRE((flags & LH_GEMM_SPLITK_MASK) == 0, "gemm: split-K requests apply to 16-bit inputs only");
+    LH_REQUIRE(tile == LH_GEMM_TILE_AUTO || tile >= LH_GEMM_TILE_128x128,
+               "gemm: f32 inputs take the 128x128, 128x64 and 64x64 tiles");
     return gemm32(g, s);
   }
+  LH_REQUIRE((flags & LH_GEMM_TILE_MASK) <= LH_GEMM_TILE_128x128,
+             "gemm: 16-bit inputs take the 256x256, 256x128, 128x256 and 128x128 tiles");
   return gemm16(g, ab_dtype, s);
 }
 

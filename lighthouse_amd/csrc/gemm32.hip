@@ -335,7 +335,8 @@ __global__ void __launch_bounds__(256) gemm32_generic(GemmArgs g) {
 
 int gemm32(const GemmArgs& g_in, hipStream_t s) {
   GemmArgs g = g_in;
-  if (g.ldc % 4 == 0 && aligned16(g.out) && (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias))) {
+  const uint32_t tile = g.flags & LH_GEMM_TILE_MASK;
+  if (tile == LH_GEMM_TILE_AUTO && g.ldc % 4 == 0 && aligned16(g.out) && (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias))) {
     const int rc = untranspose_operands<4>(g, kBK32, 4, s);
     if (rc < 0) return rc;
   }
@@ -343,6 +344,15 @@ int gemm32(const GemmArgs& g_in, hipStream_t s) {
   const bool vec_ok = !trans && g.K % kBK32 == 0 && g.lda % 4 == 0 && g.ldb % 4 == 0 && g.ldc % 4 == 0 &&
                       aligned16(g.a) && aligned16(g.b) && aligned16(g.out) &&
                       (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias));
+  if (tile != LH_GEMM_TILE_AUTO) {
+    LH_REQUIRE(vec_ok && g.N % 4 == 0 && direct32_offsets_fit(g),
+               "gemm: a tile request on f32 inputs needs untransposed operands, K %% 32 == 0, N %% 4 == 0 and 16-byte "
+               "aligned rows (M=%d N=%d K=%d)", g.M, g.N, g.K);
+    if (tile == LH_GEMM_TILE_128x128) return launch_direct32<2, 2, 4, 8>(g, s);
+    if (tile == LH_GEMM_TILE_128x64) return launch_direct32<2, 1, 4, 8>(g, s);
+    if ((int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64) <= 512) return launch_direct32<1, 1, 8>(g, s);
+    return launch_direct32<1, 1, 3>(g, s);
+  }
   if (!(vec_ok && g.N % 4 == 0) && (int64_t)g.M * g.N * g.K >= (1 << 22)) {
     // not a shape for the direct kernels as it stands: run it on padded copies of the operands
     const int rc = gemm_padded<4>(g, kBK32, 4, s, [&](const GemmArgs& p) { return gemm32(p, s); });
@@ -353,10 +363,15 @@ int gemm32(const GemmArgs& g_in, hipStream_t s) {
     const int cus = num_cus();
     const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128);
     if (t128 >= 256) {
-      // 128 x 128 or 128 x 64 tiles, one workgroup per CU: whichever needs less time in whole
-      // rounds of tiles (the narrow tile pays about 8 % more operand traffic per flop).
+      // 128 x 128 or 128 x 64 tiles, one workgroup per CU, or 64 x 64 tiles, three per CU: whichever
+      // needs less time in whole rounds of tiles (per flop the narrow tile costs about 8 % more,
+      // three resident small ones 3 %: 4096^3 1058 / 1101 / 1079 us; 3072 x 3072 x 1024, 2.25 rounds of
+      // wide tiles but exactly 3 of small ones, 206 / 181 / 164 us).
       const int64_t t64n = (int64_t)((g.M + 127) / 128) * ((g.N + 63) / 64);
+      const int64_t t64 = (int64_t)((g.M + 63) / 64) * ((g.N + 63) / 64);
       const double wide = (double)((t128 + cus - 1) / cus), narrow = (double)((t64n + cus - 1) / cus) * 0.54;
+      const double small = (double)((t64 + 3 * cus - 1) / (3 * cus)) * 0.7725;
+      if (small < wide && small < narrow) return launch_direct32<1, 1, 3>(g, s);
       if (narrow < wide) return launch_direct32<2, 1, 4, 8>(g, s);
       return launch_direct32<2, 2, 4, 8>(g, s);
     }

@@ -43,20 +43,24 @@ def _apply_matmul(fn, params: dict, notes: list[str]) -> None:
     if not params:
         return
     out_shape = fn.args[fn.arg_order[0] if fn.arg_order else 0].shape
-    if fn.attrs.ab_dtype == _lib.F32:
-        notes.append(f"stage 'matmul': tile / split-K requests apply to 16-bit operands, not to @{fn.name}; the library chooses")
-        return
+    f32 = fn.attrs.ab_dtype == _lib.F32
     flags = fn.attrs.flags
     if "tile_m" in params or "tile_n" in params:
         tile = (params.get("tile_m"), params.get("tile_n"))
         if tile not in _lib.GEMM_TILES:
             raise ValueError(f"stage 'matmul': unsupported tile {tile[0]}x{tile[1]}; choose from {sorted(_lib.GEMM_TILES)}")
-        if out_shape[0] % tile[0] == 0 and out_shape[1] % tile[1] == 0:
+        allowed = _lib.GEMM_TILES_F32 if f32 else _lib.GEMM_TILES_16BIT
+        if tile not in allowed:
+            notes.append(f"stage 'matmul': tile {tile[0]}x{tile[1]} is not one the {'f32' if f32 else '16-bit'} kernel of "
+                         f"@{fn.name} takes ({sorted(allowed)}); the library chooses")
+        elif f32 or (out_shape[0] % tile[0] == 0 and out_shape[1] % tile[1] == 0):
             flags = (flags & ~_lib.GEMM_TILE_MASK) | _lib.GEMM_TILES[tile]
         else:
             notes.append(f"stage 'matmul': tile {tile[0]}x{tile[1]} does not apply to @{fn.name} "
                          f"({out_shape[0]}x{out_shape[1]}); the library chooses")
-    if "split_k" in params:
+    if "split_k" in params and f32:
+        notes.append(f"stage 'matmul': a cut along K applies to 16-bit operands, not to @{fn.name}; the library chooses")
+    elif "split_k" in params:
         sp = params["split_k"]
         if sp not in _lib.GEMM_SPLITK:
             raise ValueError(f"stage 'matmul': unsupported split_k {sp}; choose from {sorted(_lib.GEMM_SPLITK)}")

@@ -48,6 +48,7 @@ def _tuned_db():
 
 
 _active_db = None
+_DTYPE_NAMES = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}
 
 
 def _rows_aligned16(*tensors) -> bool:
@@ -93,7 +94,8 @@ def device_info() -> dict:
 def gemm(a, b, bias=None, *, out=None, out_dtype=None, relu=False, gelu=False, accumulate_c=False,
          transpose_a=False, transpose_b=False, tile=None, split_k=None, residual=None, workspace=None):
     """out = epilogue(A @ B); see lh_hip_gemm.  `tile=(bm, bn)` requests a workgroup tile and
-    `split_k` (1 = never, 2 / 4 / 8) a cut along K for the 16-bit kernels; with neither given the
+    `split_k` (1 = never, 2 / 4 / 8) a cut along K for the 16-bit kernels (f32 inputs take the tiles
+    128x128, 128x64 and 64x64 and no cut); with neither given the
     tuned-parameter database is asked, then the library's own choice applies;
     `residual` [M, N] is added to A @ B before the epilogue (lh_hip_gemm_residual) and is left intact;
     `workspace` (uint8, see gemm_workspace_bytes) makes the call take its temporary memory from
@@ -133,18 +135,21 @@ def gemm(a, b, bias=None, *, out=None, out_dtype=None, relu=False, gelu=False, a
     flags = ((_lib.GEMM_HAS_BIAS if bias is not None else 0) | (_lib.GEMM_HAS_RELU if relu else 0)
              | (_lib.GEMM_HAS_GELU if gelu else 0) | (_lib.GEMM_ACCUMULATE_C if accumulate_c else 0)
              | (_lib.GEMM_TRANSPOSE_A if transpose_a else 0) | (_lib.GEMM_TRANSPOSE_B if transpose_b else 0))
-    if tile is None and split_k is None and a.dtype in (torch.bfloat16, torch.float16) and not (transpose_a or transpose_b):
+    if tile is None and split_k is None and not (transpose_a or transpose_b):
         db = _tuned_db()  # tuned parameters for this shape, if the database has any
         if db is not None:
-            tile, split_k = db.lookup_gemm("bf16" if a.dtype == torch.bfloat16 else "f16", M, N, K)
+            tile, split_k = db.lookup_gemm(_DTYPE_NAMES[a.dtype], M, N, K)
             # (a request needs aligned rows; tuned entries assume them)
             if (tile is not None or split_k is not None) and not _rows_aligned16(a, b, out, bias):
                 tile = split_k = None
     if tile is not None:
-        if tuple(tile) not in _lib.GEMM_TILES:
-            raise ValueError(f"unsupported tile {tile}; choose from {sorted(_lib.GEMM_TILES)}")
+        allowed = _lib.GEMM_TILES_F32 if a.dtype == torch.float32 else _lib.GEMM_TILES_16BIT
+        if tuple(tile) not in allowed:
+            raise ValueError(f"unsupported tile {tile} for {_DTYPE_NAMES[a.dtype]} inputs; choose from {sorted(allowed)}")
         flags |= _lib.GEMM_TILES[tuple(tile)]
     if split_k is not None:
+        if a.dtype == torch.float32 and split_k != 0:
+            raise ValueError("split_k applies to 16-bit inputs")
         if split_k not in _lib.GEMM_SPLITK:
             raise ValueError(f"unsupported split_k {split_k}; choose from {sorted(_lib.GEMM_SPLITK)}")
         flags |= _lib.GEMM_SPLITK[split_k]

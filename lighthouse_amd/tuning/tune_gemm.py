@@ -1,5 +1,5 @@
-"""Parameter search for the 16-bit GEMM (workgroup tile, cut along K) and the head-dimension-64
-attention kernel (query rows per wave, K/V ring depth): enumerate the settings that fit a shape,
+"""Parameter search for the GEMMs (16-bit: workgroup tile, cut along K; f32: workgroup tile) and the
+head-dimension-64 attention kernel (query rows per wave, K/V ring depth, key-range split): enumerate the settings that fit a shape,
 drop the ones a cost model already rules out, time the rest in child processes, log every trial
 and keep the winner when it beats the library's own choice.
 
@@ -9,6 +9,7 @@ examples/xegpu/tune_utils.py:35-85 (`run_with_timeout`), CSV logging of csv_logg
 per-shape JSON parameters.  Usage:
 
     python -m lighthouse_amd.tuning.tune_gemm --sizes 8192,2304,768 --dtype bf16 --db tiles.json --csv tune.csv
+    python -m lighthouse_amd.tuning.tune_gemm --sizes 8192,768,768 --dtype f32 --db tiles.json
     python -m lighthouse_amd.tuning.tune_gemm --attention 64,2048,causal --db tiles.json
 
 Without --db the packaged database (gfx950_tuned.json, the one `ops` consults by default) is updated.
@@ -24,33 +25,47 @@ from .csv_logger import CSVLogger
 from .tile_db import TileDB
 
 TILES = ((256, 256), (256, 128), (128, 256), (128, 128))
-# Relative cost per output element of the smaller tiles (more operand traffic per flop).
-_PENALTY = {(256, 256): 1.0, (256, 128): 1.1, (128, 256): 1.1, (128, 128): 1.25}
+TILES_F32 = ((128, 128), (128, 64), (64, 64))
+# Cost per flop relative to the largest tile, as the library's own tile choice prices it (16-bit:
+# measured one round of 256 tiles each at K = 2048 and 4096; 128 x 128 runs two workgroups per CU).
+_PENALTY = {(256, 256): 1.0, (256, 128): 1.155, (128, 256): 1.135, (128, 128): 1.2}
+_PENALTY_F32 = {(128, 128): 1.0, (128, 64): 1.08, (64, 64): 1.3}
 _CUS = 256
 
 
-def candidate_tiles(M: int, N: int, K: int) -> list[tuple[int, int]]:
-    """Tiles the direct-to-LDS kernel accepts for this shape (K % 64 == 0, tile divides M x N)."""
+def candidate_tiles(M: int, N: int, K: int, dtype: str = "bf16") -> list[tuple[int, int]]:
+    """Tiles the direct-to-LDS kernel accepts for this shape: 16-bit K % 64 == 0 and the tile
+    divides M x N; f32 K % 32 == 0 and N % 4 == 0 (edge tiles are clipped)."""
+    if dtype == "f32":
+        return [] if K % 32 or N % 4 else list(TILES_F32)
     if K % 64:
         return []
     return [t for t in TILES if M % t[0] == 0 and N % t[1] == 0]
 
 
-def estimate_cost(M: int, N: int, K: int, tile: tuple[int, int]) -> float:
-    """Rounds of one workgroup per CU x tile area x penalty x (K + a fixed per-round cost worth
-    about 320 k of main loop: launch, first loads, output stores)."""
-    tiles = (M // tile[0]) * (N // tile[1])
-    rounds = -(-tiles // _CUS)
-    return rounds * tile[0] * tile[1] * _PENALTY[tile] * (K + 320)
+def estimate_cost(M: int, N: int, K: int, tile: tuple[int, int], dtype: str = "bf16") -> float:
+    """Rounds of resident workgroups x tile area x cost per flop x (K + a fixed per-round cost worth
+    about 320 k of main loop: launch, first loads, output stores).  The 16-bit 128 x 128 tile runs
+    two workgroups per CU that share its rate: a round is two CUs' worth of tiles at twice the cost."""
+    tiles = -(-M // tile[0]) * -(-N // tile[1])
+    if dtype == "f32":
+        return -(-tiles // _CUS) * tile[0] * tile[1] * _PENALTY_F32[tile] * (K + 320)
+    if tile == (128, 128):
+        # short K: prologue and epilogue weigh as much as the main loop and the two co-resident
+        # workgroups cover each other's; long K and a lone workgroup per CU: nobody covers its waits
+        per_flop = 1.08 if K <= 1536 else (_PENALTY[tile] if tiles > _CUS else 1.37)
+        rounds = -(-tiles // (2 * _CUS)) * 2 if tiles > _CUS else 1
+        return rounds * tile[0] * tile[1] * per_flop * (K + 320)
+    return -(-tiles // _CUS) * tile[0] * tile[1] * _PENALTY[tile] * (K + 320)
 
 
-def prefilter(M: int, N: int, K: int, slack: float = 1.35) -> list[tuple[int, int]]:
+def prefilter(M: int, N: int, K: int, slack: float = 1.35, dtype: str = "bf16") -> list[tuple[int, int]]:
     """Candidates whose estimated cost is within `slack` of the best estimate, best first."""
-    cands = sorted(candidate_tiles(M, N, K), key=lambda t: estimate_cost(M, N, K, t))
+    cands = sorted(candidate_tiles(M, N, K, dtype), key=lambda t: estimate_cost(M, N, K, t, dtype))
     if not cands:
         return []
-    best = estimate_cost(M, N, K, cands[0])
-    return [t for t in cands if estimate_cost(M, N, K, t) <= slack * best]
+    best = estimate_cost(M, N, K, cands[0], dtype)
+    return [t for t in cands if estimate_cost(M, N, K, t, dtype) <= slack * best]
 
 
 SPLITS = (2, 4, 8)
@@ -65,9 +80,12 @@ def candidate_splits(M: int, N: int, K: int) -> list[int]:
     return [sp for sp in SPLITS if K % (64 * sp) == 0 and K // sp >= 256 and tiles * sp <= 4 * _CUS]
 
 
-def candidate_settings(M: int, N: int, K: int, exhaustive: bool = False) -> list[tuple]:
-    """(tile or None, split_k or None) pairs to time after the library's own choice (None, None)."""
-    tiles = candidate_tiles(M, N, K) if exhaustive else prefilter(M, N, K)
+def candidate_settings(M: int, N: int, K: int, exhaustive: bool = False, dtype: str = "bf16") -> list[tuple]:
+    """(tile or None, split_k or None) pairs to time after the library's own choice (None, None);
+    f32 inputs have tiles only."""
+    tiles = candidate_tiles(M, N, K, dtype) if exhaustive else prefilter(M, N, K, dtype=dtype)
+    if dtype == "f32":
+        return [(t, None) for t in tiles]
     return [(t, None) for t in tiles] + [(None, sp) for sp in candidate_splits(M, N, K)]
 
 
@@ -78,7 +96,7 @@ def _time_tile(res, M, N, K, dtype, tile, nruns, nwarmup, split_k=None):
     from .tile_db import use_db
 
     use_db(None)  # the baseline trial must be the library's own choice, not an earlier database entry
-    tdt = {"bf16": torch.bfloat16, "f16": torch.float16}[dtype]
+    tdt = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[dtype]
     a = torch.randn(M, K, device="cuda").to(tdt)
     b = torch.randn(K, N, device="cuda").to(tdt)
     out = torch.empty(M, N, device="cuda", dtype=tdt)
@@ -173,14 +191,14 @@ def tune_shape(M: int, N: int, K: int, dtype: str = "bf16", db: TileDB | None = 
     """Time the (pre-filtered) tiles and K cuts for one shape; record the fastest in `db` if it beats
     the library's own choice.  Returns the fastest row.  `isolate=False` times in this process (no
     protection against a hanging or crashing trial)."""
-    cands = candidate_settings(M, N, K, exhaustive)
+    cands = candidate_settings(M, N, K, exhaustive, dtype)
     best = base = None
     # The library's own choice (no request: its cost model, its own split-K criterion) is timed first.
     for tile, split_k in [(None, None), *cands] if cands else []:
         res = _trial(_time_tile, (M, N, K, dtype, tile, nruns, nwarmup, split_k), isolate, timeout)
         row = {"dtype": dtype, "M": M, "N": N, "K": K, "tile_m": tile[0] if tile else 0, "tile_n": tile[1] if tile else 0,
                "split_k": split_k or 0,
-               "estimate": round(estimate_cost(M, N, K, tile) / 1e6, 3) if tile else 0.0,
+               "estimate": round(estimate_cost(M, N, K, tile, dtype) / 1e6, 3) if tile else 0.0,
                "time_us": round(res["time"] * 1e6, 3),
                "tflops": round(res["throughput"], 2), "error": res["error"]}
         if logger is not None:
@@ -233,10 +251,11 @@ def tune_attention(BH: int, T: int, causal: bool, dtype: str = "bf16", db: TileD
 def main(argv: list[str] | None = None) -> int:
     from .tile_db import DEFAULT_DB_PATH
 
-    ap = argparse.ArgumentParser(description="Parameter search for the 16-bit HIP GEMM and the attention kernel.")
+    ap = argparse.ArgumentParser(description="Parameter search for the HIP GEMMs (16-bit and f32) and the attention kernel.")
     ap.add_argument("--sizes", action="append", default=[], help="GEMM M,N,K (repeatable)")
     ap.add_argument("--attention", action="append", default=[], help="attention BH,T[,causal] (repeatable; head_dim 64)")
-    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16"])
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f16", "f32"],
+                    help="GEMM operand type (f32: tiles 128x128 / 128x64 / 64x64, no cut along K); attention is 16-bit")
     ap.add_argument("--db", default=str(DEFAULT_DB_PATH), help="JSON database to update (default: the packaged one)")
     ap.add_argument("--csv", default=None, help="CSV log of every GEMM trial (attention trials: <name>_attention.csv)")
     ap.add_argument("--nruns", type=int, default=300)
@@ -246,6 +265,9 @@ def main(argv: list[str] | None = None) -> int:
     args = ap.parse_args(argv)
     if not args.sizes and not args.attention:
         print("Error: nothing to tune (give --sizes and / or --attention)", file=sys.stderr)
+        return 1
+    if args.attention and args.dtype == "f32":
+        print("Error: the attention variants exist for 16-bit tensors (--dtype bf16 / f16)", file=sys.stderr)
         return 1
     db = TileDB(args.db)
     logger = CSVLogger(args.csv)

@@ -213,8 +213,39 @@ def test_gemm_tile_request_errors():
     with pytest.raises(ValueError):
         ops.gemm(a, b, tile=(64, 64))
     with pytest.raises(ValueError):
-        ops.gemm(a.float(), b.float(), tile=(128, 128))
+        ops.gemm(a.float(), b.float(), tile=(256, 128))  # a tile of the 16-bit kernel
+    with pytest.raises(ValueError):
+        ops.gemm(a.float(), b.float(), split_k=2)
+    with pytest.raises(ValueError, match="K % 32"):
+        ops.gemm(torch.zeros(64, 48, device="cuda"), torch.zeros(48, 64, device="cuda"), tile=(64, 64))
     ops.gemm(a, b, tile=(256, 128))
+    ops.gemm(a.float(), b.float(), tile=(128, 128))
+
+
+@pytest.mark.parametrize("tile", [(128, 128), (128, 64), (64, 64)])
+@pytest.mark.parametrize("shape", [(1024, 1024, 1024), (8192, 768, 768), (200, 332, 96), (64, 64, 32), (4096, 2304, 256)])
+def test_gemm_f32_tile_requests(shape, tile):
+    """Each tile of the f32 kernel on request (edge tiles clipped): integer operands make the result
+    exact, so every tile must give the bits of the library's own choice, with and without bias +
+    ReLU, and nothing outside the output may be written."""
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K)
+    a = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    bias = rng.integers(-8, 9, (N,)).astype(np.float32)
+    da, db, dbias = _dev(a, torch.float32), _dev(b, torch.float32), _dev(bias, torch.float32)
+    ref = a.astype(np.float64) @ b.astype(np.float64)
+    out = ops.gemm(da, db, tile=tile)
+    assert np.array_equal(_host(out).astype(np.float64), ref), f"f32 gemm {shape} tile {tile}"
+    assert torch.equal(out, ops.gemm(da, db))
+    canvas = torch.full((M + 2, N + 8), 7.0, device="cuda")
+    view = canvas[1:M + 1, 4:4 + N]
+    ops.gemm(da, db, dbias, relu=True, out=view, tile=tile)
+    assert np.array_equal(_host(view).astype(np.float64), np.maximum(ref + bias, 0.0))
+    canvas[1:M + 1, 4:4 + N] = 7.0
+    assert (canvas == 7.0).all(), "the kernel wrote outside the output matrix"
 
 
 @pytest.mark.parametrize("kind", ["bf16_bias_relu", "bf16_f32_acc", "f32", "fp8"])

@@ -150,6 +150,17 @@ def test_stage_application(tmp_path):
     apply_stage(module, str(yaml_path), notes)                 # 384 % 256 != 0: left to the library
     assert module.lookup("layer").attrs.flags & 0x700 == _lib.GEMM_TILES[(256, 128)]
     assert "does not apply" in notes[-1]
+    # the f32 kernel has tiles of its own (edge tiles clipped: no divisibility rule) and no cut along K
+    f32 = parse_payload_module(NAMED)
+    yaml_path.write_text('Pipeline:\n  - kernel: "matmul{tile_m=128 tile_n=64}"\n')
+    apply_stage(f32, str(yaml_path), notes)
+    assert f32.lookup("mm").attrs.flags & 0x700 == _lib.GEMM_TILES[(128, 64)] == 0x500
+    apply_stage(module, str(yaml_path), notes)                 # not a tile of the 16-bit kernel
+    assert module.lookup("layer").attrs.flags & 0x700 == _lib.GEMM_TILES[(256, 128)] and "16-bit kernel" in notes[-1]
+    yaml_path.write_text('Pipeline:\n  - kernel: "matmul{tile_m=256 tile_n=128 split_k=1}"\n')
+    apply_stage(f32, str(yaml_path), notes)
+    assert f32.lookup("mm").attrs.flags & 0x700 == 0x500 and f32.lookup("mm").attrs.flags & _lib.GEMM_SPLITK_MASK == 0
+    assert "f32 kernel" in notes[-2] and "cut along K" in notes[-1]
 
 
 def test_stage_parameters_all_act_or_fail(tmp_path):

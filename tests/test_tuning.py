@@ -15,10 +15,19 @@ def test_candidates_and_prefilter():
     assert candidate_tiles(256, 256, 96) == []          # K must be a multiple of 64
     # 4096^3: 256 tiles of 256 x 256 are exactly one round, every smaller tile costs more
     assert prefilter(4096, 4096, 4096)[0] == (256, 256)
-    # N = 768: 96 big tiles leave CUs idle; halves and quarters are estimated cheaper
-    assert prefilter(8192, 768, 768)[0] in ((256, 128), (128, 256))
+    # N = 768: 96 big tiles leave CUs idle; halves and quarters are estimated cheaper, at short K the quarters
+    assert prefilter(8192, 768, 768)[0] == (128, 128)
+    assert prefilter(8192, 768, 4096)[0] in ((256, 128), (128, 256))
     assert estimate_cost(8192, 768, 768, (256, 256)) > estimate_cost(8192, 768, 768, (256, 128))
     assert all(t in candidate_tiles(8192, 2304, 768) for t in prefilter(8192, 2304, 768))
+    # 192 tiles of 256 x 256 in one round beat 768 of 128 x 128 in two rounds of pairs
+    assert prefilter(4096, 3072, 4096)[0] == (256, 256)
+    # f32: three tiles, edge tiles clipped, no cut along K
+    assert candidate_tiles(1000, 1000, 1024, "f32") == [(128, 128), (128, 64), (64, 64)]
+    assert candidate_tiles(1024, 1024, 1000, "f32") == [] and candidate_tiles(1024, 1022, 1024, "f32") == []
+    assert prefilter(4096, 4096, 4096, dtype="f32")[0] == (128, 128)
+    assert prefilter(8192, 768, 768, dtype="f32")[0] == (128, 64)     # 384 wide tiles = 2 rounds, 768 narrow = 3 x 0.54
+    assert all(sp is None for _, sp in candidate_settings(16, 8192, 8192, dtype="f32"))
 
 
 def _ok(res, x):
@@ -94,4 +103,4 @@ def test_settings_and_database_kinds(tmp_path):
     assert default is None or isinstance(default, TileDB)
     if default is not None:
         for key, entry in default.entries.items():
-            assert key.split(":")[0] in ("bf16", "f16", "attn") and entry["time_us"] > 0
+            assert key.split(":")[0] in ("bf16", "f16", "f32", "attn") and entry["time_us"] > 0
