@@ -142,3 +142,48 @@ def test_compiled_matmul_nodes(dtype, rtol):
         np.testing.assert_array_equal(_np(out), ref)
     else:
         assert_close(_np(out), ref, rtol, "compiled matmul nodes bf16")
+
+
+def test_reference_compile_model_examples():
+    """The three flows of the reference's torch-ingress examples at their own shapes and pass criteria:
+    a decorated matmul model called with two input shapes, each of which gets its own specialisation
+    (examples/ingress/torch/compile_model.py:60-107: [8,16] @ [16,4], then [2,4] @ [4,16], allclose
+    rtol = atol = 1e-3), `model.compile(...)` on a Linear(16, 8) with batch 2 (:113-142, rtol = atol =
+    1e-2), and the MLP of examples/ingress/torch/MLPModel/model.py (Linear(10, 32), ReLU, Linear(32, 2)
+    on a [1, 10] input)."""
+    from lighthouse_amd.ingress.torch import gpu_backend
+
+    backend = gpu_backend()
+
+    @torch.compile(dynamic=False, backend=backend)
+    class Model(nn.Module):
+        def forward(self, a, b):
+            return torch.matmul(a, b)
+
+    torch.manual_seed(0)
+    model = Model()
+    for shape_a, shape_b in (((8, 16), (16, 4)), ((2, 4), (4, 16))):
+        a, b = torch.randn(shape_a, device="cuda"), torch.randn(shape_b, device="cuda")
+        out = model(a, b)
+        assert backend.last_jit_function.kinds == ["hip.gemm"]
+        assert out.shape == (shape_a[0], shape_b[1])
+        assert torch.allclose(torch.matmul(a.cpu(), b.cpu()), out.cpu(), rtol=0.001, atol=0.001)
+
+    linear = nn.Sequential(nn.Linear(16, 8)).cuda()
+    x = torch.randn(2, 16, device="cuda")
+    with torch.no_grad():
+        out_ref = linear(x)
+        linear.compile(dynamic=False, backend=backend)
+        out = linear(x)
+    assert backend.last_jit_function.kinds == ["hip.gemm"]
+    assert torch.allclose(out_ref, out, rtol=0.01, atol=0.01)
+    assert_close(_np(out), orc.matmul(_np(x), _np(linear[0].weight).T, bias=_np(linear[0].bias)), 1e-4, "Linear(16, 8)")
+
+    mlp = nn.Sequential(nn.Linear(10, 32), nn.ReLU(), nn.Linear(32, 2)).cuda()
+    x = torch.randn(1, 10, device="cuda")
+    compiled = torch.compile(mlp, backend=backend, dynamic=False)
+    with torch.no_grad():
+        out = compiled(x)
+    assert backend.last_jit_function.kinds == ["hip.gemm", "hip.gemm"]
+    h = orc.matmul(_np(x), _np(mlp[0].weight).T, bias=_np(mlp[0].bias), relu=True)
+    assert_close(_np(out), orc.matmul(h, _np(mlp[2].weight).T, bias=_np(mlp[2].bias)), 1e-4, "MLPModel")
