@@ -5,6 +5,7 @@ The reference parses any MLIR module and lowers it with pass pipelines
 compiler, so the text front end recognises the linalg programs that map onto one kernel call and
 rejects everything else with ``ValueError``:
 
+* ``linalg.add`` of two arguments into a third (examples/basic/compile_and_run.py:25-31);
 * ``linalg.matmul`` (test/run/pipeline-check.mlir:8-14), optionally followed by a broadcast bias
   add and a ReLU in named form (``linalg.broadcast`` + ``linalg.add``, ``linalg.max`` against a
   zero fill: the ops of lighthouse/ingress/mlir_gen/named.py:5-32);
@@ -62,6 +63,10 @@ def _split_statements(body: str) -> list[str]:
     for line in body.splitlines():
         stripped = line.split("//")[0].strip()
         if not stripped:
+            continue
+        # an operation may continue on the next line with its ins(...) / outs(...) / result type
+        if not cur and out and re.match(r"(ins|outs)\s*\(|->|:\s", stripped):
+            out[-1] += " " + stripped
             continue
         cur.append(stripped)
         depth += stripped.count("{") - stripped.count("}")
@@ -144,7 +149,7 @@ def parse_function(text: str, name: str, maps: dict[str, tuple[str, ...]]) -> Pa
             elif a is not None and a.kind == "bcast":
                 val = _Value("bias", (ins[1], a.data[0]))
             else:
-                raise ValueError(f"linalg.add without a broadcast bias operand: {stmt}")
+                val = _Value("add2", (ins[0], ins[1], outs[0] if outs else None))  # plain elementwise sum
         elif op == "linalg.max":
             a, b = (env.get(x) for x in ins)
             zero = lambda v: v is not None and v.kind == "fill" and float(v.data[0]) == 0.0  # noqa: E731
@@ -171,12 +176,14 @@ def parse_function(text: str, name: str, maps: dict[str, tuple[str, ...]]) -> Pa
             versioned = f"{raw_outs[0]}@{versions[raw_outs[0]]}"
             env[versioned] = val
             cur[raw_outs[0]] = versioned
-        last = val if val.kind in ("matmul", "bias", "relu") else None
+        last = val if val.kind in ("matmul", "bias", "relu", "add2") else None
         if last is not None:
             env["__last__"] = val
     root = env.get(returned) if returned else env.get("__last__")
     if root is None:
         raise ValueError(f"@{name} computes nothing this target recognises")
+    if root.kind == "add2":
+        return _elementwise_add(name, root, env, arg_types)
     has_relu = has_bias = False
     bias_name = None
     if root.kind == "relu":
@@ -228,6 +235,33 @@ def parse_function(text: str, name: str, maps: dict[str, tuple[str, ...]]) -> Pa
     attrs = _lib.MatmulAttrs(lh_dtype(a_elem), lh_dtype(c_elem), flags)
     flops = 2 * M * N * K + (M * N if has_bias else 0) + (M * N if has_relu else 0)
     return PayloadFunction(name, "matmul", attrs, args, flops, 0, arg_order=order)
+
+
+def _elementwise_add(name: str, root: _Value, env: dict, arg_types: list) -> PayloadFunction:
+    """`linalg.add ins(%a, %b) outs(%out)` on three function arguments of one shape and type: the
+    kernel of examples/basic/compile_and_run.py:25-31 (memref<16x32xf32>)."""
+    a, b, out = root.data
+    vals = [env.get(x) for x in (a, b, out)]
+    if any(v is None or v.kind != "arg" for v in vals):
+        raise ValueError(f"@{name}: linalg.add must read two function arguments and write a third "
+                         "(results-to-arguments convention)")
+    ia, ib, io = (v.data[0] for v in vals)
+    if not (arg_types[ia] == arg_types[ib] == arg_types[io]) or io in (ia, ib):
+        raise ValueError(f"@{name}: linalg.add needs three distinct arguments of one shape and element type")
+    dims, elem = arg_types[io]
+    if len(dims) != 2:
+        raise ValueError(f"@{name}: linalg.add runs on 2-D buffers, got rank {len(dims)}")
+    if elem not in ("f32", "bf16", "f16"):
+        raise ValueError(f"@{name}: linalg.add on {elem} is not supported")
+    unused = sorted(set(range(len(arg_types))) - {ia, ib, io})
+    if unused:
+        raise ValueError(f"@{name}: arguments {unused} take no part in the sum")
+    n = 1
+    for d in dims:
+        n *= d
+    args = [ArgSpec(d, e, writable=(i == io)) for i, (d, e) in enumerate(arg_types)]
+    attrs = _lib.ElementwiseAttrs(_lib.EW_ADD, lh_dtype(elem), lh_dtype(elem), 0)
+    return PayloadFunction(name, "elementwise", attrs, args, n, 3 * n * (4 if elem == "f32" else 2), arg_order=[io, ia, ib])
 
 
 def _classify_generic(stmt, ins, outs, env, maps) -> _Value:

@@ -175,6 +175,46 @@ module {
     assert re.match(r"100 runs: [0-9.e-]+ seconds", capsys.readouterr().out)
 
 
+def test_basic_example_add_kernel(tmp_path, capsys):
+    """The kernel of examples/basic/compile_and_run.py:25-31 (`linalg.add` on three 16x32xf32 buffers)
+    through the text front end: the Runner on the example's own inputs (a, b random, out zero;
+    checked as there against a + b, :170-176) and the command line."""
+    import re
+
+    from lighthouse_amd.execution import GPUMemoryManager, Runner
+    from lighthouse_amd.ingress.mlir_text import parse_payload_module
+    from lighthouse_amd.lh_run import main
+
+    text = """
+func.func @add(%a: memref<16x32xf32>, %b: memref<16x32xf32>, %out: memref<16x32xf32>) {
+    linalg.add ins(%a, %b : memref<16x32xf32>, memref<16x32xf32>)
+               outs(%out : memref<16x32xf32>)
+    return
+}
+"""
+    module = parse_payload_module(text)
+    rng = np.random.default_rng(0)
+    a, b = rng.standard_normal((16, 32)).astype(np.float32), rng.standard_normal((16, 32)).astype(np.float32)
+    out = np.zeros((16, 32), dtype=np.float32)
+    result = {}
+
+    def read_back(inputs, *, execution_engine, memory_manager):
+        memory_manager.copy(inputs[2], out)
+        result["done"] = True
+
+    Runner(module, mem_manager_cls=GPUMemoryManager).execute("add", [a, b, out], read_back)
+    assert result["done"] and np.array_equal(out, a + b)
+    mlir = tmp_path / "add.mlir"
+    mlir.write_text(text)
+    assert main([str(mlir), "--entry-point=add", "--input-shape=16x32xf32xrnd,16x32xf32x1,16x32xf32x0", "--print-tensor=3",
+                 "--seed=7", "--stage=canonicalize"]) == 0
+    printed = capsys.readouterr().out
+    np.random.seed(7)
+    expect = np.random.rand(16, 32).astype(np.float32) + 1.0
+    vals = np.array([float(v) for v in re.findall(r"[-+]?\d+\.\d+(?:e[-+]?\d+)?", printed)], dtype=np.float32)
+    assert vals.size >= 6 and np.allclose(vals[:3], expect[0, :3], rtol=1e-5)
+
+
 @pytest.mark.parametrize("ab,res,bias_t", [("f32", "f32", "f32"), ("bf16", "bf16", "bf16"), ("bf16", "f32", "f32")])
 @pytest.mark.parametrize("variant", ["plain", "bias_relu", "bias_relu_final_tb", "acc"])
 def test_runner_mlp_payload(ab, res, bias_t, variant):

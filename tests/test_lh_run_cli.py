@@ -218,3 +218,23 @@ def test_cli_error_codes(tmp_path, capsys):
     assert bad_stage == 1
     bad_entry = main([str(f), "--entry-point", "zz", "--input-shape", "8x24xf32x1", "--stage", "cse"])
     assert bad_entry == 1
+
+
+def test_plain_add_becomes_an_elementwise_payload():
+    """`linalg.add` of two arguments into a third (examples/basic/compile_and_run.py:25-31) maps to the
+    elementwise sum kernel with the output first; anything else about it is rejected."""
+    text = """
+func.func @add(%a: memref<16x32xf32>, %b: memref<16x32xf32>, %out: memref<16x32xf32>) {
+    linalg.add ins(%a, %b : memref<16x32xf32>, memref<16x32xf32>) outs(%out : memref<16x32xf32>)
+    return
+}
+"""
+    fn = parse_payload_module(text).lookup("add")
+    assert fn.entry == "elementwise" and fn.arg_order == [2, 0, 1]
+    assert fn.attrs.kind == _lib.EW_ADD and [a.writable for a in fn.args] == [False, False, True]
+    with pytest.raises(ValueError, match="one shape"):
+        parse_payload_module(text.replace("%b: memref<16x32xf32>", "%b: memref<16x64xf32>"))
+    with pytest.raises(ValueError, match="2-D"):
+        parse_payload_module(text.replace("16x32xf32", "16xf32"))
+    with pytest.raises(ValueError, match="distinct"):
+        parse_payload_module(text.replace("outs(%out", "outs(%a"))
