@@ -203,11 +203,14 @@ class _Lowering:
                 if not isinstance(r, torch.Tensor) or tuple(r.shape) != shape or r.dtype != x.dtype:
                     raise ValueError(f"{node.name}: broadcasting / mixed-type add is not supported")
                 r = _as_2d(r)
+            _check_schedule(node.name, schedule, x2.shape[0], wt.shape[1], x2.shape[1])
             out = ops.gemm(x2, wt, b.detach() if b is not None else None, relu=act == "relu", gelu=act == "gelu",
-                           residual=r)
+                           residual=r, tile=schedule.get("tile"), split_k=schedule.get("split_k"))
             return out.view(shape)
 
-        self._emit(node.name, "hip.gemm", run, bias=b_arg is not None, activation=act, residual=add_node is not None)
+        schedule: dict = {}
+        self._emit(node.name, "hip.gemm", run, bias=b_arg is not None, activation=act, residual=add_node is not None,
+                   schedule=schedule)
 
     def _matmul(self, node, a_arg, b_arg, bias_arg=None):
         """torch.matmul / mm / `@` with a 2-D right operand (and addmm with a vector bias): one GEMM.
@@ -238,11 +241,15 @@ class _Lowering:
             shape = (*a.shape[:-1], b.shape[1])
             a2, ta = operand(a) if a.dim() == 2 else (_as_2d(a), False)
             b2, tb = operand(b)
+            _check_schedule(node.name, schedule, a2.shape[1] if ta else a2.shape[0], b.shape[1], b.shape[0])
             out = ops.gemm(a2, b2, bias.detach().contiguous() if bias is not None else None, relu=act == "relu",
-                           gelu=act == "gelu", transpose_a=ta, transpose_b=tb)
+                           gelu=act == "gelu", transpose_a=ta, transpose_b=tb, tile=schedule.get("tile"),
+                           split_k=schedule.get("split_k"))
             return out.view(shape)
 
-        self._emit(node.name, "hip.gemm", run, bias=bias_arg is not None, activation=act, residual=False)
+        schedule: dict = {}
+        self._emit(node.name, "hip.gemm", run, bias=bias_arg is not None, activation=act, residual=False,
+                   schedule=schedule)
 
     def _layer_norm(self, node, x_arg, shape, w_arg, b_arg, eps):
         if len(tuple(shape)) != 1:
@@ -507,6 +514,54 @@ class JITFunction:
         return times
 
 
+
+def _check_schedule(name: str, schedule: dict, M: int, N: int, K: int) -> None:
+    """A layer's schedule parameters may state the problem they were chosen for; running them on
+    another one is an error, not a silent fallback."""
+    want = schedule.get("mnk")
+    if want is not None and tuple(want) != (M, N, K):
+        raise ValueError(f"{name}: schedule parameters are for a {want[0]}x{want[1]}x{want[2]} matmul, the layer is "
+                         f"{M}x{N}x{K}")
+
+
+_SCHEDULE_KEYS = {"layer_kind", "m", "n", "k", "wg_m", "wg_n", "split_k"}
+
+
+def with_schedule_parameters(parameters: Sequence[dict]) -> Callable[[list[PlanStep]], list[PlanStep]]:
+    """An `fn_compile` that gives the i-th GEMM of the lowered graph the i-th entry of `parameters`,
+    the per-layer dictionaries of the reference's ScheduleParameters
+    (lighthouse/schedule/parameters.py; examples/xegpu/torch_matmul.py:219-262: layer_kind, m, n, k,
+    wg_m, wg_n, ...).  This target's kernels take `wg_m` x `wg_n` (the workgroup tile) and `split_k`;
+    every other tiling key of the XeGPU schedule has no counterpart and is an error, as is a count of
+    entries that differs from the graph's GEMMs."""
+    parameters = [dict(p) for p in parameters]
+    for p in parameters:
+        unknown = sorted(set(p) - _SCHEDULE_KEYS)
+        if unknown:
+            raise ValueError(f"schedule parameter(s) {unknown} have no counterpart on this target; it takes "
+                             f"{sorted(_SCHEDULE_KEYS)}")
+        if p.get("layer_kind", "matmul") != "matmul":
+            raise ValueError(f"schedule parameters for layer kind '{p['layer_kind']}' are not supported")
+        if ("wg_m" in p) != ("wg_n" in p):
+            raise ValueError("wg_m and wg_n come together")
+
+    def fn_compile(plan: list[PlanStep]) -> list[PlanStep]:
+        gemms = [st for st in plan if st.kind == "hip.gemm"]
+        if len(gemms) != len(parameters):
+            raise ValueError(f"{len(parameters)} schedule parameter entries for a graph of {len(gemms)} matmul layers")
+        for st, p in zip(gemms, parameters):
+            sched = st.detail["schedule"]
+            if "wg_m" in p:
+                sched["tile"] = (int(p["wg_m"]), int(p["wg_n"]))
+            if "split_k" in p:
+                sched["split_k"] = int(p["split_k"])
+            if all(key in p for key in ("m", "n", "k")):
+                sched["mnk"] = (int(p["m"]), int(p["n"]), int(p["k"]))
+        return plan
+
+    return fn_compile
+
+
 class HipBackend:
     """A PyTorch backend onto liblighthouse_hip.so; `backend(gm, example_inputs) -> JITFunction`."""
 
@@ -535,6 +590,14 @@ class HipBackend:
 
     @property
     def last_jit_function(self) -> JITFunction | None:
+        return self._last_jit_function
+
+    @property
+    def jit_function(self) -> JITFunction:
+        """The last JITFunction created (lighthouse/ingress/torch/compile.py:202-217); ValueError
+        before the first compilation."""
+        if self._last_jit_function is None:
+            raise ValueError("The backend does not have a JITFunction available. Compile the torch model first.")
         return self._last_jit_function
 
 

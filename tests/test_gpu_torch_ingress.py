@@ -187,3 +187,39 @@ def test_reference_compile_model_examples():
     assert backend.last_jit_function.kinds == ["hip.gemm", "hip.gemm"]
     h = orc.matmul(_np(x), _np(mlp[0].weight).T, bias=_np(mlp[0].bias), relu=True)
     assert_close(_np(out), orc.matmul(h, _np(mlp[2].weight).T, bias=_np(mlp[2].bias)), 1e-4, "MLPModel")
+
+
+def test_reference_torch_matmul_example():
+    """examples/xegpu/torch_matmul.py: an f16 matmul model with per-layer schedule parameters handed
+    to the backend through `fn_compile`, `model.compile(dynamic=False, backend=...)`, the result
+    checked with allclose rtol = atol = 1e-2 (:291-296), then `backend.jit_function.benchmark(a, b,
+    nruns, nwarmup)` (:299-305).  Here on 2048^3 with the workgroup tile as the parameter that acts;
+    parameters for another problem size are refused when the layer runs."""
+    from lighthouse_amd.ingress.torch import gpu_backend, with_schedule_parameters
+
+    class Model(nn.Module):
+        def forward(self, A, B):
+            return torch.matmul(A, B)
+
+    m = n = k = 2048
+    torch.manual_seed(0)
+    a = torch.randn(m, k, device="cuda", dtype=torch.float16)
+    b = torch.randn(k, n, device="cuda", dtype=torch.float16)
+    params = [{"layer_kind": "matmul", "m": m, "n": n, "k": k, "wg_m": 256, "wg_n": 128}]
+    backend = gpu_backend(with_schedule_parameters(params), device=torch.device("cuda"))
+    model = Model()
+    model.compile(dynamic=False, backend=backend)
+    out = model(a, b)
+    assert backend.jit_function.kinds == ["hip.gemm"]
+    rows = [0, 777, m - 1]
+    ref = orc.matmul(_np(a[rows]), _np(b), result_type="f16")
+    assert torch.allclose(torch.from_numpy(ref).to(torch.float16), out[rows].cpu(), rtol=0.01, atol=0.01)
+    assert_close(_np(out[rows]), ref, 2e-2, "torch_matmul example f16 2048^3")
+    unrequested = gpu_backend()
+    plain = torch.compile(Model(), backend=unrequested, dynamic=False)(a, b)
+    assert torch.equal(plain, out)                      # another tile, the same sums in the same order of k
+    times = backend.jit_function.benchmark(a, b, nruns=5, nwarmup=2)
+    assert times.shape == (5,) and (times > 0).all()
+    wrong = gpu_backend(with_schedule_parameters([{"m": 64, "n": 64, "k": 64, "wg_m": 128, "wg_n": 128}]))
+    with pytest.raises(ValueError, match="64x64x64"):
+        torch.compile(Model(), backend=wrong, dynamic=False)(a, b)

@@ -163,3 +163,29 @@ def test_plain_matmul_nodes_become_gemms():
 
     with pytest.raises(ValueError, match="addmm"):
         gpu_backend()(torch.fx.symbolic_trace(Scaled()), [torch.randn(4, 4), torch.randn(4, 4)])
+
+
+def test_schedule_parameters_reach_the_gemm_steps():
+    """Per-layer schedule parameters (the dictionaries of the reference's ScheduleParameters) set the
+    tile / K-cut request of the graph's GEMMs in order; keys without a counterpart, a wrong count and
+    a lone wg_m are errors; `backend.jit_function` raises before the first compilation."""
+    from lighthouse_amd.ingress.torch import gpu_backend, with_schedule_parameters
+    from lighthouse_amd.ingress.torch.compile import _Lowering
+
+    with pytest.raises(ValueError, match="Compile the torch model first"):
+        gpu_backend().jit_function
+    model = nn.Sequential(nn.Linear(16, 32), nn.ReLU(), nn.Linear(32, 8))
+    gm = torch.fx.symbolic_trace(model)
+    _, plan, _ = _Lowering(gm, False).lower()
+    fn = with_schedule_parameters([{"layer_kind": "matmul", "m": 4, "n": 32, "k": 16, "wg_m": 128, "wg_n": 128},
+                                   {"split_k": 2}])
+    plan = fn(plan)
+    gemms = [st for st in plan if st.kind == "hip.gemm"]
+    assert gemms[0].detail["schedule"] == {"tile": (128, 128), "mnk": (4, 32, 16)}
+    assert gemms[1].detail["schedule"] == {"split_k": 2}
+    with pytest.raises(ValueError, match="no counterpart"):
+        with_schedule_parameters([{"wg_m": 256, "wg_n": 256, "sg_m": 32}])
+    with pytest.raises(ValueError, match="come together"):
+        with_schedule_parameters([{"wg_m": 256}])
+    with pytest.raises(ValueError, match="2 matmul layers"):
+        with_schedule_parameters([{"wg_m": 256, "wg_n": 256}])(_Lowering(gm, False).lower()[1])
