@@ -205,7 +205,10 @@ def test_reference_torch_matmul_example():
     torch.manual_seed(0)
     a = torch.randn(m, k, device="cuda", dtype=torch.float16)
     b = torch.randn(k, n, device="cuda", dtype=torch.float16)
-    params = [{"layer_kind": "matmul", "m": m, "n": n, "k": k, "wg_m": 256, "wg_n": 128}]
+    from lighthouse_amd.schedule import ScheduleParameters
+
+    params = ScheduleParameters([{"layer_kind": "matmul", "m": m, "n": n, "k": k}])
+    params[0]["wg_m"], params[0]["wg_n"] = 256, 128      # (as the example's --wg-tile argument does, :237-238)
     backend = gpu_backend(with_schedule_parameters(params), device=torch.device("cuda"))
     model = Model()
     model.compile(dynamic=False, backend=backend)

@@ -281,3 +281,31 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setenv("LIGHTHOUSE_HIP_LIBRARY", "/nonexistent/liblighthouse_hip.so")
     with pytest.raises(ValueError, match="Could not find shared library"):
         _lib.load()
+
+
+def test_schedule_parameters_container(tmp_path):
+    """lighthouse/schedule/parameters.py: a verified list of per-layer dictionaries with a JSON round trip."""
+    from lighthouse_amd.schedule import ScheduleParameters
+
+    params = ScheduleParameters([{"layer_kind": "matmul", "m": 4096, "n": 4096, "k": 4096}])
+    params[0].update({"wg_m": 256, "wg_n": 256})
+    params.append({"layer_kind": "matmul", "wg_tile": [128, 128], "relu": True})
+    assert len(params) == 2 and [p["layer_kind"] for p in params] == ["matmul", "matmul"]
+    for bad, match in (("matmul", "must be a dictionary"), ({"wg_m": 1}, "layer_kind"), ({"layer_kind": 3}, "must be a string"),
+                       ({"layer_kind": "matmul", "x": object()}, "values must be"), ({"layer_kind": "matmul", 1: 2}, "keys must be")):
+        with pytest.raises(ValueError, match=match):
+            params.append(bad)
+        with pytest.raises(ValueError, match=match):
+            ScheduleParameters([bad])
+    with pytest.raises(ValueError, match="list of dictionaries"):
+        ScheduleParameters({"layer_kind": "matmul"})
+    path = tmp_path / "p.json"
+    params.to_json(path)
+    with pytest.raises(FileExistsError):
+        params.to_json(path)
+    params.to_json(path, overwrite=True)
+    again = ScheduleParameters.from_json(str(path))
+    assert list(again) == list(params)
+    del again[1]
+    again.insert(0, {"layer_kind": "attention"})
+    assert [p["layer_kind"] for p in again] == ["attention", "matmul"] and len(ScheduleParameters(None)) == 0
