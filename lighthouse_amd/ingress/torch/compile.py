@@ -524,7 +524,7 @@ def _check_schedule(name: str, schedule: dict, M: int, N: int, K: int) -> None:
                          f"{M}x{N}x{K}")
 
 
-_SCHEDULE_KEYS = {"layer_kind", "m", "n", "k", "wg_m", "wg_n", "split_k"}
+_SCHEDULE_KEYS = {"layer_kind", "m", "n", "k", "wg_m", "wg_n", "split_k", "transpose_a", "transpose_b", "source"}
 
 
 def with_schedule_parameters(parameters: Sequence[dict]) -> Callable[[list[PlanStep]], list[PlanStep]]:

@@ -1,3 +1,4 @@
+from .parameter_selector import HipParameterSelector
 from .parameters import ScheduleParameters
 
-__all__ = ["ScheduleParameters"]
+__all__ = ["HipParameterSelector", "ScheduleParameters"]

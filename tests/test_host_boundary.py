@@ -309,3 +309,33 @@ def test_schedule_parameters_container(tmp_path):
     del again[1]
     again.insert(0, {"layer_kind": "attention"})
     assert [p["layer_kind"] for p in again] == ["attention", "matmul"] and len(ScheduleParameters(None)) == 0
+
+
+def test_parameter_selector_database_then_cost_model(tmp_path):
+    """lighthouse/schedule/xegpu/xegpu_parameter_selector.py:26-85: a shape in the database gets its
+    entry, any other the cost model's first configuration; the result feeds the torch ingress."""
+    from lighthouse_amd.ingress.torch import with_schedule_parameters
+    from lighthouse_amd.schedule import HipParameterSelector, ScheduleParameters
+    from lighthouse_amd.tuning import TileDB
+
+    db = TileDB(str(tmp_path / "db.json"))
+    db.record("bf16", 16, 8192, 8192, None, 25.0, 86.0, split_k=4)
+    db.record("bf16", 8192, 768, 768, (256, 128), 20.0, 480.0)
+    db.save()
+    sel = HipParameterSelector(str(tmp_path / "db.json"))
+    assert sel.get_parameters_dict((16, 8192, 8192)) == {
+        "layer_kind": "matmul", "m": 16, "n": 8192, "k": 8192, "transpose_a": False, "transpose_b": False,
+        "source": "database", "split_k": 4}
+    hit = sel.get_parameters((8192, 768, 768))
+    assert isinstance(hit, ScheduleParameters) and (hit[0]["wg_m"], hit[0]["wg_n"], hit[0]["source"]) == (256, 128, "database")
+    miss = sel.get_parameters_dict((4096, 4096, 4096))
+    assert (miss["wg_m"], miss["wg_n"], miss["source"]) == (256, 256, "cost model")
+    assert sel.get_parameters_dict((8192, 768, 768), transpose_b=True)["source"] == "cost model"
+    assert sel.get_parameters_dict((1024, 1024, 1024), dtype="f32")["wg_m"] in (128, 64)
+    with pytest.raises(ValueError, match="did not return any valid"):
+        sel.get_parameters_dict((100, 100, 100))
+    layers = sel.get_parameters_for_layers([{"shape": (8192, 2304, 768)}, {"shape": (8192, 768, 3072)}])
+    assert len(layers) == 2 and all(p["layer_kind"] == "matmul" for p in layers)
+    with_schedule_parameters(layers)      # every key the selector writes is one the ingress accepts
+    # the packaged database loads by default
+    assert HipParameterSelector().get_parameters_dict((2048, 2048, 2048))["layer_kind"] == "matmul"
