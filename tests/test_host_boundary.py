@@ -339,3 +339,23 @@ def test_parameter_selector_database_then_cost_model(tmp_path):
     with_schedule_parameters(layers)      # every key the selector writes is one the ingress accepts
     # the packaged database loads by default
     assert HipParameterSelector().get_parameters_dict((2048, 2048, 2048))["layer_kind"] == "matmul"
+
+
+def test_torch_tensors_as_packed_arguments():
+    """lighthouse/utils/torch.py:41-83: element strides of views, rank 0, integers among the tensors."""
+    import torch
+
+    from lighthouse_amd.utils.torch import to_memref, to_packed_args
+
+    base = torch.arange(24, dtype=torch.float32).reshape(4, 6)
+    view = base[:, 1:5].t()
+    d = to_memref(view)
+    assert d.aligned == view.data_ptr() and tuple(d.shape) == (4, 4) and tuple(d.strides) == (1, 6) and d.offset == 0
+    scalar = to_memref(torch.tensor(3.0))
+    assert not hasattr(scalar, "shape") and scalar.offset == 0
+    packed = to_packed_args([base, 7, view])
+    assert len(packed) == 3
+    second = ctypes.cast(packed[1], ctypes.POINTER(ctypes.c_int64))
+    assert second[0] == 7
+    inner = ctypes.cast(packed[2], ctypes.POINTER(ctypes.POINTER(type(d))))
+    assert tuple(inner[0][0].strides) == (1, 6)
