@@ -326,6 +326,7 @@ int lh_hip_nanogpt_block(float* y, const float* x, const lh_nanogpt_block_params
     lh_strides3 sqkv = {T * 3 * C, hs, 3 * C};
     lh_strides3 so = {T * C, hs, C};
     const char* qp = reinterpret_cast<const char*>(qkv);
+    NoAttentionScratchScope own_workspace_only;  // (the block's temporaries all come from `workspace`)
     if ((rc = lh_hip_attention(att, qp, qp + (size_t)C * e, qp + (size_t)2 * C * e, B, n_head, T, hs, so, sqkv, sqkv,
                                sqkv, 0.0f, cfg.causal ? 1 : 0, dtype, s)))
       return rc;

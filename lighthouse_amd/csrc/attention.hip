@@ -34,6 +34,12 @@ struct AttnArgs {
   int cus;  // compute units of the device (causal launch order)
   int request = 0;  // LH_ATTN_ROWS_* | LH_ATTN_STAGES_* bits of the call (0: the library chooses)
   int d = 0;        // head dimension of the call (the padded kernels mask the columns from d on)
+  // Key range split between workgroups (few query blocks, long sequences): `kv_groups` workgroups
+  // per query block each take a contiguous share of its key tiles and leave (unnormalised output,
+  // offset, row sum) in `part`; attention16_merge combines them.  1: one workgroup per query block.
+  int kv_groups = 1;
+  float* part = nullptr;
+  bool allow_grid_split = true;  // the caller lets the launch take temporary memory for it
 };
 
 template <int DT>
@@ -311,8 +317,12 @@ __device__ __forceinline__ void xcd_block_of(int L, int nqb, int bhn, int& qb, i
 // output, offset, row sum) over through LDS and the first combines the two.  Same waves per CU as
 // two workgroups of 4, but the two halves of a query block's key range run side by side and end
 // together: the chain of key tiles a causal problem's heaviest query block has to walk is half as long.
-template <int DT, int NQ, int NS, bool RAGGED, int KS = 1>
+// GS = 1: the key range of a query block is split between a.kv_groups WORKGROUPS (1-D grid, query
+// blocks heaviest first, the groups of one block next to each other); each leaves its partial
+// result in a.part and attention16_merge finishes the block.
+template <int DT, int NQ, int NS, bool RAGGED, int KS = 1, int GS = 0>
 __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attention16_kernel(AttnArgs a) {
+  static_assert(!(GS && (KS != 1 || RAGGED)), "the grid split runs four waves per workgroup on whole key tiles");
   constexpr int kRowsPerWave = 32 * NQ, kRowsPerGroup = 4 * kRowsPerWave;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn_all[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -321,8 +331,13 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
   uint8_t* const smem_attn = smem_attn_all + ksplit * (NS * kAttnStageBytes);
   const int r32 = lane & 31, h = lane >> 5;
   const int nqb = (a.T + kRowsPerGroup - 1) / kRowsPerGroup;
-  int qb, bh;
-  if (a.causal) {
+  int qb, bh, grp = 0;
+  if constexpr (GS) {
+    const int per = a.Z * a.H * a.kv_groups, rem = (int)blockIdx.x % per;
+    qb = nqb - 1 - (int)blockIdx.x / per;
+    bh = rem / a.kv_groups;
+    grp = rem % a.kv_groups;
+  } else if (a.causal) {
     // (KS = 2: one workgroup per CU at a time, the others start as CUs free up: plainly heaviest first.)
     causal_block_of(blockIdx.x, gridDim.x, KS == 2 ? (int)gridDim.x : a.cus, nqb, a.Z * a.H, qb, bh);
   } else {
@@ -415,9 +430,11 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
   // This group's key tiles are t_first .. t_first + ntiles - 1; every wave of the workgroup walks
   // `steps` iterations (the larger of the two counts), because the barrier in the loop is the
   // workgroup's: a group that has run out of tiles neither loads nor computes in the rest.
-  const int steps = KS == 2 ? (ntiles_all + 1) / 2 : ntiles_all;
-  const int t_first = ksplit * steps;
-  const int ntiles = KS == 2 ? (ksplit ? ntiles_all - steps : steps) : ntiles_all;
+  const int share = GS ? (ntiles_all + a.kv_groups - 1) / a.kv_groups : 0;  // key tiles per workgroup of a split block
+  const int t_first = GS ? grp * share : ksplit * ((ntiles_all + 1) / 2);
+  const int ntiles = GS ? max(0, min(share, ntiles_all - t_first))
+                        : (KS == 2 ? (ksplit ? ntiles_all - (ntiles_all + 1) / 2 : (ntiles_all + 1) / 2) : ntiles_all);
+  const int steps = GS ? ntiles : (KS == 2 ? (ntiles_all + 1) / 2 : ntiles_all);
   constexpr int kAttnStages = NS;  // K/V ring depth, 3 or 4
 #pragma unroll
   for (int st = 0; st < kAttnStages - 1; ++st)
@@ -447,8 +464,32 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
     const bool active = wave_valid && (KS == 1 || it < ntiles) && (!a.causal || (j0 <= wq0 + kRowsPerWave - 1));
     const bool need_mask = (a.causal && (j0 + kKvTile - 1 > wq0)) || (RAGGED && j0 + kKvTile > a.T);
     const int nxt = it + kAttnStages - 1;
-    attn_tile<DT, NQ, RAGGED, !(NQ == 1 && NS == 3) && !(NQ == 2 && RAGGED), KS>(c, a, qf, acc_o, m_run, l_run, neg_m, smem_attn + (it % kAttnStages) * kAttnStageBytes,
+    attn_tile<DT, NQ, RAGGED, !(NQ == 1 && NS == 3) && !(NQ == 2 && RAGGED), KS + 2 * GS>(c, a, qf, acc_o, m_run, l_run, neg_m, smem_attn + (it % kAttnStages) * kAttnStageBytes,
                   smem_attn + (nxt % kAttnStages) * kAttnStageBytes, t_first + nxt, nxt < ntiles, j0, wq0, active, need_mask, it == 0);
+  }
+
+  if constexpr (GS) {
+    // This workgroup's share of the block: accumulators in the order of the hand-over below
+    // (block (wave, qt, j), four 16-byte groups of 64 lanes each), then offsets and row sums.  A
+    // workgroup without a visible key tile leaves offset -inf, sum 0 and zeros.
+    constexpr size_t kAccVec = (size_t)4 * NQ * 2 * 4 * 64;  // f32x4 elements
+    float* const mine = a.part + ((size_t)(qb * (a.Z * a.H) + bh) * a.kv_groups + grp) * (kAccVec * 4 + 4 * NQ * 2 * 64);
+    f32x4* const po = reinterpret_cast<f32x4*>(mine);
+    float* const ps = mine + kAccVec * 4;
+    if (wave_valid) {
+#pragma unroll
+      for (int qt = 0; qt < NQ; ++qt) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            po[(((wave * NQ + qt) * 2 + j) * 4 + g) * 64 + lane] =
+                f32x4{acc_o[qt][j][4 * g], acc_o[qt][j][4 * g + 1], acc_o[qt][j][4 * g + 2], acc_o[qt][j][4 * g + 3]};
+        ps[((wave * NQ + qt) * 2 + 0) * 64 + lane] = m_run[qt];
+        ps[((wave * NQ + qt) * 2 + 1) * 64 + lane] = l_run[qt];
+      }
+    }
+    return;
   }
 
   if constexpr (KS == 2) {
@@ -737,6 +778,83 @@ static int attention16_launch_ragged(const AttnArgs& a, hipStream_t s) {
   return check_launch("attention16");
 }
 
+// Second kernel of a launch whose query blocks were split between workgroups: one workgroup per
+// query block reads the kv_groups partial results in the order of the groups (so the result does
+// not depend on which finished first), rescales them to the common offset, normalises and writes
+// the rows.  Same thread -> element mapping as the attention kernel's own epilogue.
+template <int DT, int NQ>
+__global__ void __launch_bounds__(256) attention16_merge(AttnArgs a) {
+  constexpr int kRowsPerWave = 32 * NQ, kRowsPerGroup = 4 * kRowsPerWave;
+  constexpr size_t kAccVec = (size_t)4 * NQ * 2 * 4 * 64, kPartFloats = kAccVec * 4 + 4 * NQ * 2 * 64;
+  constexpr int kMaxGroups = 16;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r32 = lane & 31, h = lane >> 5;
+  const int bhn = a.Z * a.H, G = a.kv_groups;
+  const int qb = (int)blockIdx.x / bhn, bh = (int)blockIdx.x % bhn;
+  // blockIdx.y: which 4 columns x 64 lanes piece of the wave's rows (sub-tile qt, column block j, group q4)
+  const int qt = (int)blockIdx.y / 8, j = ((int)blockIdx.y / 4) & 1, q4 = (int)blockIdx.y & 3;
+  const int z = bh / a.H, hd = bh % a.H;
+  const int wq0 = qb * kRowsPerGroup + wave * kRowsPerWave;
+  if (wq0 >= a.T) return;
+  const float* const base = a.part + (size_t)(qb * bhn + bh) * G * kPartFloats;
+  // Offsets are per query row (equal in the two lanes that share it), sums per lane; a group that
+  // saw no visible key has offset -inf and counts as zero.  All loads of a pass are independent.
+  float f[kMaxGroups], lg[kMaxGroups];
+  f32x4 v[kMaxGroups];
+#pragma unroll
+  for (int g = 0; g < kMaxGroups; ++g) {
+    const float* p = base + (size_t)min(g, G - 1) * kPartFloats;
+    f[g] = p[kAccVec * 4 + ((wave * NQ + qt) * 2 + 0) * 64 + lane];
+    lg[g] = p[kAccVec * 4 + ((wave * NQ + qt) * 2 + 1) * 64 + lane];
+    v[g] = reinterpret_cast<const f32x4*>(p)[(((wave * NQ + qt) * 2 + j) * 4 + q4) * 64 + lane];
+  }
+  float m_all = -INFINITY;
+#pragma unroll
+  for (int g = 0; g < kMaxGroups; ++g) m_all = fmaxf(m_all, f[g]);  // (slots from G on repeat the last group)
+  float l = 0.0f;
+  f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int g = 0; g < kMaxGroups; ++g) {
+    const float w = (g >= G || f[g] == -INFINITY) ? 0.0f : exp2_fast(f[g] - m_all);
+    l += lg[g] * w;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] += v[g][e] * w;
+  }
+  const float inv_l = 1.0f / halfwave_sum(l);
+  uint16_t* orow = reinterpret_cast<uint16_t*>(a.out) + (int64_t)z * a.so.z + (int64_t)hd * a.so.h +
+                   (int64_t)(wq0 + 32 * qt + r32) * a.so.t;
+  u32x2 w = {pack2<DT>(acc[0] * inv_l, acc[1] * inv_l), pack2<DT>(acc[2] * inv_l, acc[3] * inv_l)};
+  *reinterpret_cast<u32x2*>(orow + 32 * j + 8 * q4 + 4 * h) = w;
+}
+
+// Query blocks split between `groups` workgroups each (a.T a multiple of the key tile): the
+// attention kernel leaves partial results in temporary memory, the merge kernel finishes.
+template <int DT, int NQ>
+static int attention16_launch_split(const AttnArgs& a_in, int groups, hipStream_t s) {
+  constexpr size_t kPartFloats = (size_t)4 * NQ * 2 * 4 * 64 * 4 + 4 * NQ * 2 * 64;
+  constexpr size_t lds = (size_t)4 * kAttnStageBytes;
+  auto kern = attention16_kernel<DT, NQ, 4, false, 1, 1>;
+  auto merge = attention16_merge<DT, NQ>;
+  static bool configured = false;
+  if (!configured && !planning()) {
+    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)lds));
+    configured = true;
+  }
+  const int nqb = (a_in.T + 128 * NQ - 1) / (128 * NQ), bhn = a_in.Z * a_in.H;
+  void* part = nullptr;
+  if (int rc = scratch_take(nullptr, s, kScratchAttention, (size_t)nqb * bhn * groups * kPartFloats * sizeof(float),
+                            "attention (key range split between workgroups)", &part))
+    return rc;
+  AttnArgs a = a_in;
+  a.kv_groups = groups;
+  a.part = static_cast<float*>(part);
+  LH_LAUNCH(kern, dim3(nqb * bhn * groups), dim3(256), lds, s, a);
+  if (int rc = check_launch("attention16 (split)")) return rc;
+  LH_LAUNCH(merge, dim3(nqb * bhn, NQ * 8), dim3(256), 0, s, a);
+  return check_launch("attention16_merge");
+}
+
 // Sequence lengths that are no multiple of the key tile take the instantiation that clamps the
 // last tile's loads, masks it and skips rows past the end.
 template <int DT, int NQ, int NS>
@@ -779,6 +897,32 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
     LH_REQUIRE(a.T % kKvTile == 0, "attention: 64 query rows per wave need a sequence length that is a multiple of %d",
                kKvTile);
     return attention16_launch_ragged<DT, 2, 4, false, 2>(a, s);
+  }
+  // Few query blocks and many key tiles (long sequences of a few heads): the key range of every
+  // block is split between workgroups and a second kernel merges the partial results (temporary
+  // memory: 68 KiB per workgroup).  Without the split such a problem runs one 128-row workgroup on
+  // at most every CU, each walking the whole key range (causal: the heaviest does): about 5 us +
+  // 0.77 us per key tile.  With it a workgroup walks 1 / groups of the range at 1.075 us per tile
+  // (1.61 when two share a CU, whose start-up also costs 5 us less than a lone workgroup's) and the
+  // launch pays 7.2 us (second launch, first loads) + 0.027 us per workgroup for writing and reading
+  // the partial results.  Fitted on [1,1,8192] 93.7 -> 31 us,
+  // [1,4,4096] 49.9 -> 33.5, [1,4,8192] 104 -> 83 -> (4 groups), [1,1,16384] 183 -> 78, and on
+  // [2,8,2048], which stays whole (28.4 us against 34.7 split).
+  if (!ksplit_req && !rows_req && !stages_req && a.allow_grid_split && a.T % kKvTile == 0 && 2 * groups64 <= a.cus) {
+    const int ntiles = a.T / kKvTile;
+    const double whole = 5.0 + 0.77 * ntiles;
+    int best_groups = 1;
+    double best = 0.9 * whole;  // the split has to win by a margin
+    for (int groups = 2; groups <= 16 && ntiles / groups >= 2; groups *= 2) {
+      const int64_t wgs = groups64 * groups;
+      const double t = (wgs <= a.cus ? 12.2 : 7.2) + 0.027 * (double)wgs +
+                       (double)((ntiles + groups - 1) / groups) * (wgs <= a.cus ? 1.075 : 1.61);
+      if (wgs <= 2 * (int64_t)a.cus && t < best) {
+        best = t;
+        best_groups = groups;
+      }
+    }
+    if (best_groups > 1) return attention16_launch_split<DT, 2>(a, best_groups, s);
   }
   // Unasked, the split pays where at most one 256-row workgroup falls on a CU but more than half
   // the CUs get one: a lone group of four waves leaves each SIMD with a single wave, and splitting the
@@ -1384,6 +1528,7 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   a.scale = scale;
   a.scale_log2e = scale * 1.4426950408889634f;
   a.d = (int)d;
+  a.allow_grid_split = attention_scratch_allowed();
   LH_REQUIRE((causal & ~(int32_t)(LH_ATTN_CAUSAL | LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK | LH_ATTN_KSPLIT_MASK)) == 0 &&
                  (causal & LH_ATTN_ROWS_MASK) != LH_ATTN_ROWS_MASK && (causal & LH_ATTN_STAGES_MASK) != LH_ATTN_STAGES_MASK &&
                  (causal & LH_ATTN_KSPLIT_MASK) != LH_ATTN_KSPLIT_MASK,

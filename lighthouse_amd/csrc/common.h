@@ -178,7 +178,7 @@ int pad_copy_matrix(void* dst, int64_t ld_dst, int rows_dst, int cols_dst, const
 //    device-wide synchronisation, inside a call).
 // While planning() is true (a *_workspace_bytes query on this thread) nothing is launched or
 // allocated: takes return a dummy address and add their size to `need`.
-enum ScratchSlot { kScratchTranspose = 0, kScratchPad, kScratchSplitK, kScratchSkinny, kScratchMlp, kScratchSlots };
+enum ScratchSlot { kScratchTranspose = 0, kScratchPad, kScratchSplitK, kScratchSkinny, kScratchMlp, kScratchAttention, kScratchSlots };
 struct Scratch {
   char* base = nullptr;
   size_t bytes = 0;
@@ -190,6 +190,14 @@ bool planning();
 struct PlanningScope {  // marks the calling thread as running a size query
   PlanningScope();
   ~PlanningScope();
+};
+// Entry points that run on a caller's workspace only (the nanoGPT block and forward) keep their
+// attention launches from taking pool memory: while such a scope is alive on the calling thread,
+// lh_hip_attention does not split key ranges between workgroups.
+bool attention_scratch_allowed();
+struct NoAttentionScratchScope {
+  NoAttentionScratchScope();
+  ~NoAttentionScratchScope();
 };
 #define LH_LAUNCH(...)                                        \
   do {                                                        \

@@ -140,6 +140,10 @@ static thread_local int g_planning = 0;
 bool planning() { return g_planning > 0; }
 PlanningScope::PlanningScope() { ++g_planning; }
 PlanningScope::~PlanningScope() { --g_planning; }
+static thread_local int g_no_attention_scratch = 0;
+bool attention_scratch_allowed() { return g_no_attention_scratch == 0; }
+NoAttentionScratchScope::NoAttentionScratchScope() { ++g_no_attention_scratch; }
+NoAttentionScratchScope::~NoAttentionScratchScope() { --g_no_attention_scratch; }
 
 namespace {
 struct PoolBuffer {

@@ -330,3 +330,32 @@ def test_attention_variant_request_errors():
     q128 = torch.zeros(1, 2, 256, 128, device="cuda", dtype=torch.bfloat16)
     with pytest.raises(ValueError, match="head_dim 64"):
         ops.attention(q128, q128, q128, rows_per_wave=32)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype,elt", [(torch.bfloat16, "bf16"), (torch.float16, "f16")])
+@pytest.mark.parametrize("shape", [(1, 1, 4096, 64), (1, 2, 2048, 64), (1, 3, 1024, 64), (2, 2, 512, 64), (1, 1, 8192, 64),
+                                   (1, 5, 1088, 64)])
+def test_attention_key_range_split_between_workgroups(shape, dtype, elt, causal):
+    """Few query blocks with many key tiles: the key range of every block is shared out to several
+    workgroups and a second kernel merges their (unnormalised output, offset, row sum).  Against the
+    oracle on sampled heads, on strided views with the same bits, and twice in a row (the temporary
+    memory is reused)."""
+    from lighthouse_amd import ops
+
+    Z, H, T, D = shape
+    rng = np.random.default_rng(sum(shape) + 3 * causal)
+    q, k, v = (orc.round_to(rng.standard_normal(shape).astype(np.float32), elt) for _ in range(3))
+    dq, dk, dv = (_dev(x, dtype) for x in (q, k, v))
+    out = ops.attention(dq, dk, dv, causal=causal)
+    for z, h in {(0, 0), (Z - 1, H - 1)}:
+        ref = orc.attention(q[z, h], k[z, h], v[z, h], causal=causal, result_type=elt)
+        assert_close(_host(out[z, h]), ref, 2e-2, f"split attention {shape} {elt} z={z} h={h} causal={causal}")
+    assert torch.equal(ops.attention(dq, dk, dv, causal=causal), out)
+    qs, ks, vs = (x.transpose(1, 2).contiguous().transpose(1, 2) for x in (dq, dk, dv))
+    outs = torch.empty((Z, T, H, D), dtype=dtype, device="cuda").transpose(1, 2)
+    ops.attention(qs, ks, vs, causal=causal, out=outs)
+    assert torch.equal(outs, out)
+    # one workgroup per query block (an explicit variant request) gives the same result up to the grouping of the sums
+    whole = ops.attention(dq, dk, dv, causal=causal, rows_per_wave=64, kv_split=1)
+    assert_close(_host(out), _host(whole), 2e-2, f"split vs whole {shape} {elt} causal={causal}")
