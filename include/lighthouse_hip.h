@@ -76,7 +76,8 @@ typedef enum lh_dtype {
 /* Workgroup-tile request, the counterpart of the wg_m / wg_n schedule parameters
  * (lighthouse/schedule/xegpu/mlp_schedule.py:72-78,142).  AUTO lets the library pick by shape.
  * 16-bit inputs take 256x256, 256x128, 128x256 and 128x128: the tile must divide M and N and
- * needs untransposed operands, K % 64 == 0 and 16-byte aligned rows.  f32 inputs take 128x128,
+ * needs an untransposed A (B may be stored transposed: the kernels read an [N, K] matrix with
+ * aligned rows in place), K % 64 == 0 and 16-byte aligned rows.  f32 inputs take 128x128,
  * 128x64 and 64x64 (M and N need not be multiples): untransposed operands, K % 32 == 0, N % 4 == 0
  * and 16-byte aligned rows.  A request the problem does not meet fails with LH_ERR_INVALID. */
 #define LH_GEMM_TILE_MASK 0x700u
@@ -91,7 +92,7 @@ typedef enum lh_dtype {
  * of A and rows of B and write an f32 block; a second kernel adds the blocks and runs the
  * epilogue), for problems with too few tiles to fill the CUs; the k-dimension counterpart of the
  * tile request above (lighthouse/schedule/xegpu/matmul_params.json holds such per-shape choices).
- * AUTO lets the library decide; NONE forbids the cut; 2 / 4 / 8 request it and need untransposed
+ * AUTO lets the library decide; NONE forbids the cut; 2 / 4 / 8 request it and need an untransposed A,
  * aligned operands and K / splits a multiple of 64 (runs on 128 x 128 tiles, so it excludes a tile
  * request). */
 #define LH_GEMM_SPLITK_MASK 0x3800u

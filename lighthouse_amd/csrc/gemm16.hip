@@ -221,6 +221,7 @@ struct DirectCfg {
   static constexpr int kABytes = BM * 64 * 2;             // one A stage (64 k)
   static constexpr int kBRow = BN * 2;                    // bytes of one k row of a B stage
   static constexpr int kBBytes = 32 * kBRow;              // one B stage (32 k)
+  static constexpr int kBtBytes = BN * 64 * 2;            // one stage (64 k) of a transposed B: rows n, like A
   static constexpr int kBBase = 2 * kABytes;
   static constexpr int kRingBytes = kBBase + 4 * kBBytes;
   static constexpr int kStageBytes = 8 * 32 * WTN * 2;    // output staging: 32 rows of each wave's sub-tile
@@ -253,6 +254,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t panel_resource(const void* bas
 // The direct kernels address a tile's operand panels with 32-bit byte offsets from the panel's
 // first element: 256 rows of A, K rows of B.
 static inline bool direct_offsets_fit(const GemmArgs& g) {
+  if (g.flags & LH_GEMM_TRANSPOSE_B) return g.lda < (1ll << 22) && g.ldb < (1ll << 22);  // 256 rows of B^T
   return g.lda < (1ll << 22) && (int64_t)g.K * g.ldb < (1ll << 30);
 }
 
@@ -266,6 +268,10 @@ struct DirectCtx {
   int a_off[TM];              // byte offset of the lane's A row in a stage, per m-subtile
   int a_swz[TM];
   int wave, h, b_off, b_chunk, b_swz;
+  // B stored transposed ([N, K], k contiguous): its panel is laid out, loaded and read like A's
+  int bt_src[2 * TN];         // lane's byte offset in the B^T panel for load i at k = 0
+  int bt_off[TN];             // byte offset of the lane's B^T row in a stage, per n-subtile
+  int bt_swz[TN];
 };
 
 template <int TM, int TN>
@@ -281,22 +287,33 @@ __device__ __forceinline__ void direct_load_a(const DirectCtx<TM, TN>& c, int sa
 #pragma unroll
   for (int i = 0; i < TM; ++i) dma16(rsrc, c.a_src[i], sa * 128, abuf + (8 * i + c.wave) * 1024);
 }
-// B stage `sb` (k = 32 sb .. +32): TN loads per lane.
-template <int TM, int TN>
+// B stage `sb` (k = 32 sb .. +32): TN loads per lane.  BT (B stored [N, K]): stage sb is k = 64 sb .. +64
+// of the panel's rows, 2 TN loads per lane.
+template <int TM, int TN, bool BT = false>
 __device__ __forceinline__ void direct_load_b(const DirectCtx<TM, TN>& c, int sb, uint8_t* __restrict__ bbuf) {
   const __amdgpu_buffer_rsrc_t rsrc = panel_resource(c.b_base);
+  if constexpr (BT) {
 #pragma unroll
-  for (int i = 0; i < TN; ++i) dma16(rsrc, c.b_src[i], sb * c.b_step, bbuf + (8 * i + c.wave) * 1024);
+    for (int i = 0; i < 2 * TN; ++i) dma16(rsrc, c.bt_src[i], sb * 128, bbuf + (8 * i + c.wave) * 1024);
+  } else {
+#pragma unroll
+    for (int i = 0; i < TN; ++i) dma16(rsrc, c.b_src[i], sb * c.b_step, bbuf + (8 * i + c.wave) * 1024);
+  }
 }
 
 // Fragments of 16 k: A chunk pair `kc` (0..3: which 16 of the stage's 64 k), B k-step `ks`
 // (0..1: which 16 of the stage's 32 k).
-template <int TM, int TN>
+// BT: `bs` is a 64-k stage of the transposed B; its fragments are 16-byte reads like A's, chunk pair kc.
+template <int TM, int TN, bool BT = false>
 __device__ __forceinline__ void direct_read_frags(const DirectCtx<TM, TN>& c, const uint8_t* __restrict__ as,
                                                   const uint8_t* __restrict__ bs, int kc, int ks,
                                                   DirectFrags<TM, TN>& f) {
   constexpr int row = DirectCfg<TM, TN>::kBRow;
   auto read_b = [&](int i) {
+    if constexpr (BT) {
+      f.b[i] = *reinterpret_cast<const u32x4*>(bs + c.bt_off[i] + (((2 * kc + c.h) ^ c.bt_swz[i]) << 4));
+      return;
+    }
     const int p = (c.b_chunk + 4 * i) ^ c.b_swz;
     const uint8_t* p0 = bs + ks * 16 * row + c.b_off + p * 16;
     s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p0);
@@ -391,7 +408,7 @@ __device__ __forceinline__ void direct_step_pair(const DirectCtx<TM, TN>& c, f32
 // EDGE: M and N need not be multiples of the tile (N still a multiple of 8, K of 64): loads of
 // rows / column chunks past the end are redirected to the last valid row / chunk (their products
 // land in accumulators that are never stored) and the epilogue skips what lies outside the matrix.
-template <int TM, int TN, bool EDGE>
+template <int TM, int TN, bool EDGE, bool BT = false>
 __device__ __forceinline__ void direct_place(const GemmArgs& g, int id, DirectCtx<TM, TN>& c, int& m0, int& n0) {
   using Cfg = DirectCfg<TM, TN>;
   constexpr int BM = Cfg::BM, BN = Cfg::BN;
@@ -409,7 +426,7 @@ __device__ __forceinline__ void direct_place(const GemmArgs& g, int id, DirectCt
   const uint16_t* B = reinterpret_cast<const uint16_t*>(g.b);
   const int lda = (int)g.lda, ldb = (int)g.ldb;
   c.a_base = A + (int64_t)m0 * g.lda;
-  c.b_base = B + n0;
+  c.b_base = BT ? B + (int64_t)n0 * g.ldb : B + n0;
   c.b_step = 64 * ldb;
   // A: load i of wave w fills rows (8 i + w) 8 .. +8 (1024 bytes); lane -> row += lane / 8, LDS
   // chunk p = lane % 8 holds global chunk p ^ ((row / 2) % 8).
@@ -422,12 +439,23 @@ __device__ __forceinline__ void direct_place(const GemmArgs& g, int id, DirectCt
   }
   // B: load i of wave w fills k rows (8 i + w) R .. +R with R = 1024 / row bytes; lane ->
   // row += lane / chunks-per-row, LDS chunk p holds global chunk p ^ 4 (k % 4).
+  if constexpr (BT) {
+    // B^T: exactly A's scheme on the panel's BN rows (row n of B^T = column n of B)
 #pragma unroll
-  for (int i = 0; i < TN; ++i) {
-    const int bk = (8 * i + c.wave) * Cfg::kBRowsPerLoad + lane / Cfg::kBChunks;
-    const int bc = (lane % Cfg::kBChunks) ^ (4 * (bk & 3));
-    const int bcol = EDGE ? min(bc * 8, g.N - 8 - n0) : bc * 8;  // column within the panel
-    c.b_src[i] = (bk * ldb + bcol) * 2;
+    for (int i = 0; i < 2 * TN; ++i) {
+      const int br = (8 * i + c.wave) * 8 + (lane >> 3);
+      const int bc = (lane & 7) ^ ((br >> 1) & 7);
+      const int brow = EDGE ? min(br, g.N - 1 - n0) : br;
+      c.bt_src[i] = (brow * ldb + bc * 8) * 2;
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+      const int bk = (8 * i + c.wave) * Cfg::kBRowsPerLoad + lane / Cfg::kBChunks;
+      const int bc = (lane % Cfg::kBChunks) ^ (4 * (bk & 3));
+      const int bcol = EDGE ? min(bc * 8, g.N - 8 - n0) : bc * 8;  // column within the panel
+      c.b_src[i] = (bk * ldb + bcol) * 2;
+    }
   }
 }
 
@@ -435,7 +463,7 @@ __device__ __forceinline__ void direct_place(const GemmArgs& g, int id, DirectCt
 // of 64 k.  At the barrier every read of this pair's stages has returned and the next pair's
 // stages (issued at the previous barrier, 64 k ago) are awaited in full; the pair after that is
 // then requested into this pair's buffers.
-template <int DT, int TM, int TN>
+template <int DT, int TM, int TN, bool BT = false>
 __device__ __forceinline__ void direct_step_pair_1b(const DirectCtx<TM, TN>& c, f32x16 (&acc)[TN][TM],
                                                     DirectFrags<TM, TN>& f0, const uint8_t* __restrict__ a_cur,
                                                     const uint8_t* __restrict__ a_nxt, const uint8_t* __restrict__ b0,
@@ -445,13 +473,13 @@ __device__ __forceinline__ void direct_step_pair_1b(const DirectCtx<TM, TN>& c, 
                                                     bool stores_behind) {
   using Cfg = DirectCfg<TM, TN>;
   DirectFrags<TM, TN> f1;
-  direct_read_frags(c, a_cur, b0, 1, 1, f1);
+  direct_read_frags<TM, TN, BT>(c, a_cur, b0, 1, 1, f1);
   direct_mfma<DT>(acc, f0);
   direct_interleave_hint<TM, TN>();
-  direct_read_frags(c, a_cur, b1, 2, 0, f0);
+  direct_read_frags<TM, TN, BT>(c, a_cur, b1, 2, 0, f0);
   direct_mfma<DT>(acc, f1);
   direct_interleave_hint<TM, TN>();
-  direct_read_frags(c, a_cur, b1, 3, 1, f1);
+  direct_read_frags<TM, TN, BT>(c, a_cur, b1, 3, 1, f1);
   direct_mfma<DT>(acc, f0);
   direct_interleave_hint<TM, TN>();
   // At a tile's first barrier the only operations in flight are the previous tile's stores (the
@@ -462,23 +490,32 @@ __device__ __forceinline__ void direct_step_pair_1b(const DirectCtx<TM, TN>& c, 
   else direct_wait_barrier<0>();
   if (kt + 4 < nk) {
     direct_load_a(c, kt / 2 + 2, a_refill);
-    direct_load_b(c, kt + 4, b_refill0);
-    direct_load_b(c, kt + 5, b_refill1);
+    if constexpr (BT) {
+      direct_load_b<TM, TN, true>(c, kt / 2 + 2, b_refill0);  // (b0 = b1: the pair's one 64-k stage)
+    } else {
+      direct_load_b(c, kt + 4, b_refill0);
+      direct_load_b(c, kt + 5, b_refill1);
+    }
   }
-  direct_read_frags(c, a_nxt, b2, 0, 0, f0);
+  direct_read_frags<TM, TN, BT>(c, a_nxt, b2, 0, 0, f0);
   direct_mfma<DT>(acc, f1);
   direct_interleave_hint<TM, TN>();
 }
 
-// First loads of a tile: A stages 0, 1 and B stages 0 .. 3 (nk = K / 32 >= 2).
-template <int TM, int TN>
+// First loads of a tile: A stages 0, 1 and B stages 0 .. 3 (nk = K / 32 >= 2); BT: both 64-k stages of B^T.
+template <int TM, int TN, bool BT = false>
 __device__ __forceinline__ void direct_prologue(const DirectCtx<TM, TN>& c, int nk, uint8_t* __restrict__ ring) {
   using Cfg = DirectCfg<TM, TN>;
   direct_load_a(c, 0, ring);
   if (nk > 2) direct_load_a(c, 1, ring + Cfg::kABytes);
+  if constexpr (BT) {
+    direct_load_b<TM, TN, true>(c, 0, ring + Cfg::kBBase);
+    if (nk > 2) direct_load_b<TM, TN, true>(c, 1, ring + Cfg::kBBase + Cfg::kBtBytes);
+  } else {
 #pragma unroll
-  for (int st = 0; st < 4; ++st)
-    if (st < nk) direct_load_b(c, st, ring + Cfg::kBBase + st * Cfg::kBBytes);
+    for (int st = 0; st < 4; ++st)
+      if (st < nk) direct_load_b(c, st, ring + Cfg::kBBase + st * Cfg::kBBytes);
+  }
 }
 
 // Main loop of one tile, whose first loads have been issued.
@@ -505,7 +542,7 @@ __device__ __forceinline__ void direct_load_bias(const GemmArgs& g, int n_base, 
 // those stores may stay in flight.
 // `staged`: the epilogue will want `bias` (for columns from n_base); it is loaded ahead of the
 // last two steps, whose full wait covers it.
-template <int DT, int TM, int TN, bool EDGE>
+template <int DT, int TM, int TN, bool EDGE, bool BT = false>
 __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectCtx<TM, TN>& c, f32x16 (&acc)[TN][TM],
                                                 uint8_t* smem_d, int nk, bool stores_behind, bool staged, int n_base,
                                                 u32x2 (&bias)[TN][4]) {
@@ -515,24 +552,32 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
   // two workgroups share a compute unit, 2-7 % for the 128 x 128 tile (M = 8192, N = 768, K = 3072:
   // 46.0 -> 42.9 us); a lone 128 x 128 workgroup has nobody to cover the shorter look-ahead
   // (2048^3 22.7 -> 24.2 us) and keeps two.
-  const bool one_barrier = TM * TN > 2 || g.one_barrier;
+  // A transposed B lives in the rings as two 64-k stages like A and always takes the one-barrier form.
+  const bool one_barrier = BT || TM * TN > 2 || g.one_barrier;
   uint8_t* const abuf = smem_d;
   uint8_t* const bbuf = smem_d + Cfg::kBBase;
   if (stores_behind) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(Cfg::kStagedStores) : "memory");
   else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
   DirectFrags<TM, TN> f0;
-  direct_read_frags(c, abuf, bbuf, 0, 0, f0);
+  direct_read_frags<TM, TN, BT>(c, abuf, bbuf, 0, 0, f0);
   int kt = 0;
   auto pair = [&](auto one) {
     uint8_t* a_cur = abuf + ((kt >> 1) & 1) * Cfg::kABytes;
     uint8_t* a_nxt = abuf + (((kt >> 1) + 1) & 1) * Cfg::kABytes;
-    uint8_t* b0 = bbuf + (kt & 3) * Cfg::kBBytes;
-    uint8_t* b1 = bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
-    uint8_t* b2 = bbuf + ((kt + 2) & 3) * Cfg::kBBytes;
-    if constexpr (decltype(one)::value) direct_step_pair_1b<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk, stores_behind);
-    else direct_step_pair<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
+    if constexpr (BT) {
+      uint8_t* b_cur = bbuf + ((kt >> 1) & 1) * Cfg::kBtBytes;
+      uint8_t* b_nxt = bbuf + (((kt >> 1) + 1) & 1) * Cfg::kBtBytes;
+      direct_step_pair_1b<DT, TM, TN, true>(c, acc, f0, a_cur, a_nxt, b_cur, b_cur, b_nxt, a_cur, b_cur, b_cur, kt, nk,
+                                            stores_behind);
+    } else {
+      uint8_t* b0 = bbuf + (kt & 3) * Cfg::kBBytes;
+      uint8_t* b1 = bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
+      uint8_t* b2 = bbuf + ((kt + 2) & 3) * Cfg::kBBytes;
+      if constexpr (decltype(one)::value) direct_step_pair_1b<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk, stores_behind);
+      else direct_step_pair<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
+    }
   };
-  if constexpr (TM * TN > 2) {
+  if constexpr (BT || TM * TN > 2) {
     for (; kt + 2 < nk; kt += 2) pair(std::true_type{});
   } else if (one_barrier) {
     for (; kt + 2 < nk; kt += 2) pair(std::true_type{});
@@ -542,16 +587,16 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
   {
     // Last two steps: nothing left to load; stage nk - 1 of B must have landed.
     const uint8_t* a_cur = abuf + ((kt >> 1) & 1) * Cfg::kABytes;
-    const uint8_t* b0 = bbuf + (kt & 3) * Cfg::kBBytes;
-    const uint8_t* b1 = bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
+    const uint8_t* b0 = BT ? bbuf + ((kt >> 1) & 1) * Cfg::kBtBytes : bbuf + (kt & 3) * Cfg::kBBytes;
+    const uint8_t* b1 = BT ? b0 : bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
     DirectFrags<TM, TN> f1;
     if (staged) direct_load_bias<TN, EDGE>(g, n_base, bias);
-    direct_read_frags(c, a_cur, b0, 1, 1, f1);
+    direct_read_frags<TM, TN, BT>(c, a_cur, b0, 1, 1, f1);
     direct_mfma<DT>(acc, f0);
     if (!one_barrier) direct_wait_barrier<0>();  // (one barrier per pair: awaited at the pair before)
-    direct_read_frags(c, a_cur, b1, 2, 0, f0);
+    direct_read_frags<TM, TN, BT>(c, a_cur, b1, 2, 0, f0);
     direct_mfma<DT>(acc, f1);
-    direct_read_frags(c, a_cur, b1, 3, 1, f1);
+    direct_read_frags<TM, TN, BT>(c, a_cur, b1, 3, 1, f1);
     direct_mfma<DT>(acc, f0);
     direct_mfma<DT>(acc, f1);
   }
@@ -564,7 +609,7 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
 // against bank conflicts), and leave as full row segments of 16 bytes per lane.  `ring` and
 // `stage` are separate restrict parameters so that the staging traffic does not wait for the
 // asynchronous ring writes.
-template <int DT, int TM, int TN, bool EDGE, bool HAS_NEXT>
+template <int DT, int TM, int TN, bool EDGE, bool HAS_NEXT, bool BT = false>
 __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx<TM, TN>& next, int nk,
                                               uint8_t* __restrict__ ring, uint8_t* __restrict__ stage,
                                               const f32x16 (&acc)[TN][TM], const u32x2 (&bias)[TN][4], int m0, int n0,
@@ -586,7 +631,7 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
 #pragma unroll
         for (int e = 0; e < 2; ++e) asm volatile("" ::"v"(bias[i][q][e]));
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the rings
-    if constexpr (HAS_NEXT) direct_prologue(next, nk, ring);
+    if constexpr (HAS_NEXT) direct_prologue<TM, TN, BT>(next, nk, ring);
     constexpr int RB = WTN * 2;                // bytes of a staged row
     constexpr int chunks = RB / 16;            // 16-byte chunks per staged row
     constexpr int rows_per_pass = 64 / chunks;
@@ -627,7 +672,7 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
     return;
   }
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  if constexpr (HAS_NEXT) direct_prologue(next, nk, ring);
+  if constexpr (HAS_NEXT) direct_prologue<TM, TN, BT>(next, nk, ring);
   {
     // f32 output (with or without an accumulator input), or a 16-bit output with an accumulator
     // input: the scaled f32 accumulators of a 32 x 8 QH block go through the wave's slice of `stage`
@@ -707,7 +752,9 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
 // SPLITK: the tile list is g.splits copies of the problem's tiles, copy sp working on its own K
 // columns of A / rows of B and its own block of the (f32) output; a second kernel adds the blocks.
 // For problems with few tiles and a long K (decode shapes), where the tile count cannot fill the CUs.
-template <int DT, int TM, int TN, bool EDGE, bool SPLITK = false>
+// BT: B is stored transposed ([N, K] with row stride ldb, the layout of a torch Linear weight); its
+// panel goes through the rings like A's and no transposed copy is made.
+template <int DT, int TM, int TN, bool EDGE, bool SPLITK = false, bool BT = false>
 __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
   using Cfg = DirectCfg<TM, TN>;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_d[];
@@ -718,7 +765,7 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
     if constexpr (SPLITK) {
       const int sp = t / tiles1;
       ga.a = reinterpret_cast<const uint16_t*>(g.a) + (int64_t)sp * g.K;
-      ga.b = reinterpret_cast<const uint16_t*>(g.b) + (int64_t)sp * g.K * g.ldb;
+      ga.b = reinterpret_cast<const uint16_t*>(g.b) + (BT ? (int64_t)sp * g.K : (int64_t)sp * g.K * g.ldb);
       ga.out = reinterpret_cast<float*>(g.out) + (int64_t)sp * g.M * g.ldc;
       ga.c = ga.out;
       return t - sp * tiles1;
@@ -752,15 +799,22 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
     c.b_swz = 4 * (krow & 3);
     c.b_off = krow * Cfg::kBRow + 8 * ((col >> 2) & 1);
   }
+  // (transposed B: row wn0 + 32 i + r32 of the stage, logical chunk 2 kc + h, like the A fragment)
+#pragma unroll
+  for (int i = 0; i < TN; ++i) {
+    const int r = wn0 + 32 * i + r32;
+    c.bt_off[i] = r * 128;
+    c.bt_swz[i] = (r >> 1) & 7;
+  }
 
   const int nk = g.K / 32;  // even: K is a multiple of 64
   int t = blockIdx.x;       // < ntiles: the grid is never larger than the tile list
   int m0, n0;
   {
     const int id = select(t, g_cur);
-    direct_place<TM, TN, EDGE>(SPLITK ? g_cur : g, xcd_remap(id, tiles1), c, m0, n0);
+    direct_place<TM, TN, EDGE, BT>(SPLITK ? g_cur : g, xcd_remap(id, tiles1), c, m0, n0);
   }
-  direct_prologue(c, nk, smem_d);
+  direct_prologue<TM, TN, BT>(c, nk, smem_d);
   // Without EDGE every lane issues all stores of a staged epilogue.
   const bool staged = g.out_dt != LH_F32 && !(g.flags & LH_GEMM_ACCUMULATE_C);
   const bool counted_stores = !EDGE && staged;
@@ -775,7 +829,7 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
     u32x2 bias[TN][4];
     const GemmArgs& ga = SPLITK ? g_cur : g;
-    direct_mainloop<DT, TM, TN, EDGE>(ga, c, acc, smem_d, nk, counted_stores && !first, staged, n0 + wn0 + 4 * h, bias);
+    direct_mainloop<DT, TM, TN, EDGE, BT>(ga, c, acc, smem_d, nk, counted_stores && !first, staged, n0 + wn0 + 4 * h, bias);
     first = false;
     const int tn = t + (int)gridDim.x;
     const bool more = tn < ntiles;
@@ -784,10 +838,10 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
     uint8_t* const stage = smem_d + Cfg::kRingBytes;
     if (more) {
       const int idn = select(tn, g_nxt);
-      direct_place<TM, TN, EDGE>(SPLITK ? g_nxt : g, xcd_remap(idn, tiles1), cn, m1, n1);
-      direct_finish<DT, TM, TN, EDGE, true>(ga, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0);
+      direct_place<TM, TN, EDGE, BT>(SPLITK ? g_nxt : g, xcd_remap(idn, tiles1), cn, m1, n1);
+      direct_finish<DT, TM, TN, EDGE, true, BT>(ga, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0);
     } else {
-      direct_finish<DT, TM, TN, EDGE, false>(ga, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0);
+      direct_finish<DT, TM, TN, EDGE, false, BT>(ga, cn, nk, smem_d, stage, acc, bias, m0, n0, wm0, wn0);
     }
     if (!more) break;
     if constexpr (SPLITK) g_cur = g_nxt;
@@ -798,10 +852,10 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
   }
 }
 
-template <int DT, int TM, int TN, bool EDGE>
+template <int DT, int TM, int TN, bool EDGE, bool BT = false>
 static int launch_direct_edge(const GemmArgs& g, hipStream_t s) {
   using Cfg = DirectCfg<TM, TN>;
-  auto kern = gemm16_direct<DT, TM, TN, EDGE>;
+  auto kern = gemm16_direct<DT, TM, TN, EDGE, false, BT>;
   constexpr size_t lds = Cfg::kLdsBytes;
   static bool configured = false;
   if (!configured && !planning()) {
@@ -820,8 +874,10 @@ static int launch_direct_edge(const GemmArgs& g, hipStream_t s) {
 template <int DT, int TM, int TN>
 static int launch_direct(const GemmArgs& g, hipStream_t s) {
   using Cfg = DirectCfg<TM, TN>;
-  if (g.M % Cfg::BM == 0 && g.N % Cfg::BN == 0) return launch_direct_edge<DT, TM, TN, false>(g, s);
-  return launch_direct_edge<DT, TM, TN, true>(g, s);
+  const bool whole = g.M % Cfg::BM == 0 && g.N % Cfg::BN == 0;
+  if (g.flags & LH_GEMM_TRANSPOSE_B)
+    return whole ? launch_direct_edge<DT, TM, TN, false, true>(g, s) : launch_direct_edge<DT, TM, TN, true, true>(g, s);
+  return whole ? launch_direct_edge<DT, TM, TN, false>(g, s) : launch_direct_edge<DT, TM, TN, true>(g, s);
 }
 
 // Any shape / stride / transpose; 64 x 64 x 32 tiles, 256 threads, bounds-checked.
@@ -987,9 +1043,14 @@ static int gemm16_splitk(const GemmArgs& g, uint32_t request, hipStream_t s) {
     LH_LAUNCH(kern, dim3((unsigned)(total < resident ? total : resident)), dim3(512), Cfg::kLdsBytes, s, p);
     return check_launch("gemm16_direct (split K)");
   };
-  static bool configured_edge = false, configured_whole = false;
-  const int rc = edge ? launch(gemm16_direct<DT, 2, 1, true, true>, configured_edge)
-                      : launch(gemm16_direct<DT, 2, 1, false, true>, configured_whole);
+  static bool configured_edge = false, configured_whole = false, configured_edge_bt = false, configured_whole_bt = false;
+  int rc;
+  if (g.flags & LH_GEMM_TRANSPOSE_B)
+    rc = edge ? launch(gemm16_direct<DT, 2, 1, true, true, true>, configured_edge_bt)
+              : launch(gemm16_direct<DT, 2, 1, false, true, true>, configured_whole_bt);
+  else
+    rc = edge ? launch(gemm16_direct<DT, 2, 1, true, true>, configured_edge)
+              : launch(gemm16_direct<DT, 2, 1, false, true>, configured_whole);
   if (rc) return rc;
   const int64_t groups = (int64_t)g.M * g.N / 4;
   const int rb = reduce_block(groups);
@@ -1000,12 +1061,18 @@ static int gemm16_splitk(const GemmArgs& g, uint32_t request, hipStream_t s) {
 template <int DT>
 static int gemm16_dispatch(const GemmArgs& g_in, hipStream_t s) {
   GemmArgs g = g_in;
+  // A transposed B ([N, K], k contiguous) with aligned rows goes through the direct kernels as it is
+  // (its panel is loaded and read like A's); a transposed A is copied into [M, K] first.
+  const bool b_in_place = (g.flags & LH_GEMM_TRANSPOSE_B) && g.ldb % 8 == 0 && aligned16(g.b) && g.K % kBK == 0;
   if ((g.flags & LH_GEMM_TILE_MASK) == LH_GEMM_TILE_AUTO && g.ldc % 8 == 0 && aligned16(g.out) &&
       (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias))) {
+    if (b_in_place) g.flags &= ~(uint32_t)LH_GEMM_TRANSPOSE_B;
     const int rc = untranspose_operands<2>(g, kBK, 8, s);
+    if (b_in_place) g.flags |= LH_GEMM_TRANSPOSE_B;
     if (rc < 0) return rc;
   }
-  const bool ta = g.flags & LH_GEMM_TRANSPOSE_A, tb = g.flags & LH_GEMM_TRANSPOSE_B;
+  const bool ta = g.flags & LH_GEMM_TRANSPOSE_A;
+  const bool tb = (g.flags & LH_GEMM_TRANSPOSE_B) && !b_in_place;  // a transposed B the direct kernels cannot take
   const bool vec_ok = !ta && g.K % kBK == 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 && g.ldc % 4 == 0 &&
                       aligned16(g.a) && aligned16(g.b) && aligned16(g.out) &&
                       (!(g.flags & LH_GEMM_HAS_BIAS) || aligned16(g.bias));

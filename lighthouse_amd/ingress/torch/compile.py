@@ -195,17 +195,21 @@ class _Lowering:
 
         def run(env, act=act):
             x, w, b, r = x_f(env), w_f(env), b_f(env), r_f(env)
-            wt = cache.get(w, "linear_weight", lambda t: t.t().contiguous())
+            # A 16-bit [out, in] weight is read in place as a transposed B (the direct kernels take its
+            # panel like A's); an f32 weight is transposed once and cached.
+            in_place = w.dtype != torch.float32 and w.dim() == 2 and w.stride(1) == 1
+            wt = w.detach() if in_place else cache.get(w, "linear_weight", lambda t: t.t().contiguous())
             x2 = _as_2d(x)
-            shape = (*x.shape[:-1], wt.shape[1])
+            n_out = wt.shape[0] if in_place else wt.shape[1]
+            shape = (*x.shape[:-1], n_out)
             if r is not None:
                 # x + linear(y): the accumulation starts from the residual, which is only read.
                 if not isinstance(r, torch.Tensor) or tuple(r.shape) != shape or r.dtype != x.dtype:
                     raise ValueError(f"{node.name}: broadcasting / mixed-type add is not supported")
                 r = _as_2d(r)
-            _check_schedule(node.name, schedule, x2.shape[0], wt.shape[1], x2.shape[1])
+            _check_schedule(node.name, schedule, x2.shape[0], n_out, x2.shape[1])
             out = ops.gemm(x2, wt, b.detach() if b is not None else None, relu=act == "relu", gelu=act == "gelu",
-                           residual=r, tile=schedule.get("tile"), split_k=schedule.get("split_k"))
+                           residual=r, transpose_b=in_place, tile=schedule.get("tile"), split_k=schedule.get("split_k"))
             return out.view(shape)
 
         schedule: dict = {}

@@ -135,7 +135,7 @@ def gemm(a, b, bias=None, *, out=None, out_dtype=None, relu=False, gelu=False, a
     flags = ((_lib.GEMM_HAS_BIAS if bias is not None else 0) | (_lib.GEMM_HAS_RELU if relu else 0)
              | (_lib.GEMM_HAS_GELU if gelu else 0) | (_lib.GEMM_ACCUMULATE_C if accumulate_c else 0)
              | (_lib.GEMM_TRANSPOSE_A if transpose_a else 0) | (_lib.GEMM_TRANSPOSE_B if transpose_b else 0))
-    if tile is None and split_k is None and not (transpose_a or transpose_b):
+    if tile is None and split_k is None and not transpose_a:  # (a transposed B runs on the same kernels in place)
         db = _tuned_db()  # tuned parameters for this shape, if the database has any
         if db is not None:
             tile, split_k = db.lookup_gemm(_DTYPE_NAMES[a.dtype], M, N, K)

@@ -654,34 +654,71 @@ def test_gemm_residual_input(shape, elt, out_elt):
 # ---- temporary memory: caller workspaces and the per-stream pool -------------------------------------
 
 
-@pytest.mark.parametrize("case", ["split_k", "padded", "transposed", "plain"])
+@pytest.mark.parametrize("case", ["split_k", "padded", "transposed_a", "transposed_b", "plain"])
 def test_gemm_with_caller_workspace(case):
     """lh_hip_gemm_ws: same kernels, temporaries from the caller's buffer; results equal the pooled
-    call bit for bit, a short workspace is refused before anything runs."""
+    call bit for bit, a short workspace is refused before anything runs.  A transposed A is copied
+    into [M, K] (temporary memory); a transposed B with aligned rows is read in place (none)."""
     from lighthouse_amd import ops
 
-    shapes = {"split_k": (16, 2048, 8192), "padded": (300, 520, 776), "transposed": (512, 512, 512), "plain": (512, 512, 512)}
+    shapes = {"split_k": (16, 2048, 8192), "padded": (300, 520, 776), "transposed_a": (512, 512, 512),
+              "transposed_b": (512, 512, 512), "plain": (512, 512, 512)}
     M, N, K = shapes[case]
-    tb = case == "transposed"
+    ta, tb = case == "transposed_a", case == "transposed_b"
     rng = np.random.default_rng(11)
-    a = _dev(orc.round_bf16(rng.standard_normal((M, K)).astype(np.float32)), torch.bfloat16)
+    a_h = orc.round_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    a = _dev(a_h.T.copy() if ta else a_h, torch.bfloat16)
     b_h = orc.round_bf16(rng.standard_normal((K, N)).astype(np.float32))
     b = _dev(b_h.T.copy() if tb else b_h, torch.bfloat16)
     bias = _dev(orc.round_bf16(rng.standard_normal(N).astype(np.float32)), torch.bfloat16)
-    need = ops.gemm_workspace_bytes(M, N, K, torch.bfloat16, bias=True, relu=True, transpose_b=tb)
-    assert (need > 0) == (case != "plain")
+    need = ops.gemm_workspace_bytes(M, N, K, torch.bfloat16, bias=True, relu=True, transpose_a=ta, transpose_b=tb)
+    assert (need > 0) == (case not in ("plain", "transposed_b"))
     ws = torch.empty(need, dtype=torch.uint8, device="cuda")
-    want = ops.gemm(a, b, bias, relu=True, transpose_b=tb)
-    got = ops.gemm(a, b, bias, relu=True, transpose_b=tb, workspace=ws)
+    want = ops.gemm(a, b, bias, relu=True, transpose_a=ta, transpose_b=tb)
+    got = ops.gemm(a, b, bias, relu=True, transpose_a=ta, transpose_b=tb, workspace=ws)
     assert torch.equal(got, want)
-    ref = orc.matmul(_host(a), b_h, bias=_host(bias), relu=True, result_type="bf16")
+    ref = orc.matmul(a_h, b_h, bias=_host(bias), relu=True, result_type="bf16")
     assert_close(_host(got), ref, BF16_RTOL, f"bf16 gemm {case} with a caller workspace")
     if need:
         sentinel = torch.full((M, N), 7.0, device="cuda", dtype=torch.bfloat16)
         with pytest.raises(ValueError, match="workspace too small"):
-            ops.gemm(a, b, bias, relu=True, transpose_b=tb, workspace=ws[: need - 256], out=sentinel)
+            ops.gemm(a, b, bias, relu=True, transpose_a=ta, transpose_b=tb, workspace=ws[: need - 256], out=sentinel)
         with pytest.raises(ValueError, match="workspace too small"):
-            ops.gemm(a, b, bias, relu=True, transpose_b=tb, workspace=ws[:0], out=sentinel)
+            ops.gemm(a, b, bias, relu=True, transpose_a=ta, transpose_b=tb, workspace=ws[:0], out=sentinel)
+
+
+@pytest.mark.parametrize("dtype,elt", [(torch.bfloat16, "bf16"), (torch.float16, "f16")])
+@pytest.mark.parametrize("shape", [(4096, 4096, 1024), (8192, 768, 768), (2048, 2304, 768), (512, 1024, 4096), (16, 4096, 8192),
+                                   (200, 136, 192), (1000, 520, 320), (64, 8192, 2048)])
+def test_gemm_transposed_b_in_place(shape, dtype, elt):
+    """B stored [N, K] (the layout of a torch Linear weight): the direct kernels read its panel like
+    A's, whole and edge tiles, every tile on request and the launches cut along K.  Integer operands:
+    the f32-output result is exact and equals the untransposed call bit for bit; with bias + ReLU and
+    16-bit output against the oracle; on a row-strided view of a wider buffer too."""
+    from lighthouse_amd import ops
+
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K)
+    a = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, (K, N)).astype(np.float32)
+    bias = rng.integers(-8, 9, (N,)).astype(np.float32)
+    da, db, dbt = _dev(a, dtype), _dev(b, dtype), _dev(b.T.copy(), dtype)
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    out = ops.gemm(da, dbt, transpose_b=True, out_dtype=torch.float32)
+    assert np.array_equal(_host(out).astype(np.float64), exact), f"B^T gemm {shape} {elt}"
+    assert torch.equal(out, ops.gemm(da, db, out_dtype=torch.float32))
+    assert ops.gemm_workspace_bytes(M, N, K, dtype, transpose_b=True) == ops.gemm_workspace_bytes(M, N, K, dtype)
+    ref = orc.matmul(a, b, bias=bias, relu=True, result_type=elt)
+    got = ops.gemm(da, dbt, _dev(bias, dtype), relu=True, transpose_b=True)
+    assert_close(_host(got), ref, BF16_RTOL, f"B^T gemm + bias + ReLU {shape} {elt}")
+    wide = torch.zeros(N, K + 64, device="cuda", dtype=dtype)
+    wide[:, 8:8 + K] = dbt
+    assert torch.equal(ops.gemm(da, wide[:, 8:8 + K], transpose_b=True, out_dtype=torch.float32), out)
+    for tile in [(256, 256), (256, 128), (128, 256), (128, 128)]:
+        if M % tile[0] == 0 and N % tile[1] == 0:
+            assert torch.equal(ops.gemm(da, dbt, transpose_b=True, out_dtype=torch.float32, tile=tile), out), tile
+    if K % 256 == 0 and K // 4 >= 128:
+        assert torch.equal(ops.gemm(da, dbt, transpose_b=True, out_dtype=torch.float32, split_k=4), out)
 
 
 def test_gemm_fp8_with_caller_workspace():

@@ -1,8 +1,9 @@
 """lh_hip_gemm_static: the GEMM entry point that allocates nothing (temporaries in a device array
 that is part of the library's image), called through the C ABI and compared bit for bit with
 lh_hip_gemm on the same inputs: a decode shape that is cut along K, then a smaller one (the array
-keeps the first call's contents), then problems with padded and transposed operands, then one whose
-temporaries exceed the array."""
+keeps the first call's contents), then problems with padded operands and a transposed A (copies in
+the array), a transposed B and a plain problem (no temporaries), then one whose temporaries exceed
+the array."""
 
 import ctypes
 
@@ -23,9 +24,9 @@ def _call(fn, out, a, b, bias, M, N, K, flags, stream=None):
               flags, stream)
 
 
-def _problem(M, N, K, seed, transpose_b=False):
+def _problem(M, N, K, seed, transpose_b=False, transpose_a=False):
     g = torch.Generator(device="cuda").manual_seed(seed)
-    a = torch.randn(M, K, device="cuda", generator=g).to(torch.bfloat16)
+    a = torch.randn((K, M) if transpose_a else (M, K), device="cuda", generator=g).to(torch.bfloat16)
     b = torch.randn((N, K) if transpose_b else (K, N), device="cuda", generator=g).to(torch.bfloat16)
     bias = torch.randn(N, device="cuda", generator=g).to(torch.bfloat16)
     return a, b, bias
@@ -35,9 +36,10 @@ def test_static_scratch_gemm_matches_the_pooled_entry_point():
     lib = _lib.load()
     flags = _lib.GEMM_HAS_BIAS | _lib.GEMM_HAS_RELU
     # (M, N, K, extra flags): cut along K (4 MiB of partial sums); smaller, cut along K; ragged N and K
-    # (padded copies); transposed B (untransposed copy); no temporaries at all
-    cases = [(16, 8192, 8192, 0), (16, 1024, 4096, 0), (300, 520, 776, 0), (512, 512, 512, _lib.GEMM_TRANSPOSE_B),
-             (512, 512, 512, 0)]
+    # (padded copies); transposed A (untransposed copy); then no temporaries at all: transposed B (read in
+    # place), plain
+    cases = [(16, 8192, 8192, 0), (16, 1024, 4096, 0), (300, 520, 776, 0), (512, 512, 512, _lib.GEMM_TRANSPOSE_A),
+             (512, 512, 512, _lib.GEMM_TRANSPOSE_B), (512, 512, 512, 0)]
     # The array itself becomes resident on the device when the runtime is first asked for its
     # address; one call up front keeps that out of the memory readings below.
     a, b, bias = _problem(256, 256, 256, 99)
@@ -45,8 +47,8 @@ def test_static_scratch_gemm_matches_the_pooled_entry_point():
     _lib.check(_call(lib.lh_hip_gemm_static, first, a, b, bias, 256, 256, 256, flags), "lh_hip_gemm_static")
     torch.cuda.synchronize()
     for i, (M, N, K, extra) in enumerate(cases):
-        tb = bool(extra & _lib.GEMM_TRANSPOSE_B)
-        a, b, bias = _problem(M, N, K, 100 + i, tb)
+        tb, ta = bool(extra & _lib.GEMM_TRANSPOSE_B), bool(extra & _lib.GEMM_TRANSPOSE_A)
+        a, b, bias = _problem(M, N, K, 100 + i, tb, ta)
         need = lib.lh_hip_gemm_workspace_bytes(M, N, K, a.stride(0), b.stride(0), N, _lib.BF16, _lib.BF16, flags | extra)
         assert need <= STATIC_BYTES and (need > 0) == (i < 4)
         want = torch.full((M, N), 3.0, device="cuda", dtype=torch.bfloat16)
@@ -58,7 +60,7 @@ def test_static_scratch_gemm_matches_the_pooled_entry_point():
         torch.cuda.synchronize()
         assert torch.cuda.mem_get_info()[0] >= free_before  # the call took no device memory
         assert torch.equal(got, want), (M, N, K)
-        ref = torch.relu(a.float() @ (b.float().T if tb else b.float()) + bias.float())
+        ref = torch.relu((a.float().T if ta else a.float()) @ (b.float().T if tb else b.float()) + bias.float())
         assert (got.float() - ref).abs().max() <= 2e-2 * ref.abs().max()
     # the two decode shapes again in the opposite order, back to back on one stream without a
     # synchronisation in between: the second call's kernels run after the first call's
