@@ -1011,11 +1011,22 @@ static int gemm16_splitk(const GemmArgs& g, uint32_t request, hipStream_t s) {
                kBK, 2 * kBK);
   } else {
     if (tiles * 2 > cus || g.K < 2048) return 1;
-    // With more than a quarter of the CUs busy anyway, the second kernel costs more than cutting a
-    // K of 2048 saves (M = 512, N = 4096: 24.1 us cut, 19.7 us whole; at K = 3072 the two are level).
-    if (tiles * 4 > cus && g.K < 3072) return 1;
-    while (splits < 8 && tiles * splits * 2 <= 2 * cus && (g.K / (splits * 2)) % kBK == 0 && g.K / (splits * 2) >= 512)
-      splits *= 2;
+    // Doubling the cut is taken while the k steps it saves each workgroup outweigh the f32 blocks it
+    // adds for the second kernel to read: 0.225 us per 32 k saved (half of that once the workgroups
+    // outnumber the CUs and share them), 0.62 us per MB of blocks written and read back, 2.5 us for
+    // the second kernel itself.  Measured optima this reproduces (M x N x K: cut): 1024 x 1024 x 4096: 4,
+    // 128 x 4096 x 4096: 4, 128 x 8192 x 8192: 4, 16 x 8192 x 8192: 8, 32 x 4096 x 4096: 8,
+    // 2048 x 768 x 3072: 2, 512 x 4096 x 4096: 2, 512 x 768 x 3072: 4, 512 x 4096 x 2048 and
+    // 256 x 8192 x 2048: whole.
+    const double block_mb = (double)g.M * g.N * sizeof(float) * 1e-6;
+    while (splits < 8) {
+      const int to = splits * 2;
+      if (tiles * to > 2 * cus || (g.K / to) % kBK != 0 || g.K / to < 512) break;
+      const double saved = (double)(g.K / splits - g.K / to) / 32 * 0.225 * (tiles * to > cus ? 0.5 : 1.0);
+      const double added = (splits == 1 ? to * block_mb * 0.62 + 2.5 : (to - splits) * block_mb * 0.62);
+      if (saved <= added) break;
+      splits = to;
+    }
     if (splits == 1) return 1;
   }
   void* taken = nullptr;
