@@ -78,11 +78,13 @@ def test_static_scratch_gemm_matches_the_pooled_entry_point():
 
 def test_static_scratch_gemm_refuses_what_does_not_fit():
     lib = _lib.load()
-    M, N, K = 128, 8192, 8192  # eight f32 blocks of 128 x 8192: 32 MiB
-    assert lib.lh_hip_gemm_workspace_bytes(M, N, K, K, N, N, _lib.BF16, _lib.BF16, 0) > STATIC_BYTES
+    M, N, K = 128, 8192, 8192
+    cut8 = _lib.GEMM_SPLITK[8]  # eight f32 blocks of 128 x 8192: 32 MiB (the library's own choice, four, just fits)
+    assert lib.lh_hip_gemm_workspace_bytes(M, N, K, K, N, N, _lib.BF16, _lib.BF16, 0) <= STATIC_BYTES
+    assert lib.lh_hip_gemm_workspace_bytes(M, N, K, K, N, N, _lib.BF16, _lib.BF16, cut8) > STATIC_BYTES
     a, b, _ = _problem(M, N, K, 7)
     out = torch.full((M, N), 9.0, device="cuda", dtype=torch.bfloat16)
-    rc = _call(lib.lh_hip_gemm_static, out, a, b, None, M, N, K, 0)
+    rc = _call(lib.lh_hip_gemm_static, out, a, b, None, M, N, K, cut8)
     assert rc == _lib.LH_ERR_INVALID
     assert b"static scratch holds" in lib.lh_hip_last_error()
     torch.cuda.synchronize()
