@@ -26,11 +26,19 @@ struct Mfma16<LH_BF16> {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
                                                    0, 0);
   }
+  __device__ static __forceinline__ f32x4 mma16(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                   0, 0);
+  }
 };
 template <>
 struct Mfma16<LH_F16> {
   __device__ static __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
+                                                  0);
+  }
+  __device__ static __forceinline__ f32x4 mma16(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
                                                   0);
   }
 };
@@ -203,17 +211,25 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm16_fast(GemmArgs g)
 // n-contiguous B panel is read with ds_read_b64_tr_b16, which hands each lane 4 k-values of one
 // column, i.e. the MFMA operand layout, transposing in the LDS crossbar.
 //
+// The matrix instruction is v_mfma_f32_16x16x32 (16 rows x 16 columns x 32 k), not 32x32x16: for
+// the same products it keeps the matrix cores' clock higher on random operands (a register-only
+// loop of either runs at the published peak on zeros, but at 2.02 against 1.74 PFLOP/s on N(0,1)
+// data).  A wave's sub-tile is 2 TM fragments of 16 rows by 2 TN fragments of 16 columns per 32 k.
+//
 // LDS rings: A in 2 stages of 64 k (rows of 128 bytes: every global request is a full 128-byte
-// line), B in 4 stages of 32 k.  The main loop advances 32 k per step; the barrier sits in the
-// MIDDLE of a step, after the LDS reads of the step's second k-half have been issued, so
-// fragment reads always overlap MFMAs of the previous k-half and the buffer a step has finished
-// reading is refilled right away (B: 3 stages ahead, A: on odd steps, one 64-k stage ahead).
+// line), B in 4 stages of 32 k.  The main loop advances 32 k per step, each step in two phases:
+// the MFMAs of the wave's lower TM row fragments, then of its upper ones, all against the step's
+// 2 TN column fragments.  The LDS reads of a phase fetch what the next phase needs (the other
+// half of the A fragments; in the second phase also the next step's B fragments, each after the
+// last MFMA that uses its predecessor), so reads always overlap MFMAs.  The barrier sits between
+// the two phases of a step and the buffers a step has finished reading are refilled right
+// behind it (B: 3 stages ahead, A: on odd steps, one 64-k stage ahead).
 // The large tiles (and the 128 x 128 tile when workgroups share a compute unit) run a second form
 // with one barrier per 64 k, the rings as two halves: direct_step_pair_1b.
 //
 // A wave-wide load into LDS writes 64 x 16 contiguous LDS bytes, so rows cannot be padded;
 // bank conflicts are avoided by XOR-swizzling which 16-byte chunk of a row each lane fetches
-// (A: chunk ^ ((row / 2) % 8); B: chunk ^ 4 (k % 4)).
+// (A: chunk ^ ((row / 2) % 8); B: chunk ^ 4 (k % 4) ^ 2 ((k / 8) % 2)).
 template <int TM, int TN>
 struct DirectCfg {
   static constexpr int BM = 64 * TM, BN = 128 * TN;
@@ -265,19 +281,22 @@ struct DirectCtx {
   int a_src[TM];              // lane's byte offset in the A panel for load i at k = 0
   int b_src[TN];
   int b_step;                 // bytes between B stages (32 k rows)
-  int a_off[TM];              // byte offset of the lane's A row in a stage, per m-subtile
-  int a_swz[TM];
-  int wave, h, b_off, b_chunk, b_swz;
+  // Fragment reads.  A: the lane's first row (wm0 + lane % 16) of a stage, its 16-byte chunk for the
+  // first / second 32 k of the stage's 64 (fragment jj, 16 rows further on, adds 2048 jj: the
+  // swizzle term (row / 2) % 8 does not change with 16 rows).
+  int a_rd[2];
+  int wave, b_off, b_chunk, b_swz;
   // B stored transposed ([N, K], k contiguous): its panel is laid out, loaded and read like A's
   int bt_src[2 * TN];         // lane's byte offset in the B^T panel for load i at k = 0
-  int bt_off[TN];             // byte offset of the lane's B^T row in a stage, per n-subtile
-  int bt_swz[TN];
+  int bt_rd[2];               // like a_rd, for row wn0 + lane % 16 of a B^T stage
 };
 
+// Fragments in registers: the A fragments of the lower (a[0]) and upper (a[1]) half of the wave's
+// rows, TM of 16 rows each, and the step's 2 TN B fragments of 16 columns.
 template <int TM, int TN>
 struct DirectFrags {
-  u32x4 a[TM];
-  u32x4 b[TN];
+  u32x4 a[2][TM];
+  u32x4 b[2 * TN];
 };
 
 // A stage `sa` (k = 64 sa .. +64): TM loads per lane.
@@ -301,56 +320,73 @@ __device__ __forceinline__ void direct_load_b(const DirectCtx<TM, TN>& c, int sb
   }
 }
 
-// Fragments of 16 k: A chunk pair `kc` (0..3: which 16 of the stage's 64 k), B k-step `ks`
-// (0..1: which 16 of the stage's 32 k).
-// BT: `bs` is a 64-k stage of the transposed B; its fragments are 16-byte reads like A's, chunk pair kc.
-template <int TM, int TN, bool BT = false>
-__device__ __forceinline__ void direct_read_frags(const DirectCtx<TM, TN>& c, const uint8_t* __restrict__ as,
-                                                  const uint8_t* __restrict__ bs, int kc, int ks,
-                                                  DirectFrags<TM, TN>& f) {
-  constexpr int row = DirectCfg<TM, TN>::kBRow;
-  auto read_b = [&](int i) {
-    if constexpr (BT) {
-      f.b[i] = *reinterpret_cast<const u32x4*>(bs + c.bt_off[i] + (((2 * kc + c.h) ^ c.bt_swz[i]) << 4));
-      return;
-    }
-    const int p = (c.b_chunk + 4 * i) ^ c.b_swz;
-    const uint8_t* p0 = bs + ks * 16 * row + c.b_off + p * 16;
+// A fragments of one half of the wave's rows (HALF 0: 16-row fragments 0 .. TM-1, 1: TM .. 2 TM-1)
+// for the 32 k `kc` (0 / 1) of the 64-k stage `as`.
+template <int TM, int TN, int HALF>
+__device__ __forceinline__ void direct_read_a(const DirectCtx<TM, TN>& c, const uint8_t* __restrict__ as, int kc,
+                                              u32x4 (&a)[TM]) {
+#pragma unroll
+  for (int j = 0; j < TM; ++j) a[j] = *reinterpret_cast<const u32x4*>(as + c.a_rd[kc] + 2048 * (HALF * TM + j));
+}
+// B fragment i (16 columns) of a 32-k step: from the 32-k stage `bs` of an n-contiguous B through two
+// transposing reads, or (BT) from the 32 k `kc` of the 64-k stage `bs` of a transposed B like an A fragment.
+template <int TM, int TN, bool BT>
+__device__ __forceinline__ u32x4 direct_read_b(const DirectCtx<TM, TN>& c, const uint8_t* __restrict__ bs, int kc,
+                                               int i) {
+  if constexpr (BT) {
+    return *reinterpret_cast<const u32x4*>(bs + c.bt_rd[kc] + 2048 * i);
+  } else {
+    constexpr int row = DirectCfg<TM, TN>::kBRow;
+    const int p = (c.b_chunk + 2 * i) ^ c.b_swz;
+    const uint8_t* p0 = bs + c.b_off + p * 16;
     s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p0);
     s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p0 + 4 * row));
     u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-    f.b[i] = u32x4{l2[0], l2[1], h2[0], h2[1]};
-  };
-  // In the order direct_mfma consumes them (B fragment 0 with every A fragment, then B fragment 1 ...):
-  // LDS reads return in order and the waits in front of the MFMAs count, so the fragment wanted
-  // first must be the oldest request.
-  read_b(0);
-#pragma unroll
-  for (int j = 0; j < TM; ++j)
-    f.a[j] = *reinterpret_cast<const u32x4*>(as + c.a_off[j] + (((2 * kc + c.h) ^ c.a_swz[j]) << 4));
-#pragma unroll
-  for (int i = 1; i < TN; ++i) read_b(i);
+    return u32x4{l2[0], l2[1], h2[0], h2[1]};
+  }
 }
 
-template <int DT, int TM, int TN>
-__device__ __forceinline__ void direct_mfma(f32x16 (&acc)[TN][TM], const DirectFrags<TM, TN>& f) {
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j) acc[i][j] = Mfma16<DT>::mma(f.b[i], f.a[j], acc[i][j]);
-}
-
-// Scheduling hint for one k-half: spread the TM + 2 TN LDS reads of the NEXT k-half evenly
-// between the TM TN MFMAs of the current one.
+// Scheduling hint for one phase: spread its NR LDS reads evenly between its NM MFMAs.
 template <int I, int NM, int NR>
 __device__ __forceinline__ void direct_interleave_step() {
   __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                // MFMA
   __builtin_amdgcn_sched_group_barrier(0x100, (I + 1) * NR / NM - I * NR / NM, 0);  // DS reads
   if constexpr (I + 1 < NM) direct_interleave_step<I + 1, NM, NR>();
 }
-template <int TM, int TN>
-__device__ __forceinline__ void direct_interleave_hint() {
-  direct_interleave_step<0, TM * TN, TM + 2 * TN>();
+
+// First phase of a step: the MFMAs of the lower row fragments (f.a[0]) against the step's B
+// fragments, under the reads of the same step's upper row fragments (32 k `kc` of stage `as`).
+template <int DT, int TM, int TN>
+__device__ __forceinline__ void direct_phase_lo(const DirectCtx<TM, TN>& c, f32x4 (&acc)[2 * TN][2 * TM],
+                                                DirectFrags<TM, TN>& f, const uint8_t* __restrict__ as, int kc) {
+  direct_read_a<TM, TN, 1>(c, as, kc, f.a[1]);
+#pragma unroll
+  for (int i = 0; i < 2 * TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[i][j] = Mfma16<DT>::mma16(f.b[i], f.a[0][j], acc[i][j]);
+  direct_interleave_step<0, 2 * TN * TM, TM>();
+}
+// Second phase: the MFMAs of the upper row fragments (f.a[1]) under the reads of the NEXT step's
+// lower row fragments (32 k `kc_n` of A stage `as_n`) and B fragments (stage `bs_n`; BT: its 32 k
+// `kc_n`), each B fragment requested behind the last MFMA that uses the one it replaces.
+// LOAD false: the tile's last step, nothing left to read.
+template <int DT, int TM, int TN, bool BT, bool LOAD = true>
+__device__ __forceinline__ void direct_phase_hi(const DirectCtx<TM, TN>& c, f32x4 (&acc)[2 * TN][2 * TM],
+                                                DirectFrags<TM, TN>& f, const uint8_t* __restrict__ as_n,
+                                                const uint8_t* __restrict__ bs_n, int kc_n) {
+  if constexpr (LOAD) direct_read_a<TM, TN, 0>(c, as_n, kc_n, f.a[0]);
+  u32x4 bn[2 * TN];
+#pragma unroll
+  for (int i = 0; i < 2 * TN; ++i) {
+#pragma unroll
+    for (int j = 0; j < TM; ++j) acc[i][TM + j] = Mfma16<DT>::mma16(f.b[i], f.a[1][j], acc[i][TM + j]);
+    if constexpr (LOAD) bn[i] = direct_read_b<TM, TN, BT>(c, bs_n, kc_n, i);
+  }
+  if constexpr (LOAD) {
+#pragma unroll
+    for (int i = 0; i < 2 * TN; ++i) f.b[i] = bn[i];
+    direct_interleave_step<0, 2 * TN * TM, TM + (BT ? 2 : 4) * TN>();
+  }
 }
 // Wait until at most N of this wave's loads are still in flight and all its LDS reads have
 // returned, then barrier.  One asm block: a __syncthreads() would add a release fence, i.e. a
@@ -361,47 +397,39 @@ __device__ __forceinline__ void direct_wait_barrier() {
 }
 
 
-// Steps kt (even) and kt + 1 of the main loop; both have a successor step.  On entry f0 holds
-// the fragments of (step kt, first k-half).  a_cur = A stage kt / 2, a_nxt = the next A stage,
-// b0 / b1 / b2 = B stages kt, kt + 1, kt + 2.  The refill pointers alias a_cur, b0 and b1: every
-// read of a buffer precedes the barrier after which it is refilled.  They are separate restrict
-// parameters so that the compiler does not make LDS reads wait for the asynchronous writes.
+// Steps kt (even) and kt + 1 of the main loop; both have a successor step.  On entry f holds the
+// lower row fragments and the B fragments of step kt.  a_cur = A stage kt / 2, a_nxt = the next A
+// stage, b1 / b2 = B stages kt + 1, kt + 2.  The refill pointers alias a_cur and B stages kt and
+// kt + 1: every read of a buffer precedes the barrier after which it is refilled.  They are
+// separate restrict parameters so that the compiler does not make LDS reads wait for the
+// asynchronous writes.
 //
 // In-flight loads, oldest first, when a barrier is reached (steady state):
 //   even step: [A(kt/2) B(kt+1)] [B(kt+2)] [A(kt/2+1) B(kt+3)]  -> B(kt+1) needed: TM + 2 TN may remain
 //   odd step : [B(kt+1)] [A((kt+1)/2) B(kt+2)] [B(kt+3)]        -> A needed: 2 TN may remain
 // Near the end loads are no longer issued and the waits become full waits.
 template <int DT, int TM, int TN>
-__device__ __forceinline__ void direct_step_pair(const DirectCtx<TM, TN>& c, f32x16 (&acc)[TN][TM],
-                                                 DirectFrags<TM, TN>& f0, const uint8_t* __restrict__ a_cur,
-                                                 const uint8_t* __restrict__ a_nxt, const uint8_t* __restrict__ b0,
-                                                 const uint8_t* __restrict__ b1, const uint8_t* __restrict__ b2,
-                                                 uint8_t* __restrict__ a_refill, uint8_t* __restrict__ b_refill0,
-                                                 uint8_t* __restrict__ b_refill1, int kt, int nk) {
+__device__ __forceinline__ void direct_step_pair(const DirectCtx<TM, TN>& c, f32x4 (&acc)[2 * TN][2 * TM],
+                                                 DirectFrags<TM, TN>& f, const uint8_t* __restrict__ a_cur,
+                                                 const uint8_t* __restrict__ a_nxt, const uint8_t* __restrict__ b1,
+                                                 const uint8_t* __restrict__ b2, uint8_t* __restrict__ a_refill,
+                                                 uint8_t* __restrict__ b_refill0, uint8_t* __restrict__ b_refill1,
+                                                 int kt, int nk) {
   using Cfg = DirectCfg<TM, TN>;
-  DirectFrags<TM, TN> f1;
   const bool steady = kt + 6 < nk;  // all loads of both steps are real
   // ---- even step kt
-  direct_read_frags(c, a_cur, b0, 1, 1, f1);
-  direct_mfma<DT>(acc, f0);
-  direct_interleave_hint<TM, TN>();
+  direct_phase_lo<DT>(c, acc, f, a_cur, 0);
   if (steady) direct_wait_barrier<Cfg::kWaitEven>();
   else direct_wait_barrier<0>();
   if (kt + 4 < nk) direct_load_b(c, kt + 4, b_refill0);
-  direct_read_frags(c, a_cur, b1, 2, 0, f0);
-  direct_mfma<DT>(acc, f1);
-  direct_interleave_hint<TM, TN>();
+  direct_phase_hi<DT, TM, TN, false>(c, acc, f, a_cur, b1, 1);
   // ---- odd step kt + 1
-  direct_read_frags(c, a_cur, b1, 3, 1, f1);
-  direct_mfma<DT>(acc, f0);
-  direct_interleave_hint<TM, TN>();
+  direct_phase_lo<DT>(c, acc, f, a_cur, 1);
   if (steady) direct_wait_barrier<Cfg::kWaitOdd>();
   else direct_wait_barrier<0>();
   if (kt + 4 < nk) direct_load_a(c, kt / 2 + 2, a_refill);
   if (kt + 5 < nk) direct_load_b(c, kt + 5, b_refill1);
-  direct_read_frags(c, a_nxt, b2, 0, 0, f0);
-  direct_mfma<DT>(acc, f1);
-  direct_interleave_hint<TM, TN>();
+  direct_phase_hi<DT, TM, TN, false>(c, acc, f, a_nxt, b2, 0);
 }
 
 // Source pointers of tile `id` (its position in the XCD-grouped order) and the tile's origin.
@@ -438,7 +466,9 @@ __device__ __forceinline__ void direct_place(const GemmArgs& g, int id, DirectCt
     c.a_src[i] = (arow * lda + ac * 8) * 2;
   }
   // B: load i of wave w fills k rows (8 i + w) R .. +R with R = 1024 / row bytes; lane ->
-  // row += lane / chunks-per-row, LDS chunk p holds global chunk p ^ 4 (k % 4).
+  // row += lane / chunks-per-row, LDS chunk p holds global chunk p ^ 4 (k % 4) ^ 2 ((k / 8) % 2): the
+  // four k rows a 16-lane group reads at once land in different banks, and so do the rows (8 apart)
+  // of the group next to it.
   if constexpr (BT) {
     // B^T: exactly A's scheme on the panel's BN rows (row n of B^T = column n of B)
 #pragma unroll
@@ -452,7 +482,7 @@ __device__ __forceinline__ void direct_place(const GemmArgs& g, int id, DirectCt
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
       const int bk = (8 * i + c.wave) * Cfg::kBRowsPerLoad + lane / Cfg::kBChunks;
-      const int bc = (lane % Cfg::kBChunks) ^ (4 * (bk & 3));
+      const int bc = (lane % Cfg::kBChunks) ^ (4 * (bk & 3)) ^ (2 * ((bk >> 3) & 1));
       const int bcol = EDGE ? min(bc * 8, g.N - 8 - n0) : bc * 8;  // column within the panel
       c.b_src[i] = (bk * ldb + bcol) * 2;
     }
@@ -462,26 +492,18 @@ __device__ __forceinline__ void direct_place(const GemmArgs& g, int id, DirectCt
 // The same two steps with ONE barrier, in the middle of the odd step: the rings work as two halves
 // of 64 k.  At the barrier every read of this pair's stages has returned and the next pair's
 // stages (issued at the previous barrier, 64 k ago) are awaited in full; the pair after that is
-// then requested into this pair's buffers.
+// then requested into this pair's buffers.  BT: b1 is the pair's one 64-k stage of B^T, b2 the next.
 template <int DT, int TM, int TN, bool BT = false>
-__device__ __forceinline__ void direct_step_pair_1b(const DirectCtx<TM, TN>& c, f32x16 (&acc)[TN][TM],
-                                                    DirectFrags<TM, TN>& f0, const uint8_t* __restrict__ a_cur,
-                                                    const uint8_t* __restrict__ a_nxt, const uint8_t* __restrict__ b0,
-                                                    const uint8_t* __restrict__ b1, const uint8_t* __restrict__ b2,
-                                                    uint8_t* __restrict__ a_refill, uint8_t* __restrict__ b_refill0,
-                                                    uint8_t* __restrict__ b_refill1, int kt, int nk,
-                                                    bool stores_behind) {
+__device__ __forceinline__ void direct_step_pair_1b(const DirectCtx<TM, TN>& c, f32x4 (&acc)[2 * TN][2 * TM],
+                                                    DirectFrags<TM, TN>& f, const uint8_t* __restrict__ a_cur,
+                                                    const uint8_t* __restrict__ a_nxt, const uint8_t* __restrict__ b1,
+                                                    const uint8_t* __restrict__ b2, uint8_t* __restrict__ a_refill,
+                                                    uint8_t* __restrict__ b_refill0, uint8_t* __restrict__ b_refill1,
+                                                    int kt, int nk, bool stores_behind) {
   using Cfg = DirectCfg<TM, TN>;
-  DirectFrags<TM, TN> f1;
-  direct_read_frags<TM, TN, BT>(c, a_cur, b0, 1, 1, f1);
-  direct_mfma<DT>(acc, f0);
-  direct_interleave_hint<TM, TN>();
-  direct_read_frags<TM, TN, BT>(c, a_cur, b1, 2, 0, f0);
-  direct_mfma<DT>(acc, f1);
-  direct_interleave_hint<TM, TN>();
-  direct_read_frags<TM, TN, BT>(c, a_cur, b1, 3, 1, f1);
-  direct_mfma<DT>(acc, f0);
-  direct_interleave_hint<TM, TN>();
+  direct_phase_lo<DT>(c, acc, f, a_cur, 0);
+  direct_phase_hi<DT, TM, TN, BT>(c, acc, f, a_cur, b1, 1);
+  direct_phase_lo<DT>(c, acc, f, a_cur, 1);
   // At a tile's first barrier the only operations in flight are the previous tile's stores (the
   // tile's first loads, older than they, were awaited when the main loop began): they may stay.
   // Matters for the 128 x 128 tile, whose first 64 k pass in 0.5 us (M = 8192, N = 2304, K = 768:
@@ -491,15 +513,13 @@ __device__ __forceinline__ void direct_step_pair_1b(const DirectCtx<TM, TN>& c, 
   if (kt + 4 < nk) {
     direct_load_a(c, kt / 2 + 2, a_refill);
     if constexpr (BT) {
-      direct_load_b<TM, TN, true>(c, kt / 2 + 2, b_refill0);  // (b0 = b1: the pair's one 64-k stage)
+      direct_load_b<TM, TN, true>(c, kt / 2 + 2, b_refill0);
     } else {
       direct_load_b(c, kt + 4, b_refill0);
       direct_load_b(c, kt + 5, b_refill1);
     }
   }
-  direct_read_frags<TM, TN, BT>(c, a_nxt, b2, 0, 0, f0);
-  direct_mfma<DT>(acc, f1);
-  direct_interleave_hint<TM, TN>();
+  direct_phase_hi<DT, TM, TN, BT>(c, acc, f, a_nxt, b2, 0);
 }
 
 // First loads of a tile: A stages 0, 1 and B stages 0 .. 3 (nk = K / 32 >= 2); BT: both 64-k stages of B^T.
@@ -518,34 +538,30 @@ __device__ __forceinline__ void direct_prologue(const DirectCtx<TM, TN>& c, int 
   }
 }
 
-// Main loop of one tile, whose first loads have been issued.
-// The lane's 16-bit bias values for a staged epilogue, columns n_base + 32 i + 8 q .. +4, as packed
+// The lane's 16-bit bias values for a staged epilogue, columns n_base + 16 i .. +4, as packed
 // pairs; all loads are issued back to back.  (An f32 bias is read by the epilogue itself.)
 template <int TN, bool EDGE>
-__device__ __forceinline__ void direct_load_bias(const GemmArgs& g, int n_base, u32x2 (&bias)[TN][4]) {
+__device__ __forceinline__ void direct_load_bias(const GemmArgs& g, int n_base, u32x2 (&bias)[2 * TN]) {
 #pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) bias[i][q] = u32x2{0u, 0u};
+  for (int i = 0; i < 2 * TN; ++i) bias[i] = u32x2{0u, 0u};
   if (!(g.flags & LH_GEMM_HAS_BIAS) || g.bias_dt == LH_F32) return;
 #pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const int n = n_base + 32 * i + 8 * q;
-      bias[i][q] = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.bias) + (EDGE ? min(n, g.N - 4) : n));
-    }
+  for (int i = 0; i < 2 * TN; ++i) {
+    const int n = n_base + 16 * i;
+    bias[i] = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.bias) + (EDGE ? min(n, g.N - 4) : n));
+  }
 }
 
+// Main loop of one tile, whose first loads have been issued.
 // `stores_behind`: the previous tile's staged epilogue issued exactly Cfg::kStagedStores stores
 // per lane AFTER this tile's first loads; vector memory operations complete in issue order, so
 // those stores may stay in flight.
 // `staged`: the epilogue will want `bias` (for columns from n_base); it is loaded ahead of the
 // last two steps, whose full wait covers it.
 template <int DT, int TM, int TN, bool EDGE, bool BT = false>
-__device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectCtx<TM, TN>& c, f32x16 (&acc)[TN][TM],
-                                                uint8_t* smem_d, int nk, bool stores_behind, bool staged, int n_base,
-                                                u32x2 (&bias)[TN][4]) {
+__device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectCtx<TM, TN>& c,
+                                                f32x4 (&acc)[2 * TN][2 * TM], uint8_t* smem_d, int nk,
+                                                bool stores_behind, bool staged, int n_base, u32x2 (&bias)[2 * TN]) {
   using Cfg = DirectCfg<TM, TN>;
   // One barrier per 64 k (loads one 64-k half of the rings ahead) or two (B three 32-k stages
   // ahead).  One is 1-3 % faster for every tile with a 256 side (4096^3 109.8 -> 108.3 us) and, when
@@ -558,8 +574,10 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
   uint8_t* const bbuf = smem_d + Cfg::kBBase;
   if (stores_behind) asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(Cfg::kStagedStores) : "memory");
   else asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-  DirectFrags<TM, TN> f0;
-  direct_read_frags<TM, TN, BT>(c, abuf, bbuf, 0, 0, f0);
+  DirectFrags<TM, TN> f;
+  direct_read_a<TM, TN, 0>(c, abuf, 0, f.a[0]);
+#pragma unroll
+  for (int i = 0; i < 2 * TN; ++i) f.b[i] = direct_read_b<TM, TN, BT>(c, bbuf, 0, i);
   int kt = 0;
   auto pair = [&](auto one) {
     uint8_t* a_cur = abuf + ((kt >> 1) & 1) * Cfg::kABytes;
@@ -567,14 +585,14 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
     if constexpr (BT) {
       uint8_t* b_cur = bbuf + ((kt >> 1) & 1) * Cfg::kBtBytes;
       uint8_t* b_nxt = bbuf + (((kt >> 1) + 1) & 1) * Cfg::kBtBytes;
-      direct_step_pair_1b<DT, TM, TN, true>(c, acc, f0, a_cur, a_nxt, b_cur, b_cur, b_nxt, a_cur, b_cur, b_cur, kt, nk,
+      direct_step_pair_1b<DT, TM, TN, true>(c, acc, f, a_cur, a_nxt, b_cur, b_nxt, a_cur, b_cur, b_cur, kt, nk,
                                             stores_behind);
     } else {
       uint8_t* b0 = bbuf + (kt & 3) * Cfg::kBBytes;
       uint8_t* b1 = bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
       uint8_t* b2 = bbuf + ((kt + 2) & 3) * Cfg::kBBytes;
-      if constexpr (decltype(one)::value) direct_step_pair_1b<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk, stores_behind);
-      else direct_step_pair<DT>(c, acc, f0, a_cur, a_nxt, b0, b1, b2, a_cur, b0, b1, kt, nk);
+      if constexpr (decltype(one)::value) direct_step_pair_1b<DT>(c, acc, f, a_cur, a_nxt, b1, b2, a_cur, b0, b1, kt, nk, stores_behind);
+      else direct_step_pair<DT>(c, acc, f, a_cur, a_nxt, b1, b2, a_cur, b0, b1, kt, nk);
     }
   };
   if constexpr (BT || TM * TN > 2) {
@@ -587,18 +605,13 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
   {
     // Last two steps: nothing left to load; stage nk - 1 of B must have landed.
     const uint8_t* a_cur = abuf + ((kt >> 1) & 1) * Cfg::kABytes;
-    const uint8_t* b0 = BT ? bbuf + ((kt >> 1) & 1) * Cfg::kBtBytes : bbuf + (kt & 3) * Cfg::kBBytes;
-    const uint8_t* b1 = BT ? b0 : bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
-    DirectFrags<TM, TN> f1;
+    const uint8_t* b1 = BT ? bbuf + ((kt >> 1) & 1) * Cfg::kBtBytes : bbuf + ((kt + 1) & 3) * Cfg::kBBytes;
     if (staged) direct_load_bias<TN, EDGE>(g, n_base, bias);
-    direct_read_frags<TM, TN, BT>(c, a_cur, b0, 1, 1, f1);
-    direct_mfma<DT>(acc, f0);
+    direct_phase_lo<DT>(c, acc, f, a_cur, 0);
     if (!one_barrier) direct_wait_barrier<0>();  // (one barrier per pair: awaited at the pair before)
-    direct_read_frags<TM, TN, BT>(c, a_cur, b1, 2, 0, f0);
-    direct_mfma<DT>(acc, f1);
-    direct_read_frags<TM, TN, BT>(c, a_cur, b1, 3, 1, f1);
-    direct_mfma<DT>(acc, f0);
-    direct_mfma<DT>(acc, f1);
+    direct_phase_hi<DT, TM, TN, BT>(c, acc, f, a_cur, b1, 1);
+    direct_phase_lo<DT>(c, acc, f, a_cur, 1);
+    direct_phase_hi<DT, TM, TN, BT, false>(c, acc, f, a_cur, b1, 0);
   }
 }
 
@@ -612,24 +625,23 @@ __device__ __forceinline__ void direct_mainloop(const GemmArgs& g, const DirectC
 template <int DT, int TM, int TN, bool EDGE, bool HAS_NEXT, bool BT = false>
 __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx<TM, TN>& next, int nk,
                                               uint8_t* __restrict__ ring, uint8_t* __restrict__ stage,
-                                              const f32x16 (&acc)[TN][TM], const u32x2 (&bias)[TN][4], int m0, int n0,
-                                              int wm0, int wn0) {
+                                              const f32x4 (&acc)[2 * TN][2 * TM], const u32x2 (&bias)[2 * TN], int m0,
+                                              int n0, int wm0, int wn0) {
   using Cfg = DirectCfg<TM, TN>;
   constexpr int WTN = Cfg::WTN;
   // The lane-dependent addresses below do not change from tile to tile; lane_now() has them
   // recomputed here instead of kept in registers (and spilled) across the main loop.
+  // Accumulator acc[i][j][e] of a lane: row wm0 + 16 j + lane % 16, column wn0 + 16 i + 4 (lane / 16) + e.
   const int lane = lane_now();
-  const int r32 = lane & 31, h = lane >> 5;
-  const int n_base = n0 + wn0 + 4 * h;
+  const int l16 = lane & 15, g4 = lane >> 4;
+  const int n_base = n0 + wn0 + 4 * g4;
   if (g.out_dt != LH_F32 && !(g.flags & LH_GEMM_ACCUMULATE_C)) {
     // The bias values (loaded by the main loop, whose last wait covered them) are pinned down here:
     // a wait for them placed after the ring loads below would wait for those loads as well.
 #pragma unroll
-    for (int i = 0; i < TN; ++i)
+    for (int i = 0; i < 2 * TN; ++i)
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-#pragma unroll
-        for (int e = 0; e < 2; ++e) asm volatile("" ::"v"(bias[i][q][e]));
+      for (int e = 0; e < 2; ++e) asm volatile("" ::"v"(bias[i][e]));
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the rings
     if constexpr (HAS_NEXT) direct_prologue<TM, TN, BT>(next, nk, ring);
     constexpr int RB = WTN * 2;                // bytes of a staged row
@@ -643,22 +655,20 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
 #pragma unroll
     for (int j0 = 0; j0 < TM; j0 += JB) {
 #pragma unroll
-      for (int jj = 0; jj < JB; ++jj)
+      for (int jj = 0; jj < 2 * JB; ++jj)
 #pragma unroll
-        for (int i = 0; i < TN; ++i)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int j = j0 + jj;
-            const int n = n_base + 32 * i + 8 * q;
-            const f32x4 b4 = (g.bias_dt == LH_F32)
-                                 ? bias4<DT>(g, EDGE ? min(n, g.N - 4) : n)  // the bias row ends at N
-                                 : f32x4{unpack_lo<DT>(bias[i][q][0]), unpack_hi<DT>(bias[i][q][0]),
-                                         unpack_lo<DT>(bias[i][q][1]), unpack_hi<DT>(bias[i][q][1])};
-            const u32x2 w = epilogue4_pack_bias<DT>(g, b4, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                                                    acc[i][j][4 * q + 3]);
-            *reinterpret_cast<u32x2*>(cw + (32 * jj + r32) * RB + (((4 * i + q) ^ ((r32 >> 1) & (chunks - 1))) << 4) +
-                                      8 * h) = w;
-          }
+        for (int i = 0; i < 2 * TN; ++i) {
+          const int j = 2 * j0 + jj;           // 16-row fragment; staged row 16 jj + l16
+          const int n = n_base + 16 * i;
+          const f32x4 b4 = (g.bias_dt == LH_F32)
+                               ? bias4<DT>(g, EDGE ? min(n, g.N - 4) : n)  // the bias row ends at N
+                               : f32x4{unpack_lo<DT>(bias[i][0]), unpack_hi<DT>(bias[i][0]), unpack_lo<DT>(bias[i][1]),
+                                       unpack_hi<DT>(bias[i][1])};
+          const u32x2 w = epilogue4_pack_bias<DT>(g, b4, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+          const int row = 16 * jj + l16;
+          *reinterpret_cast<u32x2*>(cw + row * RB + (((2 * i + (g4 >> 1)) ^ ((row >> 1) & (chunks - 1))) << 4) +
+                                    8 * (g4 & 1)) = w;
+        }
       // Cfg::kStagedStores stores per lane in all; the main loop's first wait counts on it.
 #pragma unroll
       for (int t = 0; t < JB * 32 / rows_per_pass; ++t) {
@@ -675,12 +685,12 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
   if constexpr (HAS_NEXT) direct_prologue<TM, TN, BT>(next, nk, ring);
   {
     // f32 output (with or without an accumulator input), or a 16-bit output with an accumulator
-    // input: the scaled f32 accumulators of a 32 x 8 QH block go through the wave's slice of `stage`
-    // so that the accumulator input is read and the result written as whole row segments (4
-    // elements per lane, 32 to 128 bytes per row) instead of pieces of 64 different rows.  Order
-    // of operations as in epilogue4 (one rounding, after the sum).
-    constexpr int QH = TN == 2 ? 4 : 2;        // accumulator column groups (of 8) per staged block
-    constexpr int RB = QH * 32;                // bytes of a staged row
+    // input: the scaled f32 accumulators of a block of 32 rows x 16 NI columns go through the wave's
+    // slice of `stage` so that the accumulator input is read and the result written as whole row
+    // segments (4 elements per lane, 64 or 128 bytes per row) instead of pieces of 64 different
+    // rows.  Order of operations as in epilogue4 (one rounding, after the sum).
+    constexpr int NI = TN;                     // 16-column fragments per staged block (2 blocks per wave)
+    constexpr int RB = NI * 64;                // bytes of a staged row
     constexpr int chunks = RB / 16;
     constexpr int rows_per_pass = 64 / chunks;
     uint8_t* cw = stage + next.wave * (32 * RB);
@@ -689,59 +699,59 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
     const bool gelu = (g.flags & LH_GEMM_HAS_GELU) != 0, relu = (g.flags & LH_GEMM_HAS_RELU) != 0;
     const int ch = lane % chunks, row0 = lane / chunks;
 #pragma unroll
-    for (int i = 0; i < TN; ++i)
+    for (int ib = 0; ib < 2; ++ib) {
+      const int n = n0 + wn0 + 16 * NI * ib + 4 * ch;  // the lane's 4 output columns
+      const bool n_ok = !EDGE || n < g.N;
+      const f32x4 b4 = bias4<DT>(g, EDGE ? min(n, g.N - 4) : n);
 #pragma unroll
-      for (int qh = 0; qh < 4 / QH; ++qh) {
-        const int n = n0 + wn0 + 32 * i + 8 * QH * qh + 4 * ch;  // the lane's 4 output columns
-        const bool n_ok = !EDGE || n < g.N;
-        const f32x4 b4 = bias4<DT>(g, EDGE ? min(n, g.N - 4) : n);
+      for (int j32 = 0; j32 < TM; ++j32) {
 #pragma unroll
-        for (int j = 0; j < TM; ++j) {
+        for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
-          for (int qq = 0; qq < QH; ++qq) {
-            const int q = QH * qh + qq;
-            const f32x4 w = {acc[i][j][4 * q] * g.alpha, acc[i][j][4 * q + 1] * g.alpha, acc[i][j][4 * q + 2] * g.alpha,
-                             acc[i][j][4 * q + 3] * g.alpha};
-            *reinterpret_cast<f32x4*>(cw + r32 * RB + (((2 * qq + h) ^ ((r32 >> 1) & (chunks - 1))) << 4)) = w;
+          for (int ii = 0; ii < NI; ++ii) {
+            const f32x4& a4 = acc[NI * ib + ii][2 * j32 + jj];
+            const f32x4 w = {a4[0] * g.alpha, a4[1] * g.alpha, a4[2] * g.alpha, a4[3] * g.alpha};
+            const int row = 16 * jj + l16;
+            *reinterpret_cast<f32x4*>(cw + row * RB + (((4 * ii + g4) ^ ((row >> 1) & (chunks - 1))) << 4)) = w;
           }
 #pragma unroll
-          for (int t = 0; t < 32 / rows_per_pass; ++t) {
-            const int row = rows_per_pass * t + row0;
-            f32x4 v = *reinterpret_cast<const f32x4*>(cw + row * RB + ((ch ^ ((row >> 1) & (chunks - 1))) << 4));
-            const int m = m0 + wm0 + 32 * j + row;
-            if (EDGE && !(n_ok && m < g.M)) continue;
-            const int64_t off = (int64_t)m * g.ldc + n;
-            if (has_c) {
-              f32x4 c4;
-              if (out32) {
-                c4 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.c) + off);
-              } else {
-                const u32x2 cc = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.c) + off);
-                c4 = f32x4{unpack_lo<DT>(cc[0]), unpack_hi<DT>(cc[0]), unpack_lo<DT>(cc[1]), unpack_hi<DT>(cc[1])};
-              }
-#pragma unroll
-              for (int e = 0; e < 4; ++e) v[e] += c4[e];
+        for (int t = 0; t < 32 / rows_per_pass; ++t) {
+          const int row = rows_per_pass * t + row0;
+          f32x4 v = *reinterpret_cast<const f32x4*>(cw + row * RB + ((ch ^ ((row >> 1) & (chunks - 1))) << 4));
+          const int m = m0 + wm0 + 32 * j32 + row;
+          if (EDGE && !(n_ok && m < g.M)) continue;
+          const int64_t off = (int64_t)m * g.ldc + n;
+          if (has_c) {
+            f32x4 c4;
+            if (out32) {
+              c4 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.c) + off);
+            } else {
+              const u32x2 cc = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.c) + off);
+              c4 = f32x4{unpack_lo<DT>(cc[0]), unpack_hi<DT>(cc[0]), unpack_lo<DT>(cc[1]), unpack_hi<DT>(cc[1])};
             }
-            if (g.flags & LH_GEMM_HAS_BIAS) {
 #pragma unroll
-              for (int e = 0; e < 4; ++e) v[e] += b4[e];
-            }
-            if (gelu) {
-#pragma unroll
-              for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
-            }
-            if (relu) {
-#pragma unroll
-              for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
-            }
-            if (out32)
-              *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(g.out) + off) = v;
-            else
-              *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(g.out) + off) =
-                  u32x2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+            for (int e = 0; e < 4; ++e) v[e] += c4[e];
           }
+          if (g.flags & LH_GEMM_HAS_BIAS) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += b4[e];
+          }
+          if (gelu) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
+          }
+          if (relu) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
+          }
+          if (out32)
+            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(g.out) + off) = v;
+          else
+            *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(g.out) + off) =
+                u32x2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
         }
       }
+    }
   }
 }
 
@@ -776,35 +786,32 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr int WN = 4;
   const int wm0 = (wave / WN) * Cfg::WTM, wn0 = (wave % WN) * Cfg::WTN;
-  const int r32 = lane & 31, h = lane >> 5;
+  const int l16 = lane & 15, g4 = lane >> 4;
 
   DirectCtx<TM, TN> c;
   c.wave = wave;
-  c.h = h;
-  // A fragment (second MFMA operand): row wm0 + 32 j + r32, logical chunk 2 kc + h.
-#pragma unroll
-  for (int j = 0; j < TM; ++j) {
-    const int r = wm0 + 32 * j + r32;
-    c.a_off[j] = r * 128;
-    c.a_swz[j] = (r >> 1) & 7;
-  }
-  // B fragment (first MFMA operand) through the transposing read: lane (grp = lane / 16,
-  // j = lane % 16) addresses k row 16 ks + 8 h + j / 4 (+4 for the second read), columns
-  // wn0 + 32 i + 16 (grp % 2) + 4 (j % 4) .. +4.
+  // A fragment jj (second MFMA operand): row wm0 + 16 jj + l16, logical 16-byte chunk 4 kc + g4 of
+  // the row's 8 (physical chunk: ^ ((row / 2) % 8); 4 kc only flips bit 2).
   {
-    const int j16 = lane & 15, grp = lane >> 4;
-    const int krow = 8 * h + (j16 >> 2);
-    const int col = wn0 + 16 * (grp & 1) + 4 * (j16 & 3);
+    const int r = wm0 + l16;
+    c.a_rd[0] = r * 128 + ((g4 ^ ((r >> 1) & 7)) << 4);
+    c.a_rd[1] = c.a_rd[0] ^ 64;
+  }
+  // B fragment i (first MFMA operand) through the transposing read: the 16 lanes of group g4
+  // address k rows 8 g4 + l16 / 4 (+4 for the second read), columns wn0 + 16 i + 4 (l16 % 4) .. +4,
+  // and each receives the 4 k-values of column wn0 + 16 i + l16.
+  {
+    const int krow = 8 * g4 + (l16 >> 2);
+    const int col = wn0 + 4 * (l16 & 3);
     c.b_chunk = col >> 3;
-    c.b_swz = 4 * (krow & 3);
+    c.b_swz = (4 * (krow & 3)) ^ (2 * ((krow >> 3) & 1));
     c.b_off = krow * Cfg::kBRow + 8 * ((col >> 2) & 1);
   }
-  // (transposed B: row wn0 + 32 i + r32 of the stage, logical chunk 2 kc + h, like the A fragment)
-#pragma unroll
-  for (int i = 0; i < TN; ++i) {
-    const int r = wn0 + 32 * i + r32;
-    c.bt_off[i] = r * 128;
-    c.bt_swz[i] = (r >> 1) & 7;
+  // (transposed B: row wn0 + 16 i + l16 of the stage, like the A fragment)
+  {
+    const int r = wn0 + l16;
+    c.bt_rd[0] = r * 128 + ((g4 ^ ((r >> 1) & 7)) << 4);
+    c.bt_rd[1] = c.bt_rd[0] ^ 64;
   }
 
   const int nk = g.K / 32;  // even: K is a multiple of 64
@@ -820,16 +827,16 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
   const bool counted_stores = !EDGE && staged;
   bool first = true;
   for (;;) {
-    f32x16 acc[TN][TM];
+    f32x4 acc[2 * TN][2 * TM];
 #pragma unroll
-    for (int i = 0; i < TN; ++i)
+    for (int i = 0; i < 2 * TN; ++i)
 #pragma unroll
-      for (int j = 0; j < TM; ++j)
+      for (int j = 0; j < 2 * TM; ++j)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-    u32x2 bias[TN][4];
+        for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.0f;
+    u32x2 bias[2 * TN];
     const GemmArgs& ga = SPLITK ? g_cur : g;
-    direct_mainloop<DT, TM, TN, EDGE, BT>(ga, c, acc, smem_d, nk, counted_stores && !first, staged, n0 + wn0 + 4 * h, bias);
+    direct_mainloop<DT, TM, TN, EDGE, BT>(ga, c, acc, smem_d, nk, counted_stores && !first, staged, n0 + wn0 + 4 * g4, bias);
     first = false;
     const int tn = t + (int)gridDim.x;
     const bool more = tn < ntiles;
@@ -1100,14 +1107,14 @@ static int gemm16_dispatch(const GemmArgs& g_in, hipStream_t s) {
     static const int bm[4] = {256, 256, 128, 128}, bn[4] = {256, 128, 256, 128};
     const int v = (int)(tile >> 8) - 1;
     LH_REQUIRE(vec_ok && !tb && g.ldc % 8 == 0 && g.M % bm[v] == 0 && g.N % bn[v] == 0 && direct_offsets_fit(g),
-               "gemm: the requested %d x %d tile needs untransposed operands, M %% %d == 0, N %% %d == 0, "
-               "K %% 64 == 0 and 16-byte aligned rows (M=%d N=%d K=%d)",
+               "gemm: the requested %d x %d tile needs an untransposed A, M %% %d == 0, N %% %d == 0, "
+               "K %% 64 == 0 and 16-byte aligned rows, also of a transposed B (M=%d N=%d K=%d)",
                bm[v], bn[v], bm[v], bn[v], g.M, g.N, g.K);
   }
   if (cut_requested)
     LH_REQUIRE(vec_ok && !tb && g.ldc % 8 == 0 && g.N % 8 == 0 && direct_offsets_fit(g),
-               "gemm: a split-K request needs untransposed operands, K %% 64 == 0, N %% 8 == 0 and 16-byte aligned rows "
-               "(M=%d N=%d K=%d)", g.M, g.N, g.K);
+               "gemm: a split-K request needs an untransposed A, K %% 64 == 0, N %% 8 == 0 and 16-byte aligned rows, "
+               "also of a transposed B (M=%d N=%d K=%d)", g.M, g.N, g.K);
   if (vec_ok) {
     if (!tb && g.ldc % 8 == 0 && g.N % 8 == 0 && direct_offsets_fit(g)) {
       if (tile == LH_GEMM_TILE_AUTO) {
