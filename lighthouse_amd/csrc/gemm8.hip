@@ -158,12 +158,16 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm8_fast(GemmArgs g) 
 // ---- direct-to-LDS kernel ---------------------------------------------------------------
 // Same structure as the 16-bit direct kernel: 256 x 256 workgroup tile, 8 waves (2 x 4, 128 x 64
 // per wave), panels global -> LDS with buffer_load_dwordx4 ... lds in their global orientation, A ring
-// 2 stages x 128 k (256 rows x 128 bytes), B ring 4 stages x 64 k (64 rows x 256 bytes), one
-// v_mfma_f32_32x32x64_f8f6f4 k-step (64 k) per main-loop step, one barrier per two steps.
+// 2 stages x 128 k (256 rows x 128 bytes), B ring 4 stages x 64 k (64 rows x 256 bytes), used as
+// two pairs of 128 k.  The matrix instruction is v_mfma_f32_16x16x128_f8f6f4: on random operands
+// the matrix cores hold a higher clock with it than with 32x32x64 (register-only loops: 4.43 against
+// 4.04 PFLOP/s; both reach the published peak on zeros).  A main-loop step is 128 k: 8 A fragments
+// of 16 rows and 4 B fragments of 16 columns per wave, in two phases (the MFMAs of the lower four
+// A fragments, then of the upper four), with one barrier per step between the phases.
 // The k-contiguous A fragment (32 bytes per lane) is two 16-byte LDS reads; the n-contiguous B
 // panel is read with ds_read_b64_tr_b8, which hands a lane 8 k-values of one column (16 lanes
 // cover 8 k-rows x 16 columns), four reads per fragment.  Swizzles: A chunk ^ ((row / 2) % 8),
-// B chunk ^ 2 (k % 8).
+// B chunk ^ 2 (k % 8) ^ ((k / 32) % 2).
 constexpr int kD8ABytes = 256 * 128;   // one A stage (128 k): 32 KiB
 constexpr int kD8BBytes = 64 * 256;    // one B stage (64 k): 16 KiB
 constexpr int kD8BBase = 2 * kD8ABytes;
@@ -194,15 +198,17 @@ struct D8Ctx {
   const uint8_t* b_base;
   uint32_t a_voff[4];
   uint32_t b_voff[2];
-  int a_off, a_swz;  // byte offset and swizzle of the lane's A row of m-subtile 0; subtile j is 32 rows
-                     // (4096 bytes) further on with the same swizzle
+  int a_rd;  // byte offset of the lane's first 16 bytes of A fragment 0 in a stage (row wm0 + lane % 16, chunk
+             // 2 (lane / 16), swizzled); its second 16 bytes are at a_rd ^ 16, fragment jj 2048 jj further on
   int64_t ldb;
-  int wave, h, b_off, b_chunk, b_swz;
+  int wave, b_off, b_chunk, b_swz;
 };
 
+// Fragments in registers: the A fragments of the lower (a[0]) and upper (a[1]) half of the wave's
+// rows, four of 16 rows each, and the step's four B fragments of 16 columns.
 struct D8Frags {
-  i32x8 a[4];
-  i32x8 b[2];
+  i32x8 a[2][4];
+  i32x8 b[4];
 };
 
 __device__ __forceinline__ void d8_load_a(const D8Ctx& c, int sa, uint8_t* __restrict__ abuf) {
@@ -216,41 +222,32 @@ __device__ __forceinline__ void d8_load_b(const D8Ctx& c, int sb, uint8_t* __res
   for (int i = 0; i < 2; ++i) dma8_16(stage_base, c.b_voff[i], 0u, bbuf + (8 * i + c.wave) * 1024);
 }
 
-// Fragments of one 64-k step: A bytes 64 kb .. +64 of the stage's rows (kb = 0 / 1), B stage bs.
-__device__ __forceinline__ void d8_read_frags(const D8Ctx& c, const uint8_t* __restrict__ as,
-                                              const uint8_t* __restrict__ bs, int kb, D8Frags& f) {
+// A fragments HALF * 4 .. + 4 (16 rows each) of the 128-k stage `as`.
+template <int HALF>
+__device__ __forceinline__ void d8_read_a(const D8Ctx& c, const uint8_t* __restrict__ as, i32x8 (&a)[4]) {
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int c0 = 4 * kb + 2 * c.h;
-    i32x4 lo = *reinterpret_cast<const i32x4*>(as + c.a_off + ((c0 ^ c.a_swz) << 4) + 4096 * j);
-    i32x4 hi = *reinterpret_cast<const i32x4*>(as + c.a_off + (((c0 + 1) ^ c.a_swz) << 4) + 4096 * j);
-    f.a[j] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-  }
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const uint8_t* p0 = bs + c.b_off + (((c.b_chunk + 2 * i) ^ c.b_swz) << 4);
-    i32x2 r[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-      r[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(p0 + q * 8 * 256));
-    f.b[i] = i32x8{r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]};
+    i32x4 lo = *reinterpret_cast<const i32x4*>(as + c.a_rd + 2048 * (4 * HALF + j));
+    i32x4 hi = *reinterpret_cast<const i32x4*>(as + (c.a_rd ^ 16) + 2048 * (4 * HALF + j));
+    a[j] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   }
 }
-
-__device__ __forceinline__ void d8_mfma(f32x16 (&acc)[2][4], const D8Frags& f) {
+// B fragment i (16 columns) of the 128 k held by the stage pair `bs` (two consecutive 64-k stages).
+__device__ __forceinline__ i32x8 d8_read_b(const D8Ctx& c, const uint8_t* __restrict__ bs, int i) {
+  const uint8_t* p0 = bs + c.b_off + (((c.b_chunk + i) ^ c.b_swz) << 4);
+  i32x2 r[4];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = mfma_f8_32(f.b[i], f.a[j], acc[i][j]);
+  for (int q = 0; q < 4; ++q)
+    r[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(p0 + q * 8 * 256));
+  return i32x8{r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]};
 }
 
-// 16 LDS reads of the next step spread over the 8 MFMAs of the current one.
+// NR LDS reads spread over the 16 MFMAs of a phase.
+template <int NR, int I = 0>
 __device__ __forceinline__ void d8_interleave_hint() {
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-  }
+  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+  __builtin_amdgcn_sched_group_barrier(0x100, (I + 1) * NR / 16 - I * NR / 16, 0);
+  if constexpr (I + 1 < 16) d8_interleave_hint<NR, I + 1>();
 }
 
 // All loads of this wave have landed and all its LDS reads have returned, then barrier.  One asm
@@ -259,32 +256,56 @@ __device__ __forceinline__ void d8_wait_barrier() {
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-// Steps kt (even) and kt + 1.  f holds the fragments of step kt on entry and of step kt + 2 on
-// exit; a step is a single MFMA k-step, so the fragments of the next step are read while the
-// current ones are multiplied.  ONE barrier per pair, between the two steps: the rings work as two
-// halves of 128 k.  At the barrier both fragment sets of this pair are in registers and the next
-// pair's stages (requested at the previous barrier, 128 k ago) are awaited in full; the pair after
-// that is then requested into this pair's buffers.  (Two barriers per pair with B requested three
-// stages ahead, as in the small tiles of the 16-bit kernel, measured 2-2.5 % slower: 8192^3 426 ->
-// 416 us.)
-__device__ __forceinline__ void d8_step_pair(const D8Ctx& c, f32x16 (&acc)[2][4], D8Frags& f,
-                                                const uint8_t* __restrict__ a_cur, const uint8_t* __restrict__ a_nxt,
-                                                const uint8_t* __restrict__ b1, const uint8_t* __restrict__ b2,
-                                                uint8_t* __restrict__ a_refill, uint8_t* __restrict__ b_refill0,
-                                                uint8_t* __restrict__ b_refill1, int kt, int nk) {
-  D8Frags g;
-  d8_read_frags(c, a_cur, b1, 1, g);  // step kt + 1
-  d8_mfma(acc, f);
-  d8_interleave_hint();
+// First phase of a step: the MFMAs of the lower row fragments under the reads of the step's upper ones.
+__device__ __forceinline__ void d8_phase_lo(const D8Ctx& c, f32x4 (&acc)[4][8], D8Frags& f,
+                                            const uint8_t* __restrict__ as) {
+  d8_read_a<1>(c, as, f.a[1]);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = mfma_f8_16(f.b[i], f.a[0][j], acc[i][j]);
+  d8_interleave_hint<8>();
+}
+// Second phase: the MFMAs of the upper row fragments under the reads of the NEXT step's lower row
+// fragments (A stage `as_n`) and B fragments (stage pair `bs_n`), each B fragment requested behind
+// the last MFMA that uses the one it replaces.  LOAD false: a tile's last step.
+template <bool LOAD = true>
+__device__ __forceinline__ void d8_phase_hi(const D8Ctx& c, f32x4 (&acc)[4][8], D8Frags& f,
+                                            const uint8_t* __restrict__ as_n, const uint8_t* __restrict__ bs_n) {
+  if constexpr (LOAD) d8_read_a<0>(c, as_n, f.a[0]);
+  i32x8 bn[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][4 + j] = mfma_f8_16(f.b[i], f.a[1][j], acc[i][4 + j]);
+    if constexpr (LOAD) bn[i] = d8_read_b(c, bs_n, i);
+  }
+  if constexpr (LOAD) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f.b[i] = bn[i];
+    d8_interleave_hint<24>();
+  }
+}
+
+// Step kt / 2 of 128 k (B stages kt and kt + 1).  f holds the step's lower A fragments and its B
+// fragments on entry and the next step's on exit.  ONE barrier, between the two phases: at the
+// barrier every fragment of this step's stages has been read and the next step's stages
+// (requested at the previous barrier, 128 k ago) are awaited in full; the step after that is then
+// requested into this step's buffers.  (Two barriers per 128 k with B requested three stages ahead,
+// as in the small tiles of the 16-bit kernel, measured 2-2.5 % slower: 8192^3 426 -> 416 us.)
+__device__ __forceinline__ void d8_step(const D8Ctx& c, f32x4 (&acc)[4][8], D8Frags& f,
+                                        const uint8_t* __restrict__ a_cur, const uint8_t* __restrict__ a_nxt,
+                                        const uint8_t* __restrict__ b_nxt, uint8_t* __restrict__ a_refill,
+                                        uint8_t* __restrict__ b_refill0, uint8_t* __restrict__ b_refill1, int kt,
+                                        int nk) {
+  d8_phase_lo(c, acc, f, a_cur);
   d8_wait_barrier();
   if (kt + 4 < nk) {
     d8_load_a(c, kt / 2 + 2, a_refill);
     d8_load_b(c, kt + 4, b_refill0);
     d8_load_b(c, kt + 5, b_refill1);
   }
-  d8_read_frags(c, a_nxt, b2, 0, f);  // step kt + 2
-  d8_mfma(acc, g);
-  d8_interleave_hint();
+  d8_phase_hi(c, acc, f, a_nxt, b_nxt);
 }
 
 // Source pointers of tile `id` (its position in the XCD-grouped order) and the tile's origin.
@@ -309,7 +330,7 @@ __device__ __forceinline__ void d8_place(const GemmArgs& g, int id, D8Ctx& c, in
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int bk = (8 * i + c.wave) * 4 + (lane >> 4);
-    const int bc = (lane & 15) ^ (2 * (bk & 7));
+    const int bc = (lane & 15) ^ (2 * (bk & 7)) ^ ((bk >> 5) & 1);
     c.b_voff[i] = (uint32_t)bk * (uint32_t)g.ldb + bc * 16;
   }
 }
@@ -324,28 +345,27 @@ __device__ __forceinline__ void d8_prologue(const D8Ctx& c, int nk, uint8_t* __r
 }
 
 // Main loop of one tile, whose first loads have been issued.
-__device__ __forceinline__ void d8_mainloop(const D8Ctx& c, f32x16 (&acc)[2][4], uint8_t* smem_8, int nk) {
+__device__ __forceinline__ void d8_mainloop(const D8Ctx& c, f32x4 (&acc)[4][8], uint8_t* smem_8, int nk) {
   uint8_t* const abuf = smem_8;
   uint8_t* const bbuf = smem_8 + kD8BBase;
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
   D8Frags f;
-  d8_read_frags(c, abuf, bbuf, 0, f);
+  d8_read_a<0>(c, abuf, f.a[0]);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f.b[i] = d8_read_b(c, bbuf, i);
   int kt = 0;
   for (; kt + 2 < nk; kt += 2) {
     uint8_t* a_cur = abuf + ((kt >> 1) & 1) * kD8ABytes;
     uint8_t* a_nxt = abuf + (((kt >> 1) + 1) & 1) * kD8ABytes;
-    uint8_t* b0 = bbuf + (kt & 3) * kD8BBytes;
-    uint8_t* b1 = bbuf + ((kt + 1) & 3) * kD8BBytes;
+    uint8_t* b0 = bbuf + (kt & 3) * kD8BBytes;         // kt is even: stages kt and kt + 1 are adjacent
     uint8_t* b2 = bbuf + ((kt + 2) & 3) * kD8BBytes;
-    d8_step_pair(c, acc, f, a_cur, a_nxt, b1, b2, a_cur, b0, b1, kt, nk);
+    d8_step(c, acc, f, a_cur, a_nxt, b2, a_cur, b0, b0 + kD8BBytes, kt, nk);
   }
   {
+    // (the last step's stages were awaited at the barrier of the step before, or at the start)
     const uint8_t* a_cur = abuf + ((kt >> 1) & 1) * kD8ABytes;
-    const uint8_t* b1 = bbuf + ((kt + 1) & 3) * kD8BBytes;
-    D8Frags gfr;  // (the last pair's stages were awaited at the barrier of the pair before, or at the start)
-    d8_read_frags(c, a_cur, b1, 1, gfr);
-    d8_mfma(acc, f);
-    d8_mfma(acc, gfr);
+    d8_phase_lo(c, acc, f, a_cur);
+    d8_phase_hi<false>(c, acc, f, a_cur, a_cur);
   }
 }
 
@@ -357,13 +377,14 @@ __device__ __forceinline__ void d8_mainloop(const D8Ctx& c, f32x16 (&acc)[2][4],
 // that the staging traffic does not wait for the asynchronous ring writes.
 template <bool HAS_NEXT>
 __device__ __forceinline__ void d8_finish(const GemmArgs& g, const D8Ctx& next, int nk, uint8_t* __restrict__ ring,
-                                          uint8_t* __restrict__ stage, const f32x16 (&acc)[2][4], int m0, int n0, int wm0,
+                                          uint8_t* __restrict__ stage, const f32x4 (&acc)[4][8], int m0, int n0, int wm0,
                                           int wn0) {
-  constexpr int TM = 4, TN = 2, RB = 128, chunks = 8, rows_per_pass = 8;
+  constexpr int TM = 4, RB = 128, chunks = 8, rows_per_pass = 8;
+  // Accumulator acc[i][j][e] of a lane: row wm0 + 16 j + lane % 16, column wn0 + 16 i + 4 (lane / 16) + e.
   const int lane = lane_now();  // keeps the addresses below out of registers during the main loop
-  const int r32 = lane & 31, h = lane >> 5;
-  const int m_base = m0 + wm0 + r32;
-  const int n_base = n0 + wn0 + 4 * h;
+  const int l16 = lane & 15, g4 = lane >> 4;
+  const int m_base = m0 + wm0 + l16;
+  const int n_base = n0 + wn0 + 4 * g4;
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the rings
   if constexpr (HAS_NEXT) d8_prologue(next, nk, ring);
   if (g.out_dt != LH_F32) {
@@ -373,17 +394,15 @@ __device__ __forceinline__ void d8_finish(const GemmArgs& g, const D8Ctx& next, 
 #pragma unroll
     for (int j0 = 0; j0 < TM; j0 += JB) {
 #pragma unroll
-      for (int jj = 0; jj < JB; ++jj)
+      for (int jj = 0; jj < 2 * JB; ++jj)
 #pragma unroll
-        for (int i = 0; i < TN; ++i)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int j = j0 + jj;
-            const u32x2 w = epilogue4_pack<LH_BF16>(g, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
-                                                    acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
-            *reinterpret_cast<u32x2*>(cw + (32 * jj + r32) * RB + (((4 * i + q) ^ ((r32 >> 1) & (chunks - 1))) << 4) +
-                                      8 * h) = w;
-          }
+        for (int i = 0; i < 4; ++i) {
+          const int j = 2 * j0 + jj;
+          const u32x2 w = epilogue4_pack<LH_BF16>(g, n_base + 16 * i, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+          const int row = 16 * jj + l16;
+          *reinterpret_cast<u32x2*>(cw + row * RB + (((2 * i + (g4 >> 1)) ^ ((row >> 1) & (chunks - 1))) << 4) +
+                                    8 * (g4 & 1)) = w;
+        }
 #pragma unroll
       for (int t = 0; t < JB * 32 / rows_per_pass; ++t) {
         const int row = rows_per_pass * t + lane / chunks, ch = lane % chunks;
@@ -394,13 +413,10 @@ __device__ __forceinline__ void d8_finish(const GemmArgs& g, const D8Ctx& next, 
     return;
   }
 #pragma unroll
-  for (int i = 0; i < TN; ++i)
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < TM; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        epilogue4<LH_BF16>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
-                           acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+    for (int j = 0; j < 8; ++j)
+      epilogue4<LH_BF16>(g, m_base + 16 * j, n_base + 16 * i, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
 }
 
 // Persistent workgroups, one per CU, each walking the tile list with the grid as stride (tile
@@ -433,18 +449,21 @@ __global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
   D8Ctx c;
   c.ldb = g.ldb;
   c.wave = wave;
-  const int r32 = lane & 31, h = lane >> 5;
-  c.h = h;
-  c.a_off = (wm0 + r32) * 128;
-  c.a_swz = (r32 >> 1) & 7;  // wm0 and 32 j are multiples of 16
+  const int l16 = lane & 15, g4 = lane >> 4;
   {
-    // Lane (grp = lane / 16, j = lane % 16) addresses k row 32 h + 8 q + j / 2 (q = 0..3), columns
-    // wn0 + 32 i + 16 (grp % 2) + 8 (j % 2) .. +8.
-    const int j16 = lane & 15, grp = lane >> 4;
-    const int krow = 32 * h + (j16 >> 1);
-    const int col = wn0 + 16 * (grp & 1) + 8 * (j16 & 1);
+    // A fragment jj: row wm0 + 16 jj + l16, its k bytes 32 g4 .. +32 = 16-byte chunks 2 g4 and 2 g4 + 1
+    // of the row's eight, swizzled with (row / 2) % 8 (the same for every jj: wm0 and 16 jj are multiples of 16).
+    const int r = wm0 + l16;
+    c.a_rd = r * 128 + (((2 * g4) ^ ((r >> 1) & 7)) << 4);
+  }
+  {
+    // B fragment i: the 16 lanes of group g4 address k rows 32 g4 + 8 q + l16 / 2 (q = 0..3) of the
+    // stage pair, columns wn0 + 16 i + 8 (l16 % 2) .. +8; each lane receives the 8 k-values per q of
+    // column wn0 + 16 i + l16.
+    const int krow = 32 * g4 + (l16 >> 1);
+    const int col = wn0 + 8 * (l16 & 1);
     c.b_chunk = col >> 4;
-    c.b_swz = 2 * (krow & 7);
+    c.b_swz = (2 * (krow & 7)) ^ (g4 & 1);
     c.b_off = krow * 256 + (col & 8);
   }
 
@@ -457,13 +476,13 @@ __global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
   }
   d8_prologue(c, nk, smem_8);
   for (;;) {
-    f32x16 acc[TN][TM];
+    f32x4 acc[4][8];  // [16-column fragment][16-row fragment]
 #pragma unroll
-    for (int i = 0; i < TN; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < TM; ++j)
+      for (int j = 0; j < 8; ++j)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.0f;
     d8_mainloop(c, acc, smem_8, nk);
     const int tn = t + (int)gridDim.x;
     const bool more = tn < ntiles;
