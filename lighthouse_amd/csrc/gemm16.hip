@@ -956,13 +956,18 @@ static int launch_fast(const GemmArgs& g, hipStream_t s) {
 
 // Tile choice for the direct kernels: 0 = 256 x 256, 1 = 256 x 128, 2 = 128 x 256, 3 = 128 x 128.
 // Cost model: rounds of resident workgroups times the tile area (edge tiles count in full) times a
-// measured cost per flop relative to the 256 x 256 tile (one round of 256 tiles each at K = 2048 and
-// 4096: 256 x 128 1.155, 128 x 256 1.135; 128 x 128 1.2 with two workgroups on a CU, 1.37 alone).
+// measured cost per flop relative to the 256 x 256 tile (256 x 128 1.19, 128 x 256 1.17; 128 x 128
+// 1.19 with two workgroups on a CU, 1.05 of it for short K, 1.30 alone).  A last round that does
+// not fill the CUs costs less than a full one: the persistent workgroups are not in step, so the
+// extra tiles run while others still finish, and fewer busy CUs hold a higher clock.  Measured at
+// M = 8192, K = 3072 and 4096: a fraction r of a round of the large tiles costs 0.6 + 0.4 r^2 of a
+// round (also when it is the only one), of the 128 x 128 tile (two workgroups per CU) 0.12 + 0.88 r.
 // The 128 x 128 tile runs two workgroups per CU, which share the CU's rate: a round is 2 CUs' worth
 // of tiles at twice a tile's cost, except when no CU gets a second tile.  For short K a tile's
 // prologue and epilogue weigh as much as its main loop, and the 128 x 128 tile, whose two
-// co-resident workgroups cover each other's, costs little more per flop than the large ones
-// (M = 8192, K = 768: N = 768 19 vs 22 us, N = 2304 39 vs 46, N = 3072 51 vs 53).  `slow_epilogue`:
+// co-resident workgroups cover each other's, costs little more per flop than the large ones.
+// On 84 shapes (M 2048 ... 8192, N 768 ... 4096, K 768 ... 4096) the choice is within 1.3 % of the best
+// explicit tile.  `slow_epilogue`:
 // an accumulator input or an f32 output is staged block by block, which the tiles with a 256 side
 // pay more for (M = 8192, N = 768, K = 3072 + residual: 49.1 / 49.6 us against 46.6 us for 128 x 128;
 // without the residual 42.6 / 43.3 against 43.0).
@@ -976,12 +981,16 @@ static int direct_variant(int M, int N, int K, bool slow_epilogue) {
     const int64_t tiles = (int64_t)((M + bm[v] - 1) / bm[v]) * ((N + bn[v] - 1) / bn[v]);
     double cost;
     if (v < 3) {
-      const double per_flop = v == 0 ? 1.0 : v == 1 ? 1.155 : 1.135;
-      cost = (double)((tiles + cus - 1) / cus) * bm[v] * bn[v] * per_flop * big;
+      const double per_flop = v == 0 ? 1.0 : v == 1 ? 1.19 : 1.17;
+      const double r = (double)(tiles % cus) / cus;
+      const double rounds = (double)(tiles / cus) + (r > 0.0 ? 0.6 + 0.4 * r * r : 0.0);
+      cost = rounds * bm[v] * bn[v] * per_flop * big;
     } else if (tiles <= cus) {
-      cost = 128.0 * 128.0 * (K <= 1536 ? 1.08 : 1.37);
+      cost = 128.0 * 128.0 * (K <= 1536 ? 1.08 : 1.30);
     } else {
-      cost = (double)((tiles + 2 * cus - 1) / (2 * cus)) * 2.0 * 128.0 * 128.0 * (K <= 1536 ? 1.08 : 1.2);
+      const double r = (double)(tiles % (2 * cus)) / (2 * cus);
+      const double rounds = (double)(tiles / (2 * cus)) + (r > 0.0 ? 0.12 + 0.88 * r : 0.0);
+      cost = rounds * 2.0 * 128.0 * 128.0 * (K <= 1536 ? 1.05 : 1.19);
     }
     if (best < 0 || cost < best_cost) {
       best = v;

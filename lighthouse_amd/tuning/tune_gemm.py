@@ -28,7 +28,7 @@ TILES = ((256, 256), (256, 128), (128, 256), (128, 128))
 TILES_F32 = ((128, 128), (128, 64), (64, 64))
 # Cost per flop relative to the largest tile, as the library's own tile choice prices it (16-bit:
 # measured one round of 256 tiles each at K = 2048 and 4096; 128 x 128 runs two workgroups per CU).
-_PENALTY = {(256, 256): 1.0, (256, 128): 1.155, (128, 256): 1.135, (128, 128): 1.2}
+_PENALTY = {(256, 256): 1.0, (256, 128): 1.19, (128, 256): 1.17, (128, 128): 1.19}
 _PENALTY_F32 = {(128, 128): 1.0, (128, 64): 1.08, (64, 64): 1.3}
 _CUS = 256
 
@@ -46,17 +46,23 @@ def candidate_tiles(M: int, N: int, K: int, dtype: str = "bf16") -> list[tuple[i
 def estimate_cost(M: int, N: int, K: int, tile: tuple[int, int], dtype: str = "bf16") -> float:
     """Rounds of resident workgroups x tile area x cost per flop x (K + a fixed per-round cost worth
     about 320 k of main loop: launch, first loads, output stores).  The 16-bit 128 x 128 tile runs
-    two workgroups per CU that share its rate: a round is two CUs' worth of tiles at twice the cost."""
+    two workgroups per CU that share its rate: a round is two CUs' worth of tiles at twice the cost.
+    For the 16-bit tiles a last round that fills a fraction r of the CUs costs 0.6 + 0.4 r^2 of a
+    round (128 x 128: 0.12 + 0.88 r), as in the library's own choice."""
     tiles = -(-M // tile[0]) * -(-N // tile[1])
     if dtype == "f32":
         return -(-tiles // _CUS) * tile[0] * tile[1] * _PENALTY_F32[tile] * (K + 320)
     if tile == (128, 128):
         # short K: prologue and epilogue weigh as much as the main loop and the two co-resident
         # workgroups cover each other's; long K and a lone workgroup per CU: nobody covers its waits
-        per_flop = 1.08 if K <= 1536 else (_PENALTY[tile] if tiles > _CUS else 1.37)
-        rounds = -(-tiles // (2 * _CUS)) * 2 if tiles > _CUS else 1
-        return rounds * tile[0] * tile[1] * per_flop * (K + 320)
-    return -(-tiles // _CUS) * tile[0] * tile[1] * _PENALTY[tile] * (K + 320)
+        if tiles <= _CUS:
+            return tile[0] * tile[1] * (1.08 if K <= 1536 else 1.30) * (K + 320)
+        full, rest = divmod(tiles, 2 * _CUS)
+        rounds = full + (0.12 + 0.88 * rest / (2 * _CUS) if rest else 0.0)
+        return rounds * 2 * tile[0] * tile[1] * (1.05 if K <= 1536 else _PENALTY[tile]) * (K + 320)
+    full, rest = divmod(tiles, _CUS)
+    rounds = full + (0.6 + 0.4 * (rest / _CUS) ** 2 if rest else 0.0)
+    return rounds * tile[0] * tile[1] * _PENALTY[tile] * (K + 320)
 
 
 def prefilter(M: int, N: int, K: int, slack: float = 1.35, dtype: str = "bf16") -> list[tuple[int, int]]:

@@ -15,12 +15,15 @@ def test_candidates_and_prefilter():
     assert candidate_tiles(256, 256, 96) == []          # K must be a multiple of 64
     # 4096^3: 256 tiles of 256 x 256 are exactly one round, every smaller tile costs more
     assert prefilter(4096, 4096, 4096)[0] == (256, 256)
-    # N = 768: 96 big tiles leave CUs idle; halves and quarters are estimated cheaper, at short K the quarters
+    # N = 768: 96 big tiles leave CUs idle; the quarters (384 tiles, three quarters of a round of pairs) are cheapest
     assert prefilter(8192, 768, 768)[0] == (128, 128)
-    assert prefilter(8192, 768, 4096)[0] in ((256, 128), (128, 256))
+    assert prefilter(8192, 768, 4096)[0] == (128, 128)
+    # a partial last round costs less than a full one: 1152 quarter tiles (2.25 rounds of pairs) beat 576 halves
+    assert prefilter(8192, 2304, 3072)[0] == (128, 128)
+    assert estimate_cost(8192, 2304, 3072, (128, 128)) < 2.5 * estimate_cost(8192, 1024, 3072, (128, 128))
     assert estimate_cost(8192, 768, 768, (256, 256)) > estimate_cost(8192, 768, 768, (256, 128))
     assert all(t in candidate_tiles(8192, 2304, 768) for t in prefilter(8192, 2304, 768))
-    # 192 tiles of 256 x 256 in one round beat 768 of 128 x 128 in two rounds of pairs
+    # 192 tiles of 256 x 256 in three quarters of a round beat 768 of 128 x 128 in a round and a half of pairs
     assert prefilter(4096, 3072, 4096)[0] == (256, 256)
     # f32: three tiles, edge tiles clipped, no cut along K
     assert candidate_tiles(1000, 1000, 1024, "f32") == [(128, 128), (128, 64), (64, 64)]
