@@ -163,15 +163,17 @@ def cpu_baseline_gemm_bf16(n: int, seconds_naive: float = 8.0, seconds_tiled: fl
     return result
 
 
-def probe_mfma_rate(dtype_code: int, random_operands: bool, iters: int):
+def probe_mfma_rate(dtype_code: int, random_operands: bool, iters: int, wide: bool = False):
     """TFLOP/s of a register-only MFMA loop on every SIMD (lighthouse_amd/csrc/probe.hip, built as a
-    library of its own beside the product library); None when it has not been built."""
+    library of its own beside the product library); None when it has not been built.  The loop issues
+    the instruction the GEMM kernels use (16x16x32 for 16-bit, 16x16x128 for fp8, 32x32x2 for f32);
+    `wide`: the 32x32x16 / 32x32x64 form of the same products."""
     path = ROOT / "lighthouse_amd" / "lib" / "liblighthouse_probe.so"
     if not path.is_file():
         return None
     lib = ctypes.CDLL(str(path))
     out = ctypes.c_double(0.0)
-    rc = lib.lh_probe_mfma_rate(ctypes.c_int32(dtype_code), ctypes.c_int32(1 if random_operands else 0),
+    rc = lib.lh_probe_mfma_rate(ctypes.c_int32(dtype_code), ctypes.c_int32((1 if random_operands else 0) | (2 if wide else 0)),
                                 ctypes.c_int64(iters), ctypes.byref(out))
     return round(out.value, 1) if rc == 0 else None
 
@@ -406,8 +408,11 @@ def main() -> int:
         # Register-only MFMA loops: what the matrix cores sustain on zero and on random operands.
         extras["mfma_register_loop_tflops"] = {
             f"{name}_{kind}": probe_mfma_rate(code, kind == "random", iters)
-            for name, code, iters in (("bf16", 1, 20000), ("fp8", 3, 10000), ("f32", 0, 20000))  # lh_dtype codes
+            for name, code, iters in (("bf16", 1, 10000), ("fp8", 3, 5000), ("f32", 0, 20000))  # lh_dtype codes
             for kind in ("zero", "random")}
+        # the wider instruction forms of the same products: the same rate on zeros, lower on random operands
+        extras["mfma_register_loop_tflops"]["bf16_random_32x32x16"] = probe_mfma_rate(1, True, 20000, wide=True)
+        extras["mfma_register_loop_tflops"]["fp8_random_32x32x64"] = probe_mfma_rate(3, True, 10000, wide=True)
 
     cpu = None
     if not args.no_cpu_baseline:

@@ -10,48 +10,87 @@
 
 namespace lh {
 
-// 8 waves per workgroup, one workgroup per CU; each wave keeps 8 independent 32x32 accumulators
-// and 4 + 4 operand fragments in registers.
-template <int DT>
+// 8 waves per workgroup, one workgroup per CU; each wave keeps the accumulators of a 128 x 64
+// sub-tile and 8 + 4 operand fragments (two sets, alternating) in registers and issues the
+// instructions the GEMM kernels use: v_mfma_f32_16x16x32 (16-bit), v_mfma_scale_f32_16x16x128_f8f6f4
+// (fp8), v_mfma_f32_32x32x2 (f32).  WIDE: the 32x32x16 / 32x32x64 forms of the same products instead,
+// which reach the same rate on zeros and a lower one on random operands.
+template <int DT, bool WIDE>
 __global__ void __launch_bounds__(512) mfma_rate_kernel(float* out, const u32x4* frag, int iters) {
-  u32x4 fa[4], fb[4];
+  u32x4 fa[8], fb[8];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < 8; ++i) {
     fa[i] = frag[i * 512 + threadIdx.x];
-    fb[i] = frag[(4 + i) * 512 + threadIdx.x];
+    fb[i] = frag[(8 + i) * 512 + threadIdx.x];
   }
-  f32x16 c[8];
+  if constexpr (DT == LH_F32 || WIDE) {
+    f32x16 c[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) c[i][e] = 0.0f;
-  for (int it = 0; it < iters; ++it) {
+      for (int e = 0; e < 16; ++e) c[i][e] = 0.0f;
+    for (int it = 0; it < iters; ++it) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const u32x4 b0 = fb[i + 2 * (it & 1)], a0 = fa[j];
-        if constexpr (DT == LH_BF16) {
-          c[4 * i + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, b0),
-                                                                 __builtin_bit_cast(bf16x8, a0), c[4 * i + j], 0, 0, 0);
-        } else if constexpr (DT == LH_F8E4M3) {
-          const u32x4 a1 = fa[(j + 1) & 3], b1 = fb[(i + 1 + 2 * (it & 1)) & 3];
-          i32x8 a = {(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3], (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
-          i32x8 b = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
-          c[4 * i + j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b, a, c[4 * i + j], 0, 0, 0, 0, 0, 0);
-        } else {
-          c[4 * i + j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, b0[it & 3]),
-                                                              __builtin_bit_cast(float, a0[it & 3]), c[4 * i + j], 0,
-                                                              0, 0);
+        for (int j = 0; j < 4; ++j) {
+          const u32x4 b0 = fb[i + 2 * (it & 1)], a0 = fa[j];
+          if constexpr (DT == LH_BF16) {
+            c[4 * i + j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, b0),
+                                                                   __builtin_bit_cast(bf16x8, a0), c[4 * i + j], 0, 0, 0);
+          } else if constexpr (DT == LH_F8E4M3) {
+            const u32x4 a1 = fa[(j + 1) & 3], b1 = fb[(i + 1 + 2 * (it & 1)) & 3];
+            i32x8 a = {(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3], (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
+            i32x8 b = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+            c[4 * i + j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(b, a, c[4 * i + j], 0, 0, 0, 0, 0, 0);
+          } else {
+            c[4 * i + j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, b0[it & 3]),
+                                                                __builtin_bit_cast(float, a0[it & 3]), c[4 * i + j], 0,
+                                                                0, 0);
+          }
         }
-      }
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s += c[i][e];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+  } else {
+    // 4 column fragments x 8 row fragments of 16: the same 128 x 64 sub-tile, twice the k per instruction
+    f32x4 c[4][8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) c[i][j][e] = 0.0f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const u32x4 b0 = fb[i + 4 * (it & 1)], a0 = fa[j];
+          if constexpr (DT == LH_BF16) {
+            c[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, b0),
+                                                              __builtin_bit_cast(bf16x8, a0), c[i][j], 0, 0, 0);
+          } else {
+            const u32x4 a1 = fa[(j + 1) & 7], b1 = fb[(i + 1 + 4 * (it & 1)) & 7];
+            i32x8 a = {(int)a0[0], (int)a0[1], (int)a0[2], (int)a0[3], (int)a1[0], (int)a1[1], (int)a1[2], (int)a1[3]};
+            i32x8 b = {(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3], (int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]};
+            c[i][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(b, a, c[i][j], 0, 0, 0, 0, 0, 0);
+          }
+        }
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s += c[i][j][e];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = s;
   }
-  float s = 0.0f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) s += c[i][e];
-  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
 }
 
 }  // namespace lh
@@ -65,13 +104,16 @@ using namespace lh;
   } while (0)
 
 // Returns 0, -1 (bad arguments) or -3 (HIP runtime failure).
+// random_operands: 0 = zeros, 1 = random; bit 1 set (2, 3) = the 32x32 instruction forms of the 16-bit / fp8 products.
 extern "C" int lh_probe_mfma_rate(int32_t dtype, int32_t random_operands, int64_t iters, double* tflops) {
+  const bool wide = (random_operands & 2) != 0 || dtype == LH_F32;
+  random_operands &= 1;
   if (!(tflops && iters > 0 && iters < (1ll << 30))) return -1;
   if (!(dtype == LH_BF16 || dtype == LH_F8E4M3 || dtype == LH_F32)) return -1;
   int dev = 0, cus = 0;
   PROBE_CHECK(hipGetDevice(&dev));
   PROBE_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  const size_t nfrag = 8 * 512;
+  const size_t nfrag = 16 * 512;
   std::vector<uint32_t> host(nfrag * 4, 0u);
   if (random_operands) {
     // Values of magnitude close to 1 with random signs and mantissas (what N(0,1) inputs look like
@@ -104,9 +146,11 @@ extern "C" int lh_probe_mfma_rate(int32_t dtype, int32_t random_operands, int64_
   PROBE_CHECK(hipEventCreate(&e0));
   PROBE_CHECK(hipEventCreate(&e1));
   auto launch = [&]() {
-    if (dtype == LH_BF16) hipLaunchKernelGGL(mfma_rate_kernel<LH_BF16>, dim3(cus), dim3(512), 0, nullptr, out, frag, (int)iters);
-    else if (dtype == LH_F8E4M3) hipLaunchKernelGGL(mfma_rate_kernel<LH_F8E4M3>, dim3(cus), dim3(512), 0, nullptr, out, frag, (int)iters);
-    else hipLaunchKernelGGL(mfma_rate_kernel<LH_F32>, dim3(cus), dim3(512), 0, nullptr, out, frag, (int)iters);
+    if (dtype == LH_BF16 && wide) hipLaunchKernelGGL((mfma_rate_kernel<LH_BF16, true>), dim3(cus), dim3(512), 0, nullptr, out, frag, (int)iters);
+    else if (dtype == LH_BF16) hipLaunchKernelGGL((mfma_rate_kernel<LH_BF16, false>), dim3(cus), dim3(512), 0, nullptr, out, frag, (int)iters);
+    else if (dtype == LH_F8E4M3 && wide) hipLaunchKernelGGL((mfma_rate_kernel<LH_F8E4M3, true>), dim3(cus), dim3(512), 0, nullptr, out, frag, (int)iters);
+    else if (dtype == LH_F8E4M3) hipLaunchKernelGGL((mfma_rate_kernel<LH_F8E4M3, false>), dim3(cus), dim3(512), 0, nullptr, out, frag, (int)iters);
+    else hipLaunchKernelGGL((mfma_rate_kernel<LH_F32, true>), dim3(cus), dim3(512), 0, nullptr, out, frag, (int)iters);
   };
   launch();  // warm-up
   PROBE_CHECK(hipEventRecord(e0, nullptr));
@@ -121,7 +165,9 @@ extern "C" int lh_probe_mfma_rate(int32_t dtype, int32_t random_operands, int64_
   PROBE_CHECK(hipFree(frag));
   PROBE_CHECK(hipFree(out));
   if (rc) return rc;
-  const double flop_per_mfma = dtype == LH_BF16 ? 32768.0 : dtype == LH_F8E4M3 ? 131072.0 : 4096.0;
-  *tflops = (double)iters * 8.0 * flop_per_mfma * 8.0 * cus / ((double)ms * 1e-3) / 1e12;
+  // flop per wave and iteration: 8 (wide) or 32 instructions on the 128 x 64 sub-tile
+  const double flop_per_iter = wide ? 8.0 * (dtype == LH_BF16 ? 32768.0 : dtype == LH_F8E4M3 ? 131072.0 : 4096.0)
+                                    : 32.0 * (dtype == LH_BF16 ? 16384.0 : 65536.0);
+  *tflops = (double)iters * flop_per_iter * 8.0 * cus / ((double)ms * 1e-3) / 1e12;
   return 0;
 }
