@@ -852,9 +852,17 @@ __global__ void __launch_bounds__(512) gemm16_direct(GemmArgs g) {
     }
     if (!more) break;
     if constexpr (SPLITK) g_cur = g_nxt;
-    c = cn;
-    m0 = m1;
-    n0 = n1;
+    if constexpr (TN == 2) {
+      // The next tile's load offsets are computed again rather than carried through the epilogue in
+      // registers: the 256-wide tiles spilled them (16 bytes per lane), and a kernel that touches
+      // scratch memory at all pays for it at every dispatch (4096^3 100.5 -> 99.4 us without).
+      const int idn = select(tn, g_cur);
+      direct_place<TM, TN, EDGE, BT>(SPLITK ? g_cur : g, xcd_remap(idn, tiles1), c, m0, n0);
+    } else {
+      c = cn;
+      m0 = m1;
+      n0 = n1;
+    }
     t = tn;
   }
 }
