@@ -435,7 +435,7 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "bf16 GEMM M=N=K=4096, A,B ~ N(0,1), f32 accumulation, bf16 output, no epilogue",
-                   "kernel": "gemm16_direct<bf16> (256x256 tile, 8 waves, direct-to-LDS rings)"},
+                   "kernel": "gemm16_direct<bf16> (256x256 tile, 8 waves, v_mfma_f32_16x16x32, direct-to-LDS rings)"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_BF16_TFLOPS, "traffic": headline_traffic_bytes()},
         "cpu_baseline": cpu,
