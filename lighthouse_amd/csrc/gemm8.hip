@@ -2,7 +2,10 @@
 // out = out_dtype((Aq . Bq)_f32 * (scale_a * scale_b)).  The benchmark's quantised
 // configuration; the reference has no fp8 payload.
 //
-// Large kernel: workgroup tile 256 x 256 x 128, 8 waves, v_mfma_f32_32x32x64_f8f6f4, A and B
+// Direct kernel (M and N multiples of 256, the benchmark shape): described at gemm8_direct below;
+// v_mfma_f32_16x16x128_f8f6f4 on panels that go global -> LDS without passing through registers.
+//
+// Register-staged kernel (other row counts): workgroup tile 256 x 256 x 128, 8 waves, v_mfma_f32_32x32x64_f8f6f4, A and B
 // panels double-buffered in LDS with k contiguous; the row-major B ([K,N]) is transposed in
 // registers with byte permutes on its way into LDS.  The MFMA pairs equal (lane half,
 // register, byte) positions of its two operands, so any k order inside a 64-wide k-step is
