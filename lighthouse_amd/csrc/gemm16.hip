@@ -698,6 +698,37 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
     const bool has_c = (g.flags & LH_GEMM_ACCUMULATE_C) != 0;
     const bool gelu = (g.flags & LH_GEMM_HAS_GELU) != 0, relu = (g.flags & LH_GEMM_HAS_RELU) != 0;
     const int ch = lane % chunks, row0 = lane / chunks;
+    // The 128 x 128 tile requests its whole accumulator input up front (8 row segments per lane, all
+    // in flight at once) instead of block by block between the stores of the blocks before, which the
+    // loads cannot pass (input and output may be the same buffer): one exposed memory latency per
+    // tile instead of eight.  The larger tiles have no registers for that.
+    constexpr bool kPreloadC = TM * TN == 2;
+    constexpr int NPASS = 32 / rows_per_pass;
+    f32x4 cin[kPreloadC ? 2 * TM * NPASS : 1];
+    if constexpr (kPreloadC) {
+      if (has_c) {
+#pragma unroll
+        for (int ib = 0; ib < 2; ++ib)
+#pragma unroll
+          for (int j32 = 0; j32 < TM; ++j32)
+#pragma unroll
+            for (int t = 0; t < NPASS; ++t) {
+              const int n = n0 + wn0 + 16 * NI * ib + 4 * ch;
+              const int m = m0 + wm0 + 32 * j32 + rows_per_pass * t + row0;
+              f32x4 c4 = {0.0f, 0.0f, 0.0f, 0.0f};
+              if (!EDGE || (n < g.N && m < g.M)) {
+                const int64_t off = (int64_t)m * g.ldc + n;
+                if (out32) {
+                  c4 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.c) + off);
+                } else {
+                  const u32x2 cc = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.c) + off);
+                  c4 = f32x4{unpack_lo<DT>(cc[0]), unpack_hi<DT>(cc[0]), unpack_lo<DT>(cc[1]), unpack_hi<DT>(cc[1])};
+                }
+              }
+              cin[(ib * TM + j32) * NPASS + t] = c4;
+            }
+      }
+    }
 #pragma unroll
     for (int ib = 0; ib < 2; ++ib) {
       const int n = n0 + wn0 + 16 * NI * ib + 4 * ch;  // the lane's 4 output columns
@@ -723,7 +754,9 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
           const int64_t off = (int64_t)m * g.ldc + n;
           if (has_c) {
             f32x4 c4;
-            if (out32) {
+            if constexpr (kPreloadC) {
+              c4 = cin[(ib * TM + j32) * NPASS + t];
+            } else if (out32) {
               c4 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.c) + off);
             } else {
               const u32x2 cc = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.c) + off);
