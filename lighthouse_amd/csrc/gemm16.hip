@@ -652,33 +652,45 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
     constexpr int JB = HAS_NEXT ? 1 : TM;
     uint8_t* cw = HAS_NEXT ? stage + next.wave * (32 * RB) : ring + next.wave * (TM * 32 * RB);
     uint16_t* outp = reinterpret_cast<uint16_t*>(g.out);
+    // One variant of the bias / activation code per tile, chosen here, not per element group.
+    epi_dispatch(g, [&](auto variant) {
+      using E = decltype(variant);
+      f32x4 b4[2 * TN];
 #pragma unroll
-    for (int j0 = 0; j0 < TM; j0 += JB) {
-#pragma unroll
-      for (int jj = 0; jj < 2 * JB; ++jj)
+      for (int i = 0; i < 2 * TN; ++i) b4[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      if (epi_has_bias<E>(g)) {
 #pragma unroll
         for (int i = 0; i < 2 * TN; ++i) {
-          const int j = 2 * j0 + jj;           // 16-row fragment; staged row 16 jj + l16
           const int n = n_base + 16 * i;
-          const f32x4 b4 = (g.bias_dt == LH_F32)
-                               ? bias4<DT>(g, EDGE ? min(n, g.N - 4) : n)  // the bias row ends at N
-                               : f32x4{unpack_lo<DT>(bias[i][0]), unpack_hi<DT>(bias[i][0]), unpack_lo<DT>(bias[i][1]),
-                                       unpack_hi<DT>(bias[i][1])};
-          const u32x2 w = epilogue4_pack_bias<DT>(g, b4, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
-          const int row = 16 * jj + l16;
-          *reinterpret_cast<u32x2*>(cw + row * RB + (((2 * i + (g4 >> 1)) ^ ((row >> 1) & (chunks - 1))) << 4) +
-                                    8 * (g4 & 1)) = w;
+          b4[i] = (g.bias_dt == LH_F32)
+                      ? bias4<DT>(g, EDGE ? min(n, g.N - 4) : n)  // the bias row ends at N
+                      : f32x4{unpack_lo<DT>(bias[i][0]), unpack_hi<DT>(bias[i][0]), unpack_lo<DT>(bias[i][1]),
+                              unpack_hi<DT>(bias[i][1])};
         }
-      // Cfg::kStagedStores stores per lane in all; the main loop's first wait counts on it.
-#pragma unroll
-      for (int t = 0; t < JB * 32 / rows_per_pass; ++t) {
-        const int row = rows_per_pass * t + lane / chunks, ch = lane % chunks;
-        u32x4 w = *reinterpret_cast<const u32x4*>(cw + row * RB + ((ch ^ ((row >> 1) & (chunks - 1))) << 4));
-        const int m = m0 + wm0 + 32 * j0 + row;
-        if (!EDGE || (m < g.M && n0 + wn0 + ch * 8 < g.N))
-          *reinterpret_cast<u32x4*>(outp + (int64_t)m * g.ldc + n0 + wn0 + ch * 8) = w;
       }
-    }
+#pragma unroll
+      for (int j0 = 0; j0 < TM; j0 += JB) {
+#pragma unroll
+        for (int jj = 0; jj < 2 * JB; ++jj)
+#pragma unroll
+          for (int i = 0; i < 2 * TN; ++i) {
+            const int j = 2 * j0 + jj;           // 16-row fragment; staged row 16 jj + l16
+            const u32x2 w = epi_pack4<DT, E>(g, b4[i], acc[i][j]);
+            const int row = 16 * jj + l16;
+            *reinterpret_cast<u32x2*>(cw + row * RB + (((2 * i + (g4 >> 1)) ^ ((row >> 1) & (chunks - 1))) << 4) +
+                                      8 * (g4 & 1)) = w;
+          }
+        // Cfg::kStagedStores stores per lane in all; the main loop's first wait counts on it.
+#pragma unroll
+        for (int t = 0; t < JB * 32 / rows_per_pass; ++t) {
+          const int row = rows_per_pass * t + lane / chunks, ch = lane % chunks;
+          u32x4 w = *reinterpret_cast<const u32x4*>(cw + row * RB + ((ch ^ ((row >> 1) & (chunks - 1))) << 4));
+          const int m = m0 + wm0 + 32 * j0 + row;
+          if (!EDGE || (m < g.M && n0 + wn0 + ch * 8 < g.N))
+            *reinterpret_cast<u32x4*>(outp + (int64_t)m * g.ldc + n0 + wn0 + ch * 8) = w;
+        }
+      }
+    });
     return;
   }
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -694,19 +706,29 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
     constexpr int chunks = RB / 16;
     constexpr int rows_per_pass = 64 / chunks;
     uint8_t* cw = stage + next.wave * (32 * RB);
-    const bool out32 = g.out_dt == LH_F32;
-    const bool has_c = (g.flags & LH_GEMM_ACCUMULATE_C) != 0;
-    const bool gelu = (g.flags & LH_GEMM_HAS_GELU) != 0, relu = (g.flags & LH_GEMM_HAS_RELU) != 0;
     const int ch = lane % chunks, row0 = lane / chunks;
-    // The 128 x 128 tile requests its whole accumulator input up front (8 row segments per lane, all
-    // in flight at once) instead of block by block between the stores of the blocks before, which the
-    // loads cannot pass (input and output may be the same buffer): one exposed memory latency per
-    // tile instead of eight.  The larger tiles have no registers for that.
-    constexpr bool kPreloadC = TM * TN == 2;
-    constexpr int NPASS = 32 / rows_per_pass;
-    f32x4 cin[kPreloadC ? 2 * TM * NPASS : 1];
-    if constexpr (kPreloadC) {
-      if (has_c) {
+    // The output type, the accumulator input and the bias / activation variant are fixed per tile:
+    // out32 / has_c as compile-time booleans, the variant from epi_dispatch_linear (an activation
+    // takes the variant that tests the flags).
+    auto body = [&](auto variant, auto out32_c, auto has_c_c) {
+      using E = decltype(variant);
+      constexpr bool out32 = decltype(out32_c)::value, has_c = decltype(has_c_c)::value;
+      // The 128 x 128 tile requests its whole accumulator input up front (8 row segments per lane, all
+      // in flight at once) instead of block by block between the stores of the blocks before, which the
+      // loads cannot pass (input and output may be the same buffer): one exposed memory latency per
+      // tile instead of eight.  The larger tiles have no registers for that.
+      constexpr bool kPreloadC = TM * TN == 2 && has_c;
+      constexpr int NPASS = 32 / rows_per_pass;
+      auto load_c = [&](int64_t off) -> f32x4 {
+        if constexpr (out32) {
+          return *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.c) + off);
+        } else {
+          const u32x2 cc = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.c) + off);
+          return f32x4{unpack_lo<DT>(cc[0]), unpack_hi<DT>(cc[0]), unpack_lo<DT>(cc[1]), unpack_hi<DT>(cc[1])};
+        }
+      };
+      f32x4 cin[kPreloadC ? 2 * TM * NPASS : 1];
+      if constexpr (kPreloadC) {
 #pragma unroll
         for (int ib = 0; ib < 2; ++ib)
 #pragma unroll
@@ -716,75 +738,75 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
               const int n = n0 + wn0 + 16 * NI * ib + 4 * ch;
               const int m = m0 + wm0 + 32 * j32 + rows_per_pass * t + row0;
               f32x4 c4 = {0.0f, 0.0f, 0.0f, 0.0f};
-              if (!EDGE || (n < g.N && m < g.M)) {
-                const int64_t off = (int64_t)m * g.ldc + n;
-                if (out32) {
-                  c4 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.c) + off);
-                } else {
-                  const u32x2 cc = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.c) + off);
-                  c4 = f32x4{unpack_lo<DT>(cc[0]), unpack_hi<DT>(cc[0]), unpack_lo<DT>(cc[1]), unpack_hi<DT>(cc[1])};
-                }
-              }
+              if (!EDGE || (n < g.N && m < g.M)) c4 = load_c((int64_t)m * g.ldc + n);
               cin[(ib * TM + j32) * NPASS + t] = c4;
             }
       }
-    }
 #pragma unroll
-    for (int ib = 0; ib < 2; ++ib) {
-      const int n = n0 + wn0 + 16 * NI * ib + 4 * ch;  // the lane's 4 output columns
-      const bool n_ok = !EDGE || n < g.N;
-      const f32x4 b4 = bias4<DT>(g, EDGE ? min(n, g.N - 4) : n);
+      for (int ib = 0; ib < 2; ++ib) {
+        const int n = n0 + wn0 + 16 * NI * ib + 4 * ch;  // the lane's 4 output columns
+        const bool n_ok = !EDGE || n < g.N;
+        f32x4 b4 = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (epi_has_bias<E>(g)) b4 = bias4<DT>(g, EDGE ? min(n, g.N - 4) : n);
 #pragma unroll
-      for (int j32 = 0; j32 < TM; ++j32) {
+        for (int j32 = 0; j32 < TM; ++j32) {
 #pragma unroll
-        for (int jj = 0; jj < 2; ++jj)
+          for (int jj = 0; jj < 2; ++jj)
 #pragma unroll
-          for (int ii = 0; ii < NI; ++ii) {
-            const f32x4& a4 = acc[NI * ib + ii][2 * j32 + jj];
-            const f32x4 w = {a4[0] * g.alpha, a4[1] * g.alpha, a4[2] * g.alpha, a4[3] * g.alpha};
-            const int row = 16 * jj + l16;
-            *reinterpret_cast<f32x4*>(cw + row * RB + (((4 * ii + g4) ^ ((row >> 1) & (chunks - 1))) << 4)) = w;
-          }
-#pragma unroll
-        for (int t = 0; t < 32 / rows_per_pass; ++t) {
-          const int row = rows_per_pass * t + row0;
-          f32x4 v = *reinterpret_cast<const f32x4*>(cw + row * RB + ((ch ^ ((row >> 1) & (chunks - 1))) << 4));
-          const int m = m0 + wm0 + 32 * j32 + row;
-          if (EDGE && !(n_ok && m < g.M)) continue;
-          const int64_t off = (int64_t)m * g.ldc + n;
-          if (has_c) {
-            f32x4 c4;
-            if constexpr (kPreloadC) {
-              c4 = cin[(ib * TM + j32) * NPASS + t];
-            } else if (out32) {
-              c4 = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.c) + off);
-            } else {
-              const u32x2 cc = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.c) + off);
-              c4 = f32x4{unpack_lo<DT>(cc[0]), unpack_hi<DT>(cc[0]), unpack_lo<DT>(cc[1]), unpack_hi<DT>(cc[1])};
+            for (int ii = 0; ii < NI; ++ii) {
+              const f32x4& a4 = acc[NI * ib + ii][2 * j32 + jj];
+              f32x4 w = a4;
+              if constexpr (E::kAlpha) w = f32x4{a4[0] * g.alpha, a4[1] * g.alpha, a4[2] * g.alpha, a4[3] * g.alpha};
+              const int row = 16 * jj + l16;
+              *reinterpret_cast<f32x4*>(cw + row * RB + (((4 * ii + g4) ^ ((row >> 1) & (chunks - 1))) << 4)) = w;
             }
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] += c4[e];
-          }
-          if (g.flags & LH_GEMM_HAS_BIAS) {
+          for (int t = 0; t < 32 / rows_per_pass; ++t) {
+            const int row = rows_per_pass * t + row0;
+            f32x4 v = *reinterpret_cast<const f32x4*>(cw + row * RB + ((ch ^ ((row >> 1) & (chunks - 1))) << 4));
+            const int m = m0 + wm0 + 32 * j32 + row;
+            if (EDGE && !(n_ok && m < g.M)) continue;
+            const int64_t off = (int64_t)m * g.ldc + n;
+            if constexpr (has_c) {
+              f32x4 c4;
+              if constexpr (kPreloadC) c4 = cin[(ib * TM + j32) * NPASS + t];
+              else c4 = load_c(off);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] += b4[e];
-          }
-          if (gelu) {
+              for (int e = 0; e < 4; ++e) v[e] += c4[e];
+            }
+            if constexpr (E::kAny) {
+              if (g.flags & LH_GEMM_HAS_BIAS) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
-          }
-          if (relu) {
+                for (int e = 0; e < 4; ++e) v[e] += b4[e];
+              }
+              if (g.flags & LH_GEMM_HAS_GELU) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
+                for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
+              }
+              if (g.flags & LH_GEMM_HAS_RELU) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
+              }
+            } else if constexpr (E::kBias) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) v[e] += b4[e];
+            }
+            if constexpr (out32)
+              *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(g.out) + off) = v;
+            else
+              *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(g.out) + off) =
+                  u32x2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
           }
-          if (out32)
-            *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(g.out) + off) = v;
-          else
-            *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(g.out) + off) =
-                u32x2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
         }
       }
-    }
+    };
+    const bool out32 = g.out_dt == LH_F32;
+    const bool has_c = (g.flags & LH_GEMM_ACCUMULATE_C) != 0;
+    epi_dispatch_linear(g, [&](auto variant) {
+      if (out32 && has_c) body(variant, std::true_type{}, std::true_type{});
+      else if (out32) body(variant, std::true_type{}, std::false_type{});
+      else body(variant, std::false_type{}, std::true_type{});  // a 16-bit output comes here only with an accumulator input
+    });
   }
 }
 

@@ -394,32 +394,50 @@ __device__ __forceinline__ void d8_finish(const GemmArgs& g, const D8Ctx& next, 
     constexpr int JB = HAS_NEXT ? 1 : TM;
     uint8_t* cw = HAS_NEXT ? stage + next.wave * (32 * RB) : ring + next.wave * (TM * 32 * RB);
     uint16_t* outp = reinterpret_cast<uint16_t*>(g.out);
+    // One variant of the scale / bias / activation code per tile (epi_dispatch), not a test of the
+    // call's flags per element group.
+    epi_dispatch(g, [&](auto variant) {
+      using E = decltype(variant);
+      f32x4 b4[4];
 #pragma unroll
-    for (int j0 = 0; j0 < TM; j0 += JB) {
+      for (int i = 0; i < 4; ++i) b4[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      if (epi_has_bias<E>(g)) {
 #pragma unroll
-      for (int jj = 0; jj < 2 * JB; ++jj)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int j = 2 * j0 + jj;
-          const u32x2 w = epilogue4_pack<LH_BF16>(g, n_base + 16 * i, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
-          const int row = 16 * jj + l16;
-          *reinterpret_cast<u32x2*>(cw + row * RB + (((2 * i + (g4 >> 1)) ^ ((row >> 1) & (chunks - 1))) << 4) +
-                                    8 * (g4 & 1)) = w;
-        }
-#pragma unroll
-      for (int t = 0; t < JB * 32 / rows_per_pass; ++t) {
-        const int row = rows_per_pass * t + lane / chunks, ch = lane % chunks;
-        u32x4 w = *reinterpret_cast<const u32x4*>(cw + row * RB + ((ch ^ ((row >> 1) & (chunks - 1))) << 4));
-        *reinterpret_cast<u32x4*>(outp + (int64_t)(m0 + wm0 + 32 * j0 + row) * g.ldc + n0 + wn0 + ch * 8) = w;
+        for (int i = 0; i < 4; ++i) b4[i] = bias4<LH_BF16>(g, n_base + 16 * i);
       }
-    }
+#pragma unroll
+      for (int j0 = 0; j0 < TM; j0 += JB) {
+#pragma unroll
+        for (int jj = 0; jj < 2 * JB; ++jj)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int j = 2 * j0 + jj;
+            const u32x2 w = epi_pack4<LH_BF16, E>(g, b4[i], acc[i][j]);
+            const int row = 16 * jj + l16;
+            *reinterpret_cast<u32x2*>(cw + row * RB + (((2 * i + (g4 >> 1)) ^ ((row >> 1) & (chunks - 1))) << 4) +
+                                      8 * (g4 & 1)) = w;
+          }
+#pragma unroll
+        for (int t = 0; t < JB * 32 / rows_per_pass; ++t) {
+          const int row = rows_per_pass * t + lane / chunks, ch = lane % chunks;
+          u32x4 w = *reinterpret_cast<const u32x4*>(cw + row * RB + ((ch ^ ((row >> 1) & (chunks - 1))) << 4));
+          *reinterpret_cast<u32x4*>(outp + (int64_t)(m0 + wm0 + 32 * j0 + row) * g.ldc + n0 + wn0 + ch * 8) = w;
+        }
+      }
+    });
     return;
   }
+  // f32 output (the blocks of a cut along K among them): no accumulator input in this kernel
+  epi_dispatch_linear(g, [&](auto variant) {
+    using E = decltype(variant);
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i) {
+      f32x4 b4 = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (epi_has_bias<E>(g)) b4 = bias4<LH_BF16>(g, n_base + 16 * i);
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
-      epilogue4<LH_BF16>(g, m_base + 16 * j, n_base + 16 * i, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+      for (int j = 0; j < 8; ++j) epi_store4<LH_BF16, E, true, false>(g, m_base + 16 * j, n_base + 16 * i, b4, acc[i][j]);
+    }
+  });
 }
 
 // Persistent workgroups, one per CU, each walking the tile list with the grid as stride (tile

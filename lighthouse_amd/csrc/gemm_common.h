@@ -117,6 +117,142 @@ __device__ __forceinline__ u32x2 epilogue4_pack(const GemmArgs& g, int n, float 
   return epilogue4_pack_bias<DT>(g, bias4<DT>(g, n), v0, v1, v2, v3);
 }
 
+// ---- epilogue variants fixed at compile time ----------------------------------------------
+// The functions above test the flags of the call for every group of 4 elements.  In a tile
+// kernel whose epilogue is unrolled over the tile that is a handful of scalar branches around a
+// few vector instructions, a hundred times over, in code that runs once per tile and is cold in
+// the instruction cache each time: the 256 x 256 bf16 tile spent 5.2 us converting and staging
+// 128 KiB of output that way, 2.5 us without the tests.  The tile kernels therefore choose ONE
+// variant per tile (epi_dispatch: a chain of wave-uniform branches at the top of the epilogue)
+// and run straight-line code specialised for it; EpiAny keeps the run-time tests for the
+// combinations that have no variant of their own.  Same operations in the same order either way
+// (a scale of exactly 1 is skipped: x * 1 == x bit for bit).
+template <bool ALPHA, bool BIAS, int ACT>  // ACT: 0 none, 1 ReLU, 2 tanh-GELU
+struct EpiFixed {
+  static constexpr bool kAny = false, kAlpha = ALPHA, kBias = BIAS;
+  static constexpr int kAct = ACT;
+};
+struct EpiAny {
+  static constexpr bool kAny = true, kAlpha = true, kBias = true;
+  static constexpr int kAct = -1;
+};
+template <typename E>
+__device__ __forceinline__ bool epi_has_bias(const GemmArgs& g) {
+  if constexpr (E::kAny) return (g.flags & LH_GEMM_HAS_BIAS) != 0;
+  else return E::kBias;
+}
+// Scale, bias and activation on 4 values, in epilogue4's order.
+template <typename E>
+__device__ __forceinline__ void epi_apply4(const GemmArgs& g, const f32x4& bias, float (&v)[4]) {
+  if constexpr (E::kAny) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] *= g.alpha;
+    if (g.flags & LH_GEMM_HAS_BIAS) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] += bias[e];
+    }
+    if (g.flags & LH_GEMM_HAS_GELU) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
+    }
+    if (g.flags & LH_GEMM_HAS_RELU) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if constexpr (E::kAlpha) v[e] *= g.alpha;
+      if constexpr (E::kBias) v[e] += bias[e];
+      if constexpr (E::kAct == 2) v[e] = gelu_tanh(v[e]);
+      if constexpr (E::kAct == 1) v[e] = relu_nan(v[e]);
+    }
+  }
+}
+// 4 accumulator values -> two packed dwords of a 16-bit output (no accumulator input).
+template <int DT, typename E>
+__device__ __forceinline__ u32x2 epi_pack4(const GemmArgs& g, const f32x4& bias, const f32x4& a) {
+  float v[4] = {a[0], a[1], a[2], a[3]};
+  epi_apply4<E>(g, bias, v);
+  return u32x2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+}
+// Calls f with the variant of the call: unscaled or scaled accumulators without bias, with a
+// bias, and (unscaled) with a bias followed by ReLU or GELU; anything else takes EpiAny.
+template <typename F>
+__device__ __forceinline__ void epi_dispatch(const GemmArgs& g, F&& f) {
+  const uint32_t k = g.flags & (LH_GEMM_HAS_BIAS | LH_GEMM_HAS_GELU | LH_GEMM_HAS_RELU);
+  if (g.alpha == 1.0f) {
+    if (k == 0) return f(EpiFixed<false, false, 0>{});
+    if (k == LH_GEMM_HAS_BIAS) return f(EpiFixed<false, true, 0>{});
+    if (k == (LH_GEMM_HAS_BIAS | LH_GEMM_HAS_RELU)) return f(EpiFixed<false, true, 1>{});
+    if (k == (LH_GEMM_HAS_BIAS | LH_GEMM_HAS_GELU)) return f(EpiFixed<false, true, 2>{});
+  } else {
+    if (k == 0) return f(EpiFixed<true, false, 0>{});
+    if (k == LH_GEMM_HAS_BIAS) return f(EpiFixed<true, true, 0>{});
+  }
+  f(EpiAny{});
+}
+// The same without the activation variants, for epilogues that also specialise on the output
+// type and the accumulator input (residual adds, f32 outputs, split-K blocks).
+template <typename F>
+__device__ __forceinline__ void epi_dispatch_linear(const GemmArgs& g, F&& f) {
+  const uint32_t k = g.flags & (LH_GEMM_HAS_BIAS | LH_GEMM_HAS_GELU | LH_GEMM_HAS_RELU);
+  if (g.alpha == 1.0f) {
+    if (k == 0) return f(EpiFixed<false, false, 0>{});
+    if (k == LH_GEMM_HAS_BIAS) return f(EpiFixed<false, true, 0>{});
+  }
+  f(EpiAny{});
+}
+// epilogue4 with the variant, the output type and the presence of an accumulator input fixed.
+template <int DT, typename E, bool OUT32, bool HAS_C>
+__device__ __forceinline__ void epi_store4(const GemmArgs& g, int m, int n, const f32x4& bias, const f32x4& a) {
+  float v[4] = {a[0], a[1], a[2], a[3]};
+  const int64_t off = (int64_t)m * g.ldc + n;
+  if constexpr (HAS_C) {
+    // (the accumulator input is added to the scaled accumulator before the bias, as in epilogue4)
+    if constexpr (E::kAlpha) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] *= g.alpha;
+    }
+    if constexpr (OUT32) {
+      const f32x4 c = *reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(g.c) + off);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] += c[e];
+    } else {
+      const u32x2 c = *reinterpret_cast<const u32x2*>(reinterpret_cast<const uint16_t*>(g.c) + off);
+      v[0] += unpack_lo<DT>(c[0]); v[1] += unpack_hi<DT>(c[0]);
+      v[2] += unpack_lo<DT>(c[1]); v[3] += unpack_hi<DT>(c[1]);
+    }
+    if constexpr (E::kAny) {
+      if (g.flags & LH_GEMM_HAS_BIAS) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += bias[e];
+      }
+      if (g.flags & LH_GEMM_HAS_GELU) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
+      }
+      if (g.flags & LH_GEMM_HAS_RELU) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if constexpr (E::kBias) v[e] += bias[e];
+        if constexpr (E::kAct == 2) v[e] = gelu_tanh(v[e]);
+        if constexpr (E::kAct == 1) v[e] = relu_nan(v[e]);
+      }
+    }
+  } else {
+    epi_apply4<E>(g, bias, v);
+  }
+  if constexpr (OUT32)
+    *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(g.out) + off) = f32x4{v[0], v[1], v[2], v[3]};
+  else
+    *reinterpret_cast<u32x2*>(reinterpret_cast<uint16_t*>(g.out) + off) = u32x2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
+}
+
 // Transposed operands (A stored [K,M], B stored [N,K]) of a problem the direct kernels would
 // otherwise take are first transposed into temporary memory (one extra pass over that
 // operand, about a tenth of a 4096^3 problem's time) instead of running the slower kernels that
