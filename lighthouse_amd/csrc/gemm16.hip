@@ -655,19 +655,16 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
     // One variant of the bias / activation code per tile, chosen here, not per element group.
     epi_dispatch(g, [&](auto variant) {
       using E = decltype(variant);
-      f32x4 b4[2 * TN];
-#pragma unroll
-      for (int i = 0; i < 2 * TN; ++i) b4[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-      if (epi_has_bias<E>(g)) {
-#pragma unroll
-        for (int i = 0; i < 2 * TN; ++i) {
-          const int n = n_base + 16 * i;
-          b4[i] = (g.bias_dt == LH_F32)
-                      ? bias4<DT>(g, EDGE ? min(n, g.N - 4) : n)  // the bias row ends at N
-                      : f32x4{unpack_lo<DT>(bias[i][0]), unpack_hi<DT>(bias[i][0]), unpack_lo<DT>(bias[i][1]),
-                              unpack_hi<DT>(bias[i][1])};
-        }
-      }
+      // The bias of fragment i's 4 columns, converted where it is used (a converted copy of all of
+      // them would be 8 TN more live registers in an epilogue that has none to spare).
+      auto bias_of = [&](int i) -> f32x4 {
+        if constexpr (!E::kAny && !E::kBias) return f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        const int n = n_base + 16 * i;
+        return (g.bias_dt == LH_F32)
+                   ? bias4<DT>(g, EDGE ? min(n, g.N - 4) : n)  // the bias row ends at N
+                   : f32x4{unpack_lo<DT>(bias[i][0]), unpack_hi<DT>(bias[i][0]), unpack_lo<DT>(bias[i][1]),
+                           unpack_hi<DT>(bias[i][1])};
+      };
 #pragma unroll
       for (int j0 = 0; j0 < TM; j0 += JB) {
 #pragma unroll
@@ -675,7 +672,7 @@ __device__ __forceinline__ void direct_finish(const GemmArgs& g, const DirectCtx
 #pragma unroll
           for (int i = 0; i < 2 * TN; ++i) {
             const int j = 2 * j0 + jj;           // 16-row fragment; staged row 16 jj + l16
-            const u32x2 w = epi_pack4<DT, E>(g, b4[i], acc[i][j]);
+            const u32x2 w = epi_pack4<DT, E>(g, bias_of(i), acc[i][j]);
             const int row = 16 * jj + l16;
             *reinterpret_cast<u32x2*>(cw + row * RB + (((2 * i + (g4 >> 1)) ^ ((row >> 1) & (chunks - 1))) << 4) +
                                       8 * (g4 & 1)) = w;

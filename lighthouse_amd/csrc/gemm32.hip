@@ -8,8 +8,6 @@
 // LDS read and issues 4 MFMAs, and reads the 4 matching B rows with 4-byte reads that are
 // contiguous across the lanes of a half wave.  As in the 16-bit kernel the B panel is the first
 // MFMA operand, so a lane's accumulator holds 4 consecutive columns of one row.
-#include <type_traits>
-
 #include "gemm_common.h"
 
 namespace lh {
@@ -248,31 +246,15 @@ __global__ void __launch_bounds__(NW * 64) gemm32_direct(GemmArgs g) {
     const int elane = lane_now();  // as in direct32_place
     const int m_base = em0 + wm0 + (elane & 31);
     const int n_base = en0 + wn0 + 4 * (elane >> 5);
-    // One variant of the scale / bias / activation code per tile (epi_dispatch) and the accumulator
-    // input as a compile-time flag, instead of tests of the call's flags for every 4 elements.
-    auto store_tile = [&](auto variant, auto has_c_c) {
-      using E = decltype(variant);
-      constexpr bool has_c = decltype(has_c_c)::value;
 #pragma unroll
-      for (int i = 0; i < TN; ++i)
+    for (int i = 0; i < TN; ++i)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = n_base + 32 * i + 8 * q;
-          if (EDGE && n >= g.N) continue;
-          f32x4 b4 = {0.0f, 0.0f, 0.0f, 0.0f};
-          if (epi_has_bias<E>(g)) b4 = bias4<LH_F32>(g, n);
+      for (int j = 0; j < WTM; ++j)
 #pragma unroll
-          for (int j = 0; j < WTM; ++j)
-            if (!EDGE || m_base + 32 * j < g.M)
-              epi_store4<LH_F32, E, true, has_c>(g, m_base + 32 * j, n, b4,
-                                                 f32x4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
-                                                       acc[i][j][4 * q + 3]});
-        }
-    };
-    if (g.flags & LH_GEMM_ACCUMULATE_C)
-      epi_dispatch_linear(g, [&](auto variant) { store_tile(variant, std::true_type{}); });
-    else
-      epi_dispatch(g, [&](auto variant) { store_tile(variant, std::false_type{}); });
+        for (int q = 0; q < 4; ++q)
+          if (!EDGE || (m_base + 32 * j < g.M && n_base + 32 * i + 8 * q < g.N))
+            epilogue4<LH_F32>(g, m_base + 32 * j, n_base + 32 * i + 8 * q, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                              acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
     if (!more) break;
     t = tn;
   }

@@ -176,8 +176,9 @@ __device__ __forceinline__ u32x2 epi_pack4(const GemmArgs& g, const f32x4& bias,
   epi_apply4<E>(g, bias, v);
   return u32x2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
 }
-// Calls f with the variant of the call: unscaled or scaled accumulators without bias, with a
-// bias, and (unscaled) with a bias followed by ReLU or GELU; anything else takes EpiAny.
+// Calls f with the variant of the call: unscaled accumulators without a bias, with a bias, with a
+// bias followed by ReLU or GELU, scaled accumulators without a bias (the fp8 payload); anything
+// else takes EpiAny.
 template <typename F>
 __device__ __forceinline__ void epi_dispatch(const GemmArgs& g, F&& f) {
   const uint32_t k = g.flags & (LH_GEMM_HAS_BIAS | LH_GEMM_HAS_GELU | LH_GEMM_HAS_RELU);
@@ -186,9 +187,8 @@ __device__ __forceinline__ void epi_dispatch(const GemmArgs& g, F&& f) {
     if (k == LH_GEMM_HAS_BIAS) return f(EpiFixed<false, true, 0>{});
     if (k == (LH_GEMM_HAS_BIAS | LH_GEMM_HAS_RELU)) return f(EpiFixed<false, true, 1>{});
     if (k == (LH_GEMM_HAS_BIAS | LH_GEMM_HAS_GELU)) return f(EpiFixed<false, true, 2>{});
-  } else {
-    if (k == 0) return f(EpiFixed<true, false, 0>{});
-    if (k == LH_GEMM_HAS_BIAS) return f(EpiFixed<true, true, 0>{});
+  } else if (k == 0) {
+    return f(EpiFixed<true, false, 0>{});
   }
   f(EpiAny{});
 }
