@@ -31,12 +31,15 @@ TRAFFIC_FILE = ROOT / "profiles" / "gemm16_direct_bf16_4096_traffic.json"
 PREWARM_SECONDS = 0.25
 
 
-def headline_traffic_bytes():
+def headline_traffic():
+    """(HBM bytes per launch of the headline kernel, the commit the counters were read on), or
+    (None, None) without the tracked summary."""
     try:
         with open(TRAFFIC_FILE) as f:
-            return float(json.load(f)["traffic_bytes"])
+            d = json.load(f)
+        return float(d["traffic_bytes"]), str(d["measured_on_commit"])
     except (OSError, KeyError, ValueError):
-        return None
+        return None, None
 
 
 def time_region(fn, steps, warmup):
@@ -75,9 +78,9 @@ def prewarm(fn, seconds=PREWARM_SECONDS, chunk=50):
 def _cpu_lib():
     lib_path = ROOT / "oracle" / "_build" / "libcpu_ref.so"
     if not lib_path.is_file():
-        from lighthouse_amd import build as lh_build
+        from oracle import build as oracle_build
 
-        lh_build.build_oracle()
+        oracle_build.build()
     return ctypes.CDLL(str(lib_path))
 
 
@@ -254,6 +257,125 @@ def compiled_block_step(torch, gen, B, T, C, H):
     return step
 
 
+def headline_operands(torch, n=4096):
+    g = torch.Generator(device="cuda").manual_seed(0xC0FFEE + 2)
+    a = torch.randn(n, n, device="cuda", generator=g).to(torch.bfloat16)
+    b = torch.randn(n, n, device="cuda", generator=g).to(torch.bfloat16)
+    bias = torch.randn(n, device="cuda", generator=g).to(torch.bfloat16)
+    out = torch.empty(n, n, device="cuda", dtype=torch.bfloat16)
+    return a, b, bias, out, g
+
+
+def quantize_e4m3(torch, x):
+    """Per-tensor quantisation of the benchmark's fp8 configuration: scale = amax / 448, codes =
+    e4m3(x / scale), round to nearest even.  -> (codes, scale)"""
+    scale = float(x.abs().max().item()) / 448.0
+    return (x / scale).to(torch.float8_e4m3fn), scale
+
+
+def fp8_operands(torch, g, n8=8192):
+    a8, sa = quantize_e4m3(torch, torch.randn(n8, n8, device="cuda", generator=g))
+    b8, sb = quantize_e4m3(torch, torch.randn(n8, n8, device="cuda", generator=g))
+    return a8, sa, b8, sb
+
+
+# `--only NAME`: one workload of the benchmark line, launched --steps times with nothing else in the
+# process, for rocprofv3 (`rocprofv3 ... -- python3 bench.py --only NAME --steps K`).  Each entry
+# builds its operands and returns the step.
+def _only_copy(torch, ops):
+    # Calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain copy of 256 MiB
+    # (lh_hip_cast f32 -> f32 reads and writes every byte exactly once).
+    src = torch.ones(64 * 1024 * 1024, device="cuda")
+    dst = torch.empty_like(src)
+    return lambda: ops.cast(src, torch.float32, out=dst)
+
+
+def _only_attention(torch, ops):
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q, k, v = (torch.randn((4, 16, 2048, 64), device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
+    o = torch.empty_like(q)
+
+    def step():
+        ops.attention(q, k, v, out=o)
+        ops.attention(q, k, v, causal=True, out=o)
+
+    return step
+
+
+def _only_block_bf16(torch, ops):
+    return block_step(torch, torch.Generator(device="cuda").manual_seed(4), torch.bfloat16)
+
+
+def _only_gemm_bf16(torch, ops):
+    a, b, _, out, _ = headline_operands(torch)
+    return lambda: ops.gemm(a, b, out=out)
+
+
+def _only_gemm_bf16_qkv(torch, ops):
+    # the nanoGPT block's first GEMM: M = 8192, N = 2304, K = 768 with a bias (the 128 x 128 tile)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = torch.randn(8192, 768, device="cuda", generator=g).to(torch.bfloat16)
+    b = (torch.randn(768, 2304, device="cuda", generator=g) * 0.02).to(torch.bfloat16)
+    bias = torch.zeros(2304, device="cuda", dtype=torch.bfloat16)
+    out = torch.empty(8192, 2304, device="cuda", dtype=torch.bfloat16)
+    return lambda: ops.gemm(a, b, bias, out=out)
+
+
+def _only_gemm_fp8(torch, ops):
+    a8, sa, b8, sb = fp8_operands(torch, torch.Generator(device="cuda").manual_seed(6))
+    o8 = torch.empty(8192, 8192, device="cuda", dtype=torch.bfloat16)
+    return lambda: ops.gemm_fp8(a8, b8, sa, sb, out=o8)
+
+
+def _only_gemm_fp8_decode(torch, ops):
+    a8, sa, b8, sb = fp8_operands(torch, torch.Generator(device="cuda").manual_seed(6))
+    a8d = a8[:16].contiguous()
+    o8d = torch.empty(16, 8192, device="cuda", dtype=torch.bfloat16)
+    rot = Rotation(lambda: b8.clone(), 8192 * 8192)  # more B matrices than the memory-side cache holds
+    return lambda: ops.gemm_fp8(a8d, rot.next(), sa, sb, out=o8d)
+
+
+def _only_gemm_f32(torch, ops):
+    g = torch.Generator(device="cuda").manual_seed(7)
+    a32 = torch.rand(1024, 1024, device="cuda", generator=g) * 2 - 1
+    b32 = torch.rand(1024, 1024, device="cuda", generator=g) * 2 - 1
+    bias32 = torch.rand(1024, device="cuda", generator=g) * 2 - 1
+    o32 = torch.empty(1024, 1024, device="cuda")
+    return lambda: ops.gemm(a32, b32, bias32, relu=True, out=o32)
+
+
+def _only_layer_norm(torch, ops):
+    M, C = 8192, 768
+    x = torch.randn(M, C, device="cuda", generator=torch.Generator(device="cuda").manual_seed(8))
+    gam, bet = torch.ones(C, device="cuda"), torch.zeros(C, device="cuda")
+    rot = Rotation(lambda: (x.clone(), torch.empty_like(x)), 2 * M * C * 4)
+
+    def step():
+        xi, yi = rot.next()
+        ops.layer_norm(xi, gam, bet, out=yi)
+
+    return step
+
+
+def _only_gelu(torch, ops):
+    M, C = 8192, 3072
+    h = torch.randn(M, C, device="cuda", generator=torch.Generator(device="cuda").manual_seed(9))
+    rot = Rotation(lambda: (h.clone(), torch.empty_like(h)), 2 * M * C * 4)
+
+    def step():
+        hi, oi = rot.next()
+        ops.gelu_tanh(hi, out=oi)
+
+    return step
+
+
+ONLY_WORKLOADS = {
+    "copy": _only_copy, "attention": _only_attention, "block_bf16": _only_block_bf16, "gemm_bf16": _only_gemm_bf16,
+    "gemm_bf16_qkv": _only_gemm_bf16_qkv, "gemm_fp8": _only_gemm_fp8, "gemm_fp8_decode": _only_gemm_fp8_decode,
+    "gemm_f32": _only_gemm_f32, "layer_norm": _only_layer_norm, "gelu": _only_gelu,
+}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -261,8 +383,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
-    ap.add_argument("--only", choices=["gemm_bf16", "attention", "copy", "block_bf16"], default=None,
-                    help="profiling aid: run just this kernel --steps times and exit (no JSON line)")
+    ap.add_argument("--only", choices=sorted(ONLY_WORKLOADS), default=None,
+                    help="profiling aid: run just this workload --steps times and exit (no JSON line)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (one MI355X per box); use --gpus 1",
@@ -274,42 +396,14 @@ def main() -> int:
     from lighthouse_amd import ops
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
-    if args.only == "copy":
-        # Calibration for the FETCH_SIZE / WRITE_SIZE counters: a plain copy of 256 MiB
-        # (lh_hip_cast f32 -> f32 reads and writes every byte exactly once).
-        src = torch.ones(64 * 1024 * 1024, device="cuda")
-        dst = torch.empty_like(src)
-        for _ in range(args.steps):
-            ops.cast(src, torch.float32, out=dst)
-        torch.cuda.synchronize()
-        return 0
-    if args.only == "attention":
-        g = torch.Generator(device="cuda").manual_seed(3)
-        q, k, v = (torch.randn((4, 16, 2048, 64), device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
-        o = torch.empty_like(q)
-        for _ in range(args.steps):
-            ops.attention(q, k, v, out=o)
-            ops.attention(q, k, v, causal=True, out=o)
-        torch.cuda.synchronize()
-        return 0
-    if args.only == "block_bf16":
-        step = block_step(torch, torch.Generator(device="cuda").manual_seed(4), torch.bfloat16)
+    if args.only is not None:
+        step = ONLY_WORKLOADS[args.only](torch, ops)
         for _ in range(args.steps):
             step()
         torch.cuda.synchronize()
         return 0
     n = 4096
-    g = torch.Generator(device="cuda").manual_seed(0xC0FFEE + 2)
-    a = torch.randn(n, n, device="cuda", generator=g).to(torch.bfloat16)
-    b = torch.randn(n, n, device="cuda", generator=g).to(torch.bfloat16)
-    bias = torch.randn(n, device="cuda", generator=g).to(torch.bfloat16)
-    out = torch.empty(n, n, device="cuda", dtype=torch.bfloat16)
-
-    if args.only == "gemm_bf16":
-        for _ in range(args.steps):
-            ops.gemm(a, b, out=out)
-        torch.cuda.synchronize()
-        return 0
+    a, b, bias, out, g = headline_operands(torch)
     flops = 2.0 * n * n * n
     headline = lambda: ops.gemm(a, b, out=out)  # noqa: E731
     prewarm_launches, prewarm_ms = prewarm(headline)
@@ -328,6 +422,12 @@ def main() -> int:
             return work * steps / e
 
         extras["gemm_bf16_4096_bias_relu_tflops"] = rate(lambda: ops.gemm(a, b, bias, relu=True, out=out), flops) / 1e12
+        # the same 4096 x 4096 output over four times the K: the kernel's steady-state rate, with the
+        # per-launch cost (entry, first loads, output stores, the gap to the next launch) a quarter as heavy
+        ak = torch.randn(n, 4 * n, device="cuda", generator=g).to(torch.bfloat16)
+        bk = torch.randn(4 * n, n, device="cuda", generator=g).to(torch.bfloat16)
+        extras["gemm_bf16_4096x4096x16384_tflops"] = rate(lambda: ops.gemm(ak, bk, out=out), 4 * flops, 50, 20) / 1e12
+        del ak, bk
         shape = (4, 16, 2048, 64)
         q, k, v = (torch.randn(shape, device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
         o = torch.empty_like(q)
@@ -340,16 +440,15 @@ def main() -> int:
         o32 = torch.empty(1024, 1024, device="cuda")
         extras["gemm_f32_1024_bias_relu_tflops"] = rate(lambda: ops.gemm(a32, b32, bias32, relu=True, out=o32), 2.0 * 1024**3) / 1e12
         n8 = 8192
-        a8 = (torch.randn(n8, n8, device="cuda", generator=g)).clamp(-4, 4).to(torch.float8_e4m3fn)
-        b8 = (torch.randn(n8, n8, device="cuda", generator=g)).clamp(-4, 4).to(torch.float8_e4m3fn)
+        a8, sa8, b8, sb8 = fp8_operands(torch, g, n8)  # seeded N(0,1) matrices, scale = amax / 448 per tensor
         o8 = torch.empty(n8, n8, device="cuda", dtype=torch.bfloat16)
-        extras["gemm_fp8_8192_tflops"] = rate(lambda: ops.gemm_fp8(a8, b8, 0.01, 0.01, out=o8), 2.0 * n8**3, 20, 5) / 1e12
+        extras["gemm_fp8_8192_tflops"] = rate(lambda: ops.gemm_fp8(a8, b8, sa8, sb8, out=o8), 2.0 * n8**3, 20, 5) / 1e12
         a8d = a8[:16].contiguous()
         o8d = torch.empty(16, n8, device="cuda", dtype=torch.bfloat16)
         dec_bytes = n8 * n8 + 16 * n8 + 16 * n8 * 2
-        extras["gemm_fp8_decode_16x8192x8192_cached_gbs"] = rate(lambda: ops.gemm_fp8(a8d, b8, 0.01, 0.01, out=o8d), dec_bytes) / 1e9
+        extras["gemm_fp8_decode_16x8192x8192_cached_gbs"] = rate(lambda: ops.gemm_fp8(a8d, b8, sa8, sb8, out=o8d), dec_bytes) / 1e9
         rot8 = Rotation(lambda: b8.clone(), n8 * n8)
-        extras["gemm_fp8_decode_16x8192x8192_gbs"] = rate(lambda: ops.gemm_fp8(a8d, rot8.next(), 0.01, 0.01, out=o8d), dec_bytes) / 1e9
+        extras["gemm_fp8_decode_16x8192x8192_gbs"] = rate(lambda: ops.gemm_fp8(a8d, rot8.next(), sa8, sb8, out=o8d), dec_bytes) / 1e9
         del a8, b8, o8, rot8
         # Beyond the named configurations: head dimension 128 and a bf16 decode shape.
         q128, k128, v128 = (torch.randn(4, 16, 2048, 128, device="cuda", generator=g).to(torch.bfloat16) for _ in range(3))
@@ -418,6 +517,7 @@ def main() -> int:
     if not args.no_cpu_baseline:
         cpu = cpu_baseline_gemm_bf16(n)
 
+    traffic, traffic_commit = headline_traffic()
     line = {
         "metric": "GEMM & flash-attn TFLOP/s, % of MI355X MFMA peak; speedup vs host-CPU lh-run",
         "value": value,
@@ -437,7 +537,7 @@ def main() -> int:
         "config": {"workload": "bf16 GEMM M=N=K=4096, A,B ~ N(0,1), f32 accumulation, bf16 output, no epilogue",
                    "kernel": "gemm16_direct<bf16> (256x256 tile, 8 waves, v_mfma_f32_16x16x32, direct-to-LDS rings)"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": headline_traffic_bytes()},
+                     "frac": achieved / PEAK_BF16_TFLOPS, "traffic": traffic, "traffic_commit": traffic_commit},
         "cpu_baseline": cpu,
         "pct_of_mfma_peak": 100.0 * value / PEAK_BF16_TFLOPS,
         "speedup_vs_cpu": (value / cpu["value"]) if cpu else None,

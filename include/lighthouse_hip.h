@@ -160,6 +160,14 @@ int lh_hip_gemm(void* out, const void* a, const void* b, const void* bias, int64
  */
 size_t lh_hip_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                                    int32_t ab_dtype, int32_t out_dtype, uint32_t flags);
+/*
+ * The same query for given operands: an operand that is not 16-byte aligned runs on a padded copy in
+ * the workspace, which this variant counts (the pointers are not dereferenced).  lh_hip_gemm_ws and
+ * lh_hip_gemm_static compute their need this way and refuse before anything is launched.
+ */
+size_t lh_hip_gemm_workspace_bytes_for(const void* out, const void* a, const void* b, const void* bias, int64_t M,
+                                       int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype,
+                                       int32_t out_dtype, uint32_t flags);
 int lh_hip_gemm_ws(void* out, const void* a, const void* b, const void* bias, int64_t M, int64_t N, int64_t K,
                    int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype, int32_t out_dtype, uint32_t flags,
                    void* workspace, size_t workspace_bytes, void* stream);
@@ -249,6 +257,21 @@ typedef struct lh_strides3 {
 int lh_hip_attention(void* out, const void* q, const void* k, const void* v, int64_t Z, int64_t H, int64_t T,
                      int64_t d, lh_strides3 so, lh_strides3 sq, lh_strides3 sk, lh_strides3 sv, float scale,
                      int32_t causal, int32_t dtype, void* stream);
+/*
+ * lh_hip_attention with its temporary memory in a caller workspace (256-byte aligned) of at least
+ * lh_hip_attention_workspace_bytes(...) bytes, for callers that cannot let the library allocate:
+ * the only temporaries of an attention call are the partial results of a key range split between
+ * workgroups, which the library chooses for 16-bit problems with few query blocks and long
+ * sequences (0 bytes for every other problem, the benchmark's among them; a call that requests
+ * LH_ATTN_KSPLIT_1, a row count or a ring depth never splits and needs none).  A workspace that is
+ * too small fails with LH_ERR_INVALID before anything is launched.  No counterpart in the
+ * reference, whose payloads receive every buffer as an argument (lighthouse/execution/runner.py:196-215).
+ */
+size_t lh_hip_attention_workspace_bytes(int64_t Z, int64_t H, int64_t T, int64_t d, lh_strides3 so, lh_strides3 sq,
+                                        lh_strides3 sk, lh_strides3 sv, int32_t causal, int32_t dtype);
+int lh_hip_attention_ws(void* out, const void* q, const void* k, const void* v, int64_t Z, int64_t H, int64_t T,
+                        int64_t d, lh_strides3 so, lh_strides3 sq, lh_strides3 sk, lh_strides3 sv, float scale,
+                        int32_t causal, int32_t dtype, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Row LayerNorm, emit_layer_norm_generics

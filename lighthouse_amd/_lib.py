@@ -132,6 +132,7 @@ PROTOTYPES = {
     "lh_hip_release_scratch": (_i32, []),
     "lh_hip_gemm": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp]),
     "lh_hip_gemm_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32]),
+    "lh_hip_gemm_workspace_bytes_for": (_sz, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32]),
     "lh_hip_gemm_ws": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp, _sz, _vp]),
     "lh_hip_gemm_static": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp]),
     "lh_hip_gemm_residual": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32, _u32, _vp]),
@@ -140,6 +141,9 @@ PROTOTYPES = {
     "lh_hip_gemm_fp8_ws": (_i32, [_vp, _vp, _vp, _f32, _f32, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _vp, _sz, _vp]),
     "lh_hip_attention": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, Strides3, Strides3, Strides3, Strides3,
                                 _f32, _i32, _i32, _vp]),
+    "lh_hip_attention_workspace_bytes": (_sz, [_i64, _i64, _i64, _i64, Strides3, Strides3, Strides3, Strides3, _i32, _i32]),
+    "lh_hip_attention_ws": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, Strides3, Strides3, Strides3, Strides3,
+                                   _f32, _i32, _i32, _vp, _sz, _vp]),
     "lh_hip_layer_norm": (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _f32, _i32, _i32, _vp]),
     "lh_hip_softmax": (_i32, [_vp, _vp, _i64, _i64, _i32, _vp]),
     "lh_hip_gelu_tanh": (_i32, [_vp, _vp, _i64, _i32, _vp]),

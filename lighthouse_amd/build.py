@@ -1,8 +1,8 @@
-"""Build liblighthouse_hip.so (gfx950) and, for the tests, the CPU checker library.
+"""Build liblighthouse_hip.so (gfx950).
 
-Usage: ``python -m lighthouse_amd.build`` or ``lighthouse_amd.build.build_all()``.
+Usage: ``python -m lighthouse_amd.build`` or ``lighthouse_amd.build.build_hip()``.
 hipcc cross-compiles for gfx950 without a GPU present.  Objects go to ``build/``,
-the libraries to ``lighthouse_amd/lib/`` and ``oracle/_build/`` (all git-ignored).
+the libraries to ``lighthouse_amd/lib/`` (all git-ignored).
 """
 
 from __future__ import annotations
@@ -18,7 +18,6 @@ CSRC = ROOT / "lighthouse_amd" / "csrc"
 LIB_DIR = ROOT / "lighthouse_amd" / "lib"
 LIB_PATH = LIB_DIR / "liblighthouse_hip.so"
 PROBE_LIB = LIB_DIR / "liblighthouse_probe.so"  # bench.py's MFMA-rate probe, not part of the product library
-ORACLE_LIB = ROOT / "oracle" / "_build" / "libcpu_ref.so"
 
 HIP_SOURCES = ["runtime.hip", "gemm16.hip", "gemm32.hip", "gemm8.hip", "attention.hip", "rowwise.hip", "api.hip"]
 
@@ -66,23 +65,5 @@ def build_hip(verbose: bool = False) -> Path:
     return LIB_PATH
 
 
-def build_oracle(verbose: bool = False) -> Path:
-    ORACLE_LIB.parent.mkdir(parents=True, exist_ok=True)
-    cmd = [
-        os.environ.get("CC", "gcc"), "-O3", "-march=x86-64-v3", "-ffp-contract=off", "-fopenmp", "-shared", "-fPIC",
-        str(ROOT / "oracle" / "cpu_ref.c"), "-o", str(ORACLE_LIB), "-lm",
-    ]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    _run(cmd)
-    return ORACLE_LIB
-
-
-def build_all(verbose: bool = False) -> None:
-    build_hip(verbose)
-    build_oracle(verbose)
-
-
 if __name__ == "__main__":
-    build_all(verbose=True)
-    print(f"built {LIB_PATH}\nbuilt {ORACLE_LIB}")
+    print(f"built {build_hip(verbose=True)}")

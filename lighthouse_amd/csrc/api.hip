@@ -55,16 +55,23 @@ int gemm_run(void* out, const void* c, const void* a, const void* b, const void*
   return gemm16(g, ab_dtype, s);
 }
 
-// Temporary bytes gemm_run would take for this problem (aligned operands assumed): the dispatch
-// code itself is run with launches and allocations switched off.
-static size_t gemm_need(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int ab_dtype,
-                        int out_dtype, int bias_dtype, uint32_t flags) {
+// Temporary bytes gemm_run would take for this problem: the dispatch code itself is run with launches
+// and allocations switched off.  The operand pointers are never dereferenced here; only their
+// alignment matters (an operand that is not 16-byte aligned runs on a padded copy, which is part
+// of the need).  The overload without pointers assumes aligned operands.
+static size_t gemm_need(const void* out, const void* a, const void* b, const void* bias, int64_t M, int64_t N, int64_t K,
+                        int64_t lda, int64_t ldb, int64_t ldc, int ab_dtype, int out_dtype, int bias_dtype,
+                        uint32_t flags) {
   PlanningScope plan;
   Scratch ws;
-  void* const fake = reinterpret_cast<void*>(uintptr_t(1) << 20);
-  const int rc = gemm_run(fake, fake, fake, fake, (flags & LH_GEMM_HAS_BIAS) ? fake : nullptr, M, N, K, lda, ldb, ldc,
-                          ab_dtype, out_dtype, bias_dtype, flags, nullptr, &ws);
+  const int rc = gemm_run(const_cast<void*>(out), out, a, b, (flags & LH_GEMM_HAS_BIAS) ? bias : nullptr, M, N, K, lda, ldb,
+                          ldc, ab_dtype, out_dtype, bias_dtype, flags, nullptr, &ws);
   return rc ? 0 : ws.need;
+}
+static size_t gemm_need(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int ab_dtype,
+                        int out_dtype, int bias_dtype, uint32_t flags) {
+  void* const fake = reinterpret_cast<void*>(uintptr_t(1) << 20);
+  return gemm_need(fake, fake, fake, fake, M, N, K, lda, ldb, ldc, ab_dtype, out_dtype, bias_dtype, flags);
 }
 
 static int gemm8_run(void* out, const void* a_q, const void* b_q, float scale_a, float scale_b, int64_t M, int64_t N,
@@ -149,6 +156,14 @@ size_t lh_hip_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int64_t lda,
   return gemm_need(M, N, K, lda, ldb, ldc, ab_dtype, out_dtype, out_dtype, flags);
 }
 
+size_t lh_hip_gemm_workspace_bytes_for(const void* out, const void* a, const void* b, const void* bias, int64_t M,
+                                       int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype,
+                                       int32_t out_dtype, uint32_t flags) {
+  if (gemm_common_checks("lh_hip_gemm_workspace_bytes_for", out, a, b, bias, M, N, K, lda, ldb, ldc, flags)) return 0;
+  if (gemm_dtype_checks("lh_hip_gemm_workspace_bytes_for", ab_dtype, out_dtype)) return 0;
+  return gemm_need(out, a, b, bias, M, N, K, lda, ldb, ldc, ab_dtype, out_dtype, out_dtype, flags);
+}
+
 int lh_hip_gemm_ws(void* out, const void* a, const void* b, const void* bias, int64_t M, int64_t N, int64_t K,
                    int64_t lda, int64_t ldb, int64_t ldc, int32_t ab_dtype, int32_t out_dtype, uint32_t flags,
                    void* workspace, size_t workspace_bytes, void* stream) {
@@ -156,6 +171,12 @@ int lh_hip_gemm_ws(void* out, const void* a, const void* b, const void* bias, in
   if (rc) return rc;
   if ((rc = gemm_dtype_checks("lh_hip_gemm_ws", ab_dtype, out_dtype))) return rc;
   if ((rc = workspace_checks("lh_hip_gemm_ws", workspace, workspace_bytes))) return rc;
+  // The need of THESE operands (their alignment included), checked before anything is launched.
+  const size_t need = gemm_need(out, a, b, bias, M, N, K, lda, ldb, ldc, ab_dtype, out_dtype, out_dtype, flags);
+  LH_REQUIRE(need <= workspace_bytes,
+             "lh_hip_gemm_ws: workspace too small: this call needs %zu bytes of temporary memory, %zu were given "
+             "(lh_hip_gemm_workspace_bytes_for gives the need of operands that are not 16-byte aligned)",
+             need, workspace_bytes);
   Scratch ws;
   // An empty workspace still must not fall back to the pool: the base stays non-null.
   ws.base = workspace ? static_cast<char*>(workspace) : reinterpret_cast<char*>(uintptr_t(256));
@@ -170,8 +191,8 @@ int lh_hip_gemm_static(void* out, const void* a, const void* b, const void* bias
   int rc = gemm_common_checks("lh_hip_gemm_static", out, a, b, bias, M, N, K, lda, ldb, ldc, flags);
   if (rc) return rc;
   if ((rc = gemm_dtype_checks("lh_hip_gemm_static", ab_dtype, out_dtype))) return rc;
-  // What the dispatch would take for aligned operands, known before anything is launched.
-  const size_t need = gemm_need(M, N, K, lda, ldb, ldc, ab_dtype, out_dtype, out_dtype, flags);
+  // What the dispatch takes for these operands (their alignment included), known before anything is launched.
+  const size_t need = gemm_need(out, a, b, bias, M, N, K, lda, ldb, ldc, ab_dtype, out_dtype, out_dtype, flags);
   LH_REQUIRE(need <= LH_STATIC_SCRATCH_BYTES,
              "lh_hip_gemm_static: this problem needs %zu bytes of temporary memory, the static scratch holds %zu "
              "(use lh_hip_gemm_ws with a workspace of that size)",

@@ -40,6 +40,7 @@ struct AttnArgs {
   int kv_groups = 1;
   float* part = nullptr;
   bool allow_grid_split = true;  // the caller lets the launch take temporary memory for it
+  Scratch* ws = nullptr;         // where that memory comes from: a caller workspace, or (nullptr) the stream's pool
 };
 
 template <int DT>
@@ -843,7 +844,7 @@ static int attention16_launch_split(const AttnArgs& a_in, int groups, hipStream_
   }
   const int nqb = (a_in.T + 128 * NQ - 1) / (128 * NQ), bhn = a_in.Z * a_in.H;
   void* part = nullptr;
-  if (int rc = scratch_take(nullptr, s, kScratchAttention, (size_t)nqb * bhn * groups * kPartFloats * sizeof(float),
+  if (int rc = scratch_take(a_in.ws, s, kScratchAttention, (size_t)nqb * bhn * groups * kPartFloats * sizeof(float),
                             "attention (key range split between workgroups)", &part))
     return rc;
   AttnArgs a = a_in;
@@ -1498,9 +1499,11 @@ int attention_launch(const AttnArgs& a, int dtype, hipStream_t s) {
 
 using namespace lh;
 
-extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const void* v, int64_t Z, int64_t H,
-                                int64_t T, int64_t d, lh_strides3 so, lh_strides3 sq, lh_strides3 sk, lh_strides3 sv,
-                                float scale, int32_t causal, int32_t dtype, void* stream) {
+// `ws`: the call's temporary memory comes from this workspace (nullptr: from the stream's pool, unless
+// a NoAttentionScratchScope forbids that).
+static int attention_run(void* out, const void* q, const void* k, const void* v, int64_t Z, int64_t H, int64_t T,
+                         int64_t d, lh_strides3 so, lh_strides3 sq, lh_strides3 sk, lh_strides3 sv, float scale,
+                         int32_t causal, int32_t dtype, void* stream, Scratch* ws) {
   LH_REQUIRE(out && q && k && v, "lh_hip_attention: null pointer");
   LH_REQUIRE(dtype == LH_BF16 || dtype == LH_F16 || dtype == LH_F32, "lh_hip_attention: unsupported dtype %d", dtype);
   LH_REQUIRE(Z > 0 && H > 0 && T > 0, "lh_hip_attention: empty problem Z=%lld H=%lld T=%lld", (long long)Z,
@@ -1528,7 +1531,8 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
   a.scale = scale;
   a.scale_log2e = scale * 1.4426950408889634f;
   a.d = (int)d;
-  a.allow_grid_split = attention_scratch_allowed();
+  a.ws = ws;
+  a.allow_grid_split = ws != nullptr || attention_scratch_allowed();
   LH_REQUIRE((causal & ~(int32_t)(LH_ATTN_CAUSAL | LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK | LH_ATTN_KSPLIT_MASK)) == 0 &&
                  (causal & LH_ATTN_ROWS_MASK) != LH_ATTN_ROWS_MASK && (causal & LH_ATTN_STAGES_MASK) != LH_ATTN_STAGES_MASK &&
                  (causal & LH_ATTN_KSPLIT_MASK) != LH_ATTN_KSPLIT_MASK,
@@ -1547,4 +1551,34 @@ extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const v
     return attention_generic_launch(a, (int)d, dtype, reinterpret_cast<hipStream_t>(stream));
   }
   return attention_launch(a, dtype, reinterpret_cast<hipStream_t>(stream));
+}
+
+extern "C" int lh_hip_attention(void* out, const void* q, const void* k, const void* v, int64_t Z, int64_t H,
+                                int64_t T, int64_t d, lh_strides3 so, lh_strides3 sq, lh_strides3 sk, lh_strides3 sv,
+                                float scale, int32_t causal, int32_t dtype, void* stream) {
+  return attention_run(out, q, k, v, Z, H, T, d, so, sq, sk, sv, scale, causal, dtype, stream, nullptr);
+}
+
+extern "C" size_t lh_hip_attention_workspace_bytes(int64_t Z, int64_t H, int64_t T, int64_t d, lh_strides3 so,
+                                                   lh_strides3 sq, lh_strides3 sk, lh_strides3 sv, int32_t causal,
+                                                   int32_t dtype) {
+  PlanningScope plan;
+  Scratch ws;
+  void* const fake = reinterpret_cast<void*>(uintptr_t(1) << 20);
+  const int rc = attention_run(fake, fake, fake, fake, Z, H, T, d, so, sq, sk, sv, 0.0f, causal, dtype, nullptr, &ws);
+  return rc ? 0 : ws.need;
+}
+
+extern "C" int lh_hip_attention_ws(void* out, const void* q, const void* k, const void* v, int64_t Z, int64_t H,
+                                   int64_t T, int64_t d, lh_strides3 so, lh_strides3 sq, lh_strides3 sk,
+                                   lh_strides3 sv, float scale, int32_t causal, int32_t dtype, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+  LH_REQUIRE(workspace != nullptr || workspace_bytes == 0, "lh_hip_attention_ws: null workspace of %zu bytes",
+             workspace_bytes);
+  LH_REQUIRE((reinterpret_cast<uintptr_t>(workspace) & 255u) == 0, "lh_hip_attention_ws: workspace must be 256-byte aligned");
+  Scratch ws;
+  // An empty workspace still must not fall back to the pool: the base stays non-null.
+  ws.base = workspace ? static_cast<char*>(workspace) : reinterpret_cast<char*>(uintptr_t(256));
+  ws.bytes = workspace_bytes;
+  return attention_run(out, q, k, v, Z, H, T, d, so, sq, sk, sv, scale, causal, dtype, stream, &ws);
 }

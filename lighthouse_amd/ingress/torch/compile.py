@@ -207,7 +207,8 @@ class _Lowering:
                 if not isinstance(r, torch.Tensor) or tuple(r.shape) != shape or r.dtype != x.dtype:
                     raise ValueError(f"{node.name}: broadcasting / mixed-type add is not supported")
                 r = _as_2d(r)
-            _check_schedule(node.name, schedule, x2.shape[0], n_out, x2.shape[1])
+            # (a Linear multiplies by its [out, in] weight transposed)
+            _check_schedule(node.name, schedule, x2.shape[0], n_out, x2.shape[1], False, True)
             out = ops.gemm(x2, wt, b.detach() if b is not None else None, relu=act == "relu", gelu=act == "gelu",
                            residual=r, transpose_b=in_place, tile=schedule.get("tile"), split_k=schedule.get("split_k"))
             return out.view(shape)
@@ -245,7 +246,7 @@ class _Lowering:
             shape = (*a.shape[:-1], b.shape[1])
             a2, ta = operand(a) if a.dim() == 2 else (_as_2d(a), False)
             b2, tb = operand(b)
-            _check_schedule(node.name, schedule, a2.shape[1] if ta else a2.shape[0], b.shape[1], b.shape[0])
+            _check_schedule(node.name, schedule, a2.shape[1] if ta else a2.shape[0], b.shape[1], b.shape[0], ta, tb)
             out = ops.gemm(a2, b2, bias.detach().contiguous() if bias is not None else None, relu=act == "relu",
                            gelu=act == "gelu", transpose_a=ta, transpose_b=tb, tile=schedule.get("tile"),
                            split_k=schedule.get("split_k"))
@@ -519,13 +520,17 @@ class JITFunction:
 
 
 
-def _check_schedule(name: str, schedule: dict, M: int, N: int, K: int) -> None:
-    """A layer's schedule parameters may state the problem they were chosen for; running them on
-    another one is an error, not a silent fallback."""
+def _check_schedule(name: str, schedule: dict, M: int, N: int, K: int, ta: bool, tb: bool) -> None:
+    """A layer's schedule parameters may state the problem they were chosen for (shape, and which
+    operands are stored transposed); running them on another one is an error, not a silent fallback."""
     want = schedule.get("mnk")
     if want is not None and tuple(want) != (M, N, K):
         raise ValueError(f"{name}: schedule parameters are for a {want[0]}x{want[1]}x{want[2]} matmul, the layer is "
                          f"{M}x{N}x{K}")
+    for key, have in (("transpose_a", ta), ("transpose_b", tb)):
+        if key in schedule and bool(schedule[key]) != bool(have):
+            raise ValueError(f"{name}: schedule parameters were chosen for {key}={bool(schedule[key])}, the layer's "
+                             f"operand is {'stored transposed' if have else 'not transposed'}")
 
 
 _SCHEDULE_KEYS = {"layer_kind", "m", "n", "k", "wg_m", "wg_n", "split_k", "transpose_a", "transpose_b", "source"}
@@ -536,6 +541,8 @@ def with_schedule_parameters(parameters: Sequence[dict]) -> Callable[[list[PlanS
     the per-layer dictionaries of the reference's ScheduleParameters
     (lighthouse/schedule/parameters.py; examples/xegpu/torch_matmul.py:219-262: layer_kind, m, n, k,
     wg_m, wg_n, ...).  This target's kernels take `wg_m` x `wg_n` (the workgroup tile) and `split_k`;
+    `m`, `n`, `k`, `transpose_a` and `transpose_b` state the problem the entry was chosen for and are
+    checked against the layer when it runs (`source` is informational);
     every other tiling key of the XeGPU schedule has no counterpart and is an error, as is a count of
     entries that differs from the graph's GEMMs."""
     parameters = [dict(p) for p in parameters]
@@ -561,6 +568,9 @@ def with_schedule_parameters(parameters: Sequence[dict]) -> Callable[[list[PlanS
                 sched["split_k"] = int(p["split_k"])
             if all(key in p for key in ("m", "n", "k")):
                 sched["mnk"] = (int(p["m"]), int(p["n"]), int(p["k"]))
+            for key in ("transpose_a", "transpose_b"):
+                if key in p:
+                    sched[key] = bool(p[key])
         return plan
 
     return fn_compile

@@ -173,13 +173,33 @@ def gemm(a, b, bias=None, *, out=None, out_dtype=None, relu=False, gelu=False, a
 
 
 def gemm_workspace_bytes(M, N, K, dtype, out_dtype=None, *, lda=None, ldb=None, ldc=None, bias=False, relu=False,
-                         accumulate_c=False, transpose_a=False, transpose_b=False) -> int:
-    """Bytes of temporary memory `gemm(..., workspace=...)` needs for this problem (0 for most)."""
+                         gelu=False, accumulate_c=False, transpose_a=False, transpose_b=False, tile=None, split_k=None,
+                         operands=None) -> int:
+    """Bytes of temporary memory `gemm(..., workspace=...)` needs for this problem (0 for most).
+    `tile` and `split_k` are the requests of the `gemm` call the workspace is for (a requested cut
+    along K needs its f32 blocks whatever the library would have chosen itself).  The plain query
+    assumes 16-byte aligned operands; `operands=(out, a, b, bias_or_None)` asks for those tensors,
+    whose alignment then counts (an unaligned operand runs on a padded copy in the workspace)."""
     flags = ((_lib.GEMM_HAS_BIAS if bias else 0) | (_lib.GEMM_HAS_RELU if relu else 0)
-             | (_lib.GEMM_ACCUMULATE_C if accumulate_c else 0)
+             | (_lib.GEMM_HAS_GELU if gelu else 0) | (_lib.GEMM_ACCUMULATE_C if accumulate_c else 0)
              | (_lib.GEMM_TRANSPOSE_A if transpose_a else 0) | (_lib.GEMM_TRANSPOSE_B if transpose_b else 0))
+    if tile is not None:
+        if tuple(tile) not in _lib.GEMM_TILES:
+            raise ValueError(f"unsupported tile {tile}")
+        flags |= _lib.GEMM_TILES[tuple(tile)]
+    if split_k is not None:
+        if split_k not in _lib.GEMM_SPLITK:
+            raise ValueError(f"unsupported split_k {split_k}; choose from {sorted(_lib.GEMM_SPLITK)}")
+        flags |= _lib.GEMM_SPLITK[split_k]
     lda = lda or (M if transpose_a else K)
     ldb = ldb or (K if transpose_b else N)
+    if operands is not None:
+        out, a, b, bias_t = operands
+        if (bias_t is not None) != bool(bias):
+            raise ValueError("operands and the bias flag disagree")
+        return int(_lib.load().lh_hip_gemm_workspace_bytes_for(
+            out.data_ptr(), a.data_ptr(), b.data_ptr(), bias_t.data_ptr() if bias_t is not None else None, M, N, K,
+            a.stride(0), b.stride(0), out.stride(0), lh_dtype(dtype), lh_dtype(out_dtype or dtype), flags))
     return int(_lib.load().lh_hip_gemm_workspace_bytes(M, N, K, lda, ldb, ldc or N, lh_dtype(dtype),
                                                        lh_dtype(out_dtype or dtype), flags))
 
@@ -214,20 +234,25 @@ def gemm_fp8(a_q, b_q, scale_a: float, scale_b: float, *, out=None, out_dtype=to
     return out
 
 
-def gemm_fp8_workspace_bytes(M, N, K, out_dtype=torch.bfloat16) -> int:
-    return int(_lib.load().lh_hip_gemm_fp8_workspace_bytes(M, N, K, K, N, N, lh_dtype(out_dtype)))
+def gemm_fp8_workspace_bytes(M, N, K, out_dtype=torch.bfloat16, *, lda=None, ldb=None, ldc=None) -> int:
+    """Bytes of temporary memory `gemm_fp8(..., workspace=...)` needs; the row strides default to
+    those of contiguous operands."""
+    return int(_lib.load().lh_hip_gemm_fp8_workspace_bytes(M, N, K, lda or K, ldb or N, ldc or N, lh_dtype(out_dtype)))
 
 
 def _strides3(t) -> _lib.Strides3:
     return _lib.Strides3(t.stride(0), t.stride(1), t.stride(2))
 
 
-def attention(q, k, v, *, causal=False, scale=None, out=None, rows_per_wave=None, stages=None, kv_split=None):
+def attention(q, k, v, *, causal=False, scale=None, out=None, rows_per_wave=None, stages=None, kv_split=None,
+              workspace=None):
     """Fused attention forward on [Z,H,T,d] tensors (any strides with unit stride along d).
     `rows_per_wave` (32 or 64), `stages` (3 or 4, K/V ring of the 32-row kernel) and `kv_split`
     (2: two wave groups per workgroup on halves of the key range, 1: never) request a
     kernel variant for 16-bit tensors with head dimension 64; with none given the
-    tuned-parameter database is asked, then the library chooses by shape."""
+    tuned-parameter database is asked, then the library chooses by shape.
+    `workspace` (uint8, see attention_workspace_bytes) makes the call take its temporary memory
+    from there instead of the library's pool (lh_hip_attention_ws)."""
     if q.dim() != 4 or q.shape != k.shape or q.shape != v.shape:
         raise ValueError("attention expects Q, K, V of equal 4-D shape [Z,H,T,d]")
     _require(q.dtype in _FLOATS and k.dtype == q.dtype and v.dtype == q.dtype,
@@ -252,12 +277,33 @@ def attention(q, k, v, *, causal=False, scale=None, out=None, rows_per_wave=None
              f"kv_split one of {sorted(_lib.ATTN_KSPLIT)[1:]}")
     word = ((_lib.ATTN_CAUSAL if causal else 0) | _lib.ATTN_ROWS[rows_per_wave or 0] | _lib.ATTN_STAGES[stages or 0]
             | _lib.ATTN_KSPLIT[kv_split or 0])
+    if workspace is not None:
+        _require(workspace.dtype == torch.uint8 and workspace.dim() == 1 and workspace.is_contiguous(),
+                 "workspace must be a contiguous uint8 vector")
+        _need_cuda(workspace)
+        _lib.check(_lib.load().lh_hip_attention_ws(
+            out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), Z, H, T, d,
+            _strides3(out), _strides3(q), _strides3(k), _strides3(v),
+            float(scale) if scale is not None else 1.0 / math.sqrt(d), word, lh_dtype(q.dtype),
+            workspace.data_ptr() if workspace.numel() else None, workspace.numel(), _stream()), "attention")
+        return out
     _lib.check(_lib.load().lh_hip_attention(
         out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), Z, H, T, d,
         _strides3(out), _strides3(q), _strides3(k), _strides3(v),
         float(scale) if scale is not None else 1.0 / math.sqrt(d), word, lh_dtype(q.dtype), _stream()),
         "attention")
     return out
+
+
+def attention_workspace_bytes(Z, H, T, d, dtype, *, causal=False, rows_per_wave=None, stages=None, kv_split=None) -> int:
+    """Bytes of temporary memory `attention(..., workspace=...)` needs for contiguous [Z,H,T,d]
+    tensors: the partial results of a key range split between workgroups, which the library
+    chooses for 16-bit problems with few query blocks and long sequences; 0 for everything else
+    and for every call that requests a kernel variant."""
+    word = ((_lib.ATTN_CAUSAL if causal else 0) | _lib.ATTN_ROWS[rows_per_wave or 0] | _lib.ATTN_STAGES[stages or 0]
+            | _lib.ATTN_KSPLIT[kv_split or 0])
+    st = _lib.Strides3(H * T * d, T * d, d)
+    return int(_lib.load().lh_hip_attention_workspace_bytes(Z, H, T, d, st, st, st, st, word, lh_dtype(dtype)))
 
 
 def layer_norm(x, gamma, beta, eps=1e-5, *, out=None, out_dtype=None):

@@ -9,7 +9,7 @@ ingress) and the `kernel:` stage of a descriptor understand."""
 from __future__ import annotations
 
 from ..tuning.tile_db import DEFAULT_DB_PATH, TileDB
-from ..tuning.tune_gemm import prefilter
+from ..tuning.tune_gemm import candidate_splits, prefilter
 from .parameters import ScheduleParameters
 
 
@@ -22,7 +22,10 @@ class HipParameterSelector:
                             **kwargs) -> dict:
         """{"layer_kind": "matmul", "m", "n", "k", then "wg_m" + "wg_n" or "split_k", "source"}.
         A database entry wins (untransposed operands only: tuned entries assume them); otherwise the
-        cost model's cheapest tile; a shape no tile of the direct kernels takes is an error."""
+        cost model's cheapest tile; a shape no tile of the direct kernels takes is an error.  A tile
+        request switches the library's own cut along K off, so for a shape the library may cut (too
+        few tiles for the compute units, a long K) the cost model names no tile and the library
+        chooses ("source": "library")."""
         m, n, k = (int(x) for x in shape)
         dtype = kwargs.get("dtype", self.dtype)
         params = {"layer_kind": "matmul", "m": m, "n": n, "k": k, "transpose_a": bool(transpose_a),
@@ -34,8 +37,12 @@ class HipParameterSelector:
             candidates = prefilter(m, n, k, dtype=dtype)
             if not candidates:
                 raise ValueError(f"Cost model did not return any valid configurations for matmul {(m, n, k)}.")
-            tile = candidates[0]
-            params["source"] = "cost model"
+            if dtype != "f32" and candidate_splits(m, n, k):
+                tile = None
+                params["source"] = "library"
+            else:
+                tile = candidates[0]
+                params["source"] = "cost model"
         if tile is not None:
             params["wg_m"], params["wg_n"] = int(tile[0]), int(tile[1])
         if split_k is not None:

@@ -356,15 +356,19 @@ def test_gemm_bf16_4096_properties():
     # (|err| <= 2^-7 |ref| + 0.02).  An element is ~N(0, 64^2) here, a lost 16-wide k-slice ~N(0, 4^2).
     for got, want in ((_host(out[rows][:, cols]), ref), (_host(out_epi[rows][:, cols]), ref_epi)):
         assert (np.abs(got - want) <= 2.0**-7 * np.abs(want) + 0.02).all()
-    # Whole sampled rows of an integer problem at the same size, exact against numpy: any wrong,
-    # missing or doubled product changes an integer.
+    # The WHOLE result of an integer problem at the same size, bit for bit: with |values| <= 3 every
+    # product and every partial sum (<= 9 * 4096) is an integer that f32, f64 and bf16-free int64 all
+    # hold exactly, so the CPU's f64 product is the only correct answer; any wrong, missing or doubled
+    # product in any tile changes an integer.  The bf16 output of the same problem must be that
+    # integer rounded once.
     ai = torch.randint(-3, 4, (n, n), device="cuda", generator=g).to(torch.bfloat16)
     bint = torch.randint(-3, 4, (n, n), device="cuda", generator=g).to(torch.bfloat16)
     exact = ops.gemm(ai, bint, out_dtype=torch.float32)
-    want = ai[rows].float().cpu().numpy().astype(np.int64) @ bint.float().cpu().numpy().astype(np.int64)
-    np.testing.assert_array_equal(_host(exact[rows]).astype(np.int64), want)
-    cols_want = ai.float().cpu().numpy().astype(np.int64) @ bint[:, cols].float().cpu().numpy().astype(np.int64)
-    np.testing.assert_array_equal(_host(exact[:, cols]).astype(np.int64), cols_want)
+    want = ai.cpu().double() @ bint.cpu().double()
+    assert torch.equal(exact.cpu().double(), want)
+    assert torch.equal(ops.gemm(ai, bint).cpu(), want.to(torch.bfloat16))
+    want_epi = torch.relu(want + bias.cpu().double()).to(torch.bfloat16)
+    assert torch.equal(ops.gemm(ai, bint, bias, relu=True).cpu(), want_epi)
     # Small-integer matrices: every partial sum is exact, so linearity must hold bit for bit.
     a1 = torch.randint(-2, 3, (n, n), device="cuda", generator=g).to(torch.bfloat16)
     a2 = torch.randint(-2, 3, (n, n), device="cuda", generator=g).to(torch.bfloat16)
@@ -426,24 +430,50 @@ def test_gemm_fp8_all_codes():
 
 
 def test_gemm_fp8_8192_properties():
-    """The benchmark's 8192^3 problem (four tiles per persistent workgroup): sampled rows against
-    the oracle, and with B the identity the output is exactly the scaled, bf16-rounded A."""
+    """The benchmark's 8192^3 problem (four tiles per persistent workgroup), quantised as the
+    benchmark states (seeded N(0,1) f32 matrices, scale = amax / 448 per tensor): sampled rows against
+    the oracle; with B the identity the output is exactly the scaled, bf16-rounded A; and the WHOLE
+    result of an integer-valued problem of the same size bit for bit."""
     from lighthouse_amd import ops
 
     n = 8192
     g = torch.Generator(device="cuda").manual_seed(13)
-    a = torch.randn(n, n, device="cuda", generator=g).clamp(-4, 4).to(torch.float8_e4m3fn)
-    b = torch.randn(n, n, device="cuda", generator=g).clamp(-4, 4).to(torch.float8_e4m3fn)
-    out = ops.gemm_fp8(a, b, 0.5, 0.25)
+
+    def quantise(x):
+        # the oracle's recipe (quantize_per_tensor_e4m3) on the device: f32 scale = amax / 448, then
+        # round to nearest even; a slab of the codes is compared with the oracle's own quantiser
+        amax = float(x.abs().max().item())
+        scale = np.float32(np.float32(amax) / np.float32(orc.E4M3_MAX))
+        q = (x / float(scale)).to(torch.float8_e4m3fn)
+        slab = slice(4000, 4064)
+        np.testing.assert_array_equal(q.view(torch.uint8)[slab].cpu().numpy(), orc.e4m3_quant(_host(x[slab]) / scale))
+        return q, float(scale)
+
+    xa = torch.randn(n, n, device="cuda", generator=g)
+    xb = torch.randn(n, n, device="cuda", generator=g)
+    a, sa = quantise(xa)
+    b, sb = quantise(xb)
+    del xa, xb
+    out = ops.gemm_fp8(a, b, sa, sb)
     rows = [0, 1, 255, 256, 4095, 4096, 8190, 8191]
     a_codes = a.view(torch.uint8)[rows].cpu().numpy()
     b_codes = b.view(torch.uint8).cpu().numpy()
-    ref = orc.matmul_fp8(a_codes, b_codes, 0.5, 0.25)
-    assert_close(_host(out[rows]), ref, FP8_RTOL, "fp8 GEMM 8192^3 (sampled rows)", report=True)
+    ref = orc.matmul_fp8(a_codes, b_codes, sa, sb)
+    assert_close(_host(out[rows]), ref, FP8_RTOL, "fp8 GEMM 8192^3, amax/448 scales (sampled rows)", report=True)
     eye = torch.eye(n, device="cuda").to(torch.float8_e4m3fn)
     out_id = ops.gemm_fp8(a, eye, 0.5, 0.25)
     expect = (a.float() * 0.125).to(torch.bfloat16)
     assert torch.equal(out_id, expect)
+    del out, out_id, expect, eye
+    # Integers -3 .. 3 are e4m3 values and every partial sum (<= 9 * 8192) is exact in f32: the CPU's
+    # f32 product is the one correct result, for all 1024 tiles of the launch.
+    ai = torch.randint(-3, 4, (n, n), device="cuda", generator=g).float()
+    bi = torch.randint(-3, 4, (n, n), device="cuda", generator=g).float()
+    got = ops.gemm_fp8(ai.to(torch.float8_e4m3fn), bi.to(torch.float8_e4m3fn), 1.0, 1.0, out_dtype=torch.float32)
+    want = ai.cpu() @ bi.cpu()
+    assert torch.equal(got.cpu(), want)
+    got16 = ops.gemm_fp8(ai.to(torch.float8_e4m3fn), bi.to(torch.float8_e4m3fn), 0.5, 0.25)
+    assert torch.equal(got16.cpu(), (want * 0.125).to(torch.bfloat16))
 
 
 @pytest.mark.parametrize("shape", [(16, 1024, 8192), (7, 384, 4096), (1, 128, 2048), (16, 2048, 384),

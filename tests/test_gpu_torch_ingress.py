@@ -226,3 +226,13 @@ def test_reference_torch_matmul_example():
     wrong = gpu_backend(with_schedule_parameters([{"m": 64, "n": 64, "k": 64, "wg_m": 128, "wg_n": 128}]))
     with pytest.raises(ValueError, match="64x64x64"):
         torch.compile(Model(), backend=wrong, dynamic=False)(a, b)
+    # parameters chosen for a transposed operand on a layer whose operand is not: refused as well;
+    # with the flags the layer has they pass (the selector writes them)
+    from lighthouse_amd.schedule import HipParameterSelector
+
+    sel = HipParameterSelector().get_parameters((m, n, k), transpose_a=False, transpose_b=False)
+    ok = gpu_backend(with_schedule_parameters(sel), device=torch.device("cuda"))
+    assert torch.equal(torch.compile(Model(), backend=ok, dynamic=False)(a, b), out)
+    tb = gpu_backend(with_schedule_parameters([{"m": m, "n": n, "k": k, "transpose_b": True}]))
+    with pytest.raises(ValueError, match="transpose_b=True"):
+        torch.compile(Model(), backend=tb, dynamic=False)(a, b)

@@ -332,6 +332,9 @@ def test_parameter_selector_database_then_cost_model(tmp_path):
     assert (miss["wg_m"], miss["wg_n"], miss["source"]) == (256, 256, "cost model")
     assert sel.get_parameters_dict((8192, 768, 768), transpose_b=True)["source"] == "cost model"
     assert sel.get_parameters_dict((1024, 1024, 1024), dtype="f32")["wg_m"] in (128, 64)
+    # a decode shape the library would cut along K: no tile request (it would switch the cut off)
+    decode = sel.get_parameters_dict((128, 8192, 8192))
+    assert decode["source"] == "library" and "wg_m" not in decode and "split_k" not in decode
     with pytest.raises(ValueError, match="did not return any valid"):
         sel.get_parameters_dict((100, 100, 100))
     layers = sel.get_parameters_for_layers([{"shape": (8192, 2304, 768)}, {"shape": (8192, 768, 3072)}])

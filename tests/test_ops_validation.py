@@ -193,7 +193,24 @@ def test_workspace_queries_run_without_a_gpu():
     assert ops.gemm_workspace_bytes(4096, 4100, 4096, bf16) >= (4096 * 4104 * 2) * 2
     assert ops.gemm_workspace_bytes(4096, 4096, 4096, bf16, transpose_a=True) == 4096 * 4096 * 2
     assert ops.gemm_workspace_bytes(1024, 1024, 1024, f32) == 0
+    # a requested cut along K needs its own blocks, whatever the library would have chosen (four here)
+    assert ops.gemm_workspace_bytes(128, 8192, 8192, bf16) == 4 * 128 * 8192 * 4
+    assert ops.gemm_workspace_bytes(128, 8192, 8192, bf16, split_k=8) == 8 * 128 * 8192 * 4
+    assert ops.gemm_workspace_bytes(128, 8192, 8192, bf16, split_k=1) == 0
+    assert ops.gemm_workspace_bytes(16, 8192, 8192, bf16, tile=(128, 128)) == 0  # a tile request switches the cut off
+    # the pointer-aware query counts the padded copy of an operand that is not 16-byte aligned
+    fake = 1 << 20
+    args = (1024, 1024, 1024, 1024, 1024, 1024, _lib.BF16, _lib.BF16, 0)
+    assert lib.lh_hip_gemm_workspace_bytes_for(fake, fake, fake, None, *args) == 0
+    assert lib.lh_hip_gemm_workspace_bytes_for(fake, fake + 2, fake, None, *args) >= 1024 * 1024 * 2
     assert ops.gemm_fp8_workspace_bytes(8192, 8192, 8192) == 0
+    # attention: only a key range split between workgroups takes temporary memory
+    assert ops.attention_workspace_bytes(4, 16, 2048, 64, bf16) == 0
+    assert ops.attention_workspace_bytes(4, 16, 2048, 64, bf16, causal=True) == 0
+    assert ops.attention_workspace_bytes(1, 1, 8192, 64, bf16) > 0
+    assert ops.attention_workspace_bytes(1, 1, 8192, 64, bf16, kv_split=1) == 0
+    assert ops.attention_workspace_bytes(1, 1, 8192, 64, f32) == 0
+    assert ops.attention_workspace_bytes(1, 1, 8192, 128, bf16) == 0
     assert ops.gemm_fp8_workspace_bytes(16, 8192, 8192) > 0
     base = ops.nanogpt_block_workspace_bytes(8, 1024, 768, bf16)
     rows = 8 * 1024

@@ -23,9 +23,9 @@ GOLDEN = json.loads((Path(__file__).parent / "golden" / "lh_run_pipeline_check.j
 def cref():
     path = ROOT / "oracle" / "_build" / "libcpu_ref.so"
     if not path.is_file():
-        from lighthouse_amd import build as lh_build
+        from oracle import build as oracle_build
 
-        lh_build.build_oracle()
+        oracle_build.build()
     return ctypes.CDLL(str(path))
 
 

@@ -93,3 +93,64 @@ def test_static_scratch_gemm_refuses_what_does_not_fit():
         _lib.check(rc, "lh_hip_gemm_static")
     # argument validation is the plain entry point's
     assert _call(lib.lh_hip_gemm_static, out, a, b, None, 0, N, K, 0) == _lib.LH_ERR_INVALID
+
+
+def test_static_scratch_gemm_with_misaligned_operands():
+    """Operands that are not 16-byte aligned run on padded copies, which the pointer-less workspace
+    query does not count; the entry points that must not allocate compute the need from the actual
+    pointers, so the call either matches lh_hip_gemm bit for bit or is refused up front with the
+    output untouched, never half way through."""
+    lib = _lib.load()
+    flags = _lib.GEMM_HAS_BIAS | _lib.GEMM_HAS_RELU
+    g = torch.Generator(device="cuda").manual_seed(5)
+
+    def shifted(rows, cols, ld):
+        # an [rows, cols] matrix with row stride ld whose first element sits 2 bytes past an aligned address
+        buf = torch.randn(rows * ld + 8, device="cuda", generator=g).to(torch.bfloat16)
+        return buf[1:1 + rows * ld].view(rows, ld)[:, :cols]
+
+    # small: the padded copies fit the array
+    M, N, K = 384, 512, 512
+    a, b = shifted(M, K, K + 8), shifted(K, N, N + 8)
+    bias = torch.randn(N, device="cuda", generator=g).to(torch.bfloat16)
+    assert a.data_ptr() % 16 == 2 and b.data_ptr() % 16 == 2
+    want = torch.full((M, N), 3.0, device="cuda", dtype=torch.bfloat16)
+    got = torch.full((M, N), 5.0, device="cuda", dtype=torch.bfloat16)
+    plain = lib.lh_hip_gemm_workspace_bytes(M, N, K, a.stride(0), b.stride(0), N, _lib.BF16, _lib.BF16, flags)
+    exact = lib.lh_hip_gemm_workspace_bytes_for(got.data_ptr(), a.data_ptr(), b.data_ptr(), bias.data_ptr(), M, N, K,
+                                                a.stride(0), b.stride(0), N, _lib.BF16, _lib.BF16, flags)
+    assert plain == 0 and 0 < exact <= STATIC_BYTES
+    _lib.check(_call(lib.lh_hip_gemm, want, a, b, bias, M, N, K, flags), "lh_hip_gemm")
+    _lib.check(_call(lib.lh_hip_gemm_static, got, a, b, bias, M, N, K, flags), "lh_hip_gemm_static")
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    ref = torch.relu(a.float() @ b.float() + bias.float())
+    assert (got.float() - ref).abs().max() <= 2e-2 * ref.abs().max()
+    # the workspace entry point with exactly that many bytes, and refused up front with one byte short of a block
+    ws = torch.empty(exact, device="cuda", dtype=torch.uint8)
+    got2 = torch.full((M, N), 5.0, device="cuda", dtype=torch.bfloat16)
+    rc = lib.lh_hip_gemm_ws(got2.data_ptr(), a.data_ptr(), b.data_ptr(), bias.data_ptr(), M, N, K, a.stride(0), b.stride(0),
+                            N, _lib.BF16, _lib.BF16, flags, ws.data_ptr(), exact, None)
+    _lib.check(rc, "lh_hip_gemm_ws")
+    torch.cuda.synchronize()
+    assert torch.equal(got2, want)
+    got2.fill_(7.0)
+    rc = lib.lh_hip_gemm_ws(got2.data_ptr(), a.data_ptr(), b.data_ptr(), bias.data_ptr(), M, N, K, a.stride(0), b.stride(0),
+                            N, _lib.BF16, _lib.BF16, flags, ws.data_ptr(), exact - 256, None)
+    assert rc == _lib.LH_ERR_INVALID and b"workspace too small" in lib.lh_hip_last_error()
+    torch.cuda.synchronize()
+    assert bool((got2 == 7.0).all())
+    # large, with a transposed and misaligned A: more than the array holds although the aligned query
+    # says otherwise; refused before the transpose kernel (or anything else) is enqueued
+    M, N, K = 4096, 2048, 2048
+    a_t, b = shifted(K, M, M + 8), shifted(K, N, N + 8)
+    out = torch.full((M, N), 9.0, device="cuda", dtype=torch.bfloat16)
+    fl = _lib.GEMM_TRANSPOSE_A
+    aligned_need = lib.lh_hip_gemm_workspace_bytes(M, N, K, a_t.stride(0), b.stride(0), N, _lib.BF16, _lib.BF16, fl)
+    exact = lib.lh_hip_gemm_workspace_bytes_for(out.data_ptr(), a_t.data_ptr(), b.data_ptr(), None, M, N, K, a_t.stride(0),
+                                                b.stride(0), N, _lib.BF16, _lib.BF16, fl)
+    assert exact > STATIC_BYTES >= 0 and exact > aligned_need
+    rc = _call(lib.lh_hip_gemm_static, out, a_t, b, None, M, N, K, fl)
+    assert rc == _lib.LH_ERR_INVALID and b"static scratch holds" in lib.lh_hip_last_error()
+    torch.cuda.synchronize()
+    assert bool((out == 9.0).all())  # nothing ran
