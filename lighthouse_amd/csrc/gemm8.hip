@@ -170,7 +170,7 @@ __global__ void __launch_bounds__(WAVES_M* WAVES_N * 64) gemm8_fast(GemmArgs g) 
 // The k-contiguous A fragment (32 bytes per lane) is two 16-byte LDS reads; the n-contiguous B
 // panel is read with ds_read_b64_tr_b8, which hands a lane 8 k-values of one column (16 lanes
 // cover 8 k-rows x 16 columns), four reads per fragment.  Swizzles: A chunk ^ ((row / 2) % 8),
-// B chunk ^ 2 (k % 8) ^ ((k / 32) % 2).
+// B chunk ^ 2 (k % 8) ^ ((k / 16) % 2).
 constexpr int kD8ABytes = 256 * 128;   // one A stage (128 k): 32 KiB
 constexpr int kD8BBytes = 64 * 256;    // one B stage (64 k): 16 KiB
 constexpr int kD8BBase = 2 * kD8ABytes;
@@ -202,7 +202,7 @@ struct D8Ctx {
   uint32_t a_voff[4];
   uint32_t b_voff[2];
   int a_rd;  // byte offset of the lane's first 16 bytes of A fragment 0 in a stage (row wm0 + lane % 16, chunk
-             // 2 (lane / 16), swizzled); its second 16 bytes are at a_rd ^ 16, fragment jj 2048 jj further on
+             // lane / 16, swizzled); its second 16 bytes (chunk + 4) are at a_rd ^ 64, fragment jj 2048 jj further on
   int64_t ldb;
   int wave, b_off, b_chunk, b_swz;
 };
@@ -231,7 +231,7 @@ __device__ __forceinline__ void d8_read_a(const D8Ctx& c, const uint8_t* __restr
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     i32x4 lo = *reinterpret_cast<const i32x4*>(as + c.a_rd + 2048 * (4 * HALF + j));
-    i32x4 hi = *reinterpret_cast<const i32x4*>(as + (c.a_rd ^ 16) + 2048 * (4 * HALF + j));
+    i32x4 hi = *reinterpret_cast<const i32x4*>(as + (c.a_rd ^ 64) + 2048 * (4 * HALF + j));
     a[j] = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
   }
 }
@@ -240,8 +240,9 @@ __device__ __forceinline__ i32x8 d8_read_b(const D8Ctx& c, const uint8_t* __rest
   const uint8_t* p0 = bs + c.b_off + (((c.b_chunk + i) ^ c.b_swz) << 4);
   i32x2 r[4];
 #pragma unroll
-  for (int q = 0; q < 4; ++q)
-    r[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) i32x2*)(p0 + q * 8 * 256));
+  for (int q = 0; q < 4; ++q)  // k rows 16 g4 + 8 (q % 2) + 64 (q / 2) + ...: the k order of the A fragment
+    r[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+        (__attribute__((address_space(3))) i32x2*)(p0 + (q & 1) * 8 * 256 + (q >> 1) * 64 * 256));
   return i32x8{r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]};
 }
 
@@ -333,7 +334,7 @@ __device__ __forceinline__ void d8_place(const GemmArgs& g, int id, D8Ctx& c, in
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int bk = (8 * i + c.wave) * 4 + (lane >> 4);
-    const int bc = (lane & 15) ^ (2 * (bk & 7)) ^ ((bk >> 5) & 1);
+    const int bc = (lane & 15) ^ (2 * (bk & 7)) ^ ((bk >> 4) & 1);
     c.b_voff[i] = (uint32_t)bk * (uint32_t)g.ldb + bc * 16;
   }
 }
@@ -472,16 +473,20 @@ __global__ void __launch_bounds__(512) gemm8_direct(GemmArgs g) {
   c.wave = wave;
   const int l16 = lane & 15, g4 = lane >> 4;
   {
-    // A fragment jj: row wm0 + 16 jj + l16, its k bytes 32 g4 .. +32 = 16-byte chunks 2 g4 and 2 g4 + 1
-    // of the row's eight, swizzled with (row / 2) % 8 (the same for every jj: wm0 and 16 jj are multiples of 16).
+    // A fragment jj: row wm0 + 16 jj + l16.  The lane's 32 k values are the 16-byte chunks g4 and g4 + 4
+    // of the row's eight (k = 16 g4 .. +16 and 64 + 16 g4 .. +16), not two neighbouring chunks: the matrix
+    // instruction only needs A and B to agree on which k a lane holds, and with the four lane groups
+    // on four neighbouring chunks a 16-byte read is free of bank conflicts (on chunks 2 g4 and 2 g4 + 1
+    // every such read took twice as long: SQ_LDS_BANK_CONFLICT 3.5e7 per 8192^3 launch against 1e6).
+    // Swizzled with (row / 2) % 8 (the same for every jj: wm0 and 16 jj are multiples of 16).
     const int r = wm0 + l16;
-    c.a_rd = r * 128 + (((2 * g4) ^ ((r >> 1) & 7)) << 4);
+    c.a_rd = r * 128 + ((g4 ^ ((r >> 1) & 7)) << 4);
   }
   {
-    // B fragment i: the 16 lanes of group g4 address k rows 32 g4 + 8 q + l16 / 2 (q = 0..3) of the
-    // stage pair, columns wn0 + 16 i + 8 (l16 % 2) .. +8; each lane receives the 8 k-values per q of
-    // column wn0 + 16 i + l16.
-    const int krow = 32 * g4 + (l16 >> 1);
+    // B fragment i: the 16 lanes of group g4 address k rows 16 g4 + 8 (q % 2) + 64 (q / 2) + l16 / 2
+    // (q = 0..3) of the stage pair, the k values of the lane's A chunks, columns
+    // wn0 + 16 i + 8 (l16 % 2) .. +8; each lane receives the 8 k-values per q of column wn0 + 16 i + l16.
+    const int krow = 16 * g4 + (l16 >> 1);
     const int col = wn0 + 8 * (l16 & 1);
     c.b_chunk = col >> 4;
     c.b_swz = (2 * (krow & 7)) ^ (g4 & 1);
