@@ -311,3 +311,54 @@ def _numel(shape) -> int:
     for d in shape:
         n *= int(d)
     return n
+
+
+# ---- payload modules by name --------------------------------------------------------------
+# The reference's command line runs whatever MLIR module it is given (lighthouse/lh_run.py:103-127);
+# for the payloads it ships no MLIR text of (attention, LayerNorm, softmax, the elementwise
+# kernels, the nanoGPT block: its examples build them with the generators above), this target's
+# command line accepts the generator call itself as the module: ``gen:KIND{key=value ...}`` with
+# the generator's own keyword names, the descriptor grammar's option syntax.
+_GENERATORS = {
+    "matmul": (generate_gpu_matmul_payload, {"M", "N", "K", "ab_type", "c_type"},
+               {"transpose_a", "transpose_b", "has_bias", "has_relu", "accumulate_c", "result_type", "has_gelu"}),
+    "attention": (generate_gpu_attention_payload, {"Z", "H", "n_ctx", "n_head", "dtype"}, {"causal"}),
+    "layer_norm": (generate_gpu_layer_norm_payload, {"M", "N", "dtype"}, {"eps", "result_type"}),
+    "softmax": (generate_gpu_softmax_payload, {"M", "N", "dtype"}, set()),
+    "elementwise": (generate_gpu_elementwise_payload, {"kind", "M", "N", "dtype"}, {"dst_dtype"}),
+    "nanogpt_block": (generate_nanogpt_block_payload, {"B", "T", "C", "n_head", "dtype"}, {"eps"}),
+}
+
+
+def is_generated_module(spec: str) -> bool:
+    return spec.startswith("gen:")
+
+
+def generate_payload_module(spec: str, func_name: str) -> PayloadModule:
+    """``gen:attention{Z=4 H=16 n_ctx=2048 n_head=64 dtype=bf16 causal}`` -> the module that
+    ``generate_gpu_attention_payload(func_name, Z=4, ...)`` builds.  Unknown kinds, unknown or
+    missing keys are errors."""
+    from ..pipeline.descriptor import Descriptor
+
+    desc = Descriptor(spec[len("gen:"):])
+    kind, params = desc.basename, {**desc.args, **desc.opts}
+    if kind not in _GENERATORS:
+        raise ValueError(f"no payload generator named '{kind}'; known: {sorted(_GENERATORS)}")
+    fn, required, optional = _GENERATORS[kind]
+    unknown = sorted(set(params) - required - optional)
+    missing = sorted(required - set(params))
+    if unknown or missing:
+        raise ValueError(f"gen:{kind}: " + "; ".join(
+            ([f"unknown key(s) {unknown}"] if unknown else []) + ([f"missing key(s) {missing}"] if missing else []))
+            + f" (it takes {sorted(required)} and optionally {sorted(optional)})")
+    return fn(func_name, **params)
+
+
+def default_input_shapes(fn: PayloadFunction) -> str:
+    """The ``--input-shape`` string for a generated function when the caller gives none: every
+    argument in order, outputs zero-filled, inputs uniform random (``rnd``), byte workspaces zero."""
+    parts = []
+    for a in fn.args:
+        init = "0" if a.writable or a.elem == "i8" else "rnd"
+        parts.append("x".join(str(d) for d in a.shape) + f"x{a.elem}x{init}")
+    return ",".join(parts)

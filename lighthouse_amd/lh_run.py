@@ -5,7 +5,11 @@ Same command line as lighthouse/lh_run.py:14-145 (``payload_module --entry-point
 [--print-optimized-module] [--print-mlir-after-all]``), same output lines (``N runs: T seconds``,
 ``Output: <array>``) and exit codes (1 on FileNotFoundError / OSError / ValueError, 130 on
 Ctrl-C).  The payload module is MLIR text of one of the matmul forms this target has a kernel for
-(see ingress/mlir_text.py).  A ``--stage`` that names a pipeline descriptor with a ``kernel:`` stage
+(see ingress/mlir_text.py), or, for the payloads the reference builds with its Python generators and
+ships no MLIR text of (attention, LayerNorm, softmax, elementwise, the nanoGPT block), the generator
+call itself: ``gen:attention{Z=4 H=16 n_ctx=2048 n_head=64 dtype=bf16 causal}`` (see
+ingress/payloads.py:generate_payload_module; ``--input-shape`` may then be left out: outputs are
+zero-filled, inputs uniform random).  A ``--stage`` that names a pipeline descriptor with a ``kernel:`` stage
 (descriptors/gfx950/<pipeline>/<dtype>.yaml) sets that kernel's request flags (every parameter of
 such a stage acts; an unknown one is an error); MLIR pass /
 transform stages have no counterpart here (the kernels are already lowered) and are skipped with a
@@ -24,7 +28,7 @@ from . import _lib
 from .execution.init import KernelArgumentParser
 from .execution.runner import Runner
 from .ingress.mlir_text import load_payload_module
-from .ingress.payloads import PayloadModule
+from .ingress.payloads import PayloadModule, default_input_shapes, generate_payload_module, is_generated_module
 from .pipeline.descriptor import Descriptor, PipelineDescriptor
 
 
@@ -121,10 +125,11 @@ def main(argv: list[str] | None = None) -> int:
         parser = argparse.ArgumentParser(
             prog="lh-run",
             description="Lighthouse runner, HIP target: runs a payload function of an MLIR module on the GPU.")
-        parser.add_argument("payload_module", type=str, help="Path to the payload MLIR module.")
+        parser.add_argument("payload_module", type=str,
+                            help="Path to the payload MLIR module, or gen:KIND{key=value ...} for a generated payload.")
         parser.add_argument("--entry-point", type=str, required=True,
                             help="Name of the entrypoint function in the payload MLIR module.")
-        parser.add_argument("--input-shape", required=True,
+        parser.add_argument("--input-shape", required=False, default=None,
                             help="Shape of the input tensors in format: DIMS(MxNx...)xTYPE(f16/f32/f64/bf16/i8)"
                                  "xINIT(0/1/rnd/id). For multiple inputs, separate by comma.")
         parser.add_argument("--seed", type=int, default=0, help="Random seed for initializing input tensors.")
@@ -142,7 +147,14 @@ def main(argv: list[str] | None = None) -> int:
 
         np.random.seed(args.seed if args.seed else int(datetime.now().timestamp()))
 
-        module = load_payload_module(args.payload_module, [args.entry_point])
+        if is_generated_module(args.payload_module):
+            module = generate_payload_module(args.payload_module, args.entry_point)
+            if args.input_shape is None:
+                args.input_shape = default_input_shapes(module.lookup(args.entry_point))
+        else:
+            module = load_payload_module(args.payload_module, [args.entry_point])
+        if args.input_shape is None:
+            raise ValueError("--input-shape is required for a module read from MLIR text")
         notes: list[str] = []
         for stage in args.stage:
             apply_stage(module, stage, notes)

@@ -453,3 +453,54 @@ module {{
     Runner(module).execute("entry", [a, b, bias, c])
     assert_close(c, orc.matmul(a, b, c=c0, bias=bias, relu=True, accumulate_c=True), 1e-4,
                  what="generic-form fixture 256x1024x2048 f32")
+
+
+def test_lh_run_cli_generated_payloads(capsys):
+    """The payloads the reference builds with its generators (no MLIR text of them exists) from the
+    command line: `gen:KIND{...}` as the module, every packaged descriptor of the kind as a stage,
+    output printed and checked against the oracle on the CLI's own seeded inputs; --benchmark prints
+    the reference's line."""
+    import re
+
+    from lighthouse_amd.execution import TargetInfo
+    from lighthouse_amd.lh_run import main
+    from lighthouse_amd.pipeline import find_pipeline_file
+
+    np.set_printoptions(threshold=10_000_000, linewidth=200, precision=8)
+    target = TargetInfo("gfx950", [])
+
+    def numbers(text):
+        return np.array([float(v) for v in re.findall(r"[-+]?(?:\d+\.\d*|\d+)(?:e[-+]?\d+)?|nan|inf", text.split("Output:", 1)[1])],
+                        dtype=np.float64)
+
+    # LayerNorm 64 x 96 f32: out, x, gamma, beta in the payload's order
+    stage = str(find_pipeline_file(target, "layer_norm", "f32"))
+    spec = "gen:layer_norm{M=64 N=96 dtype=f32}"
+    assert main([spec, "--entry-point=payload", "--stage", stage, "--seed=5", "--print-tensor=1"]) == 0
+    got = numbers(capsys.readouterr().out).reshape(64, 96)
+    np.random.seed(5)
+    _ = np.zeros((64, 96))  # (the zero-filled output draws nothing)
+    x, g, b = np.random.rand(64, 96).astype(np.float32), np.random.rand(96).astype(np.float32), np.random.rand(96).astype(np.float32)
+    assert np.allclose(got, orc.layer_norm(x, g, b), rtol=1e-4, atol=1e-5)
+    # attention [1, 2, 128, 64] f32, causal, with explicit input shapes
+    stage = str(find_pipeline_file(target, "attention", "f32"))
+    shapes = ",".join(["1x2x128x64xf32x0"] + ["1x2x128x64xf32xrnd"] * 3)
+    assert main(["gen:attention{Z=1 H=2 n_ctx=128 n_head=64 dtype=f32 causal}", "--entry-point=attn", "--stage", stage,
+                 "--input-shape", shapes, "--seed=9", "--print-tensor=1"]) == 0
+    got = numbers(capsys.readouterr().out).reshape(1, 2, 128, 64)
+    np.random.seed(9)
+    q, k, v = (np.random.rand(1, 2, 128, 64).astype(np.float32) for _ in range(3))
+    assert np.allclose(got, orc.attention(q, k, v, causal=True), rtol=1e-4, atol=1e-5)
+    # softmax, GELU and a bf16 matmul with bias + ReLU run and benchmark
+    for spec, pipeline, dt in (("gen:softmax{M=32 N=256 dtype=f32}", "softmax", "f32"),
+                               ("gen:elementwise{kind=gelu M=32 N=256 dtype=f32}", "element_wise", "f32"),
+                               ("gen:matmul{M=256 N=256 K=128 ab_type=bf16 c_type=f32 result_type=bf16 has_bias has_relu}",
+                                "matmul", "bf16"),
+                               ("gen:nanogpt_block{B=1 T=128 C=128 n_head=2 dtype=bf16}", "nanogpt_block", "bf16")):
+        stage = str(find_pipeline_file(target, pipeline, dt))
+        assert main([spec, "--entry-point=f", "--stage", stage, "--seed=3", "--benchmark"]) == 0, spec
+        assert re.match(r"100 runs: [0-9.e-]+ seconds", capsys.readouterr().out)
+    # errors: unknown kind, unknown / missing keys, and MLIR text still needs --input-shape
+    for bad in ("gen:conv{M=1}", "gen:softmax{M=32 N=256}", "gen:softmax{M=32 N=256 dtype=f32 tile=4}"):
+        assert main([bad, "--entry-point=f", "--stage=cse"]) == 1
+        assert "Error:" in capsys.readouterr().err

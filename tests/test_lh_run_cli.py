@@ -238,3 +238,26 @@ func.func @add(%a: memref<16x32xf32>, %b: memref<16x32xf32>, %out: memref<16x32x
         parse_payload_module(text.replace("16x32xf32", "16xf32"))
     with pytest.raises(ValueError, match="distinct"):
         parse_payload_module(text.replace("outs(%out", "outs(%a"))
+
+
+def test_generated_payload_modules(capsys):
+    """`gen:KIND{...}` as lh-run's module: the generator's own keyword names in the descriptor
+    grammar; default input shapes follow the payload's argument list (outputs zero, inputs random)."""
+    from lighthouse_amd.ingress.payloads import default_input_shapes, generate_payload_module, is_generated_module
+
+    assert is_generated_module("gen:softmax{M=2 N=4 dtype=f32}") and not is_generated_module("payload.mlir")
+    fn = generate_payload_module("gen:attention{Z=4 H=16 n_ctx=2048 n_head=64 dtype=bf16 causal}", "attn").lookup("attn")
+    assert fn.entry == "attention" and fn.attrs.causal == 1 and fn.args[0].writable
+    assert default_input_shapes(fn) == ",".join(["4x16x2048x64xbf16x0"] + ["4x16x2048x64xbf16xrnd"] * 3)
+    fn = generate_payload_module("gen:matmul{M=256 N=512 K=128 ab_type=bf16 c_type=f32 result_type=bf16 has_bias has_relu}",
+                                 "mm").lookup("mm")
+    assert fn.entry == "matmul" and fn.attrs.flags == _lib.GEMM_HAS_BIAS | _lib.GEMM_HAS_RELU
+    assert default_input_shapes(fn) == "256x512xbf16x0,256x128xbf16xrnd,128x512xbf16xrnd,512xbf16xrnd"
+    blk = generate_payload_module("gen:nanogpt_block{B=8 T=1024 C=768 n_head=12 dtype=bf16}", "blk").lookup("blk")
+    assert blk.entry == "nanogpt_block" and default_input_shapes(blk).endswith("xi8x0")
+    for bad, match in (("gen:conv{M=1}", "no payload generator"), ("gen:softmax{M=32 N=256}", "missing key"),
+                       ("gen:softmax{M=32 N=256 dtype=f32 tile=4}", "unknown key")):
+        with pytest.raises(ValueError, match=match):
+            generate_payload_module(bad, "f")
+        assert main([bad, "--entry-point=f", "--stage=cse"]) == 1
+        assert "Error:" in capsys.readouterr().err
