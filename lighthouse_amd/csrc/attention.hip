@@ -17,6 +17,8 @@
 // the V^T P^T product (no LDS round trip or cross-lane shuffle for P).  V^T fragments are read
 // from the row-major V tile with the transposing LDS read, in the key order the accumulator
 // layout produces.
+#include <type_traits>
+
 #include "common.h"
 
 namespace lh {
@@ -103,8 +105,10 @@ struct AttnCtx {
   int k_row, v_row;          // bytes per key (row strides), for the clamped loads of a partial tile
   int key_local[2];          // the key of the tile that load i of this lane fetches
   int wave, r32, h;
-  int k_off[2], k_swz[2];    // K fragment: byte offset of the lane's row, its swizzle, per key sub-tile
-  int v_off, v_swz;          // V fragment through the transposing read
+  // Fragment reads: lane-constant byte offsets within a stage, formed once per workgroup (a tile
+  // then adds the stage's base to each: one vector instruction per address).
+  int k_rd[4];               // K fragment of key sub-tile 0, k-step sd (sub-tile 1: + 32 rows = 4096 bytes)
+  int v_rd[2];               // V^T fragment (transposing read) of head-dim sub-tile j, keys 0 .. 15 of the tile
 };
 
 // RAGGED (sequence length T no multiple of the key tile): keys of the last, partial tile that lie
@@ -135,7 +139,7 @@ __device__ __forceinline__ void attn_issue_loads(const AttnCtx& c, int jt, int T
 template <int DT, int NQ, bool RAGGED, bool AHEAD, int KS = 1>
 __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, const u32x4 (&qf)[NQ][4],
                                           f32x16 (&acc_o)[NQ][2], float (&m_run)[NQ], float (&l_run)[NQ],
-                                          f32x16 (&neg_m)[NQ], const uint8_t* __restrict__ rd,
+                                          f32x16 (&neg_m)[NQ], bool (&has_offset)[NQ], const uint8_t* __restrict__ rd,
                                           uint8_t* __restrict__ wr, int next_jt,
                                           bool prefetch, int j0, int wq0, bool active, bool need_mask, bool first) {
   if (prefetch) attn_issue_loads<RAGGED>(c, next_jt, a.T, wr);
@@ -155,7 +159,7 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int sd = 0; sd < 4; ++sd)
-      kf[i][sd] = *reinterpret_cast<const u32x4*>(ks + c.k_off[i] + (((2 * sd + c.h) ^ c.k_swz[i]) << 4));
+      kf[i][sd] = *reinterpret_cast<const u32x4*>(ks + c.k_rd[sd] + 4096 * i);
   if constexpr (AHEAD) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int i = 0; i < 2; ++i)
@@ -194,19 +198,24 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
     // `first` (the workgroup's first key tile: no row has an offset yet, l and acc are zero) goes
     // straight to the slow path, without the pass that would only find that out and without
     // rescaling zeros.
+    // `has_offset` (wave-uniform, set on the slow path): every row of the sub-tile has an offset, so
+    // the fast path's only test is the partial row sum; a sub-tile with a row that has none yet goes
+    // straight to the slow path, like the first tile.
     const float mc = m_run[qt];
     float p[2][16];
     float l_tile = 0.0f;
     bool move_offset = true;
-    if (!first) {
+    if (!first && has_offset[qt]) {
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          p[i][v] = exp2_fast(s_acc[qt][i][v]);
-          l_tile += p[i][v];
-        }
-      move_offset = __builtin_amdgcn_ballot_w64(!(l_tile <= kOffsetSlack) || mc == -INFINITY) != 0;
+        for (int v = 0; v < 16; ++v) p[i][v] = exp2_fast(s_acc[qt][i][v]);
+      l_tile = p[0][0];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int v = (i == 0 ? 1 : 0); v < 16; ++v) l_tile += p[i][v];
+      move_offset = __builtin_amdgcn_ballot_w64(!(l_tile <= kOffsetSlack)) != 0;
     }
     if (move_offset) {
       float mx = fmaxf(s_acc[qt][0][0], s_acc[qt][1][0]);
@@ -220,6 +229,7 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
       const float delta = m_safe - m_old;
       const float alpha = exp2_fast(mc - m_safe);
       m_run[qt] = m_new;
+      has_offset[qt] = __builtin_amdgcn_ballot_w64(m_new == -INFINITY) == 0;
       if (!first) {
         l_run[qt] *= alpha;
 #pragma unroll
@@ -227,14 +237,15 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
 #pragma unroll
           for (int v = 0; v < 16; ++v) acc_o[qt][j][v] *= alpha;
       }
-      l_tile = 0.0f;
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          p[i][v] = exp2_fast(s_acc[qt][i][v] - delta);
-          l_tile += p[i][v];
-        }
+        for (int v = 0; v < 16; ++v) p[i][v] = exp2_fast(s_acc[qt][i][v] - delta);
+      l_tile = p[0][0];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int v = (i == 0 ? 1 : 0); v < 16; ++v) l_tile += p[i][v];
 #pragma unroll
       for (int v = 0; v < 16; ++v) neg_m[qt][v] = -m_safe;
       asm volatile("" : "+v"(neg_m[qt]));  // a register block, not a constant to re-create per tile
@@ -256,7 +267,7 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
     for (int u = 0; u < 2; ++u)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const uint8_t* p0 = vs + (32 * i + 16 * u) * 128 + c.v_off + (((4 * j) ^ c.v_swz) << 4);
+        const uint8_t* p0 = vs + (32 * i + 16 * u) * 128 + c.v_rd[j];
         attn_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) attn_s16x4*)p0);
         attn_s16x4 hi =
             __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) attn_s16x4*)(p0 + 8 * 128));
@@ -376,12 +387,9 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
     c.v_src[i] = key * c.v_row + ((p ^ (4 * ((key >> 1) & 1))) << 4);
   }
   // K fragment (first MFMA operand of S^T): key 32 i + r32, logical chunk 2 sd + h.
+  // (key sub-tile 1, 32 rows further on, has the same swizzle: 32 / 2 is a multiple of 8)
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int key = 32 * i + r32;
-    c.k_off[i] = key * 128;
-    c.k_swz[i] = (key >> 1) & 7;
-  }
+  for (int sd = 0; sd < 4; ++sd) c.k_rd[sd] = r32 * 128 + (((2 * sd + h) ^ ((r32 >> 1) & 7)) << 4);
   // V^T fragment (first MFMA operand of O^T) through the transposing read.  Lane (grp = lane/16,
   // j16 = lane % 16) addresses key row 4 h + j16 / 4 of the k-step (+8 for the second read),
   // head-dim columns 32 j + 16 (grp % 2) + 4 (j16 % 4) .. +4.  The slot order of the 8 values a
@@ -391,8 +399,10 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
     const int j16 = lane & 15, grp = lane >> 4;
     const int krow = 4 * h + (j16 >> 2);
     const int col = 16 * (grp & 1) + 4 * (j16 & 3);
-    c.v_swz = 4 * ((krow >> 1) & 1);  // unchanged by + 8, + 16 u, + 32 i
-    c.v_off = krow * 128 + 8 * ((col >> 2) & 1) + (((col >> 3) ^ 0) << 4);
+    const int v_swz = 4 * ((krow >> 1) & 1);  // unchanged by + 8, + 16 u, + 32 i
+    const int v_off = krow * 128 + 8 * ((col >> 2) & 1) + ((col >> 3) << 4);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) c.v_rd[j] = v_off + (((4 * j) ^ v_swz) << 4);
   }
   // Q fragments: second MFMA operand of S^T = K Q^T; lane (q = r32, half h) holds
   // Q[q][16 sd + 8 h .. +8] for the 4 k-steps over the head dimension, for both sub-tiles.
@@ -441,6 +451,9 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
   for (int st = 0; st < kAttnStages - 1; ++st)
     if (st < ntiles) attn_issue_loads<RAGGED>(c, t_first + st, a.T, smem_attn + st * kAttnStageBytes);
 
+  bool has_offset[NQ];
+#pragma unroll
+  for (int qt = 0; qt < NQ; ++qt) has_offset[qt] = false;
   for (int it = 0; it < steps; ++it) {
     // 4 loads per lane and stage; the NS - 2 younger stages may stay in flight.  One asm block: a
     // __syncthreads() would add a fence that waits for ALL outstanding loads.
@@ -465,8 +478,9 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
     const bool active = wave_valid && (KS == 1 || it < ntiles) && (!a.causal || (j0 <= wq0 + kRowsPerWave - 1));
     const bool need_mask = (a.causal && (j0 + kKvTile - 1 > wq0)) || (RAGGED && j0 + kKvTile > a.T);
     const int nxt = it + kAttnStages - 1;
-    attn_tile<DT, NQ, RAGGED, !(NQ == 1 && NS == 3) && !(NQ == 2 && RAGGED), KS + 2 * GS>(c, a, qf, acc_o, m_run, l_run, neg_m, smem_attn + (it % kAttnStages) * kAttnStageBytes,
-                  smem_attn + (nxt % kAttnStages) * kAttnStageBytes, t_first + nxt, nxt < ntiles, j0, wq0, active, need_mask, it == 0);
+    attn_tile<DT, NQ, RAGGED, !(NQ == 1 && NS == 3) && !(NQ == 2 && RAGGED), KS + 2 * GS>(
+        c, a, qf, acc_o, m_run, l_run, neg_m, has_offset, smem_attn + (it % kAttnStages) * kAttnStageBytes,
+        smem_attn + (nxt % kAttnStages) * kAttnStageBytes, t_first + nxt, nxt < ntiles, j0, wq0, active, need_mask, it == 0);
   }
 
   if constexpr (GS) {
