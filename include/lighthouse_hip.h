@@ -240,7 +240,13 @@ int lh_hip_gemm_fp8_ws(void* out, const void* a_q, const void* b_q, float scale_
  * and, for the 32-row kernel, the depth of the K/V ring (3 stages: three workgroups per CU; 4: two);
  * LH_ATTN_KSPLIT_2 gives a workgroup of the 64-row kernel two groups of four waves that walk the two
  * halves of the key range side by side and are combined at the end (LH_ATTN_KSPLIT_1: never).
- * 0 lets the library choose by shape.  A request that does not apply fails with LH_ERR_INVALID. */
+ * 0 lets the library choose by shape.  A request that does not apply fails with LH_ERR_INVALID.
+ * LH_ATTN_SCALE_F32 selects where the softmax scale is applied: by default Q is multiplied by
+ * scale * log2(e) once and rounded to the element type again (one rounding more than the reference,
+ * inside every tolerance of the payload); with this bit Q stays as stored and every score is scaled in
+ * f32, as ReplaceWithFusedAttentionOp does (replace_with_fused_attention.py:386), at one more
+ * vector instruction per score (about 7 % of the time at [4,16,2048,64]).  The f32 kernel always
+ * scales in f32. */
 #define LH_ATTN_CAUSAL 0x1
 #define LH_ATTN_ROWS_MASK 0x300
 #define LH_ATTN_ROWS_32 0x100
@@ -251,6 +257,7 @@ int lh_hip_gemm_fp8_ws(void* out, const void* a_q, const void* b_q, float scale_
 #define LH_ATTN_KSPLIT_MASK 0x3000
 #define LH_ATTN_KSPLIT_1 0x1000
 #define LH_ATTN_KSPLIT_2 0x2000
+#define LH_ATTN_SCALE_F32 0x4000
 typedef struct lh_strides3 {
   int64_t z, h, t;
 } lh_strides3;

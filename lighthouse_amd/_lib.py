@@ -36,6 +36,7 @@ ATTN_CAUSAL = 1
 ATTN_ROWS = {0: 0, 32: 0x100, 64: 0x200}
 ATTN_STAGES = {0: 0, 3: 0x400, 4: 0x800}
 ATTN_KSPLIT = {0: 0, 1: 0x1000, 2: 0x2000}
+ATTN_SCALE_F32 = 0x4000  # scores scaled in f32 (the reference's rounding points) instead of Q scaled once
 
 # lh_elementwise_kind
 EW_SOFTMAX, EW_GELU, EW_BIAS, EW_ADD, EW_CAST = range(5)

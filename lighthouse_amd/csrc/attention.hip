@@ -35,6 +35,7 @@ struct AttnArgs {
   int causal;
   int cus;  // compute units of the device (causal launch order)
   int request = 0;  // LH_ATTN_ROWS_* | LH_ATTN_STAGES_* bits of the call (0: the library chooses)
+  bool scale_f32 = false;  // LH_ATTN_SCALE_F32: Q stays as stored and the scores are scaled in f32
   int d = 0;        // head dimension of the call (the padded kernels mask the columns from d on)
   // Key range split between workgroups (few query blocks, long sequences): `kv_groups` workgroups
   // per query block each take a contiguous share of its key tiles and leave (unnormalised output,
@@ -136,7 +137,10 @@ __device__ __forceinline__ void attn_issue_loads(const AttnCtx& c, int jt, int T
 // is the ring slot that receives a later tile meanwhile (separate restrict pointers so that LDS
 // reads do not wait for the asynchronous writes).
 // (KS only separates the instantiations of the two kernels that share the other parameters.)
-template <int DT, int NQ, bool RAGGED, bool AHEAD, int KS = 1>
+// SX: Q holds the stored values, the accumulators start from zero and every score is scaled and
+// offset in f32 afterwards (one fused multiply-add each): the reference's rounding points exactly
+// (S scaled in f32, replace_with_fused_attention.py:386), at one more vector instruction per score.
+template <int DT, int NQ, bool RAGGED, bool AHEAD, int KS = 1, bool SX = false>
 __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, const u32x4 (&qf)[NQ][4],
                                           f32x16 (&acc_o)[NQ][2], float (&m_run)[NQ], float (&l_run)[NQ],
                                           f32x16 (&neg_m)[NQ], bool (&has_offset)[NQ], const uint8_t* __restrict__ rd,
@@ -167,11 +171,21 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
     for (int sd = 0; sd < 4; ++sd)
 #pragma unroll
       for (int qt = 0; qt < NQ; ++qt)
-        s_acc[qt][i] = mfma16<DT>(kf[i][sd], qf[qt][sd], sd == 0 ? neg_m[qt] : s_acc[qt][i]);
-  // A use of neg_m behind its last MFMA: without it the compiler treats that MFMA as the end of the
-  // block's life, accumulates in place and first copies the block (16 moves per tile and sub-tile).
+        s_acc[qt][i] = mfma16<DT>(kf[i][sd], qf[qt][sd], sd == 0 ? (SX ? f32x16{} : neg_m[qt]) : s_acc[qt][i]);
+  if constexpr (SX) {
+    // exponent = S * scale * log2(e) - offset, in f32 (neg_m[qt][0] is minus the lane's offset)
 #pragma unroll
-  for (int qt = 0; qt < NQ; ++qt) asm volatile("" ::"v"(neg_m[qt]));
+    for (int qt = 0; qt < NQ; ++qt)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s_acc[qt][i][v] = __builtin_fmaf(s_acc[qt][i][v], a.scale_log2e, neg_m[qt][0]);
+  } else {
+    // A use of neg_m behind its last MFMA: without it the compiler treats that MFMA as the end of the
+    // block's life, accumulates in place and first copies the block (16 moves per tile and sub-tile).
+#pragma unroll
+    for (int qt = 0; qt < NQ; ++qt) asm volatile("" ::"v"(neg_m[qt]));
+  }
   // s_acc[qt][i][v] = S[q = wq0 + 32 qt + r32][key = j0 + 32 i + 8 (v/4) + 4 h + v%4] scale log2e - offset
   u32x4 pf[NQ][2][2];
 #pragma unroll
@@ -248,7 +262,7 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
         for (int v = (i == 0 ? 1 : 0); v < 16; ++v) l_tile += p[i][v];
 #pragma unroll
       for (int v = 0; v < 16; ++v) neg_m[qt][v] = -m_safe;
-      asm volatile("" : "+v"(neg_m[qt]));  // a register block, not a constant to re-create per tile
+      if constexpr (!SX) asm volatile("" : "+v"(neg_m[qt]));  // a register block, not a constant to re-create per tile
     }
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -332,8 +346,9 @@ __device__ __forceinline__ void xcd_block_of(int L, int nqb, int bhn, int& qb, i
 // GS = 1: the key range of a query block is split between a.kv_groups WORKGROUPS (1-D grid, query
 // blocks heaviest first, the groups of one block next to each other); each leaves its partial
 // result in a.part and attention16_merge finishes the block.
-template <int DT, int NQ, int NS, bool RAGGED, int KS = 1, int GS = 0>
+template <int DT, int NQ, int NS, bool RAGGED, int KS = 1, int GS = 0, bool SX = false>
 __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attention16_kernel(AttnArgs a) {
+  static_assert(!(SX && (KS != 1 || GS)), "scores scaled in f32: one group of four waves per workgroup, no grid split");
   static_assert(!(GS && (KS != 1 || RAGGED)), "the grid split runs four waves per workgroup on whole key tiles");
   constexpr int kRowsPerWave = 32 * NQ, kRowsPerGroup = 4 * kRowsPerWave;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn_all[];
@@ -415,7 +430,8 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
       const u32x4 raw = *reinterpret_cast<const u32x4*>(Q + (int64_t)row * a.sq.t + 16 * sd + 8 * h);
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        qf[qt][sd][e] = pack2<DT>(unpack_lo<DT>(raw[e]) * a.scale_log2e, unpack_hi<DT>(raw[e]) * a.scale_log2e);
+        qf[qt][sd][e] = SX ? raw[e]
+                           : pack2<DT>(unpack_lo<DT>(raw[e]) * a.scale_log2e, unpack_hi<DT>(raw[e]) * a.scale_log2e);
     }
 
   f32x16 acc_o[NQ][2];
@@ -433,7 +449,7 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
     l_run[qt] = 0.0f;
 #pragma unroll
     for (int v = 0; v < 16; ++v) neg_m[qt][v] = 0.0f;
-    asm volatile("" : "+v"(neg_m[qt]));
+    if constexpr (!SX) asm volatile("" : "+v"(neg_m[qt]));
   }
 
   const int kv_end = a.causal ? min(a.T, q0 + kRowsPerGroup) : a.T;
@@ -478,7 +494,7 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
     const bool active = wave_valid && (KS == 1 || it < ntiles) && (!a.causal || (j0 <= wq0 + kRowsPerWave - 1));
     const bool need_mask = (a.causal && (j0 + kKvTile - 1 > wq0)) || (RAGGED && j0 + kKvTile > a.T);
     const int nxt = it + kAttnStages - 1;
-    attn_tile<DT, NQ, RAGGED, !(NQ == 1 && NS == 3) && !(NQ == 2 && RAGGED), KS + 2 * GS>(
+    attn_tile<DT, NQ, RAGGED, !(NQ == 1 && NS == 3) && !(NQ == 2 && RAGGED), KS + 2 * GS, SX>(
         c, a, qf, acc_o, m_run, l_run, neg_m, has_offset, smem_attn + (it % kAttnStages) * kAttnStageBytes,
         smem_attn + (nxt % kAttnStages) * kAttnStageBytes, t_first + nxt, nxt < ntiles, j0, wq0, active, need_mask, it == 0);
   }
@@ -777,9 +793,12 @@ __global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
     }
 }
 
-template <int DT, int NQ, int NS, bool RAGGED, int KS = 1>
+template <int DT, int NQ, int NS, bool RAGGED, int KS = 1, bool SX = false>
 static int attention16_launch_ragged(const AttnArgs& a, hipStream_t s) {
-  auto kern = attention16_kernel<DT, NQ, NS, RAGGED, KS>;
+  if constexpr (KS == 1 && !SX) {
+    if (a.scale_f32) return attention16_launch_ragged<DT, NQ, NS, RAGGED, 1, true>(a, s);
+  }
+  auto kern = attention16_kernel<DT, NQ, NS, RAGGED, KS, 0, SX>;
   constexpr size_t lds = (size_t)KS * NS * kAttnStageBytes;
   static bool configured = false;
   if (!configured && !planning()) {
@@ -906,6 +925,7 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
     return attention16_launch_nq<DT, 2, 4>(a, s);
   }
   if (ksplit_req == LH_ATTN_KSPLIT_2) {
+    LH_REQUIRE(!a.scale_f32, "attention: LH_ATTN_SCALE_F32 exists for one group of four waves per workgroup (not with LH_ATTN_KSPLIT_2)");
     // Two groups of four waves per workgroup, each on half of the key tiles (64 rows per wave, 4 stages).
     LH_REQUIRE(rows_req != LH_ATTN_ROWS_32 && stages_req != LH_ATTN_STAGES_3,
                "attention: the split key range exists for 64 query rows per wave and a 4-stage ring only");
@@ -923,7 +943,8 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
   // the partial results.  Fitted on [1,1,8192] 93.7 -> 31 us,
   // [1,4,4096] 49.9 -> 33.5, [1,4,8192] 104 -> 83 -> (4 groups), [1,1,16384] 183 -> 78, and on
   // [2,8,2048], which stays whole (28.4 us against 34.7 split).
-  if (!ksplit_req && !rows_req && !stages_req && a.allow_grid_split && a.T % kKvTile == 0 && 2 * groups64 <= a.cus) {
+  if (!ksplit_req && !rows_req && !stages_req && !a.scale_f32 && a.allow_grid_split && a.T % kKvTile == 0 &&
+      2 * groups64 <= a.cus) {
     const int ntiles = a.T / kKvTile;
     const double whole = 5.0 + 0.77 * ntiles;
     int best_groups = 1;
@@ -944,7 +965,7 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
   // rows instead (the 32-row kernel) halves the reuse of every K/V fragment.  Non-causal
   // [1,16,4096] 77 -> 72 us, [1,8,8192] 152 -> 132 us.  Causal problems are bound by the
   // total of their key tiles, not by the longest chain ([4,16,2048] 47 -> 53 us with the split).
-  if (!ksplit_req && !rows_req && !stages_req && !a.causal && a.T % kKvTile == 0 && groups64 <= a.cus &&
+  if (!ksplit_req && !rows_req && !stages_req && !a.scale_f32 && !a.causal && a.T % kKvTile == 0 && groups64 <= a.cus &&
       2 * groups64 > a.cus)
     return attention16_launch_ragged<DT, 2, 4, false, 2>(a, s);
   if (rows_req == LH_ATTN_ROWS_32 || stages_req) {
@@ -1547,15 +1568,17 @@ static int attention_run(void* out, const void* q, const void* k, const void* v,
   a.d = (int)d;
   a.ws = ws;
   a.allow_grid_split = ws != nullptr || attention_scratch_allowed();
-  LH_REQUIRE((causal & ~(int32_t)(LH_ATTN_CAUSAL | LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK | LH_ATTN_KSPLIT_MASK)) == 0 &&
+  LH_REQUIRE((causal & ~(int32_t)(LH_ATTN_CAUSAL | LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK | LH_ATTN_KSPLIT_MASK |
+                                  LH_ATTN_SCALE_F32)) == 0 &&
                  (causal & LH_ATTN_ROWS_MASK) != LH_ATTN_ROWS_MASK && (causal & LH_ATTN_STAGES_MASK) != LH_ATTN_STAGES_MASK &&
                  (causal & LH_ATTN_KSPLIT_MASK) != LH_ATTN_KSPLIT_MASK,
              "lh_hip_attention: unknown bits 0x%x in the causal / request word", causal);
   a.causal = (causal & LH_ATTN_CAUSAL) ? 1 : 0;
   a.request = causal & (LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK | LH_ATTN_KSPLIT_MASK);
-  LH_REQUIRE(a.request == 0 || (fast && dtype != LH_F32),
-             "lh_hip_attention: query-row / ring-depth requests apply to 16-bit tensors with head_dim %d and aligned rows",
-             kHeadDim);
+  a.scale_f32 = (causal & LH_ATTN_SCALE_F32) != 0;
+  LH_REQUIRE((a.request == 0 && !a.scale_f32) || (fast && dtype != LH_F32),
+             "lh_hip_attention: query-row / ring-depth / score-scaling requests apply to 16-bit tensors with head_dim %d "
+             "and aligned rows", kHeadDim);
   a.cus = num_cus();
   if (!fast) {
     if (vec_ok) {  // 16-bit tensors with another head dimension the matrix-core kernel takes

@@ -37,7 +37,7 @@ from .pipeline.descriptor import Descriptor, PipelineDescriptor
 # describe a kernel it does not select.
 KERNEL_PARAMETERS = {
     "matmul": {"tile_m", "tile_n", "split_k"},
-    "attention": {"q_rows_per_wave", "kv_stages", "kv_split"},
+    "attention": {"q_rows_per_wave", "kv_stages", "kv_split", "scale_f32"},
     "matmul_fp8": set(), "mlp": set(), "layer_norm": set(), "elementwise": set(), "nanogpt_block": set(),
     "gpt_fused": set(),
 }
@@ -79,14 +79,17 @@ def _apply_attention(fn, params: dict, notes: list[str]) -> None:
     if rows not in _lib.ATTN_ROWS or stages not in _lib.ATTN_STAGES or split not in _lib.ATTN_KSPLIT:
         raise ValueError(f"stage 'attention': q_rows_per_wave must be 32 or 64, kv_stages 3 or 4 and kv_split 1 or 2, "
                          f"got {rows} / {stages} / {split}")
-    if not (rows or stages or split):
+    scale_f32 = params.get("scale_f32", False)
+    if scale_f32 not in (True, False):
+        raise ValueError(f"stage 'attention': scale_f32 is a flag, got {scale_f32}")
+    if not (rows or stages or split or scale_f32):
         return
     if fn.attrs.dtype == _lib.F32 or fn.args[0].shape[-1] != 64:
         notes.append(f"stage 'attention': variant requests apply to 16-bit tensors with head dimension 64, not to "
                      f"@{fn.name}; the library chooses")
         return
     fn.attrs.causal = ((fn.attrs.causal & _lib.ATTN_CAUSAL) | _lib.ATTN_ROWS[rows] | _lib.ATTN_STAGES[stages]
-                       | _lib.ATTN_KSPLIT[split])
+                       | _lib.ATTN_KSPLIT[split] | (_lib.ATTN_SCALE_F32 if scale_f32 else 0))
 
 
 def apply_stage(module: PayloadModule, stage: str, notes: list[str]) -> None:

@@ -245,14 +245,17 @@ def _strides3(t) -> _lib.Strides3:
 
 
 def attention(q, k, v, *, causal=False, scale=None, out=None, rows_per_wave=None, stages=None, kv_split=None,
-              workspace=None):
+              workspace=None, scale_in_f32=False):
     """Fused attention forward on [Z,H,T,d] tensors (any strides with unit stride along d).
     `rows_per_wave` (32 or 64), `stages` (3 or 4, K/V ring of the 32-row kernel) and `kv_split`
     (2: two wave groups per workgroup on halves of the key range, 1: never) request a
     kernel variant for 16-bit tensors with head dimension 64; with none given the
     tuned-parameter database is asked, then the library chooses by shape.
     `workspace` (uint8, see attention_workspace_bytes) makes the call take its temporary memory
-    from there instead of the library's pool (lh_hip_attention_ws)."""
+    from there instead of the library's pool (lh_hip_attention_ws).
+    `scale_in_f32` (16-bit tensors, head dimension 64): Q stays as stored and every score is scaled
+    in f32, the reference's rounding points exactly (LH_ATTN_SCALE_F32; about 7 % slower), instead
+    of Q multiplied by the scale once and rounded to the element type again."""
     if q.dim() != 4 or q.shape != k.shape or q.shape != v.shape:
         raise ValueError("attention expects Q, K, V of equal 4-D shape [Z,H,T,d]")
     _require(q.dtype in _FLOATS and k.dtype == q.dtype and v.dtype == q.dtype,
@@ -276,7 +279,7 @@ def attention(q, k, v, *, causal=False, scale=None, out=None, rows_per_wave=None
              f"rows_per_wave must be one of {sorted(_lib.ATTN_ROWS)[1:]}, stages one of {sorted(_lib.ATTN_STAGES)[1:]}, "
              f"kv_split one of {sorted(_lib.ATTN_KSPLIT)[1:]}")
     word = ((_lib.ATTN_CAUSAL if causal else 0) | _lib.ATTN_ROWS[rows_per_wave or 0] | _lib.ATTN_STAGES[stages or 0]
-            | _lib.ATTN_KSPLIT[kv_split or 0])
+            | _lib.ATTN_KSPLIT[kv_split or 0] | (_lib.ATTN_SCALE_F32 if scale_in_f32 else 0))
     if workspace is not None:
         _require(workspace.dtype == torch.uint8 and workspace.dim() == 1 and workspace.is_contiguous(),
                  "workspace must be a contiguous uint8 vector")
@@ -295,13 +298,14 @@ def attention(q, k, v, *, causal=False, scale=None, out=None, rows_per_wave=None
     return out
 
 
-def attention_workspace_bytes(Z, H, T, d, dtype, *, causal=False, rows_per_wave=None, stages=None, kv_split=None) -> int:
+def attention_workspace_bytes(Z, H, T, d, dtype, *, causal=False, rows_per_wave=None, stages=None, kv_split=None,
+                              scale_in_f32=False) -> int:
     """Bytes of temporary memory `attention(..., workspace=...)` needs for contiguous [Z,H,T,d]
     tensors: the partial results of a key range split between workgroups, which the library
     chooses for 16-bit problems with few query blocks and long sequences; 0 for everything else
     and for every call that requests a kernel variant."""
     word = ((_lib.ATTN_CAUSAL if causal else 0) | _lib.ATTN_ROWS[rows_per_wave or 0] | _lib.ATTN_STAGES[stages or 0]
-            | _lib.ATTN_KSPLIT[kv_split or 0])
+            | _lib.ATTN_KSPLIT[kv_split or 0] | (_lib.ATTN_SCALE_F32 if scale_in_f32 else 0))
     st = _lib.Strides3(H * T * d, T * d, d)
     return int(_lib.load().lh_hip_attention_workspace_bytes(Z, H, T, d, st, st, st, st, word, lh_dtype(dtype)))
 

@@ -387,3 +387,44 @@ def test_attention_key_range_split_between_workgroups(shape, dtype, elt, causal)
             ops.attention(dq, dk, dv, causal=causal, workspace=ws[:need - 256], out=untouched)
         torch.cuda.synchronize()
         assert bool((untouched == 3.0).all())
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype,elt", [(torch.bfloat16, "bf16"), (torch.float16, "f16")])
+@pytest.mark.parametrize("shape", [(2, 3, 512, 64), (4, 16, 2048, 64), (1, 2, 200, 64), (8, 12, 1024, 64)])
+def test_attention_scores_scaled_in_f32(shape, dtype, elt, causal):
+    """LH_ATTN_SCALE_F32: Q as stored, scores scaled in f32 (replace_with_fused_attention.py:386) instead of Q
+    multiplied by the scale once and rounded again.  Same tolerance; the error against the f64 oracle
+    is not larger than the default's (it is about a fifth smaller in bf16 at the benchmark size, whose
+    figures are printed); every kernel variant that has the form; the others refuse it."""
+    from lighthouse_amd import ops
+
+    Z, H, T, D = shape
+    rng = np.random.default_rng(sum(shape) + 5 * causal)
+    q, k, v = (orc.round_to(rng.standard_normal(shape).astype(np.float32), elt) for _ in range(3))
+    dq, dk, dv = (_dev(x, dtype) for x in (q, k, v))
+    default = _host(ops.attention(dq, dk, dv, causal=causal))
+    exact = _host(ops.attention(dq, dk, dv, causal=causal, scale_in_f32=True))
+    heads = [(0, 0), (Z - 1, H - 1)] if Z * H > 8 else [(z, h) for z in range(Z) for h in range(H)]
+    err_default = err_exact = 0.0
+    for z, h in heads:
+        ref = orc.attention(q[z, h], k[z, h], v[z, h], causal=causal, result_type=elt)
+        assert_close(exact[z, h], ref, 2e-2, f"attention scaled in f32 {shape} {elt} z={z} h={h} causal={causal}",
+                     report=shape == (4, 16, 2048, 64) and elt == "bf16" and (z, h) == heads[-1])
+        rms = float(np.sqrt(np.mean(ref.astype(np.float64) ** 2)))
+        err_default = max(err_default, float(np.sqrt(np.mean((default[z, h] - ref) ** 2))) / rms)
+        err_exact = max(err_exact, float(np.sqrt(np.mean((exact[z, h] - ref) ** 2))) / rms)
+    assert err_exact <= 1.05 * err_default, (err_exact, err_default)
+    if shape == (4, 16, 2048, 64) and elt == "bf16":
+        print(f"attention bf16 [4,16,2048,64] causal={causal}: rms error / rms reference {err_default:.3e} with Q scaled once, "
+              f"{err_exact:.3e} with the scores scaled in f32")
+    if T % 64 == 0:
+        for rows in (32, 64):
+            got = ops.attention(dq, dk, dv, causal=causal, scale_in_f32=True, rows_per_wave=rows)
+            ref = orc.attention(q[0, 0], k[0, 0], v[0, 0], causal=causal, result_type=elt)
+            assert_close(_host(got[0, 0]), ref, 2e-2, f"attention scaled in f32, {rows} rows per wave")
+        with pytest.raises(ValueError, match="LH_ATTN_SCALE_F32"):
+            ops.attention(dq, dk, dv, causal=causal, scale_in_f32=True, kv_split=2)
+    q32 = torch.zeros(1, 1, 128, 64, device="cuda")
+    with pytest.raises(ValueError, match="16-bit"):
+        ops.attention(q32, q32, q32, scale_in_f32=True)

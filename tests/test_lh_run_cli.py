@@ -197,6 +197,9 @@ def test_stage_parameters_all_act_or_fail(tmp_path):
     y.write_text('Pipeline:\n  - kernel: "attention{q_rows_per_wave=48}"\n')
     with pytest.raises(ValueError, match="q_rows_per_wave"):
         apply_stage(att, str(y), notes)
+    y.write_text('Pipeline:\n  - kernel: "attention{q_rows_per_wave=64 scale_f32}"\n')
+    apply_stage(att, str(y), notes)
+    assert att.lookup("payload").attrs.causal == _lib.ATTN_CAUSAL | _lib.ATTN_ROWS[64] | _lib.ATTN_SCALE_F32
     # every packaged descriptor parses and applies: none carries a parameter that does nothing
     target = TargetInfo("gfx950", [])
     for pipeline, dtypes in {"matmul": ["bf16", "f16", "f32", "f8E4M3FN"], "attention": ["bf16", "f16", "f32"],
