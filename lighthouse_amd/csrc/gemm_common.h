@@ -91,34 +91,8 @@ __device__ __forceinline__ f32x4 bias4(const GemmArgs& g, int n) {
   return r;
 }
 
-// Bias / activation / conversion for 4 consecutive columns of a 16-bit output, returned as two
-// packed dwords (no accumulator input); same order of operations as epilogue4.  `bias` comes from
-// bias4 (loaded ahead of time by kernels that have other loads in flight).
-template <int DT>
-__device__ __forceinline__ u32x2 epilogue4_pack_bias(const GemmArgs& g, f32x4 bias, float v0, float v1, float v2,
-                                                     float v3) {
-  float v[4] = {v0 * g.alpha, v1 * g.alpha, v2 * g.alpha, v3 * g.alpha};
-  if (g.flags & LH_GEMM_HAS_BIAS) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) v[e] += bias[e];
-  }
-  if (g.flags & LH_GEMM_HAS_GELU) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) v[e] = gelu_tanh(v[e]);
-  }
-  if (g.flags & LH_GEMM_HAS_RELU) {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) v[e] = relu_nan(v[e]);
-  }
-  return u32x2{pack2<DT>(v[0], v[1]), pack2<DT>(v[2], v[3])};
-}
-template <int DT>
-__device__ __forceinline__ u32x2 epilogue4_pack(const GemmArgs& g, int n, float v0, float v1, float v2, float v3) {
-  return epilogue4_pack_bias<DT>(g, bias4<DT>(g, n), v0, v1, v2, v3);
-}
-
 // ---- epilogue variants fixed at compile time ----------------------------------------------
-// The functions above test the flags of the call for every group of 4 elements.  In a tile
+// epilogue4 tests the flags of the call for every group of 4 elements.  In a tile
 // kernel whose epilogue is unrolled over the tile that is a handful of scalar branches around a
 // few vector instructions, a hundred times over, in code that runs once per tile and is cold in
 // the instruction cache each time: the 256 x 256 bf16 tile spent 5.2 us converting and staging
