@@ -302,6 +302,19 @@ def _only_attention(torch, ops):
     return step
 
 
+def _only_attention_f32(torch, ops):
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q64, k64, v64 = (torch.randn((4, 16, 2048, 64), device="cuda", generator=g) for _ in range(3))
+    q128, k128, v128 = (torch.randn((4, 16, 2048, 128), device="cuda", generator=g) for _ in range(3))
+    o64, o128 = torch.empty_like(q64), torch.empty_like(q128)
+
+    def step():
+        ops.attention(q64, k64, v64, out=o64)
+        ops.attention(q128, k128, v128, out=o128)
+
+    return step
+
+
 def _only_block_bf16(torch, ops):
     return block_step(torch, torch.Generator(device="cuda").manual_seed(4), torch.bfloat16)
 
@@ -370,7 +383,7 @@ def _only_gelu(torch, ops):
 
 
 ONLY_WORKLOADS = {
-    "copy": _only_copy, "attention": _only_attention, "block_bf16": _only_block_bf16, "gemm_bf16": _only_gemm_bf16,
+    "copy": _only_copy, "attention": _only_attention, "attention_f32": _only_attention_f32, "block_bf16": _only_block_bf16, "gemm_bf16": _only_gemm_bf16,
     "gemm_bf16_qkv": _only_gemm_bf16_qkv, "gemm_fp8": _only_gemm_fp8, "gemm_fp8_decode": _only_gemm_fp8_decode,
     "gemm_f32": _only_gemm_f32, "layer_norm": _only_layer_norm, "gelu": _only_gelu,
 }
@@ -456,6 +469,12 @@ def main() -> int:
         extras["attention_bf16_d128_noncausal_tflops"] = rate(
             lambda: ops.attention(q128, k128, v128, out=o128), 4.0 * 4 * 16 * 2048 * 2048 * 128) / 1e12
         del q128, k128, v128, o128
+        for dh in (64, 128):
+            qf, kf, vf = (torch.randn(4, 16, 2048, dh, device="cuda", generator=g) for _ in range(3))
+            of = torch.empty_like(qf)
+            extras[f"attention_f32_d{dh}_noncausal_tflops"] = rate(
+                lambda: ops.attention(qf, kf, vf, out=of), 4.0 * 4 * 16 * 2048 * 2048 * dh, 10, 3) / 1e12
+            del qf, kf, vf, of
         ad = torch.randn(16, n8, device="cuda", generator=g).to(torch.bfloat16)
         bd = torch.randn(n8, n8, device="cuda", generator=g).to(torch.bfloat16)
         od = torch.empty(16, n8, device="cuda", dtype=torch.bfloat16)

@@ -1446,6 +1446,214 @@ int attention16_anyd(const AttnArgs& a, int d, int dtype, hipStream_t s) {
   return 1;
 }
 
+// f32 tensors, head dimensions that are multiples of 4 up to 256, other than 64
+// (v_mfma_f32_32x32x2_f32, D = 32 DB columns): the structure of attention16_anyd_kernel.  A
+// workgroup owns 128 query rows (4 waves x 32); K and V tiles of 64 keys are copied through
+// registers into LDS rows of D + 8 floats (with that pad the V reads of the two half waves, 4 key
+// rows apart, fall on different banks), two barriers per tile.  The copy is not overlapped with
+// the arithmetic of the same workgroup: a tile is 2 D MFMAs of 64 cycles per wave, and up to
+// D = 128 a second workgroup on the CU computes meanwhile.  Scores are scaled in f32 after the
+// product, P stays f32 and the statistics follow the plain online-softmax recurrence, exactly as
+// in attention32_kernel.  Q fragments live in registers up to D = 96; above, each tile re-reads
+// them from global memory (32 KiB per wave at most, cache hits) and the registers go to the output
+// accumulators.  Any sequence length: keys past the end are loaded from
+// the last key and masked, rows past the end are computed on the last row and not stored.
+// PAD: the head dimension a.d is a multiple of 4 below D; the 16-byte chunks of Q, K and V from
+// column a.d on are zeros, and output columns from a.d on are not stored.
+template <int DB, bool PAD>
+__global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention32_anyd_kernel(AttnArgs a) {
+  constexpr int D = 32 * DB;
+  constexpr int KROW = D + 8;  // floats per LDS row
+  const int d_real = PAD ? a.d : D;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem_anyd32[];
+  float* Ks = reinterpret_cast<float*>(smem_anyd32);  // [64][KROW]
+  float* Vs = Ks + kKvTile * KROW;                    // [64][KROW]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r32 = lane & 31, h = lane >> 5;
+  const int nqb = (a.T + kQBlock - 1) / kQBlock;
+  // (launch order as in attention16_anyd_kernel: causal blocks heaviest first)
+  const int bhn = a.Z * a.H;
+  int qb = nqb - 1 - (int)blockIdx.x / bhn, bh = (int)blockIdx.x % bhn;
+  if (!a.causal) xcd_block_of((int)(blockIdx.y * gridDim.x + blockIdx.x), nqb, bhn, qb, bh);
+  const int z = bh / a.H, hd = bh % a.H;
+  const int q0 = qb * kQBlock, wq0 = q0 + 32 * wave;
+  const bool wave_valid = wq0 < a.T;
+
+  const float* Q = reinterpret_cast<const float*>(a.q) + (int64_t)z * a.sq.z + (int64_t)hd * a.sq.h;
+  const float* K = reinterpret_cast<const float*>(a.k) + (int64_t)z * a.sk.z + (int64_t)hd * a.sk.h;
+  const float* V = reinterpret_cast<const float*>(a.v) + (int64_t)z * a.sv.z + (int64_t)hd * a.sv.h;
+  float* O = reinterpret_cast<float*>(a.out) + (int64_t)z * a.so.z + (int64_t)hd * a.so.h;
+
+  // Lane (q = r32, half h) holds Q[q][8 kk + 4 h + t], kk = 0 .. D / 8 - 1, t = 0 .. 3.
+  const float* qrow = Q + (int64_t)min(wq0 + r32, a.T - 1) * a.sq.t;
+  auto q_fragment = [&](const float* qrow, int kk) -> f32x4 {
+    const bool inside = !PAD || 8 * kk + 4 * h < d_real;
+    f32x4 raw = *reinterpret_cast<const f32x4*>(qrow + (inside ? 8 * kk + 4 * h : 0));
+    if (PAD && !inside) raw = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    return raw;
+  };
+  constexpr bool Q_REGS = DB <= 3;
+  f32x4 qf[Q_REGS ? D / 8 : 1];
+  if constexpr (Q_REGS) {
+#pragma unroll
+    for (int kk = 0; kk < D / 8; ++kk) qf[kk] = q_fragment(qrow, kk);
+  }
+
+  f32x16 acc_o[DB];
+#pragma unroll
+  for (int j = 0; j < DB; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc_o[j][v] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+
+  constexpr int CPR = D / 4;                           // 16-byte chunks per key row
+  constexpr int RPP = 256 / CPR;                       // key rows per pass of the 256 threads
+  constexpr int NPASS = (kKvTile + RPP - 1) / RPP;
+  const int row0 = tid / CPR, ch = tid % CPR;
+  const bool loader = row0 < RPP;  // (256 is no multiple of CPR for some D: the last threads copy nothing)
+  const bool inside = !PAD || 4 * ch < d_real;
+  const int col = inside ? 4 * ch : 0;
+  const int kv_end = a.causal ? min(a.T, q0 + kQBlock) : a.T;
+  const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
+  for (int jt = 0; jt < ntiles; ++jt) {
+    const int j0 = jt * kKvTile;
+    __syncthreads();  // the previous tile has been consumed
+    // D / 4 16-byte chunks per key row: thread (row0, ch) copies chunk ch of rows row0, row0 + RPP, ...
+    // (a thread's column, and whether it lies inside the head dimension, never change).
+#pragma unroll
+    for (int pass = 0; pass < NPASS; ++pass) {
+      const int key = pass * RPP + row0;
+      if (loader && ((pass + 1) * RPP <= kKvTile || key < kKvTile)) {
+        const int kg = min(j0 + key, a.T - 1);
+        f32x4 kv = *reinterpret_cast<const f32x4*>(K + (int64_t)kg * a.sk.t + col);
+        f32x4 vv = *reinterpret_cast<const f32x4*>(V + (int64_t)kg * a.sv.t + col);
+        // (a chunk past the head dimension loads the row's first chunk and drops it: no branch around the loads)
+        if (PAD && !inside) kv = vv = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        *reinterpret_cast<f32x4*>(Ks + key * KROW + 4 * ch) = kv;
+        *reinterpret_cast<f32x4*>(Vs + key * KROW + 4 * ch) = vv;
+      }
+      if (pass % 8 == 7) asm volatile("" ::: "memory");  // (at most 8 passes, 64 registers, in flight)
+    }
+    __syncthreads();
+    if (!wave_valid || (a.causal && j0 > wq0 + 31)) continue;
+    f32x16 s_acc[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s_acc[i][v] = 0.0f;
+    // (the address is opaque per tile: the loads stay inside the loop and the fragments out of registers)
+    const float* qrow_tile = qrow;
+    if constexpr (!Q_REGS) asm volatile("" : "+v"(qrow_tile));
+    // The two key sub-tiles alternate so that consecutive MFMAs never depend on each other.
+#pragma unroll
+    for (int kk = 0; kk < D / 8; ++kk) {
+      f32x4 q4;
+      if constexpr (Q_REGS) q4 = qf[kk];
+      else q4 = q_fragment(qrow_tile, kk);
+      if constexpr (!Q_REGS) {
+        if (kk % 4 == 3) asm volatile("" ::: "memory");  // (no more than 4 fragments fetched ahead)
+      }
+      f32x4 kf[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) kf[i] = *reinterpret_cast<const f32x4*>(Ks + (32 * i + r32) * KROW + 8 * kk + 4 * h);
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) s_acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[i][t], q4[t], s_acc[i], 0, 0, 0);
+    }
+    // s_acc[i][v] = S[q = wq0 + r32][key = j0 + 32 i + 8 (v / 4) + 4 h + v % 4] (unscaled)
+    if ((a.causal && j0 + kKvTile - 1 > wq0) || j0 + kKvTile > a.T) {
+      // last visible key of the row: its own index under the causal mask, and never past the end
+      const int last = a.causal ? min(wq0 + r32, a.T - 1) : a.T - 1;
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+          if (j0 + 32 * i + 8 * (v >> 2) + 4 * h + (v & 3) > last) s_acc[i][v] = -INFINITY;
+    }
+    float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
+#pragma unroll
+    for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[0][v]), s_acc[1][v]);
+    mx = halfwave_max(mx);
+    const float m_new = fmaxf(m_run, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+    const float alpha = exp2_fast((m_run - m_safe) * a.scale_log2e);
+    const float mc = m_safe * a.scale_log2e;
+    float l_tile = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        s_acc[i][v] = exp2_fast(s_acc[i][v] * a.scale_log2e - mc);
+        l_tile += s_acc[i][v];
+      }
+    l_run = l_run * alpha + l_tile;
+    m_run = m_new;
+#pragma unroll
+    for (int j = 0; j < DB; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc_o[j][v] *= alpha;
+    // O^T += V^T P^T, one key pair per MFMA: lane (d = r32, half h) reads V[key][32 j + r32].
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const float* vrow = Vs + (32 * i + 8 * (v >> 2) + 4 * h + (v & 3)) * KROW + r32;
+#pragma unroll
+        for (int j = 0; j < DB; ++j)
+          acc_o[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vrow[32 * j], s_acc[i][v], acc_o[j], 0, 0, 0);
+        if (v % 4 == 3) asm volatile("" ::: "memory");  // (V fragments of 4 keys fetched ahead, not of all 64)
+      }
+  }
+  // acc_o[j][v] = O[q = wq0 + r32][d = 32 j + 8 (v / 4) + 4 h + v % 4] * l
+  if (!wave_valid) return;
+  const float inv_l = 1.0f / halfwave_sum(l_run);
+  if (wq0 + r32 >= a.T) return;  // (after the cross-lane sum, which needs every lane)
+  float* orow = O + (int64_t)(wq0 + r32) * a.so.t;
+#pragma unroll
+  for (int j = 0; j < DB; ++j)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 w = {acc_o[j][4 * g] * inv_l, acc_o[j][4 * g + 1] * inv_l, acc_o[j][4 * g + 2] * inv_l,
+                       acc_o[j][4 * g + 3] * inv_l};
+      if (!PAD || 32 * j + 8 * g + 4 * h < d_real) *reinterpret_cast<f32x4*>(orow + 32 * j + 8 * g + 4 * h) = w;
+    }
+}
+
+template <int DB, bool PAD>
+static int attention32_anyd_launch(const AttnArgs& a, hipStream_t s) {
+  constexpr size_t lds = (size_t)2 * kKvTile * (32 * DB + 8) * 4;
+  auto kern = attention32_anyd_kernel<DB, PAD>;
+  static bool configured = false;
+  if (!configured && !planning()) {
+    LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     (int)lds));
+    configured = true;
+  }
+  const int nqb = (a.T + kQBlock - 1) / kQBlock;
+  const dim3 grid = a.causal ? dim3(nqb * a.Z * a.H) : dim3(nqb, a.Z * a.H);
+  LH_LAUNCH(kern, grid, dim3(256), lds, s, a);
+  return check_launch("attention32_anyd");
+}
+
+// f32 tensors with 16-byte aligned rows and a head dimension other than 64.  Returns 1 when the head
+// dimension is no multiple of 4.
+int attention32_anyd(const AttnArgs& a, int d, hipStream_t s) {
+  if (d % 4 != 0 || d < 4 || d > 256) return 1;
+  const bool pad = d % 32 != 0;
+  switch ((d + 31) / 32) {
+    case 1: return pad ? attention32_anyd_launch<1, true>(a, s) : attention32_anyd_launch<1, false>(a, s);
+    case 2: return attention32_anyd_launch<2, true>(a, s);  // (64 itself has attention32_kernel)
+    case 3: return pad ? attention32_anyd_launch<3, true>(a, s) : attention32_anyd_launch<3, false>(a, s);
+    case 4: return pad ? attention32_anyd_launch<4, true>(a, s) : attention32_anyd_launch<4, false>(a, s);
+    case 5: return pad ? attention32_anyd_launch<5, true>(a, s) : attention32_anyd_launch<5, false>(a, s);
+    case 6: return pad ? attention32_anyd_launch<6, true>(a, s) : attention32_anyd_launch<6, false>(a, s);
+    case 7: return pad ? attention32_anyd_launch<7, true>(a, s) : attention32_anyd_launch<7, false>(a, s);
+    default: return pad ? attention32_anyd_launch<8, true>(a, s) : attention32_anyd_launch<8, false>(a, s);
+  }
+}
+
 // Any sequence length and head dimension up to 256: one wave per query row, keys in chunks of 64
 // (one per lane), the same online-softmax recurrence and rounding points as the fast kernels
 // (f32 statistics, P rounded to the element type before P V, output rounded once).  Throughput is
@@ -1588,8 +1796,9 @@ static int attention_run(void* out, const void* q, const void* k, const void* v,
              "and aligned rows", kHeadDim);
   a.cus = num_cus();
   if (!fast) {
-    if (vec_ok) {  // 16-bit tensors with another head dimension the matrix-core kernel takes
-      const int rc = attention16_anyd(a, (int)d, dtype, reinterpret_cast<hipStream_t>(stream));
+    if (vec_ok) {  // another head dimension that a matrix-core kernel takes
+      const hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+      const int rc = dtype == LH_F32 ? attention32_anyd(a, (int)d, st) : attention16_anyd(a, (int)d, dtype, st);
       if (rc <= 0) return rc;
     }
     return attention_generic_launch(a, (int)d, dtype, reinterpret_cast<hipStream_t>(stream));

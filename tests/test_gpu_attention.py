@@ -221,13 +221,87 @@ def test_attention_padded_head_dims_on_the_matrix_cores(shape, dtype, elt, causa
 
 
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(2, 3, 256, 128), (1, 2, 333, 128), (1, 2, 512, 32), (1, 2, 200, 96), (1, 1, 384, 160),
+                                   (1, 1, 130, 192), (1, 1, 320, 224), (1, 2, 257, 256), (1, 1, 1, 128), (2, 2, 64, 32),
+                                   (8, 2, 384, 96)])
+def test_attention_f32_other_head_dims_on_the_matrix_cores(shape, causal):
+    """f32 tensors with head_dim 32, 96, ..., 256: the f32 matrix-core kernel for head dimensions
+    other than 64 (K and V tiles copied through registers), at sequence lengths that are and are not
+    multiples of the 64-key tile and the 128-row query block; also on head-innermost views."""
+    from lighthouse_amd import ops
+
+    Z, H, T, D = shape
+    rng = np.random.default_rng(sum(shape) + 2 * causal)
+    q, k, v = (rng.standard_normal(shape).astype(np.float32) for _ in range(3))
+    ref = orc.attention(q, k, v, causal=causal, result_type="f32")
+    out = ops.attention(_dev(q, torch.float32), _dev(k, torch.float32), _dev(v, torch.float32), causal=causal)
+    assert_close(_host(out), ref, 1e-4, f"attention f32 {shape} causal={causal}")
+    qs, ks, vs = (_dev(x, torch.float32).transpose(1, 2).contiguous().transpose(1, 2) for x in (q, k, v))
+    outs = torch.empty((Z, T, H, D), dtype=torch.float32, device="cuda").transpose(1, 2)
+    ops.attention(qs, ks, vs, causal=causal, out=outs)
+    assert torch.equal(outs, out)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(1, 2, 200, 4), (2, 2, 130, 24), (1, 3, 257, 36), (1, 2, 64, 60), (2, 1, 300, 68),
+                                   (1, 2, 129, 100), (1, 1, 200, 124), (1, 1, 140, 132), (1, 1, 131, 180),
+                                   (1, 1, 150, 200), (1, 1, 70, 252)])
+def test_attention_f32_padded_head_dims_on_the_matrix_cores(shape, causal):
+    """f32 head dimensions that are multiples of 4 but not of 32 run on the next wider f32
+    matrix-core kernel with the columns from head_dim on masked.  The tensors are views into wider
+    buffers whose other columns hold NaN (inputs) or a marker (output): the result is that of the
+    head dimension itself and nothing outside it is written."""
+    from lighthouse_amd import ops
+
+    Z, H, T, D = shape
+    W = D + 4 * (1 + (T + D) % 3)  # row stride of the buffers
+    rng = np.random.default_rng(sum(shape) + 5 * causal)
+    q, k, v = (rng.standard_normal(shape).astype(np.float32) for _ in range(3))
+    ref = orc.attention(q, k, v, causal=causal, result_type="f32")
+
+    def widened(x):
+        buf = torch.full((Z, H, T, W), float("nan"), dtype=torch.float32, device="cuda")
+        buf[..., :D] = _dev(x, torch.float32)
+        return buf[..., :D]
+
+    out_buf = torch.full((Z, H, T, W), 7.0, dtype=torch.float32, device="cuda")
+    out = out_buf[..., :D]
+    ops.attention(widened(q), widened(k), widened(v), causal=causal, out=out)
+    assert_close(_host(out), ref, 1e-4, f"attention f32 {shape} causal={causal}")
+    assert torch.all(out_buf[..., D:] == 7.0), "columns past head_dim were written"
+    out_c = ops.attention(_dev(q, torch.float32), _dev(k, torch.float32), _dev(v, torch.float32), causal=causal)
+    assert torch.equal(out_c, out)
+
+
+def test_attention_f32_head_dim_128_runs_at_matrix_core_speed():
+    """[2, 8, 1024, 128] f32: 34 GFLOP.  The matrix-core kernel takes well under a millisecond; the
+    one-wave-per-row kernel that other f32 head dimensions (not multiples of 4) still use takes
+    tens of milliseconds.  The bound sits between the two with a wide margin on either side."""
+    from lighthouse_amd import ops
+
+    q, k, v = (torch.randn(2, 8, 1024, 128, device="cuda") for _ in range(3))
+    o = torch.empty_like(q)
+    for _ in range(3):
+        ops.attention(q, k, v, out=o)
+    torch.cuda.synchronize()
+    beg, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    beg.record()
+    for _ in range(10):
+        ops.attention(q, k, v, out=o)
+    end.record()
+    torch.cuda.synchronize()
+    ms = beg.elapsed_time(end) / 10
+    assert ms < 3.0, f"f32 head_dim 128 attention took {ms:.2f} ms per call"
+
+
+@pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype,elt,rtol", [(torch.bfloat16, "bf16", 2e-2), (torch.float32, "f32", 1e-4)])
 @pytest.mark.parametrize("shape", [(1, 2, 100, 40), (2, 1, 77, 64), (1, 1, 130, 128), (1, 3, 64, 64), (1, 1, 1, 8),
                                    (1, 1, 200, 256), (1, 2, 100, 36), (1, 1, 70, 100), (1, 1, 33, 3)])
 def test_attention_any_shape(shape, dtype, elt, rtol, causal):
-    """Head dimensions (and element types) the MFMA kernels do not take run on the generic kernel
-    with the same rounding points (16-bit head dimensions that are multiples of 8 and f32 head_dim 64
-    take the MFMA kernels at any sequence length)."""
+    """Head dimensions the MFMA kernels do not take (16-bit: not a multiple of 8; f32: not a multiple
+    of 4) run on the generic kernel with the same rounding points; the others take the MFMA kernels at
+    any sequence length."""
     from lighthouse_amd import ops
 
     rng = np.random.default_rng(sum(shape) + causal)
