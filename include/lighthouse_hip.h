@@ -224,9 +224,9 @@ int lh_hip_gemm_fp8_ws(void* out, const void* a_q, const void* b_q, float scale_
  * with f32 running max / sum / accumulator.  Tensors are [Z,H,T,d] with element strides
  * (sz, sh, st) per tensor and unit stride along d, so (T, H*d) projection buffers can be
  * passed as strided views without a copy (examples/xegpu/nanoGPT_payload.py:198-217).
- * dtype in {BF16, F16, F32}; d <= 256.  The matrix-core kernels take every 16-bit d that is a
- * multiple of 8 and every f32 d that is a multiple of 4, with 16-byte aligned rows, at any T; every
- * other problem runs on a generic kernel.  A 16-bit problem with few query blocks and a long sequence (fewer
+ * dtype in {BF16, F16, F32}; 1 <= d <= 256, any T.  Every problem runs on the matrix cores: with
+ * 16-byte accesses when rows are 16-byte aligned and d is a multiple of 8 (16-bit) or 4 (f32), with
+ * element accesses otherwise.  A 16-bit problem with few query blocks and a long sequence (fewer
  * 128-row blocks than compute units) has the key range of every block split between workgroups;
  * the partial results (68 KiB per workgroup, at most 35 MiB) live in the library's pool of
  * temporary buffers of the stream, like the K-cut blocks of lh_hip_gemm.  The nanoGPT block and

@@ -993,6 +993,74 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
   return attention16_launch_nq<DT, 2, 4>(a, s);
 }
 
+// How the register-copy kernels below treat a head dimension d under their compiled width D:
+// kRowsExact: d == D.  kRowsChunks: rows are 16-byte aligned and d is a whole number of 16-byte
+// chunks; a chunk from column d on reads as zeros (its load goes to the row's first chunk and is
+// dropped: no branch) and is not stored.  kRowsElements: any d, any alignment; element loads and
+// stores, a column from d on reads as zero (its load goes to the row's last element).
+constexpr int kRowsExact = 0, kRowsChunks = 1, kRowsElements = 2;
+
+// Columns c .. c + 7 of a 16-bit row.
+template <int ROWS>
+__device__ __forceinline__ u32x4 row_chunk16(const uint16_t* row, int c, int d) {
+  if constexpr (ROWS == kRowsElements) {
+    u32x4 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int c0 = c + 2 * e, c1 = c0 + 1;
+      uint32_t lo = row[min(c0, d - 1)], hi = row[min(c1, d - 1)];
+      if (c0 >= d) lo = 0u;
+      if (c1 >= d) hi = 0u;
+      r[e] = lo | (hi << 16);
+    }
+    return r;
+  } else {
+    const bool inside = ROWS == kRowsExact || c < d;
+    u32x4 raw = *reinterpret_cast<const u32x4*>(row + (inside ? c : 0));
+    if (ROWS != kRowsExact && !inside) raw = u32x4{0u, 0u, 0u, 0u};
+    return raw;
+  }
+}
+// Columns c .. c + 3 of a 16-bit row, stored.
+template <int ROWS>
+__device__ __forceinline__ void store_chunk16(uint16_t* row, int c, int d, u32x2 w) {
+  if constexpr (ROWS == kRowsElements) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (c + e < d) row[c + e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+  } else {
+    if (ROWS == kRowsExact || c < d) *reinterpret_cast<u32x2*>(row + c) = w;
+  }
+}
+// Columns c .. c + 3 of an f32 row.
+template <int ROWS>
+__device__ __forceinline__ f32x4 row_chunk32(const float* row, int c, int d) {
+  if constexpr (ROWS == kRowsElements) {
+    f32x4 r;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      r[e] = row[min(c + e, d - 1)];
+      if (c + e >= d) r[e] = 0.0f;
+    }
+    return r;
+  } else {
+    const bool inside = ROWS == kRowsExact || c < d;
+    f32x4 raw = *reinterpret_cast<const f32x4*>(row + (inside ? c : 0));
+    if (ROWS != kRowsExact && !inside) raw = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    return raw;
+  }
+}
+template <int ROWS>
+__device__ __forceinline__ void store_chunk32(float* row, int c, int d, f32x4 w) {
+  if constexpr (ROWS == kRowsElements) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (c + e < d) row[c + e] = w[e];
+  } else {
+    if (ROWS == kRowsExact || c < d) *reinterpret_cast<f32x4*>(row + c) = w;
+  }
+}
+
 // 16-bit tensors, head dimension D = 32 DB (32, 96, 128, 192, 256; 64 and 128 for padded calls): the same
 // transposed formulation on the matrix cores (S^T = K Q^T, O^T = V^T P^T, a lane owns a query row)
 // without the streaming machinery of the head-dimension-64 kernel.  A workgroup owns 128 query
@@ -1000,13 +1068,13 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
 // with rows padded by 16 bytes (V^T fragments through ds_read_b64_tr_b16), two barriers per tile.  Row statistics follow the plain online-softmax recurrence (maximum per
 // tile).  Any sequence length: keys past the end are loaded from the last key and masked, rows
 // past the end are computed on the last row and not stored.
-// PAD: the head dimension a.d is a multiple of 8 below D.  The 16-byte chunks of Q, K and V from
-// column a.d on are zeros in registers and LDS (they add nothing to S, and their output columns
-// are not stored), so the result is that of head dimension a.d exactly.
-template <int DT, int DB, bool PAD>
-__global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kernel(AttnArgs a) {
+// ROWS != kRowsExact: the head dimension a.d lies below D (or the rows are not 16-byte aligned).
+// The columns of Q, K and V from a.d on are zeros in registers and LDS (they add nothing to S, and
+// their output columns are not stored), so the result is that of head dimension a.d exactly.
+template <int DT, int DB, int ROWS>
+__global__ void __launch_bounds__(256, (DB <= 2 || (DB == 3 && ROWS != kRowsElements) ? 2 : 1)) attention16_anyd_kernel(AttnArgs a) {
   constexpr int D = 32 * DB;
-  const int d_real = PAD ? a.d : D;
+  const int d_real = ROWS != kRowsExact ? a.d : D;
   constexpr int KROW = D + 8;  // elements per LDS row
   extern __shared__ __attribute__((aligned(16))) uint8_t smem_anyd[];
   uint16_t* Ks = reinterpret_cast<uint16_t*>(smem_anyd);  // [64][KROW]
@@ -1039,15 +1107,14 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
     const int row = min(wq0 + r32, a.T - 1);
 #pragma unroll
     for (int sd = 0; sd < D / 16; ++sd) {
-      const bool inside = !PAD || 16 * sd + 8 * h < d_real;
-      u32x4 raw = *reinterpret_cast<const u32x4*>(Q + (int64_t)row * a.sq.t + (inside ? 16 * sd + 8 * h : 0));
-      if (PAD && !inside) raw = u32x4{0u, 0u, 0u, 0u};
+      const u32x4 raw = row_chunk16<ROWS>(Q + (int64_t)row * a.sq.t, 16 * sd + 8 * h, d_real);
       u32x4 scaled;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
         scaled[e] = pack2<DT>(unpack_lo<DT>(raw[e]) * a.scale_log2e, unpack_hi<DT>(raw[e]) * a.scale_log2e);
       if constexpr (Q_LDS) q_lds[sd * 64] = scaled;
       else qf[sd] = scaled;
+      if constexpr (ROWS == kRowsElements) asm volatile("" ::: "memory");  // (one chunk's element loads at a time)
     }
   }
   f32x16 acc_o[DB];
@@ -1066,19 +1133,20 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
   for (int jt = 0; jt < ntiles; ++jt) {
     const int j0 = jt * kKvTile;
     __syncthreads();  // the previous tile has been consumed
+    // (opaque per tile: the masks and clamped columns that depend on it are formed where they are used
+    // and not kept in registers across the loop)
+    int d_tile = d_real;
+    if constexpr (ROWS != kRowsExact) asm volatile("" : "+s"(d_tile));
     // 8 D 16-byte chunks per tile and tensor, DB per thread: chunk c = key c / (D / 8), columns 8 (c % (D / 8)) .. +8.
 #pragma unroll
     for (int i = 0; i < DB; ++i) {
       const int c = tid + 256 * i, key = c / (D / 8), ch = c % (D / 8);
       const int kg = min(j0 + key, a.T - 1);
-      // (a masked chunk loads the row's first chunk and drops it: no branch around the loads)
-      const bool inside = !PAD || 8 * ch < d_real;
-      const int col = inside ? 8 * ch : 0;
-      u32x4 kv = *reinterpret_cast<const u32x4*>(K + (int64_t)kg * a.sk.t + col);
-      u32x4 vv = *reinterpret_cast<const u32x4*>(V + (int64_t)kg * a.sv.t + col);
-      if (PAD && !inside) kv = vv = u32x4{0u, 0u, 0u, 0u};
+      const u32x4 kv = row_chunk16<ROWS>(K + (int64_t)kg * a.sk.t, 8 * ch, d_tile);
+      const u32x4 vv = row_chunk16<ROWS>(V + (int64_t)kg * a.sv.t, 8 * ch, d_tile);
       *reinterpret_cast<u32x4*>(Ks + key * KROW + 8 * ch) = kv;
       *reinterpret_cast<u32x4*>(Vs + key * KROW + 8 * ch) = vv;
+      if constexpr (ROWS == kRowsElements) asm volatile("" ::: "memory");  // (16 element loads in flight, not 16 DB)
     }
     __syncthreads();
     if (!wave_valid || (a.causal && j0 > wq0 + 31)) continue;
@@ -1176,7 +1244,7 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention16_anyd_kerne
     for (int g = 0; g < 4; ++g) {
       u32x2 w = {pack2<DT>(acc_o[j][4 * g] * inv_l, acc_o[j][4 * g + 1] * inv_l),
                  pack2<DT>(acc_o[j][4 * g + 2] * inv_l, acc_o[j][4 * g + 3] * inv_l)};
-      if (!PAD || 32 * j + 8 * g + 4 * h < d_real) *reinterpret_cast<u32x2*>(orow + 32 * j + 8 * g + 4 * h) = w;
+      store_chunk16<ROWS>(orow, 32 * j + 8 * g + 4 * h, d_real, w);
     }
 }
 
@@ -1401,11 +1469,11 @@ static int attention16_d128_launch(const AttnArgs& a, hipStream_t s) {
   return check_launch("attention16_d128");
 }
 
-template <int DT, int DB, bool PAD = false>
+template <int DT, int DB, int ROWS = kRowsExact>
 static int attention16_anyd_launch(const AttnArgs& a, hipStream_t s) {
   constexpr int D = 32 * DB;
   constexpr size_t lds = (size_t)2 * kKvTile * (D + 8) * 2 + (DB >= 8 ? 4 * 32 * D * 2 : 0);
-  auto kern = attention16_anyd_kernel<DT, DB, PAD>;
+  auto kern = attention16_anyd_kernel<DT, DB, ROWS>;
   static bool configured = false;
   if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1418,31 +1486,39 @@ static int attention16_anyd_launch(const AttnArgs& a, hipStream_t s) {
   return check_launch("attention16_anyd");
 }
 
-// Returns 1 when no instantiation takes the head dimension.
+// `chunks`: rows are 16-byte aligned and d is a multiple of 8.  Returns 1 when d is out of range.
 template <int DT>
-static int attention16_anyd_dispatch(const AttnArgs& a, int d, hipStream_t s) {
-  switch (d) {
-    case 32: return attention16_anyd_launch<DT, 1>(a, s);
-    case 96: return attention16_anyd_launch<DT, 3>(a, s);
-    case 128: return attention16_d128_launch<DT>(a, s);
-    case 192: return attention16_anyd_launch<DT, 6>(a, s);
-    case 256: return attention16_anyd_launch<DT, 8>(a, s);
-    default: break;
+static int attention16_anyd_dispatch(const AttnArgs& a, int d, bool chunks, hipStream_t s) {
+  if (d < 1 || d > 256) return 1;
+  if (chunks) {
+    switch (d) {
+      case 32: return attention16_anyd_launch<DT, 1>(a, s);
+      case 96: return attention16_anyd_launch<DT, 3>(a, s);
+      case 128: return attention16_d128_launch<DT>(a, s);
+      case 192: return attention16_anyd_launch<DT, 6>(a, s);
+      case 256: return attention16_anyd_launch<DT, 8>(a, s);
+      default: break;
+    }
+    // Other multiples of 8: the next instantiated width, the columns from d on masked.
+    if (d < 32) return attention16_anyd_launch<DT, 1, kRowsChunks>(a, s);
+    if (d < 64) return attention16_anyd_launch<DT, 2, kRowsChunks>(a, s);
+    if (d < 96) return attention16_anyd_launch<DT, 3, kRowsChunks>(a, s);
+    if (d < 128) return attention16_anyd_launch<DT, 4, kRowsChunks>(a, s);
+    if (d < 192) return attention16_anyd_launch<DT, 6, kRowsChunks>(a, s);
+    return attention16_anyd_launch<DT, 8, kRowsChunks>(a, s);
   }
-  // Other multiples of 8: the next instantiated width, the columns from d on masked.
-  if (d % 8 != 0) return 1;
-  if (d < 32) return attention16_anyd_launch<DT, 1, true>(a, s);
-  if (d < 64) return attention16_anyd_launch<DT, 2, true>(a, s);
-  if (d < 96) return attention16_anyd_launch<DT, 3, true>(a, s);
-  if (d < 128) return attention16_anyd_launch<DT, 4, true>(a, s);
-  if (d < 192) return attention16_anyd_launch<DT, 6, true>(a, s);
-  if (d < 256) return attention16_anyd_launch<DT, 8, true>(a, s);
-  return 1;
+  // Any other head dimension or alignment: the same kernels with element loads and stores.
+  if (d <= 32) return attention16_anyd_launch<DT, 1, kRowsElements>(a, s);
+  if (d <= 64) return attention16_anyd_launch<DT, 2, kRowsElements>(a, s);
+  if (d <= 96) return attention16_anyd_launch<DT, 3, kRowsElements>(a, s);
+  if (d <= 128) return attention16_anyd_launch<DT, 4, kRowsElements>(a, s);
+  if (d <= 192) return attention16_anyd_launch<DT, 6, kRowsElements>(a, s);
+  return attention16_anyd_launch<DT, 8, kRowsElements>(a, s);
 }
 
-int attention16_anyd(const AttnArgs& a, int d, int dtype, hipStream_t s) {
-  if (dtype == LH_BF16) return attention16_anyd_dispatch<LH_BF16>(a, d, s);
-  if (dtype == LH_F16) return attention16_anyd_dispatch<LH_F16>(a, d, s);
+int attention16_anyd(const AttnArgs& a, int d, int dtype, bool chunks, hipStream_t s) {
+  if (dtype == LH_BF16) return attention16_anyd_dispatch<LH_BF16>(a, d, chunks, s);
+  if (dtype == LH_F16) return attention16_anyd_dispatch<LH_F16>(a, d, chunks, s);
   return 1;
 }
 
@@ -1458,13 +1534,13 @@ int attention16_anyd(const AttnArgs& a, int d, int dtype, hipStream_t s) {
 // them from global memory (32 KiB per wave at most, cache hits) and the registers go to the output
 // accumulators.  Any sequence length: keys past the end are loaded from
 // the last key and masked, rows past the end are computed on the last row and not stored.
-// PAD: the head dimension a.d is a multiple of 4 below D; the 16-byte chunks of Q, K and V from
-// column a.d on are zeros, and output columns from a.d on are not stored.
-template <int DB, bool PAD>
+// ROWS != kRowsExact: the head dimension a.d lies below D (or the rows are not 16-byte aligned); the
+// columns of Q, K and V from a.d on are zeros, and output columns from a.d on are not stored.
+template <int DB, int ROWS>
 __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention32_anyd_kernel(AttnArgs a) {
   constexpr int D = 32 * DB;
   constexpr int KROW = D + 8;  // floats per LDS row
-  const int d_real = PAD ? a.d : D;
+  const int d_real = ROWS != kRowsExact ? a.d : D;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem_anyd32[];
   float* Ks = reinterpret_cast<float*>(smem_anyd32);  // [64][KROW]
   float* Vs = Ks + kKvTile * KROW;                    // [64][KROW]
@@ -1487,17 +1563,12 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention32_anyd_kerne
 
   // Lane (q = r32, half h) holds Q[q][8 kk + 4 h + t], kk = 0 .. D / 8 - 1, t = 0 .. 3.
   const float* qrow = Q + (int64_t)min(wq0 + r32, a.T - 1) * a.sq.t;
-  auto q_fragment = [&](const float* qrow, int kk) -> f32x4 {
-    const bool inside = !PAD || 8 * kk + 4 * h < d_real;
-    f32x4 raw = *reinterpret_cast<const f32x4*>(qrow + (inside ? 8 * kk + 4 * h : 0));
-    if (PAD && !inside) raw = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    return raw;
-  };
+  auto q_fragment = [&](const float* qrow, int kk, int d) -> f32x4 { return row_chunk32<ROWS>(qrow, 8 * kk + 4 * h, d); };
   constexpr bool Q_REGS = DB <= 3;
   f32x4 qf[Q_REGS ? D / 8 : 1];
   if constexpr (Q_REGS) {
 #pragma unroll
-    for (int kk = 0; kk < D / 8; ++kk) qf[kk] = q_fragment(qrow, kk);
+    for (int kk = 0; kk < D / 8; ++kk) qf[kk] = q_fragment(qrow, kk, d_real);
   }
 
   f32x16 acc_o[DB];
@@ -1512,13 +1583,15 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention32_anyd_kerne
   constexpr int NPASS = (kKvTile + RPP - 1) / RPP;
   const int row0 = tid / CPR, ch = tid % CPR;
   const bool loader = row0 < RPP;  // (256 is no multiple of CPR for some D: the last threads copy nothing)
-  const bool inside = !PAD || 4 * ch < d_real;
-  const int col = inside ? 4 * ch : 0;
   const int kv_end = a.causal ? min(a.T, q0 + kQBlock) : a.T;
   const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
   for (int jt = 0; jt < ntiles; ++jt) {
     const int j0 = jt * kKvTile;
     __syncthreads();  // the previous tile has been consumed
+    // (opaque per tile: the masks and clamped columns that depend on it are formed where they are used
+    // and not kept in registers across the loop)
+    int d_tile = d_real;
+    if constexpr (ROWS != kRowsExact) asm volatile("" : "+s"(d_tile));
     // D / 4 16-byte chunks per key row: thread (row0, ch) copies chunk ch of rows row0, row0 + RPP, ...
     // (a thread's column, and whether it lies inside the head dimension, never change).
 #pragma unroll
@@ -1526,14 +1599,13 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention32_anyd_kerne
       const int key = pass * RPP + row0;
       if (loader && ((pass + 1) * RPP <= kKvTile || key < kKvTile)) {
         const int kg = min(j0 + key, a.T - 1);
-        f32x4 kv = *reinterpret_cast<const f32x4*>(K + (int64_t)kg * a.sk.t + col);
-        f32x4 vv = *reinterpret_cast<const f32x4*>(V + (int64_t)kg * a.sv.t + col);
-        // (a chunk past the head dimension loads the row's first chunk and drops it: no branch around the loads)
-        if (PAD && !inside) kv = vv = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        const f32x4 kv = row_chunk32<ROWS>(K + (int64_t)kg * a.sk.t, 4 * ch, d_tile);
+        const f32x4 vv = row_chunk32<ROWS>(V + (int64_t)kg * a.sv.t, 4 * ch, d_tile);
         *reinterpret_cast<f32x4*>(Ks + key * KROW + 4 * ch) = kv;
         *reinterpret_cast<f32x4*>(Vs + key * KROW + 4 * ch) = vv;
       }
-      if (pass % 8 == 7) asm volatile("" ::: "memory");  // (at most 8 passes, 64 registers, in flight)
+      // (at most 8 passes, 64 registers, in flight; 2 passes, 16 loads, when they are element loads)
+      if (pass % 8 == 7 || (ROWS == kRowsElements && pass % 2 == 1)) asm volatile("" ::: "memory");
     }
     __syncthreads();
     if (!wave_valid || (a.causal && j0 > wq0 + 31)) continue;
@@ -1550,9 +1622,10 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention32_anyd_kerne
     for (int kk = 0; kk < D / 8; ++kk) {
       f32x4 q4;
       if constexpr (Q_REGS) q4 = qf[kk];
-      else q4 = q_fragment(qrow_tile, kk);
+      else q4 = q_fragment(qrow_tile, kk, d_tile);
       if constexpr (!Q_REGS) {
-        if (kk % 4 == 3) asm volatile("" ::: "memory");  // (no more than 4 fragments fetched ahead)
+        // (no more than 4 fragments fetched ahead; 2 when they are element loads)
+        if (kk % 4 == 3 || (ROWS == kRowsElements && kk % 2 == 1)) asm volatile("" ::: "memory");
       }
       f32x4 kf[2];
 #pragma unroll
@@ -1617,14 +1690,14 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention32_anyd_kerne
     for (int g = 0; g < 4; ++g) {
       const f32x4 w = {acc_o[j][4 * g] * inv_l, acc_o[j][4 * g + 1] * inv_l, acc_o[j][4 * g + 2] * inv_l,
                        acc_o[j][4 * g + 3] * inv_l};
-      if (!PAD || 32 * j + 8 * g + 4 * h < d_real) *reinterpret_cast<f32x4*>(orow + 32 * j + 8 * g + 4 * h) = w;
+      store_chunk32<ROWS>(orow, 32 * j + 8 * g + 4 * h, d_real, w);
     }
 }
 
-template <int DB, bool PAD>
+template <int DB, int ROWS>
 static int attention32_anyd_launch(const AttnArgs& a, hipStream_t s) {
   constexpr size_t lds = (size_t)2 * kKvTile * (32 * DB + 8) * 4;
-  auto kern = attention32_anyd_kernel<DB, PAD>;
+  auto kern = attention32_anyd_kernel<DB, ROWS>;
   static bool configured = false;
   if (!configured && !planning()) {
     LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1637,92 +1710,30 @@ static int attention32_anyd_launch(const AttnArgs& a, hipStream_t s) {
   return check_launch("attention32_anyd");
 }
 
-// f32 tensors with 16-byte aligned rows and a head dimension other than 64.  Returns 1 when the head
-// dimension is no multiple of 4.
-int attention32_anyd(const AttnArgs& a, int d, hipStream_t s) {
-  if (d % 4 != 0 || d < 4 || d > 256) return 1;
-  const bool pad = d % 32 != 0;
+template <int DB>
+static int attention32_anyd_rows(const AttnArgs& a, int d, bool chunks, hipStream_t s) {
+  if (!chunks) return attention32_anyd_launch<DB, kRowsElements>(a, s);
+  if (d != 32 * DB) return attention32_anyd_launch<DB, kRowsChunks>(a, s);
+  return attention32_anyd_launch<DB, kRowsExact>(a, s);
+}
+
+// f32 tensors on the kernel above.  `chunks`: rows are 16-byte aligned and d is a multiple of 4.
+// Returns 1 when d is out of range.
+int attention32_anyd(const AttnArgs& a, int d, bool chunks, hipStream_t s) {
+  if (d < 1 || d > 256) return 1;
   switch ((d + 31) / 32) {
-    case 1: return pad ? attention32_anyd_launch<1, true>(a, s) : attention32_anyd_launch<1, false>(a, s);
-    case 2: return attention32_anyd_launch<2, true>(a, s);  // (64 itself has attention32_kernel)
-    case 3: return pad ? attention32_anyd_launch<3, true>(a, s) : attention32_anyd_launch<3, false>(a, s);
-    case 4: return pad ? attention32_anyd_launch<4, true>(a, s) : attention32_anyd_launch<4, false>(a, s);
-    case 5: return pad ? attention32_anyd_launch<5, true>(a, s) : attention32_anyd_launch<5, false>(a, s);
-    case 6: return pad ? attention32_anyd_launch<6, true>(a, s) : attention32_anyd_launch<6, false>(a, s);
-    case 7: return pad ? attention32_anyd_launch<7, true>(a, s) : attention32_anyd_launch<7, false>(a, s);
-    default: return pad ? attention32_anyd_launch<8, true>(a, s) : attention32_anyd_launch<8, false>(a, s);
+    case 1: return attention32_anyd_rows<1>(a, d, chunks, s);
+    case 2: return attention32_anyd_rows<2>(a, d, chunks, s);
+    case 3: return attention32_anyd_rows<3>(a, d, chunks, s);
+    case 4: return attention32_anyd_rows<4>(a, d, chunks, s);
+    case 5: return attention32_anyd_rows<5>(a, d, chunks, s);
+    case 6: return attention32_anyd_rows<6>(a, d, chunks, s);
+    case 7: return attention32_anyd_rows<7>(a, d, chunks, s);
+    default: return attention32_anyd_rows<8>(a, d, chunks, s);
   }
 }
 
-// Any sequence length and head dimension up to 256: one wave per query row, keys in chunks of 64
-// (one per lane), the same online-softmax recurrence and rounding points as the fast kernels
-// (f32 statistics, P rounded to the element type before P V, output rounded once).  Throughput is
-// not a goal here; the MFMA kernels take every shape they can.
-constexpr int kGenericMaxD = 256;
-
-template <int DT>
-__global__ void __launch_bounds__(64) attention_generic_kernel(AttnArgs a, int d) {
-  __shared__ float qs[kGenericMaxD];
-  __shared__ float ps[64];
-  const int lane = threadIdx.x;
-  const int i = blockIdx.x, bh = blockIdx.y;
-  const int z = bh / a.H, hd = bh % a.H;
-  const int64_t qoff = (int64_t)z * a.sq.z + (int64_t)hd * a.sq.h + (int64_t)i * a.sq.t;
-  const int64_t koff = (int64_t)z * a.sk.z + (int64_t)hd * a.sk.h;
-  const int64_t voff = (int64_t)z * a.sv.z + (int64_t)hd * a.sv.h;
-  const int64_t ooff = (int64_t)z * a.so.z + (int64_t)hd * a.so.h + (int64_t)i * a.so.t;
-  for (int c = lane; c < d; c += 64) qs[c] = load_as_f32<DT>(a.q, qoff + c);
-  __syncthreads();
-  float acc[kGenericMaxD / 64];
-#pragma unroll
-  for (int r = 0; r < kGenericMaxD / 64; ++r) acc[r] = 0.0f;
-  float m_run = -INFINITY, l_run = 0.0f;
-  const int kv_end = a.causal ? i + 1 : a.T;
-  for (int j0 = 0; j0 < kv_end; j0 += 64) {
-    const int j = j0 + lane;
-    float sc = -INFINITY;
-    if (j < kv_end) {
-      float dot = 0.0f;
-      for (int c = 0; c < d; ++c) dot += qs[c] * load_as_f32<DT>(a.k, koff + (int64_t)j * a.sk.t + c);
-      sc = dot * a.scale;
-    }
-    float mx = sc;
-    for (int off = 32; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-    const float m_new = fmaxf(m_run, mx);  // finite: key j0 is always valid
-    const float alpha = expf(m_run - m_new);
-    const float pexp = (j < kv_end) ? expf(sc - m_new) : 0.0f;
-    float lsum = pexp;
-    for (int off = 32; off > 0; off >>= 1) lsum += __shfl_xor(lsum, off, 64);
-    l_run = l_run * alpha + lsum;
-    m_run = m_new;
-    __syncthreads();  // previous chunk's ps fully consumed
-    ps[lane] = round_through<DT>(pexp);
-    __syncthreads();
-    const int nvalid = min(64, kv_end - j0);
-#pragma unroll
-    for (int r = 0; r < kGenericMaxD / 64; ++r) {
-      const int c = lane + 64 * r;
-      if (c < d) {
-        float s2 = 0.0f;
-        for (int jj = 0; jj < nvalid; ++jj) s2 += ps[jj] * load_as_f32<DT>(a.v, voff + (int64_t)(j0 + jj) * a.sv.t + c);
-        acc[r] = acc[r] * alpha + s2;
-      }
-    }
-  }
-#pragma unroll
-  for (int r = 0; r < kGenericMaxD / 64; ++r) {
-    const int c = lane + 64 * r;
-    if (c < d) store_from_f32<DT>(a.out, ooff + c, acc[r] / l_run);
-  }
-}
-
-int attention_generic_launch(const AttnArgs& a, int d, int dtype, hipStream_t s) {
-  const dim3 grid(a.T, a.Z * a.H);
-  if (dtype == LH_BF16) LH_LAUNCH(attention_generic_kernel<LH_BF16>, grid, dim3(64), 0, s, a, d);
-  else if (dtype == LH_F16) LH_LAUNCH(attention_generic_kernel<LH_F16>, grid, dim3(64), 0, s, a, d);
-  else LH_LAUNCH(attention_generic_kernel<LH_F32>, grid, dim3(64), 0, s, a, d);
-  return check_launch("attention_generic");
-}
+constexpr int kMaxHeadDim = 256;
 
 int attention_launch(const AttnArgs& a, int dtype, hipStream_t s) {
   if (dtype == LH_BF16) return attention16_launch<LH_BF16>(a, s);
@@ -1758,21 +1769,22 @@ static int attention_run(void* out, const void* q, const void* k, const void* v,
   LH_REQUIRE(dtype == LH_BF16 || dtype == LH_F16 || dtype == LH_F32, "lh_hip_attention: unsupported dtype %d", dtype);
   LH_REQUIRE(Z > 0 && H > 0 && T > 0, "lh_hip_attention: empty problem Z=%lld H=%lld T=%lld", (long long)Z,
              (long long)H, (long long)T);
-  if (d < 1 || d > kGenericMaxD)
-    return fail(LH_ERR_UNSUPPORTED, "lh_hip_attention: head_dim %lld not supported (1 .. %d)", (long long)d, kGenericMaxD);
+  if (d < 1 || d > kMaxHeadDim)
+    return fail(LH_ERR_UNSUPPORTED, "lh_hip_attention: head_dim %lld not supported (1 .. %d)", (long long)d, kMaxHeadDim);
   LH_REQUIRE(Z * H <= 65535 && T < (1 << 30), "lh_hip_attention: problem too large");
   const lh_strides3* ss[4] = {&so, &sq, &sk, &sv};
   const void* ps[4] = {out, q, k, v};
   for (int i = 0; i < 4; ++i) LH_REQUIRE(ss[i]->t >= d, "lh_hip_attention: row stride of tensor %d is below head_dim", i);
-  // The MFMA kernels need head_dim 64 and 16-byte aligned rows; every other problem runs on the
-  // generic kernel.
+  // The streaming kernels need head_dim 64 and 16-byte aligned rows; the register-copy kernels
+  // take every other problem, with 16-byte accesses where rows and head_dim allow them.
   const int vec = (dtype == LH_F32) ? 4 : 8;  // elements per 16-byte access
   // (the kernels mask a partial last key tile and skip rows past the end themselves)
-  bool vec_ok = true;
-  for (int i = 0; i < 4 && vec_ok; ++i)
-    vec_ok = ss[i]->t % vec == 0 && ss[i]->h % vec == 0 && ss[i]->z % vec == 0 && aligned16(ps[i]) &&
-             ss[i]->t < (1 << 24);  // (a key tile's rows are addressed with 32-bit byte offsets)
-  const bool fast = vec_ok && d == kHeadDim;
+  bool aligned = true, near = true;
+  for (int i = 0; i < 4; ++i) {
+    aligned = aligned && ss[i]->t % vec == 0 && ss[i]->h % vec == 0 && ss[i]->z % vec == 0 && aligned16(ps[i]);
+    near = near && ss[i]->t < (1 << 24);  // (the streaming kernels address a key tile's rows with 32-bit byte offsets)
+  }
+  const bool fast = aligned && near && d == kHeadDim;
   if (scale <= 0.0f) scale = 1.0f / sqrtf((float)d);
   AttnArgs a;
   a.out = out; a.q = q; a.k = k; a.v = v;
@@ -1796,12 +1808,11 @@ static int attention_run(void* out, const void* q, const void* k, const void* v,
              "and aligned rows", kHeadDim);
   a.cus = num_cus();
   if (!fast) {
-    if (vec_ok) {  // another head dimension that a matrix-core kernel takes
-      const hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-      const int rc = dtype == LH_F32 ? attention32_anyd(a, (int)d, st) : attention16_anyd(a, (int)d, dtype, st);
-      if (rc <= 0) return rc;
-    }
-    return attention_generic_launch(a, (int)d, dtype, reinterpret_cast<hipStream_t>(stream));
+    const hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const bool chunks = aligned && d % vec == 0;
+    const int rc = dtype == LH_F32 ? attention32_anyd(a, (int)d, chunks, st) : attention16_anyd(a, (int)d, dtype, chunks, st);
+    if (rc > 0) return fail(LH_ERR_UNSUPPORTED, "lh_hip_attention: no kernel for head_dim %lld", (long long)d);
+    return rc;
   }
   return attention_launch(a, dtype, reinterpret_cast<hipStream_t>(stream));
 }

@@ -295,13 +295,51 @@ def test_attention_f32_head_dim_128_runs_at_matrix_core_speed():
 
 
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype,elt,rtol", [(torch.bfloat16, "bf16", 2e-2), (torch.float16, "f16", 2e-2),
+                                            (torch.float32, "f32", 1e-4)])
+@pytest.mark.parametrize("shape", [(1, 2, 100, 1), (2, 1, 77, 3), (1, 1, 130, 7), (1, 2, 200, 33), (1, 3, 257, 64),
+                                   (1, 1, 131, 65), (2, 2, 64, 100), (1, 1, 300, 129), (1, 1, 140, 161), (1, 1, 70, 200),
+                                   (1, 1, 129, 255), (1, 2, 192, 256)])
+def test_attention_any_head_dim_and_alignment(shape, dtype, elt, rtol, causal):
+    """Head dimensions that are no multiple of 8 (16-bit) or 4 (f32), and rows that are not 16-byte
+    aligned, run on the matrix-core kernels with element loads and stores.  The tensors are views
+    that start one element into buffers with an odd row stride; the other columns hold NaN
+    (inputs) or a marker (output): the result is that of the head dimension itself, whatever the
+    alignment, and nothing outside it is written."""
+    from lighthouse_amd import ops
+
+    Z, H, T, D = shape
+    W = D + 3 + 2 * ((T + D) % 3)  # odd or even row stride, never a multiple of 16 bytes past an aligned start
+    rng = np.random.default_rng(sum(shape) + 7 * causal)
+    q, k, v = (orc.round_to(rng.standard_normal(shape).astype(np.float32), elt) for _ in range(3))
+    ref = orc.attention(q, k, v, causal=causal, result_type=elt)
+
+    def shifted(x):
+        buf = torch.full((Z, H, T, W), float("nan"), dtype=dtype, device="cuda")
+        buf[..., 1:1 + D] = _dev(x, dtype)
+        return buf[..., 1:1 + D]
+
+    out_buf = torch.full((Z, H, T, W), 7.0, dtype=dtype, device="cuda")
+    out = out_buf[..., 1:1 + D]
+    ops.attention(shifted(q), shifted(k), shifted(v), causal=causal, out=out)
+    assert_close(_host(out), ref, rtol, f"attention {shape} {elt} causal={causal}")
+    assert torch.all(out_buf[..., :1] == 7.0) and torch.all(out_buf[..., 1 + D:] == 7.0), "columns outside the view were written"
+    # contiguous tensors (aligned rows when head_dim allows) run the same kernel with wider accesses: the
+    # same bits (64 and 128 have streaming kernels of their own, with other rounding points)
+    out_c = ops.attention(_dev(q, dtype), _dev(k, dtype), _dev(v, dtype), causal=causal)
+    if D in (64, 128):
+        assert_close(_host(out_c), ref, rtol, f"attention {shape} {elt} causal={causal} contiguous")
+    else:
+        assert torch.equal(out_c, out)
+
+
+@pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("dtype,elt,rtol", [(torch.bfloat16, "bf16", 2e-2), (torch.float32, "f32", 1e-4)])
 @pytest.mark.parametrize("shape", [(1, 2, 100, 40), (2, 1, 77, 64), (1, 1, 130, 128), (1, 3, 64, 64), (1, 1, 1, 8),
                                    (1, 1, 200, 256), (1, 2, 100, 36), (1, 1, 70, 100), (1, 1, 33, 3)])
 def test_attention_any_shape(shape, dtype, elt, rtol, causal):
-    """Head dimensions the MFMA kernels do not take (16-bit: not a multiple of 8; f32: not a multiple
-    of 4) run on the generic kernel with the same rounding points; the others take the MFMA kernels at
-    any sequence length."""
+    """Small and odd shapes of every kind: each takes a matrix-core kernel (16-byte accesses where
+    rows and head_dim allow them, element accesses otherwise)."""
     from lighthouse_amd import ops
 
     rng = np.random.default_rng(sum(shape) + causal)
