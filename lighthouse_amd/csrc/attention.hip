@@ -58,7 +58,7 @@ __device__ __forceinline__ f32x16 mfma16(u32x4 a, u32x4 b, f32x16 c) {
 
 constexpr int kHeadDim = 64;
 constexpr int kKvTile = 64;
-constexpr int kQBlock = 128;        // query rows per workgroup of the f32 kernel
+constexpr int kQBlock = 128;        // query rows per workgroup of the f32 kernel and of the register-copy kernels
 constexpr int kQBlock16 = 256;      // query rows per workgroup of the 16-bit kernel (4 waves x 64)
 constexpr int kAttnStageBytes = 2 * kKvTile * kHeadDim * 2;  // K tile + V tile, 16 KiB
 constexpr float kOffsetSlack = 1024.0f;  // largest partial row sum of P the softmax offset tolerates
@@ -589,215 +589,6 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
         *reinterpret_cast<u32x2*>(orow + 32 * j + 8 * g + 4 * h) = w;
       }
   }
-}
-
-// f32 variant (all tensors f32, v_mfma_f32_32x32x2_f32): same transposed formulation; P stays
-// f32.  A workgroup owns 128 query rows (4 waves x 32).  K and V tiles of 64 keys keep their
-// global orientation in LDS (rows of 256 bytes), loaded with global_load_lds_dwordx4 one tile
-// ahead into the other of two 32 KiB stages.  Unpadded rows again: the 16-byte chunk a lane
-// fetches is XOR-swizzled, K chunk ^ (key % 16) (a lane reads 4 consecutive d of its key row),
-// V chunk ^ 8 ((key / 4) % 2) (the two half waves read rows 4 apart at the same columns).
-constexpr int kAttn32StageBytes = 2 * kKvTile * kHeadDim * 4;  // K tile + V tile
-
-struct Attn32Ctx {
-  const float* k_src[4];
-  const float* v_src[4];
-  int64_t k_step, v_step;
-  int64_t k_row, v_row;  // elements per key, for the clamped loads of a partial last tile
-  int key_local[4];      // the key of the tile that load i of this lane fetches
-  int wave, r32, h;
-  int k_off[2], k_swz[2];
-  int v_col[2];  // byte offset of the lane's V column inside a row, per head-dim sub-tile (unswizzled half)
-};
-
-
-// RAGGED: as in the 16-bit kernel, keys past the end of the sequence are fetched from the last key.
-template <bool RAGGED>
-__device__ __forceinline__ void attn32_issue(const Attn32Ctx& c, int jt, int T, uint8_t* __restrict__ stage) {
-  // (The global form of the LDS-DMA load: this kernel measured 3 % slower with the buffer form
-  // that the 16-bit kernels use, [8,12,1024,64] causal 129 -> 133 us.)
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int64_t k_off = jt * c.k_step, v_off = jt * c.v_step;
-    if constexpr (RAGGED) {
-      const int back = max(jt * kKvTile + c.key_local[i] - (T - 1), 0);
-      k_off -= back * c.k_row;
-      v_off -= back * c.v_row;
-    }
-    __builtin_amdgcn_global_load_lds(c.k_src[i] + k_off, (attn_lds_void_t*)(stage + (4 * i + c.wave) * 1024), 16, 0, 0);
-    __builtin_amdgcn_global_load_lds(c.v_src[i] + v_off, (attn_lds_void_t*)(stage + 16384 + (4 * i + c.wave) * 1024), 16,
-                                     0, 0);
-  }
-}
-
-// One key tile for the wave's 32 query rows; `wr` receives the next tile meanwhile.
-template <bool RAGGED>
-__device__ __forceinline__ void attn32_tile(const Attn32Ctx& c, const AttnArgs& a, const f32x4 (&qf)[8],
-                                            f32x16 (&acc_o)[2], float& m_run, float& l_run,
-                                            const uint8_t* __restrict__ rd, uint8_t* __restrict__ wr, int next_jt,
-                                            bool prefetch, int j0, int wq0, bool active, bool need_mask) {
-  if (prefetch) attn32_issue<RAGGED>(c, next_jt, a.T, wr);
-  if (!active) return;
-  const uint8_t* ks = rd;
-  const uint8_t* vs = rd + 16384;
-  f32x16 s_acc[2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) s_acc[i][v] = 0.0f;
-  // The two key sub-tiles alternate so that consecutive MFMAs never depend on each other.
-#pragma unroll
-  for (int kk = 0; kk < 8; ++kk) {
-    f32x4 kf[2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-      kf[i] = *reinterpret_cast<const f32x4*>(ks + c.k_off[i] + (((2 * kk + c.h) ^ c.k_swz[i]) << 4));
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-        s_acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[i][t], qf[kk][t], s_acc[i], 0, 0, 0);
-  }
-  // s_acc[i][v] = S[q = wq0 + r32][key = j0 + 32 i + 8 (v/4) + 4 h + v%4] (unscaled)
-  if (need_mask) {
-    // last visible key of the row: its own index under the causal mask, and never past the end
-    const int last = a.causal ? min(wq0 + c.r32, a.T - 1) : a.T - 1;
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        int key = j0 + 32 * i + 8 * (v >> 2) + 4 * c.h + (v & 3);
-        if (key > last) s_acc[i][v] = -INFINITY;
-      }
-  }
-  float mx = fmaxf(s_acc[0][0], s_acc[1][0]);
-#pragma unroll
-  for (int v = 1; v < 16; ++v) mx = fmaxf(fmaxf(mx, s_acc[0][v]), s_acc[1][v]);
-  mx = halfwave_max(mx);
-  const float m_new = fmaxf(m_run, mx);
-  const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-  // exp(x) as exp2(x log2 e): v_exp_f32 is accurate to about 1 ulp, the scaled argument (|x| < 100)
-  // to 1e-5 absolute, well inside the f32 tolerance of the payload.
-  const float alpha = exp2_fast((m_run - m_safe) * a.scale_log2e);
-  const float mc = m_safe * a.scale_log2e;
-  float l_tile = 0.0f;
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      s_acc[i][v] = exp2_fast(s_acc[i][v] * a.scale_log2e - mc);
-      l_tile += s_acc[i][v];
-    }
-  l_run = l_run * alpha + l_tile;
-  m_run = m_new;
-#pragma unroll
-  for (int j = 0; j < 2; ++j)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc_o[j][v] *= alpha;
-  // O^T += V^T P^T, one key (pair) per MFMA: lane (d = r32, half h) reads V[key][32 j + r32].
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      const int key = 32 * i + 8 * (v >> 2) + 4 * c.h + (v & 3);  // (key / 4) % 2 == h
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        float vf = *reinterpret_cast<const float*>(vs + key * 256 + c.v_col[j]);
-        acc_o[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf, s_acc[i][v], acc_o[j], 0, 0, 0);
-      }
-    }
-}
-
-// RAGGED: T is no multiple of the 128-row query block; the last key tile may be partial, rows past
-// the end compute on the last row and are not stored, and a wave entirely past the end only takes
-// part in the loads and barriers.
-template <bool RAGGED>
-__global__ void __launch_bounds__(256) attention32_kernel(AttnArgs a) {
-  extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn32[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r32 = lane & 31, h = lane >> 5;
-  const int nqb = (a.T + kQBlock - 1) / kQBlock;
-  int qb, bh;
-  if (a.causal) causal_block_of(blockIdx.x, gridDim.x, a.cus, nqb, a.Z * a.H, qb, bh);
-  else xcd_block_of((int)(blockIdx.y * gridDim.x + blockIdx.x), nqb, a.Z * a.H, qb, bh);
-  const int z = bh / a.H, hd = bh % a.H;
-  const int q0 = qb * kQBlock;
-  const int wq0 = q0 + wave * 32;
-  const bool wave_valid = !RAGGED || wq0 < a.T;
-  const float* Q = reinterpret_cast<const float*>(a.q) + (int64_t)z * a.sq.z + (int64_t)hd * a.sq.h;
-  const float* K = reinterpret_cast<const float*>(a.k) + (int64_t)z * a.sk.z + (int64_t)hd * a.sk.h;
-  const float* V = reinterpret_cast<const float*>(a.v) + (int64_t)z * a.sv.z + (int64_t)hd * a.sv.h;
-  float* O = reinterpret_cast<float*>(a.out) + (int64_t)z * a.so.z + (int64_t)hd * a.so.h;
-
-  Attn32Ctx c;
-  c.wave = wave; c.r32 = r32; c.h = h;
-  c.k_step = (int64_t)kKvTile * a.sk.t;
-  c.v_step = (int64_t)kKvTile * a.sv.t;
-  c.k_row = a.sk.t;
-  c.v_row = a.sv.t;
-  // Loader: load i of wave w fills keys (4 i + w) 4 .. +4; lane -> key += lane / 16, LDS chunk
-  // p = lane % 16 holds global chunk p ^ swizzle(key).
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int key = (4 * i + wave) * 4 + (lane >> 4);
-    const int p = lane & 15;
-    c.key_local[i] = key;
-    c.k_src[i] = K + (int64_t)key * a.sk.t + ((p ^ (key & 15)) << 2);
-    c.v_src[i] = V + (int64_t)key * a.sv.t + ((p ^ (8 * ((key >> 2) & 1))) << 2);
-  }
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int key = 32 * i + r32;
-    c.k_off[i] = key * 256;
-    c.k_swz[i] = key & 15;
-  }
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int col = 32 * j + r32;
-    c.v_col[j] = (((col >> 2) ^ (8 * h)) << 4) + (col & 3) * 4;
-  }
-
-  // Lane (q = r32, half h) holds Q[q][8 kk + 4 h + t], kk = 0..7, t = 0..3.
-  f32x4 qf[8];
-#pragma unroll
-  for (int kk = 0; kk < 8; ++kk)
-    qf[kk] = *reinterpret_cast<const f32x4*>(Q + (int64_t)(RAGGED ? min(wq0 + r32, a.T - 1) : wq0 + r32) * a.sq.t +
-                                             8 * kk + 4 * h);
-
-  f32x16 acc_o[2];
-#pragma unroll
-  for (int j = 0; j < 2; ++j)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc_o[j][v] = 0.0f;
-  float m_run = -INFINITY, l_run = 0.0f;
-  const int kv_end = a.causal ? min(a.T, q0 + kQBlock) : a.T;
-  const int ntiles = (kv_end + kKvTile - 1) / kKvTile;
-
-  attn32_issue<RAGGED>(c, 0, a.T, smem_attn32);
-  for (int jt = 0; jt < ntiles; ++jt) {
-    // Tile jt is the only load in flight: wait for it, and the barrier also says every wave is
-    // done reading the stage the next tile is about to overwrite.
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    const int j0 = jt * kKvTile;
-    const bool active = wave_valid && (!a.causal || (j0 <= wq0 + 31));
-    const bool need_mask = (a.causal && (j0 + kKvTile - 1 > wq0)) || (RAGGED && j0 + kKvTile > a.T);
-    attn32_tile<RAGGED>(c, a, qf, acc_o, m_run, l_run, smem_attn32 + (jt & 1) * kAttn32StageBytes,
-                smem_attn32 + ((jt + 1) & 1) * kAttn32StageBytes, jt + 1, jt + 1 < ntiles, j0, wq0, active, need_mask);
-  }
-
-  if (!wave_valid) return;
-  const float inv_l = 1.0f / halfwave_sum(l_run);
-  if (RAGGED && wq0 + r32 >= a.T) return;  // (after the cross-lane sum, which needs every lane)
-  float* orow = O + (int64_t)(wq0 + r32) * a.so.t;
-#pragma unroll
-  for (int j = 0; j < 2; ++j)
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      f32x4 w = {acc_o[j][4 * g] * inv_l, acc_o[j][4 * g + 1] * inv_l, acc_o[j][4 * g + 2] * inv_l,
-                 acc_o[j][4 * g + 3] * inv_l};
-      *reinterpret_cast<f32x4*>(orow + 32 * j + 8 * g + 4 * h) = w;
-    }
 }
 
 template <int DT, int NQ, int NS, bool RAGGED, int KS = 1, bool SX = false>
@@ -1522,18 +1313,21 @@ int attention16_anyd(const AttnArgs& a, int d, int dtype, bool chunks, hipStream
   return 1;
 }
 
-// f32 tensors, head dimensions that are multiples of 4 up to 256, other than 64
-// (v_mfma_f32_32x32x2_f32, D = 32 DB columns): the structure of attention16_anyd_kernel.  A
-// workgroup owns 128 query rows (4 waves x 32); K and V tiles of 64 keys are copied through
-// registers into LDS rows of D + 8 floats (with that pad the V reads of the two half waves, 4 key
-// rows apart, fall on different banks), two barriers per tile.  The copy is not overlapped with
-// the arithmetic of the same workgroup: a tile is 2 D MFMAs of 64 cycles per wave, and up to
-// D = 128 a second workgroup on the CU computes meanwhile.  Scores are scaled in f32 after the
-// product, P stays f32 and the statistics follow the plain online-softmax recurrence, exactly as
-// in attention32_kernel.  Q fragments live in registers up to D = 96; above, each tile re-reads
-// them from global memory (32 KiB per wave at most, cache hits) and the registers go to the output
-// accumulators.  Any sequence length: keys past the end are loaded from
-// the last key and masked, rows past the end are computed on the last row and not stored.
+// f32 tensors (all of Q, K, V and the output f32; v_mfma_f32_32x32x2_f32, D = 32 DB columns): the
+// structure of attention16_anyd_kernel, with P kept in f32.  A workgroup owns 128 query rows
+// (4 waves x 32); K and V tiles of 64 keys are copied through registers into LDS rows of D + 8
+// floats (with that pad the V reads of the two half waves, 4 key rows apart, fall on different
+// banks), two barriers per tile.  The copy is not overlapped with the arithmetic of the same
+// workgroup: a tile is 2 D MFMAs of 64 cycles per wave, and up to D = 128 a second workgroup on
+// the CU computes meanwhile.  (For D = 64 a kernel that streamed the tiles by LDS-DMA one tile ahead
+// into a second stage measured 1.5 to 3.5 % slower than this one, [4,16,2048,64] 612 against 600 us,
+// and is gone.)  Scores are scaled in f32 after the product (exp(x) as exp2(x log2 e): v_exp_f32 is
+// accurate to about 1 ulp and the scaled argument, |x| < 100, to 1e-5 absolute, well inside the f32
+// tolerance of the payload); the statistics follow the plain online-softmax recurrence.  Q
+// fragments live in registers up to D = 96; above, each tile re-reads them from global memory
+// (32 KiB per wave at most, cache hits) and the registers go to the output accumulators.  Any
+// sequence length: keys past the end are loaded from the last key and masked, rows past the end are
+// computed on the last row and not stored.
 // ROWS != kRowsExact: the head dimension a.d lies below D (or the rows are not 16-byte aligned); the
 // columns of Q, K and V from a.d on are zeros, and output columns from a.d on are not stored.
 template <int DB, int ROWS>
@@ -1548,10 +1342,12 @@ __global__ void __launch_bounds__(256, (DB <= 4 ? 2 : 1)) attention32_anyd_kerne
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r32 = lane & 31, h = lane >> 5;
   const int nqb = (a.T + kQBlock - 1) / kQBlock;
-  // (launch order as in attention16_anyd_kernel: causal blocks heaviest first)
+  // Causal blocks heaviest first; where two (three) workgroups fit a CU, a grid of up to two (three) per
+  // CU is resident at once and is dealt so that the CUs' sums stay level.
   const int bhn = a.Z * a.H;
   int qb = nqb - 1 - (int)blockIdx.x / bhn, bh = (int)blockIdx.x % bhn;
   if (!a.causal) xcd_block_of((int)(blockIdx.y * gridDim.x + blockIdx.x), nqb, bhn, qb, bh);
+  else if constexpr (DB <= 4) causal_block_of(blockIdx.x, gridDim.x, a.cus, nqb, bhn, qb, bh, DB <= 2);
   const int z = bh / a.H, hd = bh % a.H;
   const int q0 = qb * kQBlock, wq0 = q0 + 32 * wave;
   const bool wave_valid = wq0 < a.T;
@@ -1737,23 +1533,7 @@ constexpr int kMaxHeadDim = 256;
 
 int attention_launch(const AttnArgs& a, int dtype, hipStream_t s) {
   if (dtype == LH_BF16) return attention16_launch<LH_BF16>(a, s);
-  if (dtype == LH_F16) return attention16_launch<LH_F16>(a, s);
-  const int nqb32 = (a.T + kQBlock - 1) / kQBlock;
-  const dim3 grid32 = a.causal ? dim3(nqb32 * a.Z * a.H) : dim3(nqb32, a.Z * a.H);
-  auto launch = [&](auto kern, bool& configured) -> int {
-    if (!configured && !planning()) {
-      LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       2 * kAttn32StageBytes));
-      configured = true;
-    }
-    LH_LAUNCH(kern, grid32, dim3(256), 2 * kAttn32StageBytes, s, a);
-    return 0;
-  };
-  static bool configured_whole = false, configured_ragged = false;
-  const int rc = a.T % kQBlock == 0 ? launch(attention32_kernel<false>, configured_whole)
-                                    : launch(attention32_kernel<true>, configured_ragged);
-  if (rc) return rc;
-  return check_launch("attention32");
+  return attention16_launch<LH_F16>(a, s);
 }
 
 }  // namespace lh
@@ -1775,8 +1555,8 @@ static int attention_run(void* out, const void* q, const void* k, const void* v,
   const lh_strides3* ss[4] = {&so, &sq, &sk, &sv};
   const void* ps[4] = {out, q, k, v};
   for (int i = 0; i < 4; ++i) LH_REQUIRE(ss[i]->t >= d, "lh_hip_attention: row stride of tensor %d is below head_dim", i);
-  // The streaming kernels need head_dim 64 and 16-byte aligned rows; the register-copy kernels
-  // take every other problem, with 16-byte accesses where rows and head_dim allow them.
+  // The streaming kernels need 16-bit tensors, head_dim 64 and 16-byte aligned rows; the register-copy
+  // kernels take every other problem, with 16-byte accesses where rows and head_dim allow them.
   const int vec = (dtype == LH_F32) ? 4 : 8;  // elements per 16-byte access
   // (the kernels mask a partial last key tile and skip rows past the end themselves)
   bool aligned = true, near = true;
@@ -1784,7 +1564,7 @@ static int attention_run(void* out, const void* q, const void* k, const void* v,
     aligned = aligned && ss[i]->t % vec == 0 && ss[i]->h % vec == 0 && ss[i]->z % vec == 0 && aligned16(ps[i]);
     near = near && ss[i]->t < (1 << 24);  // (the streaming kernels address a key tile's rows with 32-bit byte offsets)
   }
-  const bool fast = aligned && near && d == kHeadDim;
+  const bool fast = aligned && near && d == kHeadDim && dtype != LH_F32;
   if (scale <= 0.0f) scale = 1.0f / sqrtf((float)d);
   AttnArgs a;
   a.out = out; a.q = q; a.k = k; a.v = v;
@@ -1803,7 +1583,7 @@ static int attention_run(void* out, const void* q, const void* k, const void* v,
   a.causal = (causal & LH_ATTN_CAUSAL) ? 1 : 0;
   a.request = causal & (LH_ATTN_ROWS_MASK | LH_ATTN_STAGES_MASK | LH_ATTN_KSPLIT_MASK);
   a.scale_f32 = (causal & LH_ATTN_SCALE_F32) != 0;
-  LH_REQUIRE((a.request == 0 && !a.scale_f32) || (fast && dtype != LH_F32),
+  LH_REQUIRE((a.request == 0 && !a.scale_f32) || fast,
              "lh_hip_attention: query-row / ring-depth / score-scaling requests apply to 16-bit tensors with head_dim %d "
              "and aligned rows", kHeadDim);
   a.cus = num_cus();
