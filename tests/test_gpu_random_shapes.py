@@ -129,7 +129,8 @@ def test_gemm_fp8_random_shapes_are_exact(seed):
 @pytest.mark.parametrize("seed", range(3))
 def test_attention_random_shapes_and_layouts(seed):
     """Random [Z,H,T,d] problems (every kernel family: head dimension 64, 128, other multiples of 32,
-    anything else), causal or not, in three memory layouts; the row after the last query must survive."""
+    of 8 and of 4, anything else), causal or not, in four memory layouts (one of them misaligned, inside
+    NaN padding); the row after the last query must survive."""
     from lighthouse_amd import ops
     from tests.conftest import assert_close
 
@@ -138,13 +139,13 @@ def test_attention_random_shapes_and_layouts(seed):
     for case in range(25):
         kind = rnd.choice(["bf16", "bf16", "f16", "f32"])
         dt = _DT[kind]
-        d = rnd.choice([64, 64, 64, 128, 128, 32, 96, 192, 256, 40, 80, 16, 100])
+        d = rnd.choice([64, 64, 64, 128, 128, 32, 96, 192, 256, 40, 80, 16, 100, 36, 7, 65, 130, 255])
         z, h = rnd.randint(1, 3), rnd.randint(1, 6)
         t = rnd.choice([rnd.randint(1, 300), 64 * rnd.randint(1, 12), 256 * rnd.randint(1, 4), rnd.randint(1, 1100)])
         while z * h * t * t * d > (1 << 28):
             t = max(1, t // 2)
         causal = rnd.random() < 0.5
-        layout = rnd.choice(["zhtd", "zthd", "packed"])
+        layout = rnd.choice(["zhtd", "zthd", "packed", "shifted"])
         what = f"seed {seed} case {case}: {kind} Z={z} H={h} T={t} d={d} causal={causal} {layout}"
         host = orc.round_to(rng.standard_normal((3, z, h, t, d)).astype(np.float32), kind)
         if layout == "zhtd":
@@ -152,6 +153,10 @@ def test_attention_random_shapes_and_layouts(seed):
         elif layout == "zthd":
             q, k, v = (torch.from_numpy(host[i]).to("cuda").to(dt).transpose(1, 2).contiguous().transpose(1, 2)
                        for i in range(3))
+        elif layout == "shifted":  # views that start one element into rows of d + 3 elements; NaN around them
+            wide = torch.full((3, z, h, t, d + 3), float("nan"), device="cuda", dtype=dt)
+            wide[..., 1:1 + d] = torch.from_numpy(host).to("cuda").to(dt)
+            q, k, v = (wide[i, ..., 1:1 + d] for i in range(3))
         else:  # one [Z, T, 3, H, d] tensor, as the fused QKV projection of the nanoGPT block leaves it
             packed = torch.from_numpy(host).to("cuda").to(dt).permute(1, 3, 0, 2, 4).contiguous()
             q, k, v = (packed[:, :, i].transpose(1, 2) for i in range(3))
