@@ -42,6 +42,10 @@ struct AttnArgs {
   // offset, row sum) in `part`; attention16_merge combines them.  1: one workgroup per query block.
   int kv_groups = 1;
   float* part = nullptr;
+  // Causal launches of up to a third more query blocks than fit the CUs at once (32 rows per wave,
+  // three workgroups per CU): the grid is `chain` = 3 x CUs workgroups, all resident, and the first
+  // third of them take a second query block each (see attention16_kernel).  0: one block per workgroup.
+  int chain = 0;
   bool allow_grid_split = true;  // the caller lets the launch take temporary memory for it
   Scratch* ws = nullptr;         // where that memory comes from: a caller workspace, or (nullptr) the stream's pool
 };
@@ -350,13 +354,26 @@ __device__ __forceinline__ void xcd_block_of(int L, int nqb, int bhn, int& qb, i
 // output, offset, row sum) over through LDS and the first combines the two.  Same waves per CU as
 // two workgroups of 4, but the two halves of a query block's key range run side by side and end
 // together: the chain of key tiles a causal problem's heaviest query block has to walk is half as long.
+// GS = 2 (causal, NQ = 1, NS = 3): a workgroup may take a second query block (see the loop below).
 // GS = 1: the key range of a query block is split between a.kv_groups WORKGROUPS (1-D grid, query
 // blocks heaviest first, the groups of one block next to each other); each leaves its partial
 // result in a.part and attention16_merge finishes the block.
 template <int DT, int NQ, int NS, bool RAGGED, int KS = 1, int GS = 0, bool SX = false>
-__global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attention16_kernel(AttnArgs a) {
-  static_assert(!(SX && (KS != 1 || GS)), "scores scaled in f32: one group of four waves per workgroup, no grid split");
-  static_assert(!(GS && (KS != 1 || RAGGED)), "the grid split runs four waves per workgroup on whole key tiles");
+__global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attention16_kernel(AttnArgs a_arg) {
+  static_assert(!(SX && (KS != 1 || GS == 1)), "scores scaled in f32: one group of four waves per workgroup, no grid split");
+  static_assert(!(GS == 1 && (KS != 1 || RAGGED)), "the grid split runs four waves per workgroup on whole key tiles");
+  static_assert(GS != 2 || (NQ == 1 && NS == 3 && KS == 1), "second query blocks: the 32-rows-per-wave kernel with three workgroups per CU");
+  // The instantiation whose workgroups may take a second query block reads its arguments through
+  // the kernel argument pointer, made opaque once per block: the argument loads then stay inside the
+  // loop over the blocks (held across it they cost 30 scalar registers more than there are, and
+  // their spills the last vector registers of a kernel that runs three waves per SIMD).
+  constexpr bool chained = GS == 2;
+  typedef const __attribute__((address_space(4))) AttnArgs* kernarg_ptr_t;
+  kernarg_ptr_t arg_ptr = (kernarg_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();
+  const int chain_nqb = (a_arg.T + 32 * NQ * 4 - 1) / (32 * NQ * 4), chain_bhn = a_arg.Z * a_arg.H, chain_s = a_arg.chain;
+  for (int link = 0;; ++link) {
+  if constexpr (chained) asm volatile("" : "+s"(arg_ptr));
+  const AttnArgs& a = chained ? *(const AttnArgs*)arg_ptr : a_arg;
   constexpr int kRowsPerWave = 32 * NQ, kRowsPerGroup = 4 * kRowsPerWave;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem_attn_all[];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -365,8 +382,31 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
   uint8_t* const smem_attn = smem_attn_all + ksplit * (NS * kAttnStageBytes);
   const int r32 = lane & 31, h = lane >> 5;
   const int nqb = (a.T + kRowsPerGroup - 1) / kRowsPerGroup;
+  // Chained causal launch (a.chain = S = 3 R workgroups for R CUs, resident at once, workgroup L on CU
+  // L % R; at most 4 R query blocks, ranked heaviest first): the first block of a workgroup is dealt
+  // as causal_block_of deals three per CU (CU c: ranks c, 2 R - 1 - c, 2 R + c), and the blocks
+  // beyond 3 R go to the workgroups that hold the heaviest, lightest to heaviest (rank 4 R - 1 - c
+  // after rank c), so that every CU has the same number of key tiles from the start.  With one
+  // block per workgroup those blocks start wherever a slot frees first, 30 us into a [4,16,2048]
+  // launch, and the launch ends with a quarter of the CUs working on them alone: 45.7 -> 43.7 us.
+  // (Appended to the CU's lightest workgroup instead: 45.9; to the middle one: 48.5.  The oldest
+  // workgroup of a CU wins the contested issue slots and walks its chain at a lone workgroup's pace,
+  // 1.09 us per tile, whatever else the CU holds; the younger ones share what is left.)
   int qb, bh, grp = 0;
-  if constexpr (GS) {
+  if constexpr (chained) {
+    const int R = chain_s / 3, L = (int)blockIdx.x;
+    int r = L;
+    if (link == 0) {
+      if (L >= R && L < 2 * R) r = 3 * R - 1 - L;
+    } else {
+      r = (link == 1 && L < R) ? 4 * R - 1 - L : chain_nqb * chain_bhn;
+    }
+    if (r >= chain_nqb * chain_bhn) break;
+    qb = chain_nqb - 1 - r / chain_bhn;
+    bh = r % chain_bhn;
+    // (every wave has left the rings of the block before)
+    if (link > 0) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  } else if constexpr (GS == 1) {
     const int per = a.Z * a.H * a.kv_groups, rem = (int)blockIdx.x % per;
     qb = nqb - 1 - (int)blockIdx.x / per;
     bh = rem / a.kv_groups;
@@ -464,11 +504,11 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
   // This group's key tiles are t_first .. t_first + ntiles - 1; every wave of the workgroup walks
   // `steps` iterations (the larger of the two counts), because the barrier in the loop is the
   // workgroup's: a group that has run out of tiles neither loads nor computes in the rest.
-  const int share = GS ? (ntiles_all + a.kv_groups - 1) / a.kv_groups : 0;  // key tiles per workgroup of a split block
-  const int t_first = GS ? grp * share : ksplit * ((ntiles_all + 1) / 2);
-  const int ntiles = GS ? max(0, min(share, ntiles_all - t_first))
+  const int share = GS == 1 ? (ntiles_all + a.kv_groups - 1) / a.kv_groups : 0;  // key tiles per workgroup of a split block
+  const int t_first = GS == 1 ? grp * share : ksplit * ((ntiles_all + 1) / 2);
+  const int ntiles = GS == 1 ? max(0, min(share, ntiles_all - t_first))
                         : (KS == 2 ? (ksplit ? ntiles_all - (ntiles_all + 1) / 2 : (ntiles_all + 1) / 2) : ntiles_all);
-  const int steps = GS ? ntiles : (KS == 2 ? (ntiles_all + 1) / 2 : ntiles_all);
+  const int steps = GS == 1 ? ntiles : (KS == 2 ? (ntiles_all + 1) / 2 : ntiles_all);
   constexpr int kAttnStages = NS;  // K/V ring depth, 3 or 4
 #pragma unroll
   for (int st = 0; st < kAttnStages - 1; ++st)
@@ -506,7 +546,7 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
         smem_attn + (nxt % kAttnStages) * kAttnStageBytes, t_first + nxt, nxt < ntiles, j0, wq0, active, need_mask, it == 0);
   }
 
-  if constexpr (GS) {
+  if constexpr (GS == 1) {
     // This workgroup's share of the block: accumulators in the order of the hand-over below
     // (block (wave, qt, j), four 16-byte groups of 64 lanes each), then offsets and row sums.  A
     // workgroup without a visible key tile leaves offset -inf, sum 0 and zeros.
@@ -574,21 +614,24 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
   }
 
   // acc_o[qt][j][v] = O[q = wq0 + 32 qt + r32][d = 32 j + 8 (v/4) + 4 h + v%4] * l
-  if (!wave_valid) return;
+  if (wave_valid) {
 #pragma unroll
-  for (int qt = 0; qt < NQ; ++qt) {
-    const float inv_l = 1.0f / halfwave_sum(l_run[qt]);
-    if (RAGGED && wq0 + 32 * qt + r32 >= a.T) continue;  // (after the cross-lane sum, which needs every lane)
-    uint16_t* orow = O + (int64_t)(wq0 + 32 * qt + r32) * a.so.t;
+    for (int qt = 0; qt < NQ; ++qt) {
+      const float inv_l = 1.0f / halfwave_sum(l_run[qt]);
+      if (RAGGED && wq0 + 32 * qt + r32 >= a.T) continue;  // (after the cross-lane sum, which needs every lane)
+      uint16_t* orow = O + (int64_t)(wq0 + 32 * qt + r32) * a.so.t;
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w = {pack2<DT>(acc_o[qt][j][4 * g] * inv_l, acc_o[qt][j][4 * g + 1] * inv_l),
-                   pack2<DT>(acc_o[qt][j][4 * g + 2] * inv_l, acc_o[qt][j][4 * g + 3] * inv_l)};
-        *reinterpret_cast<u32x2*>(orow + 32 * j + 8 * g + 4 * h) = w;
-      }
+        for (int g = 0; g < 4; ++g) {
+          u32x2 w = {pack2<DT>(acc_o[qt][j][4 * g] * inv_l, acc_o[qt][j][4 * g + 1] * inv_l),
+                     pack2<DT>(acc_o[qt][j][4 * g + 2] * inv_l, acc_o[qt][j][4 * g + 3] * inv_l)};
+          *reinterpret_cast<u32x2*>(orow + 32 * j + 8 * g + 4 * h) = w;
+        }
+    }
   }
+  if (!chained) break;
+  }  // (the workgroup's next query block)
 }
 
 template <int DT, int NQ, int NS, bool RAGGED, int KS = 1, bool SX = false>
@@ -596,6 +639,8 @@ static int attention16_launch_ragged(const AttnArgs& a, hipStream_t s) {
   if constexpr (KS == 1 && !SX) {
     if (a.scale_f32) return attention16_launch_ragged<DT, NQ, NS, RAGGED, 1, true>(a, s);
   }
+  constexpr bool kCanChain = NQ == 1 && NS == 3 && KS == 1;
+  const bool chained = kCanChain && a.causal && a.chain > 0;
   auto kern = attention16_kernel<DT, NQ, NS, RAGGED, KS, 0, SX>;
   constexpr size_t lds = (size_t)KS * NS * kAttnStageBytes;
   static bool configured = false;
@@ -605,6 +650,19 @@ static int attention16_launch_ragged(const AttnArgs& a, hipStream_t s) {
     configured = true;
   }
   const int nqb = (a.T + 128 * NQ - 1) / (128 * NQ);
+  if constexpr (kCanChain) {
+    if (chained) {
+      auto kern2 = attention16_kernel<DT, NQ, NS, RAGGED, KS, 2, SX>;
+      static bool configured2 = false;
+      if (!configured2 && !planning()) {
+        LH_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern2), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)lds));
+        configured2 = true;
+      }
+      LH_LAUNCH(kern2, dim3(a.chain), dim3(256 * KS), lds, s, a);
+      return check_launch("attention16");
+    }
+  }
   const dim3 grid = a.causal ? dim3(nqb * a.Z * a.H) : dim3(nqb, a.Z * a.H);
   LH_LAUNCH(kern, grid, dim3(256 * KS), lds, s, a);
   return check_launch("attention16");
@@ -778,7 +836,17 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
     // 22.3); a problem that cannot put a third one there is better off with the deeper ring
     // (causal [1,16,4096] 57.9 -> 53.9 us, [1,8,8192] 108 -> 98.8, [2,16,2048] 32.7 -> 30.6, [1,40,2048] 36.2 -> 33.7).
     const int64_t groups32 = (int64_t)((a.T + 127) / 128) * a.Z * a.H;
-    if (groups32 >= 3 * (int64_t)a.cus) return attention16_launch_nq<DT, 1, 3>(a, s);
+    if (groups32 >= 3 * (int64_t)a.cus) {
+      // Causal, 3.5 to 4 per CU, sequences from 1000 on: all resident, a second block for a third of them
+      // ([4,16,2048] 45.7 -> 43.7 us, [2,16,4096] 80.9 -> 77.8, [7,16,1024] 25.8 -> 24.9, [7,18,1000] 32.2 -> 29.6;
+      // at 3.25 per CU, or with 512-key sequences, the plain launch is 2-3 % ahead).
+      if (a.causal && a.T >= 1000 && 2 * groups32 >= 7 * (int64_t)a.cus && groups32 <= 4 * (int64_t)a.cus) {
+        AttnArgs ac = a;
+        ac.chain = 3 * a.cus;
+        return attention16_launch_nq<DT, 1, 3>(ac, s);
+      }
+      return attention16_launch_nq<DT, 1, 3>(a, s);
+    }
     return attention16_launch_nq<DT, 1, 4>(a, s);
   }
   return attention16_launch_nq<DT, 2, 4>(a, s);

@@ -220,6 +220,34 @@ def test_attention_padded_head_dims_on_the_matrix_cores(shape, dtype, elt, causa
     assert torch.equal(out_c, out)
 
 
+@pytest.mark.parametrize("dtype,elt", [(torch.bfloat16, "bf16"), (torch.float16, "f16")])
+@pytest.mark.parametrize("shape", [(14, 8, 1024, 64), (14, 8, 1000, 64), (15, 4, 2048, 64), (2, 16, 4096, 64), (1, 128, 1000, 64)])
+def test_attention_causal_second_block_per_workgroup(shape, dtype, elt):
+    """Causal problems with 3.5 to 4 128-row query blocks per compute unit (256 CUs) and sequences from
+    1000 keys on: every workgroup is resident at once and a third of them take a second query block.
+    Every (batch, head) slice against an f32 evaluation on the GPU, the first and the last one
+    against the f64 oracle; the row after the last query survives."""
+    from lighthouse_amd import ops
+
+    Z, H, T, D = shape
+    g = torch.Generator(device="cuda").manual_seed(sum(shape))
+    q, k, v = (torch.randn(shape, device="cuda", generator=g).to(dtype) for _ in range(3))
+    buf = torch.full((Z, H, T + 1, D), 55.0, device="cuda", dtype=dtype)
+    out = ops.attention(q, k, v, causal=True, out=buf[:, :, :T])
+    assert bool((buf[:, :, T] == 55.0).all()), "wrote past the last query row"
+    mask = torch.ones(T, T, dtype=torch.bool, device="cuda").tril()
+    worst = 0.0
+    for z in range(Z):
+        sc = torch.einsum("hqd,hkd->hqk", q[z].float(), k[z].float()) / D ** 0.5
+        ref = torch.einsum("hqk,hkd->hqd", torch.softmax(sc.masked_fill(~mask, float("-inf")), dim=-1), v[z].float())
+        err = ((out[z].float() - ref).abs().amax(dim=(1, 2)) / ref.abs().amax(dim=(1, 2))).max().item()
+        worst = max(worst, err)
+    assert worst <= 2e-2, f"attention {shape} {elt} causal: worst slice max|err|/max|ref| = {worst:.3e}"
+    for z, h in [(0, 0), (Z - 1, H - 1)]:
+        ref = orc.attention(_host(q[z, h]), _host(k[z, h]), _host(v[z, h]), causal=True, result_type=elt)
+        assert_close(_host(out[z, h]), ref, 2e-2, f"attention {shape} {elt} z={z} h={h} causal, second block per workgroup")
+
+
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("shape", [(2, 3, 256, 128), (1, 2, 333, 128), (1, 2, 512, 32), (1, 2, 200, 96), (1, 1, 384, 160),
                                    (1, 1, 130, 192), (1, 1, 320, 224), (1, 2, 257, 256), (1, 1, 1, 128), (2, 2, 64, 32),
