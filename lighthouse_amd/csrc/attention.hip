@@ -314,6 +314,13 @@ __device__ __forceinline__ void attn_tile(const AttnCtx& c, const AttnArgs& a, c
 // then resident at once as well, and every second round of R workgroups is dealt in reverse (CU c
 // gets ranks c, 2R - 1 - c, 2R + c: heavy + light + what is left, sums within a few tiles of each
 // other instead of the heaviest three against the lightest three).  [8,12,1024]: +3 %.
+// top - L for a round of R workgroups dealt in reverse, but with L's last three bits: workgroup ids
+// that agree modulo 8 share an XCD, and with a multiple of 8 (batch, head) pairs per query block the
+// blocks of a head then stay on one XCD's L2 (ranks move by less than 8 places).
+__device__ __forceinline__ int mirrored_rank(int top, int L, int R) {
+  return R % 8 == 0 ? (((top - L) & ~7) | (L & 7)) : top - L;
+}
+
 __device__ __forceinline__ void causal_block_of(int L, int G, int R, int nqb, int bhn, int& qb, int& bh,
                                                 bool three = false) {
   int r = L;
@@ -322,7 +329,7 @@ __device__ __forceinline__ void causal_block_of(int L, int G, int R, int nqb, in
     if (L < n2) r = R - 1 - L;
     else if (L < R) r = L - n2;
   } else if (three && G > 2 * R && G <= 3 * R && L >= R && L < 2 * R) {
-    r = 3 * R - 1 - L;
+    r = mirrored_rank(3 * R - 1, L, R);
   }
   qb = nqb - 1 - r / bhn;
   bh = r % bhn;
@@ -397,9 +404,9 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
     const int R = chain_s / 3, L = (int)blockIdx.x;
     int r = L;
     if (link == 0) {
-      if (L >= R && L < 2 * R) r = 3 * R - 1 - L;
+      if (L >= R && L < 2 * R) r = mirrored_rank(3 * R - 1, L, R);
     } else {
-      r = (link == 1 && L < R) ? 4 * R - 1 - L : chain_nqb * chain_bhn;
+      r = (link == 1 && L < R) ? mirrored_rank(4 * R - 1, L, R) : chain_nqb * chain_bhn;
     }
     if (r >= chain_nqb * chain_bhn) break;
     qb = chain_nqb - 1 - r / chain_bhn;
