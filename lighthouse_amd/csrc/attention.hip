@@ -46,6 +46,9 @@ struct AttnArgs {
   // three workgroups per CU): the grid is `chain` = 3 x CUs workgroups, all resident, and the first
   // third of them take a second query block each (see attention16_kernel).  0: one block per workgroup.
   int chain = 0;
+  // 64 rows per wave, two workgroups per CU: of every 8 key tiles, the number for which the younger
+  // workgroup's waves hold the higher priority (0: the two take turns tile by tile).
+  int pair_bias = 0;
   bool allow_grid_split = true;  // the caller lets the launch take temporary memory for it
   Scratch* ws = nullptr;         // where that memory comes from: a caller workspace, or (nullptr) the stream's pool
 };
@@ -539,8 +542,18 @@ __global__ void __launch_bounds__(256 * KS, (NQ == 1 && NS == 3 ? 3 : 2)) attent
       // and in opposite phase on the two wave slots, keeps the pair closer together (0.8 % of the
       // launch; 3.5 % before the query blocks of a head shared an XCD).  The 32-row kernels, three
       // workgroups per CU or long causal chains, lost 3-5 % with it.
+      // Even so the older workgroup of every CU ends first ([4,16,2048]: at 58.5 us, its partner at 61.9,
+      // alone for the difference).  Where a launch is a single round of two workgroups per CU the
+      // younger one therefore holds the higher priority for a.pair_bias = 6 of every 8 tiles: 72.2 ->
+      // 70.6 us (7 of 8: 71.4; 3 of 4: 71.1).  Launches of several rounds lose 1-2 % with any such bias
+      // (the slot that frees first takes the next workgroup) and keep the even turns.
       const unsigned slot = __builtin_amdgcn_s_getreg((3u << 11) | (0u << 6) | 4u);  // HW_ID: wave slot within its SIMD
-      if (((unsigned)it ^ slot) & 1u) __builtin_amdgcn_s_setprio(1);
+      unsigned high = ((unsigned)it ^ slot) & 1u;
+      if (a.pair_bias) {
+        const unsigned phase = (unsigned)it & 7u;
+        high = (slot & 1u) ? (phase < (unsigned)a.pair_bias) : (phase >= (unsigned)a.pair_bias);
+      }
+      if (high) __builtin_amdgcn_s_setprio(1);
       else __builtin_amdgcn_s_setprio(0);
     }
     const int jt = t_first + it;
@@ -855,6 +868,11 @@ static int attention16_launch(const AttnArgs& a, hipStream_t s) {
       return attention16_launch_nq<DT, 1, 3>(a, s);
     }
     return attention16_launch_nq<DT, 1, 4>(a, s);
+  }
+  if (!a.causal && groups64 == 2 * (int64_t)a.cus) {  // exactly one round of two workgroups per CU (fewer take the 32-row kernels)
+    AttnArgs ab = a;
+    ab.pair_bias = 6;
+    return attention16_launch_nq<DT, 2, 4>(ab, s);
   }
   return attention16_launch_nq<DT, 2, 4>(a, s);
 }
